@@ -1,0 +1,123 @@
+/*
+ * ornith_hip.h -- C ABI of the MI355X (gfx950) speculative-decode path.
+ *
+ * Every entry point takes plain pointers and sizes, returns an int status
+ * (ORNITH_OK == 0) and never aborts; the message for the last failure on the
+ * calling thread is available from ornith_last_error(). Pointers named d_* are
+ * device pointers obtained from ornith_alloc(); everything else is host memory.
+ * A context owns one HIP stream; all work of a context is ordered on it and a
+ * context must be used from one thread at a time (the reference's Context is
+ * !Send for the same reason, /root/reference/src/metal/mod.rs:433-519).
+ *
+ * Each declaration cites the reference interface it stands in for.
+ */
+#ifndef ORNITH_HIP_H
+#define ORNITH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* exported from the shared library (everything else is hidden) */
+#define ORNITH_API __attribute__((visibility("default")))
+
+#define ORNITH_OK 0
+#define ORNITH_ERR_INVALID 1 /* shape / mode / argument mismatch (the reference asserts) */
+#define ORNITH_ERR_HIP 2     /* a HIP call or kernel launch failed */
+#define ORNITH_ERR_IO 3      /* file could not be read / parsed */
+#define ORNITH_ERR_UNSUPPORTED 4
+
+/* activation / output element types */
+#define ORNITH_F32 0
+#define ORNITH_BF16 1
+
+/* k-quant kinds (src/ops/kquant.rs KQuant) */
+#define ORNITH_Q4K 0
+#define ORNITH_Q6K 1
+
+typedef struct ornith_ctx ornith_ctx;
+
+/* ---- runtime: replaces metal::Context (src/metal/mod.rs:433-519, 521-646, 833-879) */
+ORNITH_API int ornith_ctx_create(int device, ornith_ctx** out);
+ORNITH_API int ornith_ctx_destroy(ornith_ctx* ctx);
+/* Context::sync (src/metal/mod.rs:833-879): block until the stream is idle. */
+ORNITH_API int ornith_sync(ornith_ctx* ctx);
+/* Array::empty / alloc_exact (src/metal/mod.rs:636-646). 256-byte aligned. */
+ORNITH_API int ornith_alloc(ornith_ctx* ctx, size_t bytes, void** d_out);
+ORNITH_API int ornith_free(ornith_ctx* ctx, void* d_ptr);
+/* Array::from_slice / to_vec (src/array.rs:132-197). Both are stream ordered;
+ * download synchronises before returning, upload does not outlive `host`. */
+ORNITH_API int ornith_upload(ornith_ctx* ctx, void* d_dst, const void* host, size_t bytes);
+ORNITH_API int ornith_download(ornith_ctx* ctx, void* host, const void* d_src, size_t bytes);
+ORNITH_API int ornith_memset(ornith_ctx* ctx, void* d_dst, int byte, size_t bytes);
+ORNITH_API int ornith_copy(ornith_ctx* ctx, void* d_dst, const void* d_src, size_t bytes);
+ORNITH_API const char* ornith_last_error(void);
+/* device facts for reports: name into buf, CU count, bytes of device memory */
+ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, int* compute_units,
+                       size_t* total_mem);
+/* Event timing on the context's stream (the reference sums GPUEndTime -
+ * GPUStartTime per command buffer, src/metal/mod.rs:197-285). begin/end record
+ * events; elapsed synchronises on the end event and returns milliseconds. */
+ORNITH_API int ornith_timer_begin(ornith_ctx* ctx);
+ORNITH_API int ornith_timer_end(ornith_ctx* ctx, float* ms_out);
+
+/* ---- k-quant matrices: KMatrix (src/ops/kquant.rs:349-411) ------------------
+ * Three device tensors in the reference's layout:
+ *   Q4_K qs u32[E,O,K/8]     scales u8[E,O,K/256,12]  dm f16[E,O,K/256,2]
+ *   Q6_K qs u32[E,O,3K/16]   scales u8[E,O,K/256,16]  dm f16[E,O,K/256,1]
+ * E == 1 for a plain matrix. */
+typedef struct ornith_kmatrix {
+  int kind; /* ORNITH_Q4K / ORNITH_Q6K */
+  int E, O, K;
+  const void* d_qs;
+  const void* d_scales;
+  const void* d_dm;
+} ornith_kmatrix;
+
+/* KMatrix::check: validates kind, K % 256, and the three byte sizes. */
+ORNITH_API int ornith_kmatrix_check(const ornith_kmatrix* w, size_t qs_bytes, size_t scales_bytes,
+                         size_t dm_bytes);
+
+/* kquant::dequantize (src/ops/kquant.rs:418-433; kernels q4k.metal:64-96,
+ * q6k.metal:47-77): all E*O*K weights to out_dtype. */
+ORNITH_API int ornith_kq_dequantize(ornith_ctx* ctx, const ornith_kmatrix* w, void* d_out, int out_dtype);
+
+/* kquant::qmv (src/ops/kquant.rs:539-595): y[M,O] = x[M,K] . W^T, fp32
+ * accumulate, each row computed exactly as it would be alone. M <= 4 is the
+ * decode/verify shape; larger M loops in groups of four. */
+ORNITH_API int ornith_kq_qmv(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int x_dtype, int M,
+                  void* d_y, int y_dtype);
+
+/* kquant::gather_qmv (src/ops/kquant.rs:741-770): out[r] = x[lhs[r]] . W[rhs[r]]^T,
+ * r < rows; lhs/rhs are device u32 arrays; x has x_rows rows. Indices live on the
+ * device, so they cannot be validated here: an id past the end is clamped to the
+ * last row / expert instead of reading out of bounds. */
+ORNITH_API int ornith_kq_gather_qmv(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int x_dtype,
+                         int x_rows, const uint32_t* d_lhs, const uint32_t* d_rhs, int rows,
+                         void* d_y, int y_dtype);
+
+/* ---- self test ------------------------------------------------------------------
+ * Evaluates one of the library's scalar device functions element-wise (fp32 in,
+ * fp32 out) so their bits can be compared with a CPU evaluation. No reference
+ * counterpart: the reference calls Metal's math library
+ * (kernels/ornith_sigmoid.h:27-31, ornith_logaddexp.h:12-23), whose last bits are not
+ * reproducible off its device; this library carries its own. WAVE_SUM returns, in
+ * every element, the 64-lane butterfly sum of its wavefront (n must be a multiple of 64). */
+#define ORNITH_FN_EXP 0
+#define ORNITH_FN_LOG 1
+#define ORNITH_FN_LOG1P 2
+#define ORNITH_FN_SIGMOID_BF16 3
+#define ORNITH_FN_SIGMOID_F32 4
+#define ORNITH_FN_RSQRT 5
+#define ORNITH_FN_RECIP 6
+#define ORNITH_FN_ROUND_BF16 7
+#define ORNITH_FN_WAVE_SUM 8
+ORNITH_API int ornith_selftest_unary(ornith_ctx* ctx, int fn, const float* d_in, float* d_out, int64_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ORNITH_HIP_H */

@@ -1,0 +1,179 @@
+"""ctypes binding of libornith_hip.so (the C ABI in include/ornith_hip.h).
+
+The directory name is not a Python identifier; import it with
+``importlib.import_module("ornith-rs_amd")`` (tests/conftest.py does).
+
+There is no CPU fallback: if the shared library is missing, loading raises, and
+every operator raises ``OrnithError`` with the library's own message on failure.
+Arrays cross the boundary as raw host buffers (numpy) and opaque device pointers.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libornith_hip.so")
+
+F32, BF16 = 0, 1
+Q4K, Q6K = 0, 1
+KIND_NAMES = {Q4K: "q4k", Q6K: "q6k"}
+
+
+class OrnithError(RuntimeError):
+    pass
+
+
+class KMatrixStruct(C.Structure):
+    _fields_ = [("kind", C.c_int), ("E", C.c_int), ("O", C.c_int), ("K", C.c_int),
+                ("d_qs", C.c_void_p), ("d_scales", C.c_void_p), ("d_dm", C.c_void_p)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OrnithError(
+                f"{LIB_PATH} is missing: build it with `python ornith-rs_amd/build.py` "
+                "(there is no CPU fallback)")
+        _lib = C.CDLL(LIB_PATH)
+        _lib.ornith_last_error.restype = C.c_char_p
+    return _lib
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise OrnithError(f"{what}: [{rc}] {lib().ornith_last_error().decode()}")
+
+
+def _ptr(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+# ---- bf16 helpers on the host (numpy has no bf16; raw uint16 bits) ----------
+def f32_to_bf16(a):
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
+
+
+def bf16_to_f32(b):
+    return (np.ascontiguousarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+class DeviceBuffer:
+    """A device allocation owned by a Ctx."""
+
+    def __init__(self, ctx, nbytes):
+        self.ctx, self.nbytes = ctx, int(nbytes)
+        p = C.c_void_p()
+        _check(lib().ornith_alloc(ctx.h, C.c_size_t(self.nbytes), C.byref(p)), "ornith_alloc")
+        self.ptr = p
+
+    def upload(self, arr):
+        arr = np.ascontiguousarray(arr)
+        assert arr.nbytes <= self.nbytes, (arr.nbytes, self.nbytes)
+        _check(lib().ornith_upload(self.ctx.h, self.ptr, _ptr(arr), C.c_size_t(arr.nbytes)),
+               "ornith_upload")
+        return self
+
+    def download(self, dtype, shape):
+        out = np.empty(shape, dtype=dtype)
+        assert out.nbytes <= self.nbytes, (out.nbytes, self.nbytes)
+        _check(lib().ornith_download(self.ctx.h, _ptr(out), self.ptr, C.c_size_t(out.nbytes)),
+               "ornith_download")
+        return out
+
+    def zero(self):
+        _check(lib().ornith_memset(self.ctx.h, self.ptr, 0, C.c_size_t(self.nbytes)), "ornith_memset")
+        return self
+
+    def free(self):
+        if self.ptr:
+            lib().ornith_free(self.ctx.h, self.ptr)
+            self.ptr = None
+
+
+class KMatrix:
+    """Device-resident k-quant matrix: ops::kquant::KMatrix of the reference."""
+
+    def __init__(self, ctx, kind, qs, scales, dm, E, O, K):
+        self.ctx, self.kind, self.E, self.O, self.K = ctx, kind, E, O, K
+        qs, scales, dm = (np.ascontiguousarray(t) for t in (qs, scales, dm))
+        self.bufs = [ctx.to_device(t) for t in (qs, scales, dm)]
+        self.s = KMatrixStruct(kind, E, O, K, self.bufs[0].ptr, self.bufs[1].ptr, self.bufs[2].ptr)
+        _check(lib().ornith_kmatrix_check(C.byref(self.s), C.c_size_t(qs.nbytes),
+                                          C.c_size_t(scales.nbytes), C.c_size_t(dm.nbytes)),
+               "ornith_kmatrix_check")
+
+    def free(self):
+        for b in self.bufs:
+            b.free()
+
+
+class Ctx:
+    def __init__(self, device=0):
+        h = C.c_void_p()
+        _check(lib().ornith_ctx_create(device, C.byref(h)), "ornith_ctx_create")
+        self.h = h
+
+    def close(self):
+        if self.h:
+            lib().ornith_ctx_destroy(self.h)
+            self.h = None
+
+    def sync(self):
+        _check(lib().ornith_sync(self.h), "ornith_sync")
+
+    def alloc(self, nbytes):
+        return DeviceBuffer(self, nbytes)
+
+    def to_device(self, arr):
+        arr = np.ascontiguousarray(arr)
+        return DeviceBuffer(self, max(arr.nbytes, 1)).upload(arr)
+
+    def device_info(self):
+        name = C.create_string_buffer(256)
+        cus, mem = C.c_int(), C.c_size_t()
+        _check(lib().ornith_device_info(self.h, name, C.c_size_t(256), C.byref(cus), C.byref(mem)),
+               "ornith_device_info")
+        return name.value.decode(), cus.value, mem.value
+
+    def timer_begin(self):
+        _check(lib().ornith_timer_begin(self.h), "ornith_timer_begin")
+
+    def timer_end(self):
+        ms = C.c_float()
+        _check(lib().ornith_timer_end(self.h, C.byref(ms)), "ornith_timer_end")
+        return ms.value
+
+    # ---- ops on device buffers -------------------------------------------
+    def kq_dequantize(self, w, out, out_dtype):
+        _check(lib().ornith_kq_dequantize(self.h, C.byref(w.s), out.ptr, out_dtype), "kq_dequantize")
+
+    def kq_qmv(self, w, x, x_dtype, M, y, y_dtype):
+        _check(lib().ornith_kq_qmv(self.h, C.byref(w.s), x.ptr, x_dtype, M, y.ptr, y_dtype), "kq_qmv")
+
+    def kq_gather_qmv(self, w, x, x_dtype, x_rows, lhs, rhs, rows, y, y_dtype):
+        _check(lib().ornith_kq_gather_qmv(self.h, C.byref(w.s), x.ptr, x_dtype, x_rows, lhs.ptr,
+                                          rhs.ptr, rows, y.ptr, y_dtype), "kq_gather_qmv")
+
+    def selftest_unary(self, fn, x):
+        """Element-wise device scalar function (see ORNITH_FN_* in the header)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        din, dout = self.to_device(x), self.alloc(max(x.nbytes, 4))
+        _check(lib().ornith_selftest_unary(self.h, fn, din.ptr, dout.ptr, C.c_int64(x.size)),
+               "selftest_unary")
+        out = dout.download(np.float32, x.shape)
+        din.free()
+        dout.free()
+        return out
+
+
+FN_EXP, FN_LOG, FN_LOG1P, FN_SIGMOID_BF16, FN_SIGMOID_F32, FN_RSQRT, FN_RECIP, FN_ROUND_BF16, FN_WAVE_SUM = range(9)

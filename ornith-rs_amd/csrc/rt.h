@@ -1,0 +1,45 @@
+// Internal runtime declarations shared by the HIP translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/ornith_hip.h"
+
+struct ornith_ctx {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  int compute_units = 0;
+};
+
+// Records the message for ornith_last_error() and returns `code`.
+int ornith_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define ORN_HIP(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t e__ = (expr);                                                            \
+    if (e__ != hipSuccess)                                                              \
+      return ornith_fail(ORNITH_ERR_HIP, "%s failed: %s (%s:%d)", #expr,                \
+                         hipGetErrorString(e__), __FILE__, __LINE__);                   \
+  } while (0)
+
+#define ORN_REQUIRE(cond, ...)                                  \
+  do {                                                          \
+    if (!(cond)) return ornith_fail(ORNITH_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+// After a kernel launch: report a launch failure (bad grid, missing code object).
+#define ORN_LAUNCH_CHECK(name)                                                         \
+  do {                                                                                  \
+    hipError_t e__ = hipGetLastError();                                                 \
+    if (e__ != hipSuccess)                                                              \
+      return ornith_fail(ORNITH_ERR_HIP, "launch of %s failed: %s", name,               \
+                         hipGetErrorString(e__));                                       \
+  } while (0)
+
+static inline size_t ornith_dtype_size(int dt) { return dt == ORNITH_F32 ? 4 : 2; }

@@ -1,0 +1,132 @@
+// Context, memory and timing: the part of metal::Context
+// (/root/reference/src/metal/mod.rs:433-519) a HIP stream does not already give.
+// A stream orders every kernel after the previous one, so the reference's hazard
+// tracker, barrier epochs and command-buffer batching have no counterpart here.
+#include "rt.h"
+
+static thread_local char g_err[512] = "";
+
+int ornith_fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+extern "C" {
+
+const char* ornith_last_error(void) { return g_err; }
+
+int ornith_ctx_create(int device, ornith_ctx** out) {
+  ORN_REQUIRE(out != nullptr, "ornith_ctx_create: out is null");
+  int n = 0;
+  ORN_HIP(hipGetDeviceCount(&n));
+  ORN_REQUIRE(device >= 0 && device < n, "ornith_ctx_create: device %d of %d", device, n);
+  ORN_HIP(hipSetDevice(device));
+  hipDeviceProp_t prop;
+  ORN_HIP(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return ornith_fail(ORNITH_ERR_UNSUPPORTED,
+                       "ornith_ctx_create: device %d is %s; this library is built for gfx950 only",
+                       device, prop.gcnArchName);
+  ornith_ctx* c = new ornith_ctx();
+  c->device = device;
+  c->compute_units = prop.multiProcessorCount;
+  ORN_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+  ORN_HIP(hipEventCreate(&c->ev0));
+  ORN_HIP(hipEventCreate(&c->ev1));
+  *out = c;
+  return ORNITH_OK;
+}
+
+int ornith_ctx_destroy(ornith_ctx* ctx) {
+  if (!ctx) return ORNITH_OK;
+  (void)hipStreamSynchronize(ctx->stream);
+  (void)hipEventDestroy(ctx->ev0);
+  (void)hipEventDestroy(ctx->ev1);
+  (void)hipStreamDestroy(ctx->stream);
+  delete ctx;
+  return ORNITH_OK;
+}
+
+int ornith_sync(ornith_ctx* ctx) {
+  ORN_REQUIRE(ctx, "ornith_sync: null ctx");
+  ORN_HIP(hipStreamSynchronize(ctx->stream));
+  return ORNITH_OK;
+}
+
+int ornith_alloc(ornith_ctx* ctx, size_t bytes, void** d_out) {
+  ORN_REQUIRE(ctx && d_out, "ornith_alloc: null argument");
+  if (bytes == 0) bytes = 256;
+  ORN_HIP(hipSetDevice(ctx->device));
+  ORN_HIP(hipMalloc(d_out, bytes));
+  return ORNITH_OK;
+}
+
+int ornith_free(ornith_ctx* ctx, void* d_ptr) {
+  ORN_REQUIRE(ctx, "ornith_free: null ctx");
+  if (!d_ptr) return ORNITH_OK;
+  ORN_HIP(hipStreamSynchronize(ctx->stream));
+  ORN_HIP(hipFree(d_ptr));
+  return ORNITH_OK;
+}
+
+int ornith_upload(ornith_ctx* ctx, void* d_dst, const void* host, size_t bytes) {
+  ORN_REQUIRE(ctx && (bytes == 0 || (d_dst && host)), "ornith_upload: null argument");
+  if (bytes == 0) return ORNITH_OK;
+  ORN_HIP(hipMemcpyAsync(d_dst, host, bytes, hipMemcpyHostToDevice, ctx->stream));
+  // pageable source: the copy may still be staging from `host`; wait so the
+  // caller is free to reuse it, which is what the reference's from_slice gives.
+  ORN_HIP(hipStreamSynchronize(ctx->stream));
+  return ORNITH_OK;
+}
+
+int ornith_download(ornith_ctx* ctx, void* host, const void* d_src, size_t bytes) {
+  ORN_REQUIRE(ctx && (bytes == 0 || (d_src && host)), "ornith_download: null argument");
+  if (bytes == 0) return ORNITH_OK;
+  ORN_HIP(hipMemcpyAsync(host, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+  ORN_HIP(hipStreamSynchronize(ctx->stream));
+  return ORNITH_OK;
+}
+
+int ornith_memset(ornith_ctx* ctx, void* d_dst, int byte, size_t bytes) {
+  ORN_REQUIRE(ctx && (bytes == 0 || d_dst), "ornith_memset: null argument");
+  if (bytes == 0) return ORNITH_OK;
+  ORN_HIP(hipMemsetAsync(d_dst, byte, bytes, ctx->stream));
+  return ORNITH_OK;
+}
+
+int ornith_copy(ornith_ctx* ctx, void* d_dst, const void* d_src, size_t bytes) {
+  ORN_REQUIRE(ctx && (bytes == 0 || (d_dst && d_src)), "ornith_copy: null argument");
+  if (bytes == 0) return ORNITH_OK;
+  ORN_HIP(hipMemcpyAsync(d_dst, d_src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+  return ORNITH_OK;
+}
+
+int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, int* compute_units,
+                       size_t* total_mem) {
+  ORN_REQUIRE(ctx, "ornith_device_info: null ctx");
+  hipDeviceProp_t prop;
+  ORN_HIP(hipGetDeviceProperties(&prop, ctx->device));
+  if (name && name_len) snprintf(name, name_len, "%s (%s)", prop.name, prop.gcnArchName);
+  if (compute_units) *compute_units = prop.multiProcessorCount;
+  if (total_mem) *total_mem = prop.totalGlobalMem;
+  return ORNITH_OK;
+}
+
+int ornith_timer_begin(ornith_ctx* ctx) {
+  ORN_REQUIRE(ctx, "ornith_timer_begin: null ctx");
+  ORN_HIP(hipEventRecord(ctx->ev0, ctx->stream));
+  return ORNITH_OK;
+}
+
+int ornith_timer_end(ornith_ctx* ctx, float* ms_out) {
+  ORN_REQUIRE(ctx && ms_out, "ornith_timer_end: null argument");
+  ORN_HIP(hipEventRecord(ctx->ev1, ctx->stream));
+  ORN_HIP(hipEventSynchronize(ctx->ev1));
+  ORN_HIP(hipEventElapsedTime(ms_out, ctx->ev0, ctx->ev1));
+  return ORNITH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,49 @@
+"""The C-ABI library loads and exports every function include/*.h declares (no GPU needed)."""
+import ctypes
+import glob
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions():
+    names = []
+    for h in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(h).read(), flags=re.S)
+        names += re.findall(r"^\s*ORNITH_API\s+(?:const\s+)?(?:int|char\s*\*|void)\s*\*?\s*(ornith_\w+)\s*\(", text, flags=re.M)
+    return sorted(set(names))
+
+
+def test_library_exports_every_declared_symbol():
+    lib_path = os.path.join(ROOT, "ornith-rs_amd", "libornith_hip.so")
+    assert os.path.exists(lib_path), "build it first: python ornith-rs_amd/build.py"
+    lib = ctypes.CDLL(lib_path)
+    names = declared_functions()
+    assert len(names) >= 15
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+
+
+def test_binding_fails_loudly_without_library(orn, monkeypatch):
+    monkeypatch.setattr(orn, "_lib", None)
+    monkeypatch.setattr(orn, "LIB_PATH", "/nonexistent/libornith_hip.so")
+    try:
+        orn.lib()
+    except orn.OrnithError as e:
+        assert "no CPU fallback" in str(e)
+    else:
+        raise AssertionError("missing library did not raise")
+
+
+def test_error_path_reports_message_without_gpu(orn):
+    # argument validation happens before any HIP call
+    rc = orn.lib().ornith_kmatrix_check(None, 0, 0, 0)
+    assert rc == 1
+    assert b"null matrix" in orn.lib().ornith_last_error()
+    s = orn.KMatrixStruct(orn.Q4K, 1, 4, 300, 1, 1, 1)
+    assert orn.lib().ornith_kmatrix_check(ctypes.byref(s), 0, 0, 0) == 1
+    assert b"multiple of 256" in orn.lib().ornith_last_error()
+    s = orn.KMatrixStruct(orn.Q4K, 1, 4, 512, 1, 1, 1)
+    assert orn.lib().ornith_kmatrix_check(ctypes.byref(s), ctypes.c_size_t(4 * 2 * 128), ctypes.c_size_t(4 * 2 * 12), ctypes.c_size_t(4 * 2 * 4)) == 0
+    assert orn.lib().ornith_kmatrix_check(ctypes.byref(s), ctypes.c_size_t(4 * 2 * 128), ctypes.c_size_t(4 * 2 * 16), ctypes.c_size_t(4 * 2 * 4)) == 1
