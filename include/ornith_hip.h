@@ -99,6 +99,66 @@ ORNITH_API int ornith_kq_gather_qmv(ornith_ctx* ctx, const ornith_kmatrix* w, co
                          int x_rows, const uint32_t* d_lhs, const uint32_t* d_rhs, int rows,
                          void* d_y, int y_dtype);
 
+/* ---- Linear: ops::linear::Linear (src/ops/linear.rs:23-28), one polymorphic
+ * projection. Activations in and out are bf16. -------------------------------- */
+#define ORNITH_LIN_KQUANT 0  /* Linear::K(KMatrix) */
+#define ORNITH_LIN_AFFINE8 1 /* Linear::Mlx, mlx affine 8-bit group 64 (quantized.rs:311-333) */
+#define ORNITH_LIN_DENSE 2   /* bf16 [O,K], ops::matmul::gemv (matmul.rs:334-438) */
+typedef struct ornith_linear {
+  int mode;
+  int O, K;
+  ornith_kmatrix km;    /* KQUANT */
+  const void* d_w;      /* AFFINE8: u8[O,K] (the reference's u32[O,K/4] bytes); DENSE: bf16[O,K] */
+  const void* d_scales; /* AFFINE8: bf16[O,K/64] */
+  const void* d_biases; /* AFFINE8: bf16[O,K/64] */
+} ornith_linear;
+
+/* Linear::matmul (src/ops/linear.rs:60-110): y[M,O] = x[M,K] . W^T, bf16 in/out. */
+ORNITH_API int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_x, int M,
+                                    void* d_y);
+
+/* ops::matmul::gather_mv (src/ops/matmul.rs:649-): stacked dense bf16 experts
+ * W[E,O,K]; out[r] = x[lhs[r]] . W[rhs[r]]^T. Used by the MTP head's MoE. */
+ORNITH_API int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K,
+                                      const void* d_x, int x_rows, const uint32_t* d_lhs,
+                                      const uint32_t* d_rhs, int rows, void* d_y);
+
+/* ops::embedding::embedding (src/ops/embedding.rs:18-46): 8-bit affine g64 table
+ * rows -> bf16; ids are device u32, clamped to the table. */
+ORNITH_API int ornith_embedding(ornith_ctx* ctx, const ornith_linear* table, const uint32_t* d_ids,
+                                int n, void* d_out);
+
+/* ---- MoE block -------------------------------------------------------------- */
+/* softmax::softmax(precise) + moe::top_k -> router_top_k (src/ops/moe.rs:113-134,
+ * 688-697; kernels/moe.metal:568-614): gates bf16 [T,E] -> probabilities (bf16) ->
+ * the k winners by (value, then larger index), slots ascending; scores are the
+ * winners' probabilities. d_probs may be null. E % 64 == 0, E <= 1024, k <= 16. */
+ORNITH_API int ornith_router_topk(ornith_ctx* ctx, const void* d_gates, int T, int E, int k,
+                                  uint32_t* d_inds, void* d_scores, void* d_probs);
+
+/* elementwise::swiglu (kernels/ornith_elementwise.metal:97-105), bf16. */
+ORNITH_API int ornith_swiglu(ornith_ctx* ctx, const void* d_gate, const void* d_up, int64_t n,
+                             void* d_out);
+
+/* moe::combine -> moe_combine (src/ops/moe.rs:548-596; kernels/moe.metal:207-258). */
+ORNITH_API int ornith_moe_combine(ornith_ctx* ctx, const void* d_scores, const void* d_y,
+                                  const void* d_gate, const void* d_shared, int T, int k, int dim,
+                                  int normalize, void* d_out);
+
+typedef struct ornith_moe_weights {
+  ornith_linear router;                    /* mlp.gate [E,H] */
+  ornith_kmatrix ex_gate, ex_up, ex_down;  /* mlp.switch_mlp.{gate,up,down}_proj */
+  ornith_linear sh_gate, sh_up, sh_down;   /* mlp.shared_expert.* */
+  ornith_linear sh_egate;                  /* mlp.shared_expert_gate [1,H] */
+  int top_k;
+  int norm_topk_prob;
+} ornith_moe_weights;
+
+/* moe::sparse_moe_block (src/ops/moe.rs:662-741): x bf16 [T,H] -> out bf16 [T,H].
+ * d_inds_out (u32 [T,k]) and d_scores_out (bf16 [T,k]) may be null. T <= 64. */
+ORNITH_API int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                                void* d_out, uint32_t* d_inds_out, void* d_scores_out);
+
 /* ---- self test ------------------------------------------------------------------
  * Evaluates one of the library's scalar device functions element-wise (fp32 in,
  * fp32 out) so their bits can be compared with a CPU evaluation. No reference

@@ -177,3 +177,98 @@ class Ctx:
 
 
 FN_EXP, FN_LOG, FN_LOG1P, FN_SIGMOID_BF16, FN_SIGMOID_F32, FN_RSQRT, FN_RECIP, FN_ROUND_BF16, FN_WAVE_SUM = range(9)
+
+
+# ---- Linear / MoE ---------------------------------------------------------------
+LIN_KQUANT, LIN_AFFINE8, LIN_DENSE = 0, 1, 2
+
+
+class LinearStruct(C.Structure):
+    _fields_ = [("mode", C.c_int), ("O", C.c_int), ("K", C.c_int), ("km", KMatrixStruct),
+                ("d_w", C.c_void_p), ("d_scales", C.c_void_p), ("d_biases", C.c_void_p)]
+
+
+class MoeWeightsStruct(C.Structure):
+    _fields_ = [("router", LinearStruct), ("ex_gate", KMatrixStruct), ("ex_up", KMatrixStruct),
+                ("ex_down", KMatrixStruct), ("sh_gate", LinearStruct), ("sh_up", LinearStruct),
+                ("sh_down", LinearStruct), ("sh_egate", LinearStruct), ("top_k", C.c_int),
+                ("norm_topk_prob", C.c_int)]
+
+
+class Linear:
+    """ops::linear::Linear on the device, from host tensors.
+
+    kquant: Linear.kquant(ctx, kind, qs, scales, dm, O, K)
+    affine: Linear.affine8(ctx, w_u8[O,K], scales_bf16[O,K/64], biases_bf16[O,K/64])
+    dense:  Linear.dense(ctx, w_bf16[O,K])
+    """
+
+    def __init__(self, s, keep):
+        self.s, self.keep = s, keep
+
+    @staticmethod
+    def kquant(ctx, kind, qs, scales, dm, O, K):
+        km = KMatrix(ctx, kind, qs, scales, dm, 1, O, K)
+        return Linear(LinearStruct(LIN_KQUANT, O, K, km.s, None, None, None), [km])
+
+    @staticmethod
+    def affine8(ctx, w, scales, biases):
+        O, K = w.shape
+        bufs = [ctx.to_device(t) for t in (w, scales, biases)]
+        return Linear(LinearStruct(LIN_AFFINE8, O, K, KMatrixStruct(), bufs[0].ptr, bufs[1].ptr,
+                                   bufs[2].ptr), bufs)
+
+    @staticmethod
+    def dense(ctx, w):
+        O, K = w.shape
+        buf = ctx.to_device(w)
+        return Linear(LinearStruct(LIN_DENSE, O, K, KMatrixStruct(), buf.ptr, None, None), [buf])
+
+    def free(self):
+        for b in self.keep:
+            b.free()
+
+
+def _ctx_method(fn):
+    setattr(Ctx, fn.__name__, fn)
+    return fn
+
+
+@_ctx_method
+def linear_matmul(self, lin, x, M, y):
+    _check(lib().ornith_linear_matmul(self.h, C.byref(lin.s), x.ptr, M, y.ptr), "linear_matmul")
+
+
+@_ctx_method
+def dense_gather_mv(self, w, E, O, K, x, x_rows, lhs, rhs, rows, y):
+    _check(lib().ornith_dense_gather_mv(self.h, w.ptr, E, O, K, x.ptr, x_rows, lhs.ptr, rhs.ptr,
+                                        rows, y.ptr), "dense_gather_mv")
+
+
+@_ctx_method
+def embedding(self, table, ids, n, out):
+    _check(lib().ornith_embedding(self.h, C.byref(table.s), ids.ptr, n, out.ptr), "embedding")
+
+
+@_ctx_method
+def router_topk(self, gates, T, E, k, inds, scores, probs=None):
+    _check(lib().ornith_router_topk(self.h, gates.ptr, T, E, k, inds.ptr, scores.ptr,
+                                    probs.ptr if probs else None), "router_topk")
+
+
+@_ctx_method
+def swiglu(self, gate, up, n, out):
+    _check(lib().ornith_swiglu(self.h, gate.ptr, up.ptr, C.c_int64(n), out.ptr), "swiglu")
+
+
+@_ctx_method
+def moe_combine(self, scores, y, gate, shared, T, k, dim, normalize, out):
+    _check(lib().ornith_moe_combine(self.h, scores.ptr, y.ptr, gate.ptr, shared.ptr, T, k, dim,
+                                    int(normalize), out.ptr), "moe_combine")
+
+
+@_ctx_method
+def moe_block(self, w, x, T, out, inds=None, scores=None):
+    _check(lib().ornith_moe_block(self.h, C.byref(w), x.ptr, T, out.ptr,
+                                  inds.ptr if inds else None, scores.ptr if scores else None),
+           "moe_block")

@@ -266,7 +266,7 @@ struct LaneOf<ORNITH_Q6K, M> {
 };
 
 // One kernel for plain and gathered mat-vecs.
-//   KIND  format; LPR lanes per row (8,16,32,64); KS wavefronts per row (1,2)
+//   KIND  format; LPR lanes per row (4,8,16,32,64); KS wavefronts per row (1,2)
 //   M     activation rows sharing each weight read (1..4); gather uses M == 1
 //   grid.x covers output rows, grid.y is the gather row (1 for plain)
 template <int KIND, int LPR, int KS, int M, bool XF32, bool GATHER>
@@ -416,6 +416,7 @@ template <int KIND, int M, bool XF32, bool GATHER>
 int launch_shape(ornith_ctx* ctx, const KqArgs& a, int grid_y) {
   const int nch = (a.K >> 8) * (KIND == ORNITH_Q4K ? 8 : 4);
   switch (nch) {
+    case 4: return launch_one<KIND, 4, 1, M, XF32, GATHER>(ctx, a, grid_y);
     case 8: return launch_one<KIND, 8, 1, M, XF32, GATHER>(ctx, a, grid_y);
     case 16: return launch_one<KIND, 16, 1, M, XF32, GATHER>(ctx, a, grid_y);
     case 32: return launch_one<KIND, 32, 1, M, XF32, GATHER>(ctx, a, grid_y);
@@ -424,7 +425,7 @@ int launch_shape(ornith_ctx* ctx, const KqArgs& a, int grid_y) {
     default:
       return ornith_fail(ORNITH_ERR_UNSUPPORTED,
                          "k-quant mat-vec: K=%d is not one of the supported widths "
-                         "(Q4_K: 256,512,1024,2048,4096; Q6_K: 512,1024,2048,4096,8192)",
+                         "(Q4_K: 256,512,1024,2048,4096; Q6_K: 256,512,1024,2048,4096,8192)",
                          a.K);
   }
 }

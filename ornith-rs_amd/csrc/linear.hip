@@ -1,0 +1,166 @@
+// The non-k-quant projections and the polymorphic Linear.
+//
+// Replaces Linear::matmul (/root/reference/src/ops/linear.rs:23-110), the 8-bit
+// affine mat-vec `affine_qmv_fast` (/root/reference/src/ops/quantized.rs:311-333,
+// vendored quantized.h:283-289,756-821), the dense bf16 mat-vec and its gathered
+// form (/root/reference/src/ops/matmul.rs:334-438,649-) and the embedding lookup
+// (/root/reference/src/ops/embedding.rs:18-46).
+//
+// All are one wavefront per output row: lane l owns the 8-element chunks
+// j = l + 64c in ascending c, accumulates them in fp32 and the 64 lane sums go
+// through the butterfly. These matrices are small (router-sized or the MTP
+// head), so the layout favours a fixed summation order over tuning.
+#include "dmath.h"
+#include "rt.h"
+
+namespace {
+
+// ---- 8-bit affine, group 64 ---------------------------------------------
+__global__ __launch_bounds__(64) void affine8_qmv_kernel(const uint8_t* w, const bf16_t* scales,
+                                                         const bf16_t* biases, const bf16_t* x,
+                                                         bf16_t* y, int O, int K) {
+  const int o = blockIdx.x, m = blockIdx.y, lane = threadIdx.x;
+  const uint8_t* wr = w + (size_t)o * K;
+  const bf16_t* sr = scales + (size_t)o * (K / 64);
+  const bf16_t* br = biases + (size_t)o * (K / 64);
+  const bf16_t* xr = x + (size_t)m * K;
+  float acc_lane = 0.f;
+  for (int j = lane; j < K / 8; j += 64) {
+    const uint2 q = *reinterpret_cast<const uint2*>(wr + 8 * j);
+    const uint4 xv = *reinterpret_cast<const uint4*>(xr + 8 * j);
+    const float xs[8] = {dm_bf2f_lo(xv.x), dm_bf2f_hi(xv.x), dm_bf2f_lo(xv.y), dm_bf2f_hi(xv.y),
+                         dm_bf2f_lo(xv.z), dm_bf2f_hi(xv.z), dm_bf2f_lo(xv.w), dm_bf2f_hi(xv.w)};
+    const uint32_t qw[2] = {q.x, q.y};
+    float acc = 0.f, sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float qf = (float)((qw[i >> 2] >> (8 * (i & 3))) & 0xffu);
+      acc = dm_fma(xs[i], qf, acc);
+      sum = sum + xs[i];
+    }
+    const float s = dm_bf2f(sr[j >> 3]), b = dm_bf2f(br[j >> 3]);
+    float p = s * acc;
+    p = dm_fma(sum, b, p);
+    acc_lane = acc_lane + p;
+  }
+  const float v = dm_wave_sum<64>(acc_lane);
+  if (lane == 0) y[(size_t)m * O + o] = dm_f2bf(v);
+}
+
+// ---- dense bf16 ------------------------------------------------------------
+// grid.x covers rows four at a time (one per wavefront), grid.y is the
+// activation row; GATHER selects expert / activation row through lhs, rhs.
+template <bool GATHER>
+__global__ __launch_bounds__(256) void dense_gemv_kernel(const bf16_t* w, const bf16_t* x,
+                                                         bf16_t* y, int O, int K, int E, int x_rows,
+                                                         const uint32_t* lhs, const uint32_t* rhs) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int o = blockIdx.x * 4 + wave;
+  if (o >= O) return;
+  const int r = blockIdx.y;
+  const bf16_t* wr;
+  const bf16_t* xr;
+  if constexpr (GATHER) {
+    const uint32_t xi = min(lhs[r], (uint32_t)(x_rows - 1));
+    const uint32_t ei = min(rhs[r], (uint32_t)(E - 1));
+    wr = w + ((size_t)ei * O + o) * K;
+    xr = x + (size_t)xi * K;
+  } else {
+    wr = w + (size_t)o * K;
+    xr = x + (size_t)r * K;
+  }
+  float a = 0.f;
+  for (int j = lane; j < K / 8; j += 64) {
+    const uint4 wv = *reinterpret_cast<const uint4*>(wr + 8 * j);
+    const uint4 xv = *reinterpret_cast<const uint4*>(xr + 8 * j);
+    a = dm_fma(dm_bf2f_lo(wv.x), dm_bf2f_lo(xv.x), a);
+    a = dm_fma(dm_bf2f_hi(wv.x), dm_bf2f_hi(xv.x), a);
+    a = dm_fma(dm_bf2f_lo(wv.y), dm_bf2f_lo(xv.y), a);
+    a = dm_fma(dm_bf2f_hi(wv.y), dm_bf2f_hi(xv.y), a);
+    a = dm_fma(dm_bf2f_lo(wv.z), dm_bf2f_lo(xv.z), a);
+    a = dm_fma(dm_bf2f_hi(wv.z), dm_bf2f_hi(xv.z), a);
+    a = dm_fma(dm_bf2f_lo(wv.w), dm_bf2f_lo(xv.w), a);
+    a = dm_fma(dm_bf2f_hi(wv.w), dm_bf2f_hi(xv.w), a);
+  }
+  const float v = dm_wave_sum<64>(a);
+  if (lane == 0) y[(size_t)r * O + o] = dm_f2bf(v);
+}
+
+// ---- embedding: out = bf16(bf16(q * scale) + bias) ------------------------------
+__global__ void embedding_kernel(const uint8_t* w, const bf16_t* scales, const bf16_t* biases,
+                                 const uint32_t* ids, bf16_t* out, int V, int K) {
+  const int r = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= K) return;
+  const size_t row = min(ids[r], (uint32_t)(V - 1));
+  const float s = dm_bf2f(scales[row * (K / 64) + i / 64]);
+  const float b = dm_bf2f(biases[row * (K / 64) + i / 64]);
+  const float v = dm_rb((float)w[row * K + i] * s);
+  out[(size_t)r * K + i] = dm_f2bf(v + b);
+}
+
+}  // namespace
+
+extern "C" {
+
+int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_x, int M,
+                         void* d_y) {
+  ORN_REQUIRE(ctx && w && d_x && d_y, "linear_matmul: null argument");
+  ORN_REQUIRE(M >= 1, "linear_matmul: M=%d", M);
+  switch (w->mode) {
+    case ORNITH_LIN_KQUANT:
+      ORN_REQUIRE(w->km.O == w->O && w->km.K == w->K, "linear_matmul: k-quant dims disagree");
+      return ornith_kq_qmv(ctx, &w->km, d_x, ORNITH_BF16, M, d_y, ORNITH_BF16);
+    case ORNITH_LIN_AFFINE8:
+      ORN_REQUIRE(w->d_w && w->d_scales && w->d_biases, "linear_matmul: affine tensor missing");
+      ORN_REQUIRE(w->K % 64 == 0 && w->O >= 1 && M <= 65535, "linear_matmul: affine O=%d K=%d",
+                  w->O, w->K);
+      hipLaunchKernelGGL(affine8_qmv_kernel, dim3(w->O, M), dim3(64), 0, ctx->stream,
+                         (const uint8_t*)w->d_w, (const bf16_t*)w->d_scales,
+                         (const bf16_t*)w->d_biases, (const bf16_t*)d_x, (bf16_t*)d_y, w->O, w->K);
+      ORN_LAUNCH_CHECK("affine8_qmv_kernel");
+      return ORNITH_OK;
+    case ORNITH_LIN_DENSE:
+      ORN_REQUIRE(w->d_w, "linear_matmul: dense weight missing");
+      ORN_REQUIRE(w->K % 8 == 0 && w->O >= 1 && M <= 65535, "linear_matmul: dense O=%d K=%d", w->O,
+                  w->K);
+      hipLaunchKernelGGL(dense_gemv_kernel<false>, dim3((w->O + 3) / 4, M), dim3(256), 0,
+                         ctx->stream, (const bf16_t*)w->d_w, (const bf16_t*)d_x, (bf16_t*)d_y, w->O,
+                         w->K, 1, M, nullptr, nullptr);
+      ORN_LAUNCH_CHECK("dense_gemv_kernel");
+      return ORNITH_OK;
+    default:
+      return ornith_fail(ORNITH_ERR_INVALID, "linear_matmul: unknown mode %d", w->mode);
+  }
+}
+
+int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K, const void* d_x,
+                           int x_rows, const uint32_t* d_lhs, const uint32_t* d_rhs, int rows,
+                           void* d_y) {
+  ORN_REQUIRE(ctx && d_w && d_x && d_lhs && d_rhs && d_y, "dense_gather_mv: null argument");
+  ORN_REQUIRE(E >= 1 && O >= 1 && K % 8 == 0 && x_rows >= 1 && rows >= 0 && rows <= 65535,
+              "dense_gather_mv: E=%d O=%d K=%d rows=%d", E, O, K, rows);
+  if (rows == 0) return ORNITH_OK;
+  hipLaunchKernelGGL(dense_gemv_kernel<true>, dim3((O + 3) / 4, rows), dim3(256), 0, ctx->stream,
+                     (const bf16_t*)d_w, (const bf16_t*)d_x, (bf16_t*)d_y, O, K, E, x_rows, d_lhs,
+                     d_rhs);
+  ORN_LAUNCH_CHECK("dense_gemv_kernel<gather>");
+  return ORNITH_OK;
+}
+
+int ornith_embedding(ornith_ctx* ctx, const ornith_linear* table, const uint32_t* d_ids, int n,
+                     void* d_out) {
+  ORN_REQUIRE(ctx && table && d_ids && d_out, "embedding: null argument");
+  ORN_REQUIRE(table->mode == ORNITH_LIN_AFFINE8,
+              "embedding: table mode %d; the lookup is defined for the 8-bit affine table only",
+              table->mode);
+  ORN_REQUIRE(table->K % 64 == 0 && n >= 0 && n <= 65535, "embedding: K=%d n=%d", table->K, n);
+  if (n == 0) return ORNITH_OK;
+  hipLaunchKernelGGL(embedding_kernel, dim3((table->K + 255) / 256, n), dim3(256), 0, ctx->stream,
+                     (const uint8_t*)table->d_w, (const bf16_t*)table->d_scales,
+                     (const bf16_t*)table->d_biases, d_ids, (bf16_t*)d_out, table->O, table->K);
+  ORN_LAUNCH_CHECK("embedding_kernel");
+  return ORNITH_OK;
+}
+
+}  // extern "C"

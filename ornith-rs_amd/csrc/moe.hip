@@ -1,0 +1,250 @@
+// The sparse MoE block: router softmax + top-k, expert FFNs, shared expert, tail.
+//
+// Replaces moe::sparse_moe_block and its helpers
+// (/root/reference/src/ops/moe.rs:113-134,256-338,548-596,662-741) and the
+// kernels router_top_k / moe_combine / swiglu
+// (/root/reference/kernels/moe.metal:207-258,568-614,
+//  /root/reference/kernels/ornith_elementwise.metal:97-105) and the vendored
+// precise softmax (softmax.h:10-98).
+//
+// Rounding points are the reference's: gates, probabilities, every expert output
+// and every step of the tail are bf16; sums inside a kernel are fp32.
+#include "dmath.h"
+#include "rt.h"
+
+namespace {
+
+// One wavefront per token. Lane l holds gates [l*PER, (l+1)*PER).
+//   softmax: fp32 max, e = exp(g - max), lane-sequential sum then butterfly,
+//            p = bf16(e * (1/sum))
+//   top-k:   k rounds of (value, then larger index) selection; round r -> slot k-1-r
+// Also writes the gather index lists the expert mat-vecs use:
+//   lhs_tok[t*k+j] = t (row of x), lhs_row[t*k+j] = t*k+j (row of act).
+template <int PER>
+__global__ __launch_bounds__(64) void router_topk_kernel(const bf16_t* gates, int E, int k,
+                                                         uint32_t* inds, bf16_t* scores,
+                                                         bf16_t* probs, uint32_t* lhs_tok,
+                                                         uint32_t* lhs_row) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const bf16_t* g = gates + (size_t)t * E + lane * PER;
+  float v[PER];
+  float m = -DM_INF;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    v[i] = dm_bf2f(g[i]);
+    m = v[i] > m ? v[i] : m;
+  }
+  m = dm_wave_max<64>(m);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    v[i] = dm_exp(v[i] - m);
+    s = s + v[i];
+  }
+  const float inv = 1.0f / dm_wave_sum<64>(s);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const bf16_t pb = dm_f2bf(v[i] * inv);
+    if (probs) probs[(size_t)t * E + lane * PER + i] = pb;
+    v[i] = dm_bf2f(pb);
+  }
+  for (int r = 0; r < k; ++r) {
+    float best = -DM_INF;
+    int besti = -1;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      // ascending i, so >= keeps the larger index among equals
+      if (v[i] >= best && !(v[i] != v[i])) {
+        if (v[i] > best || besti < lane * PER + i) {
+          best = v[i];
+          besti = lane * PER + i;
+        }
+      }
+    }
+    const float wm = dm_wave_max<64>(best);
+    int cand = (best == wm) ? besti : -1;
+#pragma unroll
+    for (int sft = 32; sft >= 1; sft >>= 1) {
+      const int o = __shfl_xor(cand, sft, 64);
+      cand = o > cand ? o : cand;
+    }
+    // cand: the winning expert, identical in every lane (never -1: probabilities are
+    // finite and at most k <= E entries are ever removed)
+    const int owner = cand / PER;
+    float wv = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      if (lane == owner && i == cand - owner * PER) {
+        wv = v[i];
+        v[i] = -DM_INF;
+      }
+    }
+    if (lane == owner) {
+      const size_t slot = (size_t)t * k + (k - 1 - r);
+      inds[slot] = (uint32_t)cand;
+      scores[slot] = dm_f2bf(wv);  // already a bf16 value
+    }
+  }
+  if (lane < k) {
+    if (lhs_tok) lhs_tok[t * k + lane] = t;
+    if (lhs_row) lhs_row[t * k + lane] = t * k + lane;
+  }
+}
+
+__global__ void swiglu_kernel(const bf16_t* gate, const bf16_t* up, bf16_t* out, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float g = dm_bf2f(gate[i]);
+  const float s = dm_rb(g * dm_sigmoid_bf16(g));
+  out[i] = dm_f2bf(s * dm_bf2f(up[i]));
+}
+
+// one thread per output element; j ascends, every step rounds to bf16
+__global__ void moe_combine_kernel(const bf16_t* scores, const bf16_t* y, const bf16_t* gate,
+                                   const bf16_t* shared, bf16_t* out, int T, int k, int dim,
+                                   int normalize) {
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)T * dim) return;
+  const int t = (int)(idx / dim), c = (int)(idx - (int64_t)t * dim);
+  const bf16_t* s = scores + (size_t)t * k;
+  float denom = 0.f;
+  if (normalize)
+    for (int j = 0; j < k; ++j) denom = dm_rb(dm_bf2f(s[j]) + denom);
+  float acc = 0.f;
+  for (int j = 0; j < k; ++j) {
+    const float w = normalize ? dm_rb(dm_bf2f(s[j]) / denom) : dm_bf2f(s[j]);
+    const float weighted = dm_rb(dm_bf2f(y[((size_t)t * k + j) * dim + c]) * w);
+    acc = dm_rb(weighted + acc);
+  }
+  const float g = dm_sigmoid_bf16(dm_bf2f(gate[t]));
+  const float gated = dm_rb(g * dm_bf2f(shared[idx]));
+  out[idx] = dm_f2bf(acc + gated);
+}
+
+int launch_router(ornith_ctx* ctx, const bf16_t* gates, int T, int E, int k, uint32_t* inds,
+                  bf16_t* scores, bf16_t* probs, uint32_t* lhs_tok, uint32_t* lhs_row) {
+#define ROUTER_CASE(P)                                                                       \
+  case P:                                                                                    \
+    hipLaunchKernelGGL(router_topk_kernel<P>, dim3(T), dim3(64), 0, ctx->stream, gates, E, k, \
+                       inds, scores, probs, lhs_tok, lhs_row);                               \
+    break;
+  switch (E / 64) {
+    ROUTER_CASE(1)
+    ROUTER_CASE(2)
+    ROUTER_CASE(4)
+    ROUTER_CASE(8)
+    ROUTER_CASE(16)
+    default:
+      return ornith_fail(ORNITH_ERR_UNSUPPORTED, "router_topk: E=%d (need 64,128,256,512,1024)", E);
+  }
+#undef ROUTER_CASE
+  ORN_LAUNCH_CHECK("router_topk_kernel");
+  return ORNITH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ornith_router_topk(ornith_ctx* ctx, const void* d_gates, int T, int E, int k, uint32_t* d_inds,
+                       void* d_scores, void* d_probs) {
+  ORN_REQUIRE(ctx && d_gates && d_inds && d_scores, "router_topk: null argument");
+  ORN_REQUIRE(T >= 1 && E % 64 == 0 && k >= 1 && k <= 16 && k <= E, "router_topk: T=%d E=%d k=%d",
+              T, E, k);
+  return launch_router(ctx, (const bf16_t*)d_gates, T, E, k, d_inds, (bf16_t*)d_scores,
+                       (bf16_t*)d_probs, nullptr, nullptr);
+}
+
+int ornith_swiglu(ornith_ctx* ctx, const void* d_gate, const void* d_up, int64_t n, void* d_out) {
+  ORN_REQUIRE(ctx && d_gate && d_up && d_out && n >= 0, "swiglu: bad argument");
+  if (n == 0) return ORNITH_OK;
+  hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream,
+                     (const bf16_t*)d_gate, (const bf16_t*)d_up, (bf16_t*)d_out, n);
+  ORN_LAUNCH_CHECK("swiglu_kernel");
+  return ORNITH_OK;
+}
+
+int ornith_moe_combine(ornith_ctx* ctx, const void* d_scores, const void* d_y, const void* d_gate,
+                       const void* d_shared, int T, int k, int dim, int normalize, void* d_out) {
+  ORN_REQUIRE(ctx && d_scores && d_y && d_gate && d_shared && d_out, "moe_combine: null argument");
+  ORN_REQUIRE(T >= 1 && k >= 1 && dim >= 1, "moe_combine: T=%d k=%d dim=%d", T, k, dim);
+  const int64_t n = (int64_t)T * dim;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     ctx->stream, (const bf16_t*)d_scores, (const bf16_t*)d_y,
+                     (const bf16_t*)d_gate, (const bf16_t*)d_shared, (bf16_t*)d_out, T, k, dim,
+                     normalize);
+  ORN_LAUNCH_CHECK("moe_combine_kernel");
+  return ORNITH_OK;
+}
+
+int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                     void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
+  ORN_REQUIRE(ctx && w && d_x && d_out, "moe_block: null argument");
+  const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
+  ORN_REQUIRE(T >= 1 && T <= 64, "moe_block: T=%d (decode/verify widths only)", T);
+  ORN_REQUIRE(k >= 1 && k <= 16 && k <= E, "moe_block: top_k=%d of %d", k, E);
+  ORN_REQUIRE(w->ex_gate.E == E && w->ex_up.E == E && w->ex_down.E == E,
+              "moe_block: expert tensors carry %d/%d/%d experts, router has %d", w->ex_gate.E,
+              w->ex_up.E, w->ex_down.E, E);
+  ORN_REQUIRE(w->ex_gate.K == H && w->ex_up.K == H && w->ex_up.O == I && w->ex_down.K == I &&
+                  w->ex_down.O == H,
+              "moe_block: expert shapes do not chain (H=%d I=%d)", H, I);
+  ORN_REQUIRE(w->sh_gate.K == H && w->sh_up.K == H && w->sh_up.O == w->sh_gate.O &&
+                  w->sh_down.K == w->sh_gate.O && w->sh_down.O == H && w->sh_egate.K == H &&
+                  w->sh_egate.O == 1,
+              "moe_block: shared expert shapes do not chain");
+  const int SI = w->sh_gate.O;
+
+  const size_t need = 2 * ((size_t)T * E * 2 + (size_t)T * SI * 3 + (size_t)T * H + T +
+                           (size_t)T * k * (2 * I + I + H + 1)) +
+                      4 * (size_t)T * k * 3 + 64 * 256;
+  void* base = nullptr;
+  int rc = ornith_scratch(ctx, need, &base);
+  if (rc) return rc;
+  ScratchCursor sc(base);
+  bf16_t* gates = sc.take<bf16_t>((size_t)T * E);
+  uint32_t* inds = sc.take<uint32_t>((size_t)T * k);
+  bf16_t* scores = sc.take<bf16_t>((size_t)T * k);
+  uint32_t* lhs_tok = sc.take<uint32_t>((size_t)T * k);
+  uint32_t* lhs_row = sc.take<uint32_t>((size_t)T * k);
+  bf16_t* sg = sc.take<bf16_t>((size_t)T * SI);
+  bf16_t* su = sc.take<bf16_t>((size_t)T * SI);
+  bf16_t* sact = sc.take<bf16_t>((size_t)T * SI);
+  bf16_t* sy = sc.take<bf16_t>((size_t)T * H);
+  bf16_t* eg = sc.take<bf16_t>((size_t)T);
+  bf16_t* xg = sc.take<bf16_t>((size_t)T * k * I);
+  bf16_t* xu = sc.take<bf16_t>((size_t)T * k * I);
+  bf16_t* act = sc.take<bf16_t>((size_t)T * k * I);
+  bf16_t* y = sc.take<bf16_t>((size_t)T * k * H);
+
+#define TRY(e)          \
+  do {                  \
+    rc = (e);           \
+    if (rc) return rc;  \
+  } while (0)
+  TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
+  TRY(ornith_linear_matmul(ctx, &w->sh_gate, d_x, T, sg));
+  TRY(ornith_linear_matmul(ctx, &w->sh_up, d_x, T, su));
+  TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
+  TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, lhs_tok, lhs_row));
+  TRY(ornith_swiglu(ctx, sg, su, (int64_t)T * SI, sact));
+  TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
+  TRY(ornith_kq_gather_qmv(ctx, &w->ex_gate, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xg,
+                           ORNITH_BF16));
+  TRY(ornith_kq_gather_qmv(ctx, &w->ex_up, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xu,
+                           ORNITH_BF16));
+  TRY(ornith_swiglu(ctx, xg, xu, (int64_t)T * k * I, act));
+  TRY(ornith_kq_gather_qmv(ctx, &w->ex_down, act, ORNITH_BF16, T * k, lhs_row, inds, T * k, y,
+                           ORNITH_BF16));
+  TRY(ornith_moe_combine(ctx, scores, y, eg, sy, T, k, H, w->norm_topk_prob, d_out));
+  if (d_inds_out)
+    ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,
+                           ctx->stream));
+  if (d_scores_out)
+    ORN_HIP(hipMemcpyAsync(d_scores_out, scores, 2 * (size_t)T * k, hipMemcpyDeviceToDevice,
+                           ctx->stream));
+#undef TRY
+  return ORNITH_OK;
+}
+
+}  // extern "C"

@@ -15,6 +15,27 @@ struct ornith_ctx {
   hipStream_t stream = nullptr;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   int compute_units = 0;
+  // grow-only scratch for operators that need temporaries between their kernels;
+  // stream order makes reuse by the next operator safe.
+  void* scratch = nullptr;
+  size_t scratch_cap = 0;
+};
+
+// Returns at least `bytes` of device scratch (256-byte aligned). Growing it
+// synchronises the stream; callers that must not allocate size it once up front.
+int ornith_scratch(ornith_ctx* ctx, size_t bytes, void** out);
+
+// bump allocator over a scratch block
+struct ScratchCursor {
+  char* base;
+  size_t off = 0;
+  explicit ScratchCursor(void* p) : base(static_cast<char*>(p)) {}
+  template <typename T>
+  T* take(size_t count) {
+    T* r = reinterpret_cast<T*>(base + off);
+    off += (count * sizeof(T) + 255) & ~size_t(255);
+    return r;
+  }
 };
 
 // Records the message for ornith_last_error() and returns `code`.

@@ -14,6 +14,20 @@ int ornith_fail(int code, const char* fmt, ...) {
   return code;
 }
 
+int ornith_scratch(ornith_ctx* ctx, size_t bytes, void** out) {
+  if (bytes > ctx->scratch_cap) {
+    ORN_HIP(hipStreamSynchronize(ctx->stream));
+    if (ctx->scratch) ORN_HIP(hipFree(ctx->scratch));
+    ctx->scratch = nullptr;
+    ctx->scratch_cap = 0;
+    size_t cap = (bytes + (size_t(1) << 20) - 1) & ~((size_t(1) << 20) - 1);
+    ORN_HIP(hipMalloc(&ctx->scratch, cap));
+    ctx->scratch_cap = cap;
+  }
+  *out = ctx->scratch;
+  return ORNITH_OK;
+}
+
 extern "C" {
 
 const char* ornith_last_error(void) { return g_err; }
@@ -43,6 +57,7 @@ int ornith_ctx_create(int device, ornith_ctx** out) {
 int ornith_ctx_destroy(ornith_ctx* ctx) {
   if (!ctx) return ORNITH_OK;
   (void)hipStreamSynchronize(ctx->stream);
+  if (ctx->scratch) (void)hipFree(ctx->scratch);
   (void)hipEventDestroy(ctx->ev0);
   (void)hipEventDestroy(ctx->ev1);
   (void)hipStreamDestroy(ctx->stream);

@@ -69,7 +69,7 @@ def test_dequantize_bit_exact(orn, ctx, kind):
 
 
 SHAPES = [(Q4K, 2048, 512), (Q4K, 512, 96), (Q4K, 4096, 200), (Q4K, 1024, 64), (Q4K, 256, 40),
-          (Q6K, 2048, 256), (Q6K, 512, 2048), (Q6K, 4096, 130), (Q6K, 1024, 64), (Q6K, 8192, 32)]
+          (Q6K, 2048, 256), (Q6K, 512, 2048), (Q6K, 4096, 130), (Q6K, 1024, 64), (Q6K, 8192, 32), (Q6K, 256, 24)]
 
 
 @pytest.mark.parametrize("kind,K,O", SHAPES)

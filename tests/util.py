@@ -144,3 +144,135 @@ def global_rel(got, want):
     got = np.asarray(got, dtype=np.float64)
     want = np.asarray(want, dtype=np.float64)
     return float(np.max(np.abs(got - want)) / max(np.max(np.abs(want)), 1e-300))
+
+
+# ---- host-side model pieces: numpy tensors that feed both the oracle and the device ----
+class OrcKmat(C.Structure):
+    _fields_ = [("kind", C.c_int), ("E", C.c_int), ("O", C.c_int), ("K", C.c_int),
+                ("qs", C.c_void_p), ("scales", C.c_void_p), ("dm", C.c_void_p)]
+
+
+class OrcLinear(C.Structure):
+    _fields_ = [("mode", C.c_int), ("km", OrcKmat), ("aw", C.c_void_p), ("as_", C.c_void_p),
+                ("ab", C.c_void_p)]
+
+
+class OrcMoeWeights(C.Structure):
+    _fields_ = [("router", OrcLinear), ("ex_gate", OrcKmat), ("ex_up", OrcKmat), ("ex_down", OrcKmat),
+                ("sh_gate", OrcLinear), ("sh_up", OrcLinear), ("sh_down", OrcLinear),
+                ("sh_egate", OrcLinear), ("top_k", C.c_int), ("normalize", C.c_int)]
+
+
+def unit_sigma(kind, K):
+    """d-sigma that gives ~unit-variance outputs for N(0,1) inputs with centred weights."""
+    return 1.0 / ((168.3 if kind == Q4K else 682.9) * np.sqrt(K))
+
+
+class HostKMat:
+    def __init__(self, kind, E, O, K, tensors):
+        self.kind, self.E, self.O, self.K = kind, E, O, K
+        self.qs, self.scales, self.dm = (np.ascontiguousarray(t) for t in tensors)
+
+    @staticmethod
+    def random(rng, kind, E, O, K, sigma=None):
+        sigma = unit_sigma(kind, K) if sigma is None else sigma
+        t = make_q4k(rng, E, O, K, d_sigma=sigma, centered=True) if kind == Q4K else make_q6k(rng, E, O, K, d_sigma=sigma)
+        return HostKMat(kind, E, O, K, t)
+
+    def orc(self):
+        return OrcKmat(self.kind, self.E, self.O, self.K, p(self.qs), p(self.scales), p(self.dm))
+
+    def dev(self, orn, ctx):
+        return orn.KMatrix(ctx, self.kind, self.qs, self.scales, self.dm, self.E, self.O, self.K)
+
+    def nbytes(self):
+        return self.qs.nbytes + self.scales.nbytes + self.dm.nbytes
+
+
+class HostLinear:
+    """mode: 'kq' (HostKMat), 'affine8' (w u8, scales bf16, biases bf16), 'dense' (w bf16)."""
+
+    def __init__(self, mode, O, K, km=None, w=None, scales=None, biases=None):
+        self.mode, self.O, self.K, self.km = mode, O, K, km
+        self.w, self.scales, self.biases = w, scales, biases
+
+    @staticmethod
+    def kq(rng, kind, O, K, sigma=None):
+        return HostLinear("kq", O, K, km=HostKMat.random(rng, kind, 1, O, K, sigma))
+
+    @staticmethod
+    def affine8(rng, O, K, out_std=1.0):
+        w = rng.integers(0, 256, size=(O, K), dtype=np.uint8)
+        # weight = s*q + b, centred: b = -127.5 s; std(q) = 73.9
+        s = (out_std / (73.9 * np.sqrt(K))) * (0.5 + rng.random((O, K // 64)))
+        scales = f32_to_bf16(s.astype(np.float32))
+        biases = f32_to_bf16((-127.5 * bf16_to_f32(scales)).astype(np.float32))
+        return HostLinear("affine8", O, K, w=w, scales=scales, biases=biases)
+
+    @staticmethod
+    def dense(rng, O, K, out_std=1.0):
+        w = f32_to_bf16((rng.standard_normal((O, K)) * (out_std / np.sqrt(K))).astype(np.float32))
+        return HostLinear("dense", O, K, w=w)
+
+    def orc(self):
+        if self.mode == "kq":
+            return OrcLinear(0, self.km.orc(), None, None, None)
+        km = OrcKmat(0, 1, self.O, self.K, None, None, None)
+        if self.mode == "affine8":
+            return OrcLinear(1, km, p(self.w), p(self.scales), p(self.biases))
+        return OrcLinear(2, km, p(self.w), None, None)
+
+    def dev(self, orn, ctx):
+        if self.mode == "kq":
+            return orn.Linear.kquant(ctx, self.km.kind, self.km.qs, self.km.scales, self.km.dm, self.O, self.K)
+        if self.mode == "affine8":
+            return orn.Linear.affine8(ctx, self.w, self.scales, self.biases)
+        return orn.Linear.dense(ctx, self.w)
+
+    def nbytes(self):
+        if self.mode == "kq":
+            return self.km.nbytes()
+        return sum(t.nbytes for t in (self.w, self.scales, self.biases) if t is not None)
+
+
+class HostMoe:
+    """One sparse MoE block's weights (BASELINE config 2 mix by default:
+    routed gate/up Q4_K, down Q6_K, shared expert the same, router Q6_K, shared gate 8-bit)."""
+
+    def __init__(self, rng, H=2048, E=256, I=512, top_k=8, gate_kind=Q4K, down_kind=Q6K, router_kind=Q6K):
+        self.H, self.E, self.I, self.top_k = H, E, I, top_k
+        self.router = HostLinear.kq(rng, router_kind, E, H)
+        self.ex_gate = HostKMat.random(rng, gate_kind, E, I, H)
+        self.ex_up = HostKMat.random(rng, gate_kind, E, I, H)
+        self.ex_down = HostKMat.random(rng, down_kind, E, H, I)
+        self.sh_gate = HostLinear.kq(rng, gate_kind, I, H)
+        self.sh_up = HostLinear.kq(rng, gate_kind, I, H)
+        self.sh_down = HostLinear.kq(rng, down_kind, H, I)
+        self.sh_egate = HostLinear.affine8(rng, 1, H)
+
+    def orc(self):
+        return OrcMoeWeights(self.router.orc(), self.ex_gate.orc(), self.ex_up.orc(), self.ex_down.orc(),
+                             self.sh_gate.orc(), self.sh_up.orc(), self.sh_down.orc(), self.sh_egate.orc(),
+                             self.top_k, 1)
+
+    def dev(self, orn, ctx):
+        self._dev = [self.router.dev(orn, ctx), self.ex_gate.dev(orn, ctx), self.ex_up.dev(orn, ctx),
+                     self.ex_down.dev(orn, ctx), self.sh_gate.dev(orn, ctx), self.sh_up.dev(orn, ctx),
+                     self.sh_down.dev(orn, ctx), self.sh_egate.dev(orn, ctx)]
+        d = self._dev
+        return orn.MoeWeightsStruct(d[0].s, d[1].s, d[2].s, d[3].s, d[4].s, d[5].s, d[6].s, d[7].s,
+                                    self.top_k, 1)
+
+    def free(self):
+        for d in getattr(self, "_dev", []):
+            d.free()
+
+
+def orc_moe_block(moe, xb, T):
+    w = moe.orc()
+    out = np.empty((T, moe.H), np.uint16)
+    inds = np.empty((T, moe.top_k), np.uint32)
+    scores = np.empty((T, moe.top_k), np.uint16)
+    probs = np.empty((T, moe.E), np.uint16)
+    oracle().orc_moe_block(C.byref(w), p(xb), T, p(out), p(inds), p(scores), p(probs))
+    return out, inds, scores, probs
