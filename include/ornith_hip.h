@@ -159,6 +159,41 @@ typedef struct ornith_moe_weights {
 ORNITH_API int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                                 void* d_out, uint32_t* d_inds_out, void* d_scores_out);
 
+/* ---- norms: src/ops/norm.rs:19-220 (vendored rms_norm.metal:12-81,
+ * kernels/ornith_norm.metal:28-183). Rows of n bf16 values, n = 64 * 2^j <= 4096. */
+/* norm::rms_norm: out = w * (x * rsqrt(mean(x^2) + eps)); d_w may be null (weight 1). */
+ORNITH_API int ornith_rms_norm(ornith_ctx* ctx, const void* d_x, const void* d_w, int rows, int n,
+                               float eps, void* d_out);
+/* norm::add_rms_norm: h = a + b (rounded, written to d_h_out), out = rms_norm(h). */
+ORNITH_API int ornith_add_rms_norm(ornith_ctx* ctx, const void* d_a, const void* d_b, const void* d_w,
+                                   int rows, int n, float eps, void* d_h_out, void* d_out);
+/* norm::rms_norm_gated (Qwen3NextRMSNormGated): out = silu_f32(z) * rms_norm(y, w). */
+ORNITH_API int ornith_rms_norm_gated(ornith_ctx* ctx, const void* d_y, const void* d_w,
+                                     const void* d_z, int rows, int n, float eps, void* d_out);
+
+/* ---- gated-delta layer --------------------------------------------------------- */
+/* gdn::gdn_front (src/ops/gdn.rs:331-413, kernels/gdn_front.metal:65-190), batch 1:
+ *   conv_state bf16[K-1,D], qkv bf16[T,D], cw bf16[D,K], a,b bf16[T,Hv], a_log,dt_bias bf16[Hv]
+ *   -> q,k bf16[T,Hk,Dk], v bf16[T,Hv,Dv], beta bf16[T,Hv], g f32[T,Hv],
+ *      conv_input bf16[K-1+T,D] (the concatenated window, keep_conv_input = true).
+ * D = 2*Hk*Dk + Hv*Dv, Dk = Dv = 128. The next conv state is rows [T, T+K-1) of
+ * conv_input, or rows [keep, keep+K-1) after a rollback (qwen3_5.rs:324-348). */
+ORNITH_API int ornith_gdn_front(ornith_ctx* ctx, const void* d_conv_state, const void* d_qkv,
+                                const void* d_cw, const void* d_a, const void* d_b,
+                                const void* d_a_log, const void* d_dt_bias, int T, int K, int Hk,
+                                int Dk, int Hv, int Dv, float eps, void* d_q, void* d_k, void* d_v,
+                                void* d_beta, float* d_g, void* d_conv_input);
+/* gdn::gated_delta_kernel_into stepped per token as GatedDeltaNet::forward_capture does
+ * (src/ops/gdn.rs:131-271, kernels/gated_delta.metal:36-142, qwen3_5.rs:650-677):
+ * state_in f32[Hv,Dv,Dk] -> y bf16[T,Hv,Dv] and one state snapshot per token,
+ * d_snapshots f32[T][Hv,Dv,Dk]; snapshot T-1 is the new state, snapshot keep-1 is
+ * the state to continue from after accepting keep tokens. With T == 1 d_snapshots may
+ * alias d_state_in. */
+ORNITH_API int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k,
+                                     const void* d_v, const float* d_g, const void* d_beta,
+                                     const float* d_state_in, int T, int Hk, int Hv, int Dk, int Dv,
+                                     void* d_y, float* d_snapshots);
+
 /* ---- self test ------------------------------------------------------------------
  * Evaluates one of the library's scalar device functions element-wise (fp32 in,
  * fp32 out) so their bits can be compared with a CPU evaluation. No reference

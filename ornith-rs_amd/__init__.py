@@ -272,3 +272,35 @@ def moe_block(self, w, x, T, out, inds=None, scores=None):
     _check(lib().ornith_moe_block(self.h, C.byref(w), x.ptr, T, out.ptr,
                                   inds.ptr if inds else None, scores.ptr if scores else None),
            "moe_block")
+
+
+# ---- norms / gated-delta ----------------------------------------------------------
+@_ctx_method
+def rms_norm(self, x, w, rows, n, eps, out):
+    _check(lib().ornith_rms_norm(self.h, x.ptr, w.ptr if w else None, rows, n, C.c_float(eps), out.ptr), "rms_norm")
+
+
+@_ctx_method
+def add_rms_norm(self, a, b, w, rows, n, eps, h_out, out):
+    _check(lib().ornith_add_rms_norm(self.h, a.ptr, b.ptr, w.ptr if w else None, rows, n, C.c_float(eps),
+                                     h_out.ptr, out.ptr), "add_rms_norm")
+
+
+@_ctx_method
+def rms_norm_gated(self, y, w, z, rows, n, eps, out):
+    _check(lib().ornith_rms_norm_gated(self.h, y.ptr, w.ptr, z.ptr, rows, n, C.c_float(eps), out.ptr),
+           "rms_norm_gated")
+
+
+@_ctx_method
+def gdn_front(self, conv_state, qkv, cw, a, b, a_log, dt_bias, T, K, Hk, Dk, Hv, Dv, eps, q, k, v, beta, g,
+              conv_input):
+    _check(lib().ornith_gdn_front(self.h, conv_state.ptr, qkv.ptr, cw.ptr, a.ptr, b.ptr, a_log.ptr,
+                                  dt_bias.ptr, T, K, Hk, Dk, Hv, Dv, C.c_float(eps), q.ptr, k.ptr, v.ptr,
+                                  beta.ptr, g.ptr, conv_input.ptr), "gdn_front")
+
+
+@_ctx_method
+def gdn_recurrence(self, q, k, v, g, beta, state_in, T, Hk, Hv, Dk, Dv, y, snapshots):
+    _check(lib().ornith_gdn_recurrence(self.h, q.ptr, k.ptr, v.ptr, g.ptr, beta.ptr, state_in.ptr, T, Hk, Hv,
+                                       Dk, Dv, y.ptr, snapshots.ptr), "gdn_recurrence")

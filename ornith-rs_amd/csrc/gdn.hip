@@ -1,0 +1,243 @@
+// Gated-delta (linear attention) layer: fused front end and the recurrence.
+//
+// Replaces gdn::gdn_front and gdn::gated_delta_kernel[_into]
+// (/root/reference/src/ops/gdn.rs:131-271,331-413; kernels
+// /root/reference/kernels/gdn_front.metal:65-190,
+// /root/reference/kernels/gated_delta.metal:36-142) and the per-token snapshot
+// loop of GatedDeltaNet::forward_capture (/root/reference/src/model/qwen3_5.rs:650-677).
+//
+// Front: one wavefront per (token, 128-channel head slot); lane l holds channels
+// 2l, 2l+1 from the convolution through the q/k normalisation, so the causal
+// conv, silu, RMS and scale never leave registers. It also writes the
+// concatenated window [K-1+T, D]; the next conv state is a 3-row slice of it
+// (rows [keep, keep+3) after a rollback to `keep` tokens).
+//
+// Recurrence: the fp32 state [Hv, Dv, 128] stays in registers across the T verify
+// tokens. Eight lanes share a state row (lane j owns dk = 32m + 4j + i, which
+// makes every load and store a contiguous 128 bytes per row), one wavefront
+// carries eight rows, and the state after EACH token is written out as a
+// snapshot, so rejecting a draft is a pointer move to snapshot keep-1.
+#include "dmath.h"
+#include "rt.h"
+
+namespace {
+
+struct FrontArgs {
+  const bf16_t* conv_state;  // [S, D]
+  const bf16_t* qkv;         // [T, D]
+  const bf16_t* cw;          // [D, K]
+  const bf16_t* a_in;        // [T, Hv]
+  const bf16_t* b_in;        // [T, Hv]
+  const bf16_t* a_log;       // [Hv]
+  const bf16_t* dt_bias;     // [Hv]
+  bf16_t* q;                 // [T, Hk, 128]
+  bf16_t* k;                 // [T, Hk, 128]
+  bf16_t* v;                 // [T, Hv, 128]
+  bf16_t* beta;              // [T, Hv]
+  float* g;                  // [T, Hv]
+  bf16_t* conv_input;        // [S + T, D]
+  int T, K, Hk, Hv, D;
+  float q_scale, k_scale, eps;
+};
+
+__device__ __forceinline__ float softplus_bf16(float x) {
+  if (x != x) return x;
+  const float mx = x > 0.f ? x : 0.f, mn = x > 0.f ? 0.f : x;
+  if (mn == -DM_INF || mx == DM_INF) return mx;
+  const float d = dm_rb(mn - mx);
+  const float e = dm_rb(dm_exp(d));
+  const float l = dm_rb(dm_log1p(e));
+  return dm_rb(mx + l);
+}
+
+__global__ __launch_bounds__(64) void gdn_front_kernel(FrontArgs p) {
+  const int slot = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+  const int S = p.K - 1, D = p.D;
+  const int c0 = slot * 128 + 2 * lane;
+  const int key_dim = p.Hk * 128;
+
+  float acc0 = 0.f, acc1 = 0.f;
+  for (int i = 0; i < p.K; ++i) {
+    const int j = t + i;
+    const bf16_t* src = (j < S) ? (p.conv_state + (size_t)j * D) : (p.qkv + (size_t)(j - S) * D);
+    const uint32_t xv = *reinterpret_cast<const uint32_t*>(src + c0);
+    acc0 = dm_fma(dm_bf2f_lo(xv), dm_bf2f(p.cw[(size_t)c0 * p.K + i]), acc0);
+    acc1 = dm_fma(dm_bf2f_hi(xv), dm_bf2f(p.cw[(size_t)(c0 + 1) * p.K + i]), acc1);
+  }
+  const float cv0 = dm_rb(acc0), cv1 = dm_rb(acc1);
+  const float y0 = dm_rb(cv0 * dm_sigmoid_bf16(cv0)), y1 = dm_rb(cv1 * dm_sigmoid_bf16(cv1));
+
+  // the concatenated window
+  {
+    uint32_t* ci = reinterpret_cast<uint32_t*>(p.conv_input + (size_t)(S + t) * D + c0);
+    *ci = *reinterpret_cast<const uint32_t*>(p.qkv + (size_t)t * D + c0);
+    if (t == 0) {
+      for (int j = 0; j < S; ++j)
+        *reinterpret_cast<uint32_t*>(p.conv_input + (size_t)j * D + c0) =
+            *reinterpret_cast<const uint32_t*>(p.conv_state + (size_t)j * D + c0);
+    }
+  }
+
+  if (slot < 2 * p.Hk) {
+    float ss = dm_fma(y0, y0, 0.f);
+    ss = dm_fma(y1, y1, ss);
+    const float inv = dm_rsqrt(dm_wave_sum<64>(ss) / 128.0f + p.eps);
+    const bool is_q = slot < p.Hk;
+    bf16_t* dst = (is_q ? p.q : p.k) + (size_t)t * key_dim + (is_q ? c0 : c0 - key_dim);
+    const float sc = is_q ? p.q_scale : p.k_scale;
+    const uint32_t lo = dm_f2bf(sc * dm_rb(y0 * inv)), hi = dm_f2bf(sc * dm_rb(y1 * inv));
+    *reinterpret_cast<uint32_t*>(dst) = lo | (hi << 16);
+  } else {
+    bf16_t* dst = p.v + (size_t)t * (D - 2 * key_dim) + (c0 - 2 * key_dim);
+    *reinterpret_cast<uint32_t*>(dst) = (uint32_t)dm_f2bf(y0) | ((uint32_t)dm_f2bf(y1) << 16);
+  }
+
+  if (slot == 0) {
+    for (int h = lane; h < p.Hv; h += 64) {
+      const int i = t * p.Hv + h;
+      const float sp = softplus_bf16(dm_rb(dm_bf2f(p.a_in[i]) + dm_bf2f(p.dt_bias[h])));
+      const float decay = dm_exp(dm_bf2f(p.a_log[h]));
+      p.g[i] = dm_exp(-decay * sp);
+      p.beta[i] = dm_f2bf(dm_sigmoid_bf16(dm_bf2f(p.b_in[i])));
+    }
+  }
+}
+
+struct RecArgs {
+  const bf16_t* q;
+  const bf16_t* k;
+  const bf16_t* v;
+  const float* g;
+  const bf16_t* beta;
+  const float* state_in;  // [Hv, Dv, 128]
+  bf16_t* y;              // [T, Hv, Dv]
+  float* snapshots;       // [T][Hv, Dv, 128]
+  int T, Hk, Hv, Dv;
+};
+
+__global__ __launch_bounds__(64) void gdn_recurrence_kernel(RecArgs p) {
+  const int lane = threadIdx.x, row = lane >> 3, j = lane & 7;
+  const int hv = blockIdx.y, dv = blockIdx.x * 8 + row;
+  const int hk = hv / (p.Hv / p.Hk);
+  const size_t ssz = (size_t)p.Hv * p.Dv * 128;
+  const size_t roff = ((size_t)hv * p.Dv + dv) * 128 + 4 * j;
+
+  float s[16];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const float4 f = *reinterpret_cast<const float4*>(p.state_in + roff + 32 * m);
+    s[4 * m + 0] = f.x;
+    s[4 * m + 1] = f.y;
+    s[4 * m + 2] = f.z;
+    s[4 * m + 3] = f.w;
+  }
+  for (int t = 0; t < p.T; ++t) {
+    float kf[16], qf[16];
+    const bf16_t* kp = p.k + ((size_t)t * p.Hk + hk) * 128 + 4 * j;
+    const bf16_t* qp = p.q + ((size_t)t * p.Hk + hk) * 128 + 4 * j;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const uint2 kw = *reinterpret_cast<const uint2*>(kp + 32 * m);
+      const uint2 qw = *reinterpret_cast<const uint2*>(qp + 32 * m);
+      kf[4 * m + 0] = dm_bf2f_lo(kw.x);
+      kf[4 * m + 1] = dm_bf2f_hi(kw.x);
+      kf[4 * m + 2] = dm_bf2f_lo(kw.y);
+      kf[4 * m + 3] = dm_bf2f_hi(kw.y);
+      qf[4 * m + 0] = dm_bf2f_lo(qw.x);
+      qf[4 * m + 1] = dm_bf2f_hi(qw.x);
+      qf[4 * m + 2] = dm_bf2f_lo(qw.y);
+      qf[4 * m + 3] = dm_bf2f_hi(qw.y);
+    }
+    const float gt = p.g[t * p.Hv + hv], bt = dm_bf2f(p.beta[t * p.Hv + hv]);
+    const float vt = dm_bf2f(p.v[((size_t)t * p.Hv + hv) * p.Dv + dv]);
+    float a = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      s[e] = s[e] * gt;
+      a = dm_fma(s[e], kf[e], a);
+    }
+    const float kv = dm_wave_sum<8>(a);
+    const float delta = (vt - kv) * bt;
+    float o = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      s[e] = dm_fma(kf[e], delta, s[e]);
+      o = dm_fma(s[e], qf[e], o);
+    }
+    o = dm_wave_sum<8>(o);
+    if (j == 0) p.y[((size_t)t * p.Hv + hv) * p.Dv + dv] = dm_f2bf(o);
+    float* snap = p.snapshots + (size_t)t * ssz + roff;
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+      *reinterpret_cast<float4*>(snap + 32 * m) =
+          make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int ornith_gdn_front(ornith_ctx* ctx, const void* d_conv_state, const void* d_qkv, const void* d_cw,
+                     const void* d_a, const void* d_b, const void* d_a_log, const void* d_dt_bias,
+                     int T, int K, int Hk, int Dk, int Hv, int Dv, float eps, void* d_q, void* d_k,
+                     void* d_v, void* d_beta, float* d_g, void* d_conv_input) {
+  ORN_REQUIRE(ctx && d_conv_state && d_qkv && d_cw && d_a && d_b && d_a_log && d_dt_bias && d_q &&
+                  d_k && d_v && d_beta && d_g && d_conv_input,
+              "gdn_front: null argument");
+  ORN_REQUIRE(Dk == 128 && Dv == 128, "gdn_front: head dims %d/%d (128 only)", Dk, Dv);
+  ORN_REQUIRE(T >= 1 && T <= 65535 && K >= 2 && K <= 8 && Hk >= 1 && Hv >= Hk && Hv % Hk == 0,
+              "gdn_front: T=%d K=%d Hk=%d Hv=%d", T, K, Hk, Hv);
+  ORN_REQUIRE(d_conv_input != d_conv_state, "gdn_front: conv_input must not alias conv_state");
+  FrontArgs p{};
+  p.conv_state = (const bf16_t*)d_conv_state;
+  p.qkv = (const bf16_t*)d_qkv;
+  p.cw = (const bf16_t*)d_cw;
+  p.a_in = (const bf16_t*)d_a;
+  p.b_in = (const bf16_t*)d_b;
+  p.a_log = (const bf16_t*)d_a_log;
+  p.dt_bias = (const bf16_t*)d_dt_bias;
+  p.q = (bf16_t*)d_q;
+  p.k = (bf16_t*)d_k;
+  p.v = (bf16_t*)d_v;
+  p.beta = (bf16_t*)d_beta;
+  p.g = d_g;
+  p.conv_input = (bf16_t*)d_conv_input;
+  p.T = T;
+  p.K = K;
+  p.Hk = Hk;
+  p.Hv = Hv;
+  p.D = 2 * Hk * 128 + Hv * 128;
+  const float inv_scale = 1.0f / sqrtf((float)Dk);
+  // both scales are applied as bf16 values (the reference casts them to T)
+  uint32_t u;
+  float f = inv_scale * inv_scale;
+  memcpy(&u, &f, 4);
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+  memcpy(&p.q_scale, &u, 4);
+  f = inv_scale;
+  memcpy(&u, &f, 4);
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+  memcpy(&p.k_scale, &u, 4);
+  p.eps = eps;
+  hipLaunchKernelGGL(gdn_front_kernel, dim3(p.D / 128, T), dim3(64), 0, ctx->stream, p);
+  ORN_LAUNCH_CHECK("gdn_front_kernel");
+  return ORNITH_OK;
+}
+
+int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, const void* d_v,
+                          const float* d_g, const void* d_beta, const float* d_state_in, int T,
+                          int Hk, int Hv, int Dk, int Dv, void* d_y, float* d_snapshots) {
+  ORN_REQUIRE(ctx && d_q && d_k && d_v && d_g && d_beta && d_state_in && d_y && d_snapshots,
+              "gdn_recurrence: null argument");
+  ORN_REQUIRE(Dk == 128 && Dv % 8 == 0 && Dv >= 8, "gdn_recurrence: Dk=%d Dv=%d", Dk, Dv);
+  ORN_REQUIRE(T >= 1 && Hk >= 1 && Hv >= Hk && Hv % Hk == 0 && Hv <= 65535,
+              "gdn_recurrence: T=%d Hk=%d Hv=%d", T, Hk, Hv);
+  RecArgs p{(const bf16_t*)d_q, (const bf16_t*)d_k, (const bf16_t*)d_v, d_g, (const bf16_t*)d_beta,
+            d_state_in,         (bf16_t*)d_y,       d_snapshots,        T,   Hk, Hv, Dv};
+  hipLaunchKernelGGL(gdn_recurrence_kernel, dim3(Dv / 8, Hv), dim3(64), 0, ctx->stream, p);
+  ORN_LAUNCH_CHECK("gdn_recurrence_kernel");
+  return ORNITH_OK;
+}
+
+}  // extern "C"

@@ -276,3 +276,49 @@ def orc_moe_block(moe, xb, T):
     probs = np.empty((T, moe.E), np.uint16)
     oracle().orc_moe_block(C.byref(w), p(xb), T, p(out), p(inds), p(scores), p(probs))
     return out, inds, scores, probs
+
+
+# ---- norms / gated-delta oracle wrappers ----------------------------------------------
+def orc_rms_norm(x, w, eps=1e-6):
+    rows, n = x.shape
+    out = np.empty_like(x)
+    oracle().orc_rms_norm(p(x), p(w) if w is not None else None, rows, n, C.c_float(eps), p(out))
+    return out
+
+
+def orc_add_rms_norm(a, b, w, eps=1e-6):
+    rows, n = a.shape
+    h, out = np.empty_like(a), np.empty_like(a)
+    oracle().orc_add_rms_norm(p(a), p(b), p(w), rows, n, C.c_float(eps), p(h), p(out))
+    return h, out
+
+
+def orc_rms_norm_gated(y, w, z, eps=1e-6):
+    rows, n = y.shape
+    out = np.empty_like(y)
+    oracle().orc_rms_norm_gated(p(y), p(w), p(z), rows, n, C.c_float(eps), p(out))
+    return out
+
+
+def orc_gdn_front(conv_state, qkv, cw, a, b, a_log, dt_bias, Hk, Hv, K=4, Dk=128, Dv=128, eps=1e-6):
+    T, D = qkv.shape
+    q = np.empty((T, Hk, Dk), np.uint16); k = np.empty((T, Hk, Dk), np.uint16)
+    v = np.empty((T, Hv, Dv), np.uint16); beta = np.empty((T, Hv), np.uint16)
+    g = np.empty((T, Hv), np.float32); ci = np.empty((K - 1 + T, D), np.uint16)
+    oracle().orc_gdn_front(p(conv_state), p(qkv), p(cw), p(a), p(b), p(a_log), p(dt_bias), T, K, Hk, Dk, Hv, Dv,
+                           C.c_float(eps), p(q), p(k), p(v), p(beta), p(g), p(ci))
+    return q, k, v, beta, g, ci
+
+
+def orc_gdn_recurrence(q, k, v, g, beta, state):
+    T, Hk, Dk = q.shape
+    _, Hv, Dv = v.shape
+    y = np.empty((T, Hv, Dv), np.uint16)
+    snaps = np.empty((T, Hv, Dv, Dk), np.float32)
+    oracle().orc_gdn_recurrence(p(q), p(k), p(v), p(g), p(beta), p(np.ascontiguousarray(state)), T, Hk, Hv, Dk, Dv,
+                                p(y), p(snaps))
+    return y, snaps
+
+
+def bf16_normal(rng, shape, std=1.0):
+    return f32_to_bf16((rng.standard_normal(shape) * std).astype(np.float32))
