@@ -194,6 +194,29 @@ ORNITH_API int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const voi
                                      const float* d_state_in, int T, int Hk, int Hv, int Dk, int Dv,
                                      void* d_y, float* d_snapshots);
 
+/* ---- full-attention layer at decode / verify width ------------------------------ */
+/* ops::rope tables (src/ops/rope.rs:6-60): cos/sin f32 [npos, dims/2] for
+ * inv_freq_i = theta^(-i/(dims/2)), computed in double on the host and uploaded. */
+ORNITH_API int ornith_rope_table(ornith_ctx* ctx, int npos, int dims, double theta, float* d_cos,
+                                 float* d_sin);
+/* Attention::forward up to the cache write (src/model/qwen3_5.rs:439-463): per-head
+ * rms_norm of q and k (weights [hd]), partial RoPE at position offset + t, append of
+ * K and V at rows [offset, offset+T) of the caches bf16 [Hkv, cap, hd]
+ * (KvCache::update_and_fetch, src/model/cache.rs:38-79). qg is q_proj's output
+ * [T, Hq, 2*hd] (query | gate), kx / vx are k_proj / v_proj outputs [T, Hkv, hd].
+ * If d_offset is non-null the offset is read from device memory at run time. */
+ORNITH_API int ornith_attn_prep(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const void* d_vx,
+                                const void* d_q_norm_w, const void* d_k_norm_w, int T, int Hq, int Hkv,
+                                int hd, int rope_dims, float eps, const float* d_cos,
+                                const float* d_sin, int table_npos, int offset, const int* d_offset,
+                                int cap, void* d_q_rot, void* d_k_cache, void* d_v_cache);
+/* sdpa::attention_with_cache + sigmoid_gate (src/ops/sdpa.rs:61-83, qwen3_5.rs:465-472):
+ * query row t sees keys [0, offset + t]; out bf16 [T, Hq*hd] = sigmoid(gate) * attn. */
+ORNITH_API int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d_k_cache,
+                                        const void* d_v_cache, const void* d_qg, int T, int Hq,
+                                        int Hkv, int hd, int offset, const int* d_offset, int cap,
+                                        float scale, void* d_out);
+
 /* ---- self test ------------------------------------------------------------------
  * Evaluates one of the library's scalar device functions element-wise (fp32 in,
  * fp32 out) so their bits can be compared with a CPU evaluation. No reference

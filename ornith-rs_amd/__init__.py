@@ -304,3 +304,29 @@ def gdn_front(self, conv_state, qkv, cw, a, b, a_log, dt_bias, T, K, Hk, Dk, Hv,
 def gdn_recurrence(self, q, k, v, g, beta, state_in, T, Hk, Hv, Dk, Dv, y, snapshots):
     _check(lib().ornith_gdn_recurrence(self.h, q.ptr, k.ptr, v.ptr, g.ptr, beta.ptr, state_in.ptr, T, Hk, Hv,
                                        Dk, Dv, y.ptr, snapshots.ptr), "gdn_recurrence")
+
+
+# ---- attention ---------------------------------------------------------------------
+@_ctx_method
+def rope_table(self, npos, dims, theta):
+    half = dims // 2
+    dc, ds = self.alloc(npos * half * 4), self.alloc(npos * half * 4)
+    _check(lib().ornith_rope_table(self.h, npos, dims, C.c_double(theta), dc.ptr, ds.ptr), "rope_table")
+    return dc, ds
+
+
+@_ctx_method
+def attn_prep(self, qg, kx, vx, qw, kw, T, Hq, Hkv, hd, rope_dims, eps, cos_t, sin_t, npos, offset, cap,
+              q_rot, k_cache, v_cache, d_offset=None):
+    _check(lib().ornith_attn_prep(self.h, qg.ptr, kx.ptr, vx.ptr, qw.ptr, kw.ptr, T, Hq, Hkv, hd, rope_dims,
+                                  C.c_float(eps), cos_t.ptr, sin_t.ptr, npos, offset,
+                                  d_offset.ptr if d_offset else None, cap, q_rot.ptr, k_cache.ptr,
+                                  v_cache.ptr), "attn_prep")
+
+
+@_ctx_method
+def sdpa_decode_gated(self, q_rot, k_cache, v_cache, qg, T, Hq, Hkv, hd, offset, cap, scale, out,
+                      d_offset=None):
+    _check(lib().ornith_sdpa_decode_gated(self.h, q_rot.ptr, k_cache.ptr, v_cache.ptr, qg.ptr, T, Hq, Hkv, hd,
+                                          offset, d_offset.ptr if d_offset else None, cap, C.c_float(scale),
+                                          out.ptr), "sdpa_decode_gated")

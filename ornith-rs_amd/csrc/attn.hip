@@ -1,0 +1,374 @@
+// Full-attention layer at decode / verify width: per-head RMS + partial RoPE +
+// KV append in one kernel, split-K attention over the cache, merge + output gate.
+//
+// Replaces the middle of Attention::forward
+// (/root/reference/src/model/qwen3_5.rs:430-474): rms_norm on q/k heads,
+// rope (/root/reference/src/ops/rope.rs:6-60, vendored rope.metal:11-67),
+// KvCache::update_and_fetch (/root/reference/src/model/cache.rs:38-79),
+// attention_with_cache -> sdpa_vector[_2pass]
+// (/root/reference/src/ops/sdpa.rs:33-83,166-264, vendored sdpa_vector.h:15-318)
+// and sigmoid_gate (kernels/ornith_elementwise.metal).
+//
+// Attention is split over keys in blocks of 256 by absolute position, one
+// workgroup per (block, kv head, query row): scores are thread-per-key (one fma
+// chain over the head dimension), values are thread-per-channel (one fma chain
+// over the block's keys), so neither needs a cross-lane reduction per key. The
+// partial (max, sum, values) of each block go to scratch and a second kernel
+// merges them in ascending block order and applies the sigmoid output gate.
+// A query row only ever sees keys at or before its own position, and blocks are
+// aligned to absolute positions, so row r of a T-row verify call is bit-identical
+// to a one-row call at that position.
+#include "dmath.h"
+#include "rt.h"
+
+namespace {
+
+constexpr int ATT_KB = 256;
+
+struct PrepArgs {
+  const bf16_t* qg;  // [T, Hq, 2*hd]
+  const bf16_t* kx;  // [T, Hkv, hd]
+  const bf16_t* vx;  // [T, Hkv, hd]
+  const bf16_t* qw;  // [hd]
+  const bf16_t* kw;  // [hd]
+  const float* cos_t;  // [npos, half]
+  const float* sin_t;
+  const int* d_offset;  // optional: position of the first new row, read on the device
+  bf16_t* q_rot;      // [T, Hq, hd]
+  bf16_t* k_cache;    // [Hkv, cap, hd]
+  bf16_t* v_cache;
+  int T, Hq, Hkv, offset, cap, npos, half;
+  float eps;
+};
+
+// one wavefront per (head, token); PER = hd / 64 contiguous channels per lane
+template <int PER>
+__global__ __launch_bounds__(64) void attn_prep_kernel(PrepArgs p) {
+  constexpr int HD = 64 * PER;
+  const int hidx = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+  const int offset = p.d_offset ? *p.d_offset : p.offset;
+  const int pos = offset + t;
+  if (pos >= p.cap || pos >= p.npos) return;  // host checks the static case; device offset guarded here
+  const bf16_t* src;
+  bf16_t* dst;
+  const bf16_t* w = nullptr;
+  if (hidx < p.Hq) {
+    src = p.qg + ((size_t)t * p.Hq + hidx) * 2 * HD;
+    dst = p.q_rot + ((size_t)t * p.Hq + hidx) * HD;
+    w = p.qw;
+  } else if (hidx < p.Hq + p.Hkv) {
+    const int h = hidx - p.Hq;
+    src = p.kx + ((size_t)t * p.Hkv + h) * HD;
+    dst = p.k_cache + ((size_t)h * p.cap + pos) * HD;
+    w = p.kw;
+  } else {
+    const int h = hidx - p.Hq - p.Hkv;
+    src = p.vx + ((size_t)t * p.Hkv + h) * HD;
+    dst = p.v_cache + ((size_t)h * p.cap + pos) * HD;
+  }
+  float x[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) x[i] = dm_bf2f(src[lane * PER + i]);
+  if (w) {
+    float a = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) a = dm_fma(x[i], x[i], a);
+    const float inv = dm_rsqrt(dm_wave_sum<64>(a) / (float)HD + p.eps);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) x[i] = dm_rb(dm_bf2f(w[lane * PER + i]) * dm_rb(x[i] * inv));
+    // rotate pairs (e, e + half), e < half; the partner channel lives hl lanes away
+    const int hl = p.half / PER;
+    const bool lowg = lane < hl, rot = lane < 2 * hl;
+    const int partner = lowg ? lane + hl : lane - hl;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const float other = __shfl(x[i], partner & 63, 64);
+      if (rot) {
+        const int e = (lowg ? lane : lane - hl) * PER + i;
+        const float c = p.cos_t[(size_t)pos * p.half + e], s = p.sin_t[(size_t)pos * p.half + e];
+        float r;
+        if (lowg) {
+          r = x[i] * c;
+          r = dm_fma(-other, s, r);
+        } else {
+          r = other * s;
+          r = dm_fma(x[i], c, r);
+        }
+        x[i] = r;  // rounded on store
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < PER; ++i) dst[lane * PER + i] = dm_f2bf(x[i]);
+}
+
+struct SdpaArgs {
+  const bf16_t* q_rot;   // [T, Hq, HD]
+  const bf16_t* k_cache; // [Hkv, cap, HD]
+  const bf16_t* v_cache;
+  const bf16_t* qg;      // [T, Hq, 2*HD] (gate half read by the merge)
+  const int* d_offset;
+  float* part_m;         // [T, Hq, nblk]
+  float* part_l;         // [T, Hq, nblk]
+  float* part_o;         // [T, Hq, nblk, HD]
+  bf16_t* out;           // [T, Hq*HD]
+  int T, Hq, Hkv, offset, cap, nblk;
+  float scale;
+};
+
+// grid (nblk, Hkv, T), 256 threads. G = q heads per kv head handled together.
+template <int G, int HD>
+__global__ __launch_bounds__(256) void sdpa_partial_kernel(SdpaArgs p) {
+  const int b = blockIdx.x, hk = blockIdx.y, t = blockIdx.z, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int offset = p.d_offset ? *p.d_offset : p.offset;
+  const int last = min(offset + t, p.cap - 1);
+  if (b * ATT_KB > last) return;
+  const int gqa = p.Hq / p.Hkv;
+
+  __shared__ float qs[G][HD];
+  __shared__ float pr[G][ATT_KB];
+  __shared__ float red[G][4];
+
+  const int key = b * ATT_KB + tid;
+  const bool valid = key <= last;
+  const int nvalid = min(ATT_KB, last - b * ATT_KB + 1);
+  const bf16_t* krow = p.k_cache + ((size_t)hk * p.cap + (valid ? key : last)) * HD;
+
+  for (int g0 = 0; g0 < gqa; g0 += G) {
+    __syncthreads();
+    for (int i = tid; i < G * HD; i += 256) {
+      const int g = i / HD, d = i - g * HD;
+      const int h = hk * gqa + g0 + g;
+      qs[g][d] = (g0 + g < gqa) ? p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + h) * HD + d]) : 0.f;
+    }
+    __syncthreads();
+    float acc[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) acc[g] = 0.f;
+    for (int dc = 0; dc < HD / 8; ++dc) {
+      const uint4 kw = *reinterpret_cast<const uint4*>(krow + 8 * dc);
+      const float kf[8] = {dm_bf2f_lo(kw.x), dm_bf2f_hi(kw.x), dm_bf2f_lo(kw.y), dm_bf2f_hi(kw.y),
+                           dm_bf2f_lo(kw.z), dm_bf2f_hi(kw.z), dm_bf2f_lo(kw.w), dm_bf2f_hi(kw.w)};
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        const float4 q0 = *reinterpret_cast<const float4*>(&qs[g][8 * dc]);
+        const float4 q1 = *reinterpret_cast<const float4*>(&qs[g][8 * dc + 4]);
+        float a = acc[g];
+        a = dm_fma(q0.x, kf[0], a);
+        a = dm_fma(q0.y, kf[1], a);
+        a = dm_fma(q0.z, kf[2], a);
+        a = dm_fma(q0.w, kf[3], a);
+        a = dm_fma(q1.x, kf[4], a);
+        a = dm_fma(q1.y, kf[5], a);
+        a = dm_fma(q1.z, kf[6], a);
+        a = dm_fma(q1.w, kf[7], a);
+        acc[g] = a;
+      }
+    }
+    // block max per head
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float m = dm_wave_max<64>(valid ? acc[g] : -DM_INF);
+      if (lane == 0) red[g][wave] = m;
+    }
+    __syncthreads();
+    float mg[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float m = red[g][0];
+      m = red[g][1] > m ? red[g][1] : m;
+      m = red[g][2] > m ? red[g][2] : m;
+      m = red[g][3] > m ? red[g][3] : m;
+      mg[g] = m;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float pv = valid ? dm_exp(acc[g] - mg[g]) : 0.f;
+      pr[g][tid] = pv;
+      const float ws = dm_wave_sum<64>(pv);
+      if (lane == 0) red[g][wave] = ws;
+    }
+    __syncthreads();
+    // values: thread = channel, keys ascending
+    float o[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) o[g] = 0.f;
+    if (tid < HD) {
+      const bf16_t* vcol = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + tid;
+      for (int i = 0; i < nvalid; ++i) {
+        const float v = dm_bf2f(vcol[(size_t)i * HD]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) o[g] = dm_fma(pr[g][i], v, o[g]);
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      if (g0 + g >= gqa) continue;
+      const int h = hk * gqa + g0 + g;
+      const size_t pi = ((size_t)t * p.Hq + h) * p.nblk + b;
+      if (tid < HD) p.part_o[pi * HD + tid] = o[g];
+      if (tid == 0) {
+        float l = red[g][0] + red[g][1];
+        l = l + red[g][2];
+        l = l + red[g][3];
+        p.part_m[pi] = mg[g];
+        p.part_l[pi] = l;
+      }
+    }
+  }
+}
+
+// grid (Hq, T), HD threads: merge blocks ascending, divide, gate
+template <int HD>
+__global__ __launch_bounds__(HD) void sdpa_merge_kernel(SdpaArgs p) {
+  const int h = blockIdx.x, t = blockIdx.y, d = threadIdx.x;
+  const int offset = p.d_offset ? *p.d_offset : p.offset;
+  const int last = min(offset + t, p.cap - 1);
+  const int nb = last / ATT_KB + 1;
+  const size_t pi = ((size_t)t * p.Hq + h) * p.nblk;
+  float M = -DM_INF;
+  for (int b = 0; b < nb; ++b) M = p.part_m[pi + b] > M ? p.part_m[pi + b] : M;
+  float L = 0.f, O = 0.f;
+  for (int b = 0; b < nb; ++b) {
+    const float w = dm_exp(p.part_m[pi + b] - M);
+    L = dm_fma(p.part_l[pi + b], w, L);
+    O = dm_fma(p.part_o[(pi + b) * HD + d], w, O);
+  }
+  const float att = dm_rb(O / L);
+  const float g = dm_sigmoid_bf16(dm_bf2f(p.qg[((size_t)t * p.Hq + h) * 2 * HD + HD + d]));
+  p.out[((size_t)t * p.Hq + h) * HD + d] = dm_f2bf(g * att);
+}
+
+}  // namespace
+
+extern "C" {
+
+int ornith_rope_table(ornith_ctx* ctx, int npos, int dims, double theta, float* d_cos,
+                      float* d_sin) {
+  ORN_REQUIRE(ctx && d_cos && d_sin, "rope_table: null argument");
+  ORN_REQUIRE(npos >= 1 && dims >= 2 && dims % 2 == 0 && theta > 0, "rope_table: npos=%d dims=%d",
+              npos, dims);
+  const int half = dims / 2;
+  float* hc = (float*)malloc(sizeof(float) * (size_t)npos * half * 2);
+  if (!hc) return ornith_fail(ORNITH_ERR_INVALID, "rope_table: out of host memory");
+  float* hs = hc + (size_t)npos * half;
+  for (int i = 0; i < half; ++i) {
+    const double inv_freq = pow(theta, -(double)i / (double)half);
+    for (int pos = 0; pos < npos; ++pos) {
+      const double ang = (double)pos * inv_freq;
+      hc[(size_t)pos * half + i] = (float)cos(ang);
+      hs[(size_t)pos * half + i] = (float)sin(ang);
+    }
+  }
+  int rc = ornith_upload(ctx, d_cos, hc, sizeof(float) * (size_t)npos * half);
+  if (!rc) rc = ornith_upload(ctx, d_sin, hs, sizeof(float) * (size_t)npos * half);
+  free(hc);
+  return rc;
+}
+
+int ornith_attn_prep(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const void* d_vx,
+                     const void* d_q_norm_w, const void* d_k_norm_w, int T, int Hq, int Hkv, int hd,
+                     int rope_dims, float eps, const float* d_cos, const float* d_sin, int table_npos,
+                     int offset, const int* d_offset, int cap, void* d_q_rot, void* d_k_cache,
+                     void* d_v_cache) {
+  ORN_REQUIRE(ctx && d_qg && d_kx && d_vx && d_q_norm_w && d_k_norm_w && d_cos && d_sin && d_q_rot &&
+                  d_k_cache && d_v_cache,
+              "attn_prep: null argument");
+  ORN_REQUIRE(hd == 256 || hd == 128, "attn_prep: head_dim %d (128 or 256)", hd);
+  const int per = hd / 64, half = rope_dims / 2;
+  ORN_REQUIRE(rope_dims >= 2 * per && rope_dims <= hd && half % per == 0 &&
+                  ((half / per) & (half / per - 1)) == 0,
+              "attn_prep: rope_dims=%d does not tile head_dim %d", rope_dims, hd);
+  ORN_REQUIRE(T >= 1 && T <= 65535 && Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "attn_prep: T=%d Hq=%d Hkv=%d",
+              T, Hq, Hkv);
+  ORN_REQUIRE(offset >= 0 && offset + T <= cap && offset + T <= table_npos,
+              "attn_prep: rows [%d,%d) do not fit cache capacity %d / rope table %d", offset,
+              offset + T, cap, table_npos);
+  PrepArgs p{};
+  p.qg = (const bf16_t*)d_qg;
+  p.kx = (const bf16_t*)d_kx;
+  p.vx = (const bf16_t*)d_vx;
+  p.qw = (const bf16_t*)d_q_norm_w;
+  p.kw = (const bf16_t*)d_k_norm_w;
+  p.cos_t = d_cos;
+  p.sin_t = d_sin;
+  p.d_offset = d_offset;
+  p.q_rot = (bf16_t*)d_q_rot;
+  p.k_cache = (bf16_t*)d_k_cache;
+  p.v_cache = (bf16_t*)d_v_cache;
+  p.T = T;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.offset = offset;
+  p.cap = cap;
+  p.npos = table_npos;
+  p.half = half;
+  p.eps = eps;
+  dim3 grid(Hq + 2 * Hkv, T);
+  if (hd == 256)
+    hipLaunchKernelGGL(attn_prep_kernel<4>, grid, dim3(64), 0, ctx->stream, p);
+  else
+    hipLaunchKernelGGL(attn_prep_kernel<2>, grid, dim3(64), 0, ctx->stream, p);
+  ORN_LAUNCH_CHECK("attn_prep_kernel");
+  return ORNITH_OK;
+}
+
+int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d_k_cache,
+                             const void* d_v_cache, const void* d_qg, int T, int Hq, int Hkv, int hd,
+                             int offset, const int* d_offset, int cap, float scale, void* d_out) {
+  ORN_REQUIRE(ctx && d_q_rot && d_k_cache && d_v_cache && d_qg && d_out, "sdpa_decode: null argument");
+  ORN_REQUIRE(hd == 256 || hd == 128, "sdpa_decode: head_dim %d (128 or 256)", hd);
+  ORN_REQUIRE(T >= 1 && T <= 64 && Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "sdpa_decode: T=%d Hq=%d Hkv=%d",
+              T, Hq, Hkv);
+  ORN_REQUIRE(offset >= 0 && offset + T <= cap, "sdpa_decode: rows [%d,%d) exceed capacity %d", offset,
+              offset + T, cap);
+  // with a device-side offset the grid must cover the whole cache
+  const int nblk = d_offset ? (cap + ATT_KB - 1) / ATT_KB : (offset + T - 1) / ATT_KB + 1;
+  const size_t per = (size_t)T * Hq * nblk;
+  void* base = nullptr;
+  int rc = ornith_scratch(ctx, (per * (hd + 2)) * 4 + 1024, &base);
+  if (rc) return rc;
+  ScratchCursor sc(base);
+  SdpaArgs p{};
+  p.q_rot = (const bf16_t*)d_q_rot;
+  p.k_cache = (const bf16_t*)d_k_cache;
+  p.v_cache = (const bf16_t*)d_v_cache;
+  p.qg = (const bf16_t*)d_qg;
+  p.d_offset = d_offset;
+  p.part_m = sc.take<float>(per);
+  p.part_l = sc.take<float>(per);
+  p.part_o = sc.take<float>(per * hd);
+  p.out = (bf16_t*)d_out;
+  p.T = T;
+  p.Hq = Hq;
+  p.Hkv = Hkv;
+  p.offset = offset;
+  p.cap = cap;
+  p.nblk = nblk;
+  p.scale = scale;
+  const int gqa = Hq / Hkv;
+  dim3 grid(nblk, Hkv, T);
+#define SDPA_LAUNCH(G, HD)                                                                  \
+  hipLaunchKernelGGL((sdpa_partial_kernel<G, HD>), grid, dim3(256), 0, ctx->stream, p)
+  if (hd == 256) {
+    if (gqa >= 8) SDPA_LAUNCH(8, 256);
+    else if (gqa >= 4) SDPA_LAUNCH(4, 256);
+    else SDPA_LAUNCH(2, 256);
+  } else {
+    if (gqa >= 8) SDPA_LAUNCH(8, 128);
+    else if (gqa >= 4) SDPA_LAUNCH(4, 128);
+    else SDPA_LAUNCH(2, 128);
+  }
+#undef SDPA_LAUNCH
+  ORN_LAUNCH_CHECK("sdpa_partial_kernel");
+  if (hd == 256)
+    hipLaunchKernelGGL(sdpa_merge_kernel<256>, dim3(Hq, T), dim3(256), 0, ctx->stream, p);
+  else
+    hipLaunchKernelGGL(sdpa_merge_kernel<128>, dim3(Hq, T), dim3(128), 0, ctx->stream, p);
+  ORN_LAUNCH_CHECK("sdpa_merge_kernel");
+  return ORNITH_OK;
+}
+
+}  // extern "C"

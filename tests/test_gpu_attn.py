@@ -1,0 +1,46 @@
+"""GPU parity: attention prep (q/k norm + RoPE + KV append) and split-K decode attention
+with the output gate vs the oracle, bit for bit."""
+import numpy as np
+import pytest
+
+import util
+
+pytestmark = pytest.mark.gpu
+
+
+def _mk(rng, T, Hq, Hkv, hd, cap, offset):
+    qg = util.bf16_normal(rng, (T, Hq, 2 * hd)); kx = util.bf16_normal(rng, (T, Hkv, hd)); vx = util.bf16_normal(rng, (T, Hkv, hd))
+    qw = util.bf16_normal(rng, (hd,)); kw = util.bf16_normal(rng, (hd,))
+    kc = np.zeros((Hkv, cap, hd), np.uint16); vc = np.zeros((Hkv, cap, hd), np.uint16)
+    kc[:, :offset] = util.bf16_normal(rng, (Hkv, offset, hd)); vc[:, :offset] = util.bf16_normal(rng, (Hkv, offset, hd))
+    # rows past the end hold NaN patterns: nothing may read them
+    kc[:, offset + T:] = 0x7FC0; vc[:, offset + T:] = 0x7FC0
+    return qg, kx, vx, qw, kw, kc, vc
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,hd,cap,offset", [
+    (1, 16, 2, 256, 4096, 4000), (2, 16, 2, 256, 4096, 255), (4, 16, 2, 256, 4096, 1021),
+    (3, 4, 1, 256, 512, 0), (2, 4, 2, 128, 768, 300), (1, 2, 2, 256, 256, 7)])
+def test_attention_bit_exact(orn, ctx, T, Hq, Hkv, hd, cap, offset):
+    rng = np.random.default_rng(T * 1000 + offset)
+    qg, kx, vx, qw, kw, kc, vc = _mk(rng, T, Hq, Hkv, hd, cap, offset)
+    rd = 64 if hd == 256 else 32
+    c, s = util.orc_rope_table(cap, rd, 1e7)
+    dc, ds = ctx.rope_table(cap, rd, 1e7)
+    assert np.array_equal(dc.download(np.float32, c.shape), c) and np.array_equal(ds.download(np.float32, s.shape), s)
+    d = [ctx.to_device(a) for a in (qg, kx, vx, qw, kw)]
+    dkc, dvc = ctx.to_device(kc), ctx.to_device(vc)
+    dq, dout = ctx.alloc(T * Hq * hd * 2), ctx.alloc(T * Hq * hd * 2)
+    wkc, wvc = kc.copy(), vc.copy()
+    wq, wgate = util.orc_attn_prep(qg, kx, vx, qw, kw, rd, c, s, offset, wkc, wvc)
+    want = util.orc_sdpa(wq, wkc, wvc, wgate, offset, hd ** -0.5)
+    for use_dev_offset in (False, True):
+        doff = ctx.to_device(np.array([offset], np.int32)) if use_dev_offset else None
+        dkc.upload(kc); dvc.upload(vc)
+        ctx.attn_prep(*d, T, Hq, Hkv, hd, rd, 1e-6, dc, ds, cap, 0 if use_dev_offset else offset, cap, dq, dkc, dvc, d_offset=doff)
+        assert np.array_equal(dq.download(np.uint16, wq.shape), wq)
+        assert np.array_equal(dkc.download(np.uint16, kc.shape), wkc) and np.array_equal(dvc.download(np.uint16, vc.shape), wvc)
+        ctx.sdpa_decode_gated(dq, dkc, dvc, d[0], T, Hq, Hkv, hd, 0 if use_dev_offset else offset, cap, hd ** -0.5, dout, d_offset=doff)
+        assert np.array_equal(dout.download(np.uint16, want.shape), want), use_dev_offset
+        if doff: doff.free()
+    for b in d + [dkc, dvc, dq, dout, dc, ds]: b.free()

@@ -322,3 +322,31 @@ def orc_gdn_recurrence(q, k, v, g, beta, state):
 
 def bf16_normal(rng, shape, std=1.0):
     return f32_to_bf16((rng.standard_normal(shape) * std).astype(np.float32))
+
+
+# ---- attention oracle wrappers -------------------------------------------------------
+def orc_rope_table(npos, dims, theta):
+    half = dims // 2
+    c = np.empty((npos, half), np.float32); s = np.empty((npos, half), np.float32)
+    oracle().orc_rope_table(npos, dims, C.c_double(theta), p(c), p(s))
+    return c, s
+
+
+def orc_attn_prep(qg, kx, vx, qw, kw, rope_dims, cos_t, sin_t, offset, k_cache, v_cache, eps=1e-6):
+    """Appends into k_cache / v_cache (numpy [Hkv, cap, hd]) in place; returns q_rot, gate."""
+    T, Hq, hd2 = qg.shape
+    hd = hd2 // 2
+    Hkv, cap, _ = k_cache.shape
+    q_rot = np.empty((T, Hq, hd), np.uint16); gate = np.empty((T, Hq, hd), np.uint16)
+    oracle().orc_attn_prep(p(qg), p(kx), p(vx), p(qw), p(kw), T, Hq, Hkv, hd, rope_dims, C.c_float(eps),
+                           p(cos_t), p(sin_t), offset, cap, p(q_rot), p(gate), p(k_cache), p(v_cache))
+    return q_rot, gate
+
+
+def orc_sdpa(q_rot, k_cache, v_cache, gate, offset, scale):
+    T, Hq, hd = q_rot.shape
+    Hkv, cap, _ = k_cache.shape
+    out = np.empty((T, Hq * hd), np.uint16)
+    oracle().orc_sdpa_decode_gated(p(q_rot), p(k_cache), p(v_cache), p(gate), T, Hq, Hkv, hd, offset, cap,
+                                   C.c_float(scale), p(out))
+    return out
