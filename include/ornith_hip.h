@@ -217,6 +217,17 @@ ORNITH_API int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, co
                                         int Hkv, int hd, int offset, const int* d_offset, int cap,
                                         float scale, void* d_out);
 
+/* ---- greedy selection: src/ops/sample.rs ------------------------------------------ */
+/* greedy_token / the verify rows of generate_step_mtp (src/ops/sample.rs:134-147,
+ * src/mtp_generate.rs:237-250): tokens[r] = argmax_i bf16(logits[r,i] - lse_r), lowest
+ * index on ties; logits bf16 [rows, V]; d_lse (bf16 [rows]) may be null. */
+ORNITH_API int ornith_greedy_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V,
+                                  uint32_t* d_tokens, void* d_lse);
+/* greedy_argmax_into (src/ops/sample.rs:174-191): argmax of the raw logits, the draft
+ * chain's choice. */
+ORNITH_API int ornith_argmax_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V,
+                                  uint32_t* d_out);
+
 /* ---- self test ------------------------------------------------------------------
  * Evaluates one of the library's scalar device functions element-wise (fp32 in,
  * fp32 out) so their bits can be compared with a CPU evaluation. No reference

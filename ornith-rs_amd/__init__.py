@@ -330,3 +330,15 @@ def sdpa_decode_gated(self, q_rot, k_cache, v_cache, qg, T, Hq, Hkv, hd, offset,
     _check(lib().ornith_sdpa_decode_gated(self.h, q_rot.ptr, k_cache.ptr, v_cache.ptr, qg.ptr, T, Hq, Hkv, hd,
                                           offset, d_offset.ptr if d_offset else None, cap, C.c_float(scale),
                                           out.ptr), "sdpa_decode_gated")
+
+
+# ---- greedy selection ----------------------------------------------------------------
+@_ctx_method
+def greedy_rows(self, logits, rows, V, tokens, lse=None):
+    _check(lib().ornith_greedy_rows(self.h, logits.ptr, rows, V, tokens.ptr, lse.ptr if lse else None),
+           "greedy_rows")
+
+
+@_ctx_method
+def argmax_rows(self, logits, rows, V, out):
+    _check(lib().ornith_argmax_rows(self.h, logits.ptr, rows, V, out.ptr), "argmax_rows")

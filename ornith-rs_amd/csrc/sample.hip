@@ -1,0 +1,171 @@
+// Greedy token selection over the vocabulary.
+//
+// Replaces ops::sample::{greedy_token, greedy_argmax_into, logsumexp_last_axis,
+// argmax_last_axis_into} (/root/reference/src/ops/sample.rs:1-19,37-147,174-191):
+// target rows take argmax(logits - logsumexp(logits)) with the subtraction done in
+// bf16, draft rows take argmax of the raw logits; ties go to the lowest index
+// (vendored arg_reduce.metal:54-64).
+//
+// The vocabulary is cut into chunks of 1024, one workgroup each: pass 1 leaves
+// (max, sum exp) per chunk, pass 2 merges them in ascending chunk order into the
+// row's logsumexp and finds each chunk's best (value, lowest index), pass 3 picks
+// the winner. All of it is wavefront shuffles plus one LDS hop.
+#include "dmath.h"
+#include "rt.h"
+
+namespace {
+
+constexpr int CH = 1024;
+
+__global__ __launch_bounds__(CH) void lse_chunk_kernel(const bf16_t* logits, int V, int nch,
+                                                       float* mc, float* lc) {
+  const int c = blockIdx.x, r = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  __shared__ float red[16];
+  const int i = c * CH + tid;
+  const bool ok = i < V;
+  const float x = ok ? dm_bf2f(logits[(size_t)r * V + i]) : -DM_INF;
+  float m = dm_wave_max<64>(x);
+  if (lane == 0) red[wave] = m;
+  __syncthreads();
+  m = red[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) m = red[w] > m ? red[w] : m;
+  __syncthreads();
+  const float e = ok ? dm_exp(x - m) : 0.f;
+  const float ws = dm_wave_sum<64>(e);
+  if (lane == 0) red[wave] = ws;
+  __syncthreads();
+  if (tid == 0) {
+    float l = red[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) l = l + red[w];
+    mc[(size_t)r * nch + c] = m;
+    lc[(size_t)r * nch + c] = l;
+  }
+}
+
+// (value, index) max with lowest index on ties
+__device__ __forceinline__ void best_merge(float& v, int& i, float ov, int oi) {
+  if (ov > v || (ov == v && oi < i)) {
+    v = ov;
+    i = oi;
+  }
+}
+
+// pass 2: per chunk. USE_LSE: value = bf16(x - lse), else raw x.
+template <bool USE_LSE>
+__global__ __launch_bounds__(CH) void argmax_chunk_kernel(const bf16_t* logits, int V, int nch,
+                                                          const float* mc, const float* lc,
+                                                          float* bv, int* bi, bf16_t* lse_out) {
+  const int c = blockIdx.x, r = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  __shared__ float sv[16];
+  __shared__ int si[16];
+  __shared__ float s_lse;
+  float lse = 0.f;
+  if constexpr (USE_LSE) {
+    // every workgroup repeats the (short, sequential) merge: cheaper than another launch
+    __shared__ float smax[16];
+    float m = -DM_INF;
+    for (int k = tid; k < nch; k += CH) m = mc[(size_t)r * nch + k] > m ? mc[(size_t)r * nch + k] : m;
+    m = dm_wave_max<64>(m);
+    if (lane == 0) smax[wave] = m;
+    __syncthreads();
+    if (tid == 0) {
+      float M = smax[0];
+      for (int w = 1; w < 16; ++w) M = smax[w] > M ? smax[w] : M;
+      float L = 0.f;
+      for (int k = 0; k < nch; ++k)
+        L = dm_fma(lc[(size_t)r * nch + k], dm_exp(mc[(size_t)r * nch + k] - M), L);
+      s_lse = dm_rb(dm_log(L) + M);
+      if (c == 0 && lse_out) lse_out[r] = dm_f2bf(s_lse);
+    }
+    __syncthreads();
+    lse = s_lse;
+  }
+  const int i = c * CH + tid;
+  float v = -DM_INF;
+  int idx = 0x7fffffff;
+  if (i < V) {
+    const float x = dm_bf2f(logits[(size_t)r * V + i]);
+    v = USE_LSE ? dm_rb(x - lse) : x;
+    idx = i;
+    if (v != v) v = -DM_INF;  // NaN never wins
+  }
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) {
+    const float ov = __shfl_xor(v, s, 64);
+    const int oi = __shfl_xor(idx, s, 64);
+    best_merge(v, idx, ov, oi);
+  }
+  if (lane == 0) {
+    sv[wave] = v;
+    si[wave] = idx;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; ++w) best_merge(v, idx, sv[w], si[w]);
+    bv[(size_t)r * nch + c] = v;
+    bi[(size_t)r * nch + c] = idx;
+  }
+}
+
+// pass 3: one wavefront per row over the chunk winners
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* bv, const int* bi, int nch,
+                                                          int V, uint32_t* out) {
+  const int r = blockIdx.x, lane = threadIdx.x;
+  float v = -DM_INF;
+  int idx = 0x7fffffff;
+  for (int k = lane; k < nch; k += 64) best_merge(v, idx, bv[(size_t)r * nch + k], bi[(size_t)r * nch + k]);
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) {
+    const float ov = __shfl_xor(v, s, 64);
+    const int oi = __shfl_xor(idx, s, 64);
+    best_merge(v, idx, ov, oi);
+  }
+  if (lane == 0) out[r] = (idx >= 0 && idx < V) ? (uint32_t)idx : 0u;
+}
+
+int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens, void* d_lse,
+        bool use_lse, const char* who) {
+  ORN_REQUIRE(ctx && d_logits && d_tokens, "%s: null argument", who);
+  ORN_REQUIRE(rows >= 1 && rows <= 65535 && V >= 1, "%s: rows=%d V=%d", who, rows, V);
+  const int nch = (V + CH - 1) / CH;
+  void* base = nullptr;
+  int rc = ornith_scratch(ctx, (size_t)rows * nch * 16 + 2048, &base);
+  if (rc) return rc;
+  ScratchCursor sc(base);
+  float* mc = sc.take<float>((size_t)rows * nch);
+  float* lc = sc.take<float>((size_t)rows * nch);
+  float* bv = sc.take<float>((size_t)rows * nch);
+  int* bi = sc.take<int>((size_t)rows * nch);
+  const bf16_t* lg = (const bf16_t*)d_logits;
+  if (use_lse) {
+    hipLaunchKernelGGL(lse_chunk_kernel, dim3(nch, rows), dim3(CH), 0, ctx->stream, lg, V, nch, mc, lc);
+    ORN_LAUNCH_CHECK("lse_chunk_kernel");
+    hipLaunchKernelGGL(argmax_chunk_kernel<true>, dim3(nch, rows), dim3(CH), 0, ctx->stream, lg, V,
+                       nch, mc, lc, bv, bi, (bf16_t*)d_lse);
+  } else {
+    hipLaunchKernelGGL(argmax_chunk_kernel<false>, dim3(nch, rows), dim3(CH), 0, ctx->stream, lg, V,
+                       nch, mc, lc, bv, bi, (bf16_t*)nullptr);
+  }
+  ORN_LAUNCH_CHECK("argmax_chunk_kernel");
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, ctx->stream, bv, bi, nch, V,
+                     d_tokens);
+  ORN_LAUNCH_CHECK("argmax_final_kernel");
+  return ORNITH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ornith_greedy_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens,
+                       void* d_lse) {
+  return run(ctx, d_logits, rows, V, d_tokens, d_lse, true, "greedy_rows");
+}
+
+int ornith_argmax_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_out) {
+  return run(ctx, d_logits, rows, V, d_out, nullptr, false, "argmax_rows");
+}
+
+}  // extern "C"
