@@ -152,6 +152,12 @@ typedef struct ornith_moe_weights {
   ornith_linear sh_egate;                  /* mlp.shared_expert_gate [1,H] */
   int top_k;
   int norm_topk_prob;
+  /* the MTP head's block (sparse_moe_block_dense, src/ops/moe.rs:863-937): experts are
+   * stacked dense bf16 [E,O,K]; ex_* above then carry the dims only. */
+  int ex_dense;
+  const void* d_ex_gate;
+  const void* d_ex_up;
+  const void* d_ex_down;
 } ornith_moe_weights;
 
 /* moe::sparse_moe_block (src/ops/moe.rs:662-741): x bf16 [T,H] -> out bf16 [T,H].
@@ -187,12 +193,13 @@ ORNITH_API int ornith_gdn_front(ornith_ctx* ctx, const void* d_conv_state, const
  * (src/ops/gdn.rs:131-271, kernels/gated_delta.metal:36-142, qwen3_5.rs:650-677):
  * state_in f32[Hv,Dv,Dk] -> y bf16[T,Hv,Dv] and one state snapshot per token,
  * d_snapshots f32[T][Hv,Dv,Dk]; snapshot T-1 is the new state, snapshot keep-1 is
- * the state to continue from after accepting keep tokens. With T == 1 d_snapshots may
- * alias d_state_in. */
+ * the state to continue from after accepting keep tokens. With snapshot_every_token == 0
+ * (plain forward, no rollback wanted) only the final state is written, to slot 0.
+ * d_snapshots may alias d_state_in: a lane reads its state elements before it writes. */
 ORNITH_API int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k,
                                      const void* d_v, const float* d_g, const void* d_beta,
                                      const float* d_state_in, int T, int Hk, int Hv, int Dk, int Dv,
-                                     void* d_y, float* d_snapshots);
+                                     void* d_y, float* d_snapshots, int snapshot_every_token);
 
 /* ---- full-attention layer at decode / verify width ------------------------------ */
 /* ops::rope tables (src/ops/rope.rs:6-60): cos/sin f32 [npos, dims/2] for
@@ -227,6 +234,131 @@ ORNITH_API int ornith_greedy_rows(ornith_ctx* ctx, const void* d_logits, int row
  * chain's choice. */
 ORNITH_API int ornith_argmax_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V,
                                   uint32_t* d_out);
+
+/* ---- weights: WeightStore (src/weights.rs:41-279) -------------------------------
+ * A named-tensor store on the device. Names are the reference's
+ * (language_model.model.layers.N.linear_attn.in_proj_qkv.weight, ...). A module
+ * <path> is k-quant if it has <path>.dm (Q4_K when scales are 12 bytes a block,
+ * Q6_K when 16; .weight may be u32 or u8, same bytes), 8-bit affine if it has
+ * <path>.biases, dense bf16 otherwise -- the same three-way dispatch as
+ * WeightStore::linear (src/weights.rs:179-184). */
+#define ORNITH_DT_F32 0
+#define ORNITH_DT_BF16 1
+#define ORNITH_DT_F16 2
+#define ORNITH_DT_U8 3
+#define ORNITH_DT_U32 4
+#define ORNITH_DT_I32 5
+typedef struct ornith_weights ornith_weights;
+ORNITH_API int ornith_weights_create(ornith_ctx* ctx, ornith_weights** out);
+/* WeightStore::tensor: copies host_data to the device and records it under `name`. */
+ORNITH_API int ornith_weights_put(ornith_weights* ws, const char* name, int dtype,
+                                  const int64_t* shape, int ndim, const void* host_data);
+ORNITH_API int ornith_weights_destroy(ornith_weights* ws);
+/* number of tensors held and their total bytes (the loader's report, src/main.rs:483-488) */
+ORNITH_API int ornith_weights_stats(const ornith_weights* ws, int64_t* n_tensors, int64_t* bytes);
+
+/* TextConfig (src/model/config.rs:46-134), the fields this path reads. */
+typedef struct ornith_text_config {
+  int hidden_size, num_hidden_layers, vocab_size;
+  int num_experts, num_experts_per_tok, moe_intermediate_size, shared_expert_intermediate_size;
+  int linear_num_key_heads, linear_num_value_heads, linear_key_head_dim, linear_value_head_dim;
+  int linear_conv_kernel_dim;
+  int num_attention_heads, num_key_value_heads, head_dim, rope_dims;
+  int full_attention_interval; /* layer i is full attention iff (i+1) % interval == 0 */
+  int norm_topk_prob;
+  float rms_norm_eps;
+  double rope_theta;
+} ornith_text_config;
+
+/* ---- model: TextModel (src/model/qwen3_5.rs:102-279), caches (src/model/cache.rs) */
+typedef struct ornith_model ornith_model;
+typedef struct ornith_caches ornith_caches;
+/* TextModel::load: resolves every tensor by name; the store must outlive the model. */
+ORNITH_API int ornith_model_load(ornith_ctx* ctx, const ornith_weights* ws,
+                                 const ornith_text_config* cfg, ornith_model** out);
+ORNITH_API int ornith_model_destroy(ornith_model* m);
+/* make_cache: one KvCache (bf16 [Hkv, capacity, hd] x2) or GdnCache (conv window +
+ * fp32 state with max_window snapshot slots) per layer. capacity bounds prompt +
+ * generated tokens (the reference grows in steps of 256; here it is fixed up front). */
+ORNITH_API int ornith_caches_create(ornith_model* m, int capacity, int max_window,
+                                    ornith_caches** out);
+ORNITH_API int ornith_caches_reset(ornith_caches* c);
+ORNITH_API int ornith_caches_destroy(ornith_caches* c);
+ORNITH_API int ornith_caches_offset(const ornith_caches* c, int* offset_out);
+/* TextModel::forward_hidden (capture = 0) / forward_capture (capture = 1): T tokens
+ * (device u32) through the trunk; writes the post-norm hidden rows bf16 [T, H] and
+ * advances the caches by T. With capture, T <= max_window and every gated-delta layer
+ * keeps a state snapshot per token so ornith_model_rewind can take rows back. */
+ORNITH_API int ornith_model_forward(ornith_model* m, ornith_caches* c, const uint32_t* d_tokens, int T,
+                                    int capture, void* d_hidden_out);
+/* TrunkCapture::rewind (src/model/qwen3_5.rs:324-348): after a captured forward of T
+ * tokens keep only the first `keep` (1 <= keep <= T). Pointer moves only. */
+ORNITH_API int ornith_model_rewind(ornith_model* m, ornith_caches* c, int keep);
+/* lm_head.matmul: hidden bf16 [T, H] -> logits bf16 [T, vocab]. */
+ORNITH_API int ornith_model_logits(ornith_model* m, const void* d_hidden, int T, void* d_logits);
+
+/* ---- FR-Spec: FrSpec (src/frspec.rs:38-158) ----------------------------------------- */
+typedef struct ornith_frspec ornith_frspec;
+/* FrSpec::load: file = u32 n, then n x u32 LE; rejects n == 0, n >= vocab, ids out of
+ * range, duplicates. FrSpec::prune: row-gathers lm_head's tensors into an n-row head. */
+ORNITH_API int ornith_frspec_load(ornith_model* m, const char* path, ornith_frspec** out);
+ORNITH_API int ornith_frspec_from_ids(ornith_model* m, const uint32_t* ids, int n, ornith_frspec** out);
+ORNITH_API int ornith_frspec_destroy(ornith_frspec* f);
+/* the pruned head as a Linear (for tests: pruned row == original row) and its size */
+ORNITH_API int ornith_frspec_head(const ornith_frspec* f, ornith_linear* head_out, int* n_out);
+
+/* ---- MTP head: MtpHead (src/model/mtp.rs:96-268) ----------------------------------- */
+typedef struct ornith_mtp_head ornith_mtp_head;
+/* MtpHead::load from the mtp.* tensors (dense bf16); owns a one-layer KV cache. */
+ORNITH_API int ornith_mtp_load(ornith_model* m, const ornith_weights* ws, int capacity,
+                               ornith_mtp_head** out);
+ORNITH_API int ornith_mtp_destroy(ornith_mtp_head* h);
+/* MtpHead::hidden / forward: T rows of trunk hidden + the T token ids that follow them
+ * -> post-norm hidden bf16 [T, H] (and, if d_logits != null, logits through the pruned
+ * head when `frspec` != null, else through lm_head). Appends T rows to the head's cache. */
+ORNITH_API int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspec,
+                                  const void* d_trunk_hidden, const uint32_t* d_next_ids, int T,
+                                  void* d_hidden_out, void* d_logits);
+ORNITH_API int ornith_mtp_cache_set_offset(ornith_mtp_head* h, int offset);
+ORNITH_API int ornith_mtp_cache_offset(const ornith_mtp_head* h, int* offset_out);
+
+/* ---- generation loops ---------------------------------------------------------------- */
+/* Sampler (src/generate.rs:36-64, src/sample.rs:205-225). rows_are_independent is
+ * true for GREEDY. */
+#define ORNITH_SAMPLER_GREEDY 0
+#define ORNITH_SAMPLER_TOP_P 1
+typedef struct ornith_sampler {
+  int kind;
+  float temperature, top_p;
+  int top_k;
+  uint64_t seed;
+} ornith_sampler;
+/* on_token: return 0 to stop (FnMut(u32) -> bool); progress: (done, total) prompt tokens */
+typedef int (*ornith_token_cb)(uint32_t token, void* user);
+typedef void (*ornith_progress_cb)(size_t done, size_t total, void* user);
+
+/* generate::generate_step (src/generate.rs:162-206): prefill all but the last prompt
+ * token in chunks of prefill_step, then one step per token; the caches end holding the
+ * prompt plus exactly the tokens shown to on_token. */
+ORNITH_API int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, size_t n_prompt,
+                               const ornith_sampler* sampler, size_t max_tokens, size_t prefill_step,
+                               ornith_progress_cb progress, ornith_token_cb on_token, void* user);
+
+#define ORNITH_HISTORY_CYCLE 0     /* HistoryPolicy::Cycle */
+#define ORNITH_HISTORY_COMMITTED 1 /* HistoryPolicy::Committed (the CLI default) */
+#define ORNITH_MAX_DEPTH 8
+typedef struct ornith_mtp_stats { /* MtpStats (src/mtp_generate.rs:66-84) */
+  size_t cycles, drafted, accepted;
+  size_t reached_by_depth[ORNITH_MAX_DEPTH], accepted_by_depth[ORNITH_MAX_DEPTH];
+} ornith_mtp_stats;
+/* mtp_generate::generate_step_mtp (src/mtp_generate.rs:150-317): draft `depth` tokens
+ * with the MTP head (through the FR-Spec head if frspec != null), verify depth+1 rows in
+ * one trunk forward, accept the leading run of equal tokens, rewind, repeat. */
+ORNITH_API int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frspec* frspec,
+                                   ornith_caches* c, const uint32_t* prompt, size_t n_prompt,
+                                   const ornith_sampler* sampler, int depth, size_t max_tokens,
+                                   size_t prefill_step, int policy, ornith_progress_cb progress,
+                                   ornith_token_cb on_token, void* user, ornith_mtp_stats* stats_out);
 
 /* ---- self test ------------------------------------------------------------------
  * Evaluates one of the library's scalar device functions element-wise (fp32 in,

@@ -9,6 +9,7 @@
  * vendored quantized.h:283-289,756-821 (8-bit affine mat-vec).
  */
 #include "orc_common.h"
+#include "orc_types.h"
 
 float orc_kq_row_dot(int kind, const uint8_t* qs, const uint8_t* scales, const f16_t* dm, int K,
                      int64_t row, const float* x);
@@ -153,20 +154,7 @@ ORC_API void orc_embedding(const uint8_t* w, const bf16_t* scales, const bf16_t*
 }
 
 /* ---- the whole block ------------------------------------------------------- */
-typedef struct orc_kmat {
-  int kind, E, O, K;
-  const uint8_t* qs;
-  const uint8_t* scales;
-  const f16_t* dm;
-} orc_kmat;
 
-typedef struct orc_linear {
-  int mode; /* 0 = k-quant (km), 1 = 8-bit affine g64, 2 = dense bf16 */
-  orc_kmat km;
-  const uint8_t* aw; /* affine: u8[O,K]; dense: bf16[O,K] */
-  const bf16_t* as;
-  const bf16_t* ab;
-} orc_linear;
 
 float orc_dense_row_dot(const bf16_t* w, int K, const float* x);
 
@@ -192,15 +180,7 @@ void orc_linear_fwd(const orc_linear* L, const bf16_t* x, int M, bf16_t* y) {
   free(xf);
 }
 
-typedef struct orc_moe_weights {
-  orc_linear router;             /* [E, H] */
-  orc_kmat ex_gate, ex_up;       /* [E, I, H] */
-  orc_kmat ex_down;              /* [E, H, I] */
-  orc_linear sh_gate, sh_up;     /* [I, H] */
-  orc_linear sh_down;            /* [H, I] */
-  orc_linear sh_egate;           /* [1, H] */
-  int top_k, normalize;
-} orc_moe_weights;
+
 
 /* x [T,H] bf16 -> out [T,H] bf16; also returns router picks for the index check.
  * Optional taps (may be NULL): probs [T,E], act [T*k, I], ydown [T*k, H]. */

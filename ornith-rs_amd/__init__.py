@@ -192,7 +192,8 @@ class MoeWeightsStruct(C.Structure):
     _fields_ = [("router", LinearStruct), ("ex_gate", KMatrixStruct), ("ex_up", KMatrixStruct),
                 ("ex_down", KMatrixStruct), ("sh_gate", LinearStruct), ("sh_up", LinearStruct),
                 ("sh_down", LinearStruct), ("sh_egate", LinearStruct), ("top_k", C.c_int),
-                ("norm_topk_prob", C.c_int)]
+                ("norm_topk_prob", C.c_int), ("ex_dense", C.c_int), ("d_ex_gate", C.c_void_p),
+                ("d_ex_up", C.c_void_p), ("d_ex_down", C.c_void_p)]
 
 
 class Linear:
@@ -301,9 +302,9 @@ def gdn_front(self, conv_state, qkv, cw, a, b, a_log, dt_bias, T, K, Hk, Dk, Hv,
 
 
 @_ctx_method
-def gdn_recurrence(self, q, k, v, g, beta, state_in, T, Hk, Hv, Dk, Dv, y, snapshots):
+def gdn_recurrence(self, q, k, v, g, beta, state_in, T, Hk, Hv, Dk, Dv, y, snapshots, snap_all=True):
     _check(lib().ornith_gdn_recurrence(self.h, q.ptr, k.ptr, v.ptr, g.ptr, beta.ptr, state_in.ptr, T, Hk, Hv,
-                                       Dk, Dv, y.ptr, snapshots.ptr), "gdn_recurrence")
+                                       Dk, Dv, y.ptr, snapshots.ptr, int(snap_all)), "gdn_recurrence")
 
 
 # ---- attention ---------------------------------------------------------------------
@@ -342,3 +343,7 @@ def greedy_rows(self, logits, rows, V, tokens, lse=None):
 @_ctx_method
 def argmax_rows(self, logits, rows, V, out):
     _check(lib().ornith_argmax_rows(self.h, logits.ptr, rows, V, out.ptr), "argmax_rows")
+
+
+from .engine import *  # noqa: E402,F401,F403  (engine objects: WeightStore, TextModel, ...)
+from .engine import TextConfig, Sampler, MtpStats, WeightStore, Caches, TextModel, FrSpec, MtpHead, generate_step, generate_step_mtp, HISTORY_CYCLE, HISTORY_COMMITTED  # noqa: E402,F401

@@ -1,0 +1,246 @@
+// The two generation loops.
+//
+// Mirrors generate::{prefill, step, generate_step}
+// (/root/reference/src/generate.rs:86-206) and mtp_generate::{draft,
+// generate_step_mtp} (/root/reference/src/mtp_generate.rs:99-317): same order of
+// model calls, same points at which a token is handed to the caller, same cache
+// contract (on return the caches hold the prompt plus exactly the tokens shown to
+// on_token), same statistics. One blocking read-back per speculative cycle.
+#include <algorithm>
+#include <vector>
+
+#include "model.h"
+
+#define TRY(e)             \
+  do {                     \
+    int rc__ = (e);        \
+    if (rc__) return rc__; \
+  } while (0)
+
+namespace {
+
+// FrSpec::map_id (src/frspec.rs:140-142): dst = ids[local], one thread
+__global__ void map_id_kernel(const uint32_t* ids, int n, const uint32_t* local, uint32_t* dst) {
+  const uint32_t l = *local;
+  *dst = ids[l < (uint32_t)n ? l : (uint32_t)(n - 1)];
+}
+
+// device buffers a generation call needs, freed on scope exit
+struct Bufs {
+  ornith_ctx* ctx;
+  std::vector<void*> all;
+  explicit Bufs(ornith_ctx* c) : ctx(c) {}
+  ~Bufs() {
+    for (void* p : all) ornith_free(ctx, p);
+  }
+  int get(size_t bytes, void** out) {
+    int rc = ornith_alloc(ctx, bytes, out);
+    if (!rc) all.push_back(*out);
+    return rc;
+  }
+};
+
+int check_sampler(const ornith_sampler* s) {
+  ORN_REQUIRE(s, "sampler is null");
+  if (s->kind == ORNITH_SAMPLER_GREEDY) return ORNITH_OK;
+  return ornith_fail(ORNITH_ERR_UNSUPPORTED,
+                     "sampler kind %d: only the greedy sampler is built in this library so far",
+                     s->kind);
+}
+
+// prefill (src/generate.rs:90-136): everything but the last token, in chunks
+int prefill(ornith_model* m, ornith_caches* c, const uint32_t* prompt, size_t total, size_t step,
+            uint32_t* d_tok, void* d_hidden, ornith_progress_cb progress, void* user,
+            size_t* processed_out) {
+  size_t processed = 0;
+  if (progress) progress(0, total, user);
+  const size_t chunk = std::max<size_t>(1, std::min<size_t>(step, (size_t)m->max_rows));
+  while (total - processed > 1) {
+    const size_t n = std::min(chunk, total - processed - 1);
+    TRY(ornith_upload(m->ctx, d_tok, prompt + processed, n * 4));
+    TRY(ornith_model_forward(m, c, d_tok, (int)n, 0, d_hidden));
+    TRY(ornith_sync(m->ctx));
+    processed += n;
+    if (progress) progress(processed, total, user);
+  }
+  *processed_out = processed;
+  return ORNITH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, size_t n_prompt,
+                    const ornith_sampler* sampler, size_t max_tokens, size_t prefill_step,
+                    ornith_progress_cb progress, ornith_token_cb on_token, void* user) {
+  ORN_REQUIRE(m && c && prompt && on_token, "generate: null argument");
+  ORN_REQUIRE(n_prompt >= 1, "generate_step needs a prompt");
+  TRY(check_sampler(sampler));
+  ornith_ctx* ctx = m->ctx;
+  const size_t H = m->cfg.hidden_size, V = m->cfg.vocab_size, R = m->max_rows;
+  Bufs b(ctx);
+  uint32_t *d_tok, *d_out;
+  void *d_hidden, *d_logits;
+  TRY(b.get(R * 4, (void**)&d_tok));
+  TRY(b.get(4, (void**)&d_out));
+  TRY(b.get(R * H * 2, &d_hidden));
+  TRY(b.get(V * 2, &d_logits));
+
+  size_t processed = 0;
+  TRY(prefill(m, c, prompt, n_prompt, prefill_step, d_tok, d_hidden, progress, user, &processed));
+  // step(): run the remaining prompt tokens and sample from the last position
+  auto step = [&](const uint32_t* toks, size_t n, uint32_t* y) -> int {
+    TRY(ornith_upload(ctx, d_tok, toks, n * 4));
+    TRY(ornith_model_forward(m, c, d_tok, (int)n, 0, d_hidden));
+    TRY(ornith_model_logits(m, (char*)d_hidden + (n - 1) * H * 2, 1, d_logits));
+    TRY(ornith_greedy_rows(ctx, d_logits, 1, (int)V, d_out, nullptr));
+    return ornith_download(ctx, y, d_out, 4);
+  };
+  uint32_t y = 0;
+  TRY(step(prompt + processed, n_prompt - processed, &y));
+  if (progress) progress(n_prompt, n_prompt, user);
+  size_t n = 0;
+  for (;;) {
+    if (n == max_tokens) return ORNITH_OK;
+    uint32_t next = 0;
+    TRY(step(&y, 1, &next));
+    if (!on_token(y, user)) return ORNITH_OK;
+    y = next;
+    ++n;
+  }
+}
+
+int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frspec* frspec,
+                        ornith_caches* c, const uint32_t* prompt, size_t n_prompt,
+                        const ornith_sampler* sampler, int depth, size_t max_tokens,
+                        size_t prefill_step, int policy, ornith_progress_cb progress,
+                        ornith_token_cb on_token, void* user, ornith_mtp_stats* stats_out) {
+  ORN_REQUIRE(m && head && c && prompt && on_token, "mtp_generate: null argument");
+  ORN_REQUIRE(depth >= 1, "MTP depth must be at least 1");
+  ORN_REQUIRE(depth <= ORNITH_MAX_DEPTH && depth + 1 <= c->max_window,
+              "mtp_generate: depth %d needs a capture window of %d rows (caches have %d)", depth,
+              depth + 1, c->max_window);
+  ORN_REQUIRE(n_prompt >= 1, "generate_step_mtp needs a prompt");
+  ORN_REQUIRE(max_tokens >= 1, "mtp_generate: max_tokens must be at least 1");
+  ORN_REQUIRE(policy == ORNITH_HISTORY_CYCLE || policy == ORNITH_HISTORY_COMMITTED,
+              "mtp_generate: unknown history policy %d", policy);
+  ORN_REQUIRE(head->m == m && (!frspec || frspec->m == m), "mtp_generate: head / frspec of another model");
+  TRY(check_sampler(sampler));
+  ornith_ctx* ctx = m->ctx;
+  const size_t H = m->cfg.hidden_size, V = m->cfg.vocab_size, R = m->max_rows;
+  ornith_mtp_stats stats{};
+
+  Bufs b(ctx);
+  uint32_t *d_tok, *d_window, *d_targets, *d_local;
+  void *d_hidden, *d_h, *d_vlogits, *d_dlogits, *d_mh, *d_scratch_h;
+  const size_t W = (size_t)depth + 1;
+  TRY(b.get(R * 4, (void**)&d_tok));
+  TRY(b.get(W * 4, (void**)&d_window));
+  TRY(b.get(W * 4, (void**)&d_targets));
+  TRY(b.get(4, (void**)&d_local));
+  TRY(b.get(R * H * 2, &d_hidden));
+  TRY(b.get(H * 2, &d_h));
+  TRY(b.get(W * V * 2, &d_vlogits));
+  TRY(b.get(V * 2, &d_dlogits));
+  TRY(b.get(W * H * 2, &d_mh));
+  TRY(b.get(W * H * 2, &d_scratch_h));
+
+  size_t processed = 0;
+  TRY(prefill(m, c, prompt, n_prompt, prefill_step, d_tok, d_hidden, progress, user, &processed));
+  const size_t rows = n_prompt - processed;
+  TRY(ornith_upload(ctx, d_tok, prompt + processed, rows * 4));
+  TRY(ornith_model_forward(m, c, d_tok, (int)rows, 0, d_hidden));
+  if (progress) progress(n_prompt, n_prompt, user);
+  TRY(ornith_model_logits(m, (char*)d_hidden + (rows - 1) * H * 2, 1, d_vlogits));
+  TRY(ornith_greedy_rows(ctx, d_vlogits, 1, (int)V, d_targets, nullptr));
+  uint32_t primary = 0;
+  TRY(ornith_download(ctx, &primary, d_targets, 4));
+  TRY(ornith_copy(ctx, d_h, (char*)d_hidden + (rows - 1) * H * 2, H * 2));
+
+  size_t emitted = 0;
+  TRY(ornith_mtp_cache_set_offset(head, 0));  // make_mtp_cache()
+  const int draft_vocab = frspec ? frspec->n : (int)V;
+  std::vector<uint32_t> win(W), targets(W);
+  for (;;) {
+    if (policy == ORNITH_HISTORY_CYCLE) TRY(ornith_mtp_cache_set_offset(head, 0));
+    const int cycle_mtp_offset = head->offset;
+    const size_t left = max_tokens > emitted + 1 ? max_tokens - (emitted + 1) : 0;
+    const int want = (int)std::min<size_t>((size_t)depth, left);
+
+    // draft(): `want` chained head forwards, entirely on the device
+    std::fill(win.begin(), win.end(), 0u);
+    win[0] = primary;
+    TRY(ornith_upload(ctx, d_window, win.data(), W * 4));
+    const void* hcur = d_h;
+    for (int i = 0; i < want; ++i) {
+      void* hid = (char*)d_mh + (size_t)i * H * 2;
+      TRY(ornith_mtp_forward(head, frspec, hcur, d_window + i, 1, hid, d_dlogits));
+      if (frspec) {
+        TRY(ornith_argmax_rows(ctx, d_dlogits, 1, draft_vocab, d_local));
+        hipLaunchKernelGGL(map_id_kernel, dim3(1), dim3(1), 0, ctx->stream, frspec->d_ids, frspec->n,
+                           d_local, d_window + i + 1);
+        ORN_LAUNCH_CHECK("map_id_kernel");
+      } else {
+        TRY(ornith_argmax_rows(ctx, d_dlogits, 1, draft_vocab, d_window + i + 1));
+      }
+      hcur = hid;
+    }
+    if (want > 0) {
+      stats.cycles += 1;
+      stats.drafted += want;
+    }
+
+    // verify: one trunk forward over [primary] + drafts, every row's target at once
+    const int n_rows = want + 1;
+    TRY(ornith_model_forward(m, c, d_window, n_rows, 1, d_hidden));
+    TRY(ornith_model_logits(m, d_hidden, n_rows, d_vlogits));
+    TRY(ornith_greedy_rows(ctx, d_vlogits, n_rows, (int)V, d_targets, nullptr));
+    TRY(ornith_download(ctx, targets.data(), d_targets, (size_t)n_rows * 4));  // the cycle's one sync
+    TRY(ornith_download(ctx, win.data(), d_window, (size_t)n_rows * 4));
+
+    // accept the leading run of agreements
+    int k = 0;
+    bool have_next = false;
+    uint32_t next_primary = 0;
+    while (k < want) {
+      const uint32_t target = targets[k];
+      stats.reached_by_depth[k] += 1;
+      if (target != win[1 + k]) {
+        next_primary = target;
+        have_next = true;
+        break;
+      }
+      stats.accepted_by_depth[k] += 1;
+      stats.accepted += 1;
+      ++k;
+    }
+    if (!have_next) next_primary = targets[k];  // the bonus token
+
+    // the window put want+1 tokens into the caches; k+1 of them are committed
+    TRY(ornith_model_rewind(m, c, k + 1));
+    if (policy == ORNITH_HISTORY_COMMITTED) {
+      // keep the level-1 row (it drafted from the trunk's hidden), rebuild the rest
+      // from what the verify pass actually saw
+      TRY(ornith_mtp_cache_set_offset(head, std::min(cycle_mtp_offset + 1, head->capacity)));
+      if (k > 0) TRY(ornith_mtp_forward(head, nullptr, d_hidden, d_window + 1, k, d_scratch_h, nullptr));
+    }
+    TRY(ornith_copy(ctx, d_h, (char*)d_hidden + (size_t)k * H * 2, H * 2));
+
+    for (int i = 0; i <= k; ++i) {
+      const uint32_t t = i == 0 ? primary : win[i];
+      if (!on_token(t, user)) {
+        if (stats_out) *stats_out = stats;
+        return ORNITH_OK;
+      }
+      ++emitted;
+      if (emitted == max_tokens) {
+        if (stats_out) *stats_out = stats;
+        return ORNITH_OK;
+      }
+    }
+    primary = next_primary;
+  }
+}
+
+}  // extern "C"

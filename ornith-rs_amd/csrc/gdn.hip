@@ -113,6 +113,7 @@ struct RecArgs {
   bf16_t* y;              // [T, Hv, Dv]
   float* snapshots;       // [T][Hv, Dv, 128]
   int T, Hk, Hv, Dv;
+  int snap_all;  // 1: a snapshot per token; 0: only the final state, in slot 0
 };
 
 __global__ __launch_bounds__(64) void gdn_recurrence_kernel(RecArgs p) {
@@ -166,11 +167,13 @@ __global__ __launch_bounds__(64) void gdn_recurrence_kernel(RecArgs p) {
     }
     o = dm_wave_sum<8>(o);
     if (j == 0) p.y[((size_t)t * p.Hv + hv) * p.Dv + dv] = dm_f2bf(o);
-    float* snap = p.snapshots + (size_t)t * ssz + roff;
+    if (p.snap_all || t + 1 == p.T) {
+      float* snap = p.snapshots + (p.snap_all ? (size_t)t * ssz : 0) + roff;
 #pragma unroll
-    for (int m = 0; m < 4; ++m)
-      *reinterpret_cast<float4*>(snap + 32 * m) =
-          make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+      for (int m = 0; m < 4; ++m)
+        *reinterpret_cast<float4*>(snap + 32 * m) =
+            make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+    }
   }
 }
 
@@ -227,14 +230,16 @@ int ornith_gdn_front(ornith_ctx* ctx, const void* d_conv_state, const void* d_qk
 
 int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, const void* d_v,
                           const float* d_g, const void* d_beta, const float* d_state_in, int T,
-                          int Hk, int Hv, int Dk, int Dv, void* d_y, float* d_snapshots) {
+                          int Hk, int Hv, int Dk, int Dv, void* d_y, float* d_snapshots,
+                          int snapshot_every_token) {
   ORN_REQUIRE(ctx && d_q && d_k && d_v && d_g && d_beta && d_state_in && d_y && d_snapshots,
               "gdn_recurrence: null argument");
   ORN_REQUIRE(Dk == 128 && Dv % 8 == 0 && Dv >= 8, "gdn_recurrence: Dk=%d Dv=%d", Dk, Dv);
   ORN_REQUIRE(T >= 1 && Hk >= 1 && Hv >= Hk && Hv % Hk == 0 && Hv <= 65535,
               "gdn_recurrence: T=%d Hk=%d Hv=%d", T, Hk, Hv);
   RecArgs p{(const bf16_t*)d_q, (const bf16_t*)d_k, (const bf16_t*)d_v, d_g, (const bf16_t*)d_beta,
-            d_state_in,         (bf16_t*)d_y,       d_snapshots,        T,   Hk, Hv, Dv};
+            d_state_in,         (bf16_t*)d_y,       d_snapshots,        T,   Hk, Hv, Dv,
+            snapshot_every_token ? 1 : 0};
   hipLaunchKernelGGL(gdn_recurrence_kernel, dim3(Dv / 8, Hv), dim3(64), 0, ctx->stream, p);
   ORN_LAUNCH_CHECK("gdn_recurrence_kernel");
   return ORNITH_OK;

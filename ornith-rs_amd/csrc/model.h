@@ -1,0 +1,125 @@
+// Host-side model objects: the named-tensor store, the trunk, the MTP head, the
+// caches and the FR-Spec head. Mirrors WeightStore (/root/reference/src/weights.rs),
+// TextModel / DecoderLayer / GatedDeltaNet / Attention
+// (/root/reference/src/model/qwen3_5.rs), MtpHead (/root/reference/src/model/mtp.rs),
+// KvCache / GdnCache (/root/reference/src/model/cache.rs) and FrSpec
+// (/root/reference/src/frspec.rs). Everything here is host bookkeeping over device
+// pointers; the arithmetic lives in the .hip files.
+#pragma once
+
+#include <map>
+#include <string>
+#include <vector>
+
+#include "rt.h"
+
+struct Tensor {
+  int dtype = 0;
+  std::vector<int64_t> shape;
+  void* d = nullptr;
+  size_t bytes = 0;
+  int64_t numel() const {
+    int64_t n = 1;
+    for (auto s : shape) n *= s;
+    return n;
+  }
+};
+
+struct ornith_weights {
+  ornith_ctx* ctx = nullptr;
+  std::map<std::string, Tensor> t;
+  size_t total_bytes = 0;
+  const Tensor* find(const std::string& name) const {
+    auto it = t.find(name);
+    return it == t.end() ? nullptr : &it->second;
+  }
+};
+
+// Resolves module `path` into a Linear by the tensors present (k-quant / affine8 / dense).
+int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* out);
+// A routed k-quant module [E, O, K].
+int ws_kmatrix(const ornith_weights* ws, const std::string& path, ornith_kmatrix* out);
+// A plain tensor with an expected element count and dtype.
+int ws_tensor(const ornith_weights* ws, const std::string& name, int dtype, int64_t numel,
+              const void** out);
+
+struct GdnLayer {
+  ornith_linear in_proj_qkv, in_proj_z, out_proj, in_proj_a, in_proj_b;
+  const void *conv1d, *dt_bias, *a_log, *norm;
+};
+struct AttnLayer {
+  ornith_linear q_proj, k_proj, v_proj, o_proj;
+  const void *q_norm, *k_norm;
+};
+struct Layer {
+  bool linear = false;
+  const void *input_ln = nullptr, *post_ln = nullptr;
+  GdnLayer gdn{};
+  AttnLayer attn{};
+  ornith_moe_weights moe{};
+};
+
+struct ornith_model {
+  ornith_ctx* ctx = nullptr;
+  ornith_text_config cfg{};
+  ornith_linear embed_tokens{};
+  ornith_linear lm_head{};
+  const void* final_norm = nullptr;
+  std::vector<Layer> layers;
+  // step buffers, sized for `max_rows` activation rows
+  int max_rows = 0;
+  void* ws_buf = nullptr;
+  size_t ws_bytes = 0;
+  // rope tables, grown on demand to the largest cache capacity seen
+  float *d_cos = nullptr, *d_sin = nullptr;
+  int rope_npos = 0;
+  int key_dim() const { return cfg.linear_num_key_heads * cfg.linear_key_head_dim; }
+  int value_dim() const { return cfg.linear_num_value_heads * cfg.linear_value_head_dim; }
+  int conv_dim() const { return 2 * key_dim() + value_dim(); }
+};
+
+struct LayerCache {
+  // full attention
+  void *k = nullptr, *v = nullptr;  // bf16 [Hkv, cap, hd]
+  // gated delta
+  void* conv[2] = {nullptr, nullptr};  // bf16 [K-1+max_rows, D] each
+  float* state = nullptr;              // f32 [slots][Hv, Dv, Dk]
+};
+
+struct ornith_caches {
+  ornith_model* m = nullptr;
+  int capacity = 0, max_window = 0, conv_rows = 0;
+  std::vector<LayerCache> layers;
+  // one set of cursors serves every layer: they all advance together
+  int offset = 0;     // tokens held
+  int conv_cur = 0;   // which conv buffer holds the live window
+  int conv_off = 0;   // first row of the live K-1 rows in it
+  int state_cur = 0;  // slot holding the live recurrent state
+  int last_T = 0;     // rows of the last forward (for rewind)
+  bool last_capture = false;
+};
+
+struct ornith_frspec {
+  ornith_model* m = nullptr;
+  int n = 0, vocab = 0;
+  std::vector<uint32_t> ids;
+  uint32_t* d_ids = nullptr;
+  ornith_linear head{};
+  void* owned[3] = {nullptr, nullptr, nullptr};
+};
+
+struct ornith_mtp_head {
+  ornith_model* m = nullptr;
+  const void *pre_fc_norm_embedding, *pre_fc_norm_hidden, *input_ln, *post_ln, *norm;
+  ornith_linear fc;
+  AttnLayer attn{};
+  ornith_moe_weights moe{};
+  // one-layer KV cache
+  void *k = nullptr, *v = nullptr;
+  int capacity = 0, offset = 0;
+  void* buf = nullptr;  // step buffers
+  int max_rows = 0;
+};
+
+// grows the model's RoPE tables to cover `npos` positions
+int model_ensure_rope(ornith_model* m, int npos);

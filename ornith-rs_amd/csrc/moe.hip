@@ -229,13 +229,21 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
   TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, lhs_tok, lhs_row));
   TRY(ornith_swiglu(ctx, sg, su, (int64_t)T * SI, sact));
   TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
-  TRY(ornith_kq_gather_qmv(ctx, &w->ex_gate, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xg,
-                           ORNITH_BF16));
-  TRY(ornith_kq_gather_qmv(ctx, &w->ex_up, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xu,
-                           ORNITH_BF16));
-  TRY(ornith_swiglu(ctx, xg, xu, (int64_t)T * k * I, act));
-  TRY(ornith_kq_gather_qmv(ctx, &w->ex_down, act, ORNITH_BF16, T * k, lhs_row, inds, T * k, y,
-                           ORNITH_BF16));
+  if (w->ex_dense) {
+    ORN_REQUIRE(w->d_ex_gate && w->d_ex_up && w->d_ex_down, "moe_block: dense expert tensor missing");
+    TRY(ornith_dense_gather_mv(ctx, w->d_ex_gate, E, I, H, d_x, T, lhs_tok, inds, T * k, xg));
+    TRY(ornith_dense_gather_mv(ctx, w->d_ex_up, E, I, H, d_x, T, lhs_tok, inds, T * k, xu));
+    TRY(ornith_swiglu(ctx, xg, xu, (int64_t)T * k * I, act));
+    TRY(ornith_dense_gather_mv(ctx, w->d_ex_down, E, H, I, act, T * k, lhs_row, inds, T * k, y));
+  } else {
+    TRY(ornith_kq_gather_qmv(ctx, &w->ex_gate, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xg,
+                             ORNITH_BF16));
+    TRY(ornith_kq_gather_qmv(ctx, &w->ex_up, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xu,
+                             ORNITH_BF16));
+    TRY(ornith_swiglu(ctx, xg, xu, (int64_t)T * k * I, act));
+    TRY(ornith_kq_gather_qmv(ctx, &w->ex_down, act, ORNITH_BF16, T * k, lhs_row, inds, T * k, y,
+                             ORNITH_BF16));
+  }
   TRY(ornith_moe_combine(ctx, scores, y, eg, sy, T, k, H, w->norm_topk_prob, d_out));
   if (d_inds_out)
     ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,

@@ -1,0 +1,154 @@
+// The named-tensor store and the module resolution rules of
+// WeightStore::{tensor, linear, kquant_matrix, quant_matrix}
+// (/root/reference/src/weights.rs:101-227): a module <path> is
+//   k-quant   <path>.weight (u32 / u8 codes), <path>.scales (u8), <path>.dm (f16)
+//   affine 8  <path>.weight (u32 / u8), <path>.scales (bf16), <path>.biases (bf16)
+//   dense     <path>.weight (bf16)
+// with the tensor shapes of /root/reference/src/ops/kquant.rs:20-26.
+#include "model.h"
+
+static size_t dt_size(int dt) {
+  switch (dt) {
+    case ORNITH_DT_F32: case ORNITH_DT_U32: case ORNITH_DT_I32: return 4;
+    case ORNITH_DT_BF16: case ORNITH_DT_F16: return 2;
+    case ORNITH_DT_U8: return 1;
+    default: return 0;
+  }
+}
+
+static int kq_from(const ornith_weights* ws, const std::string& path, bool routed,
+                   ornith_kmatrix* out) {
+  const Tensor* w = ws->find(path + ".weight");
+  const Tensor* s = ws->find(path + ".scales");
+  const Tensor* d = ws->find(path + ".dm");
+  ORN_REQUIRE(w && s && d, "%s: k-quant module needs .weight, .scales and .dm", path.c_str());
+  ORN_REQUIRE(w->dtype == ORNITH_DT_U32 || w->dtype == ORNITH_DT_U8, "%s.weight must be uint32",
+              path.c_str());
+  ORN_REQUIRE(s->dtype == ORNITH_DT_U8, "%s.scales must be uint8", path.c_str());
+  ORN_REQUIRE(d->dtype == ORNITH_DT_F16, "%s.dm must be float16", path.c_str());
+  const size_t nd = s->shape.size();
+  ORN_REQUIRE(nd == (routed ? 4u : 3u), "%s.scales: expected %d dims, got %zu", path.c_str(),
+              routed ? 4 : 3, nd);
+  const int64_t per = s->shape[nd - 1], nb = s->shape[nd - 2], O = s->shape[nd - 3];
+  const int64_t E = routed ? s->shape[0] : 1;
+  ORN_REQUIRE(per == 12 || per == 16, "%s.scales: %lld bytes a block is neither Q4_K nor Q6_K",
+              path.c_str(), (long long)per);
+  out->kind = per == 12 ? ORNITH_Q4K : ORNITH_Q6K;
+  out->E = (int)E;
+  out->O = (int)O;
+  out->K = (int)(nb * 256);
+  out->d_qs = w->d;
+  out->d_scales = s->d;
+  out->d_dm = d->d;
+  return ornith_kmatrix_check(out, w->bytes, s->bytes, d->bytes);
+}
+
+int ws_kmatrix(const ornith_weights* ws, const std::string& path, ornith_kmatrix* out) {
+  return kq_from(ws, path, true, out);
+}
+
+int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* out) {
+  memset(out, 0, sizeof *out);
+  const Tensor* w = ws->find(path + ".weight");
+  ORN_REQUIRE(w, "%s.weight: no such tensor", path.c_str());
+  if (ws->find(path + ".dm")) {
+    out->mode = ORNITH_LIN_KQUANT;
+    int rc = kq_from(ws, path, false, &out->km);
+    if (rc) return rc;
+    out->O = out->km.O;
+    out->K = out->km.K;
+    return ORNITH_OK;
+  }
+  if (const Tensor* b = ws->find(path + ".biases")) {
+    const Tensor* s = ws->find(path + ".scales");
+    ORN_REQUIRE(s, "%s: affine module needs .scales", path.c_str());
+    ORN_REQUIRE(s->dtype == ORNITH_DT_BF16 && b->dtype == ORNITH_DT_BF16,
+                "%s: affine scales/biases must be bfloat16", path.c_str());
+    ORN_REQUIRE(w->dtype == ORNITH_DT_U32 || w->dtype == ORNITH_DT_U8, "%s.weight must be uint32",
+                path.c_str());
+    ORN_REQUIRE(s->shape.size() == 2 && b->shape == s->shape, "%s: scales/biases must be [O, K/64]",
+                path.c_str());
+    out->mode = ORNITH_LIN_AFFINE8;
+    out->O = (int)s->shape[0];
+    out->K = (int)s->shape[1] * 64;
+    ORN_REQUIRE(w->bytes == (size_t)out->O * out->K,
+                "%s.weight: %zu bytes is not 8-bit group-64 for [%d, %d]", path.c_str(), w->bytes,
+                out->O, out->K);
+    out->d_w = w->d;
+    out->d_scales = s->d;
+    out->d_biases = b->d;
+    return ORNITH_OK;
+  }
+  ORN_REQUIRE(w->dtype == ORNITH_DT_BF16 && w->shape.size() == 2,
+              "%s.weight: a dense projection must be bfloat16 [O, K]", path.c_str());
+  out->mode = ORNITH_LIN_DENSE;
+  out->O = (int)w->shape[0];
+  out->K = (int)w->shape[1];
+  out->d_w = w->d;
+  return ORNITH_OK;
+}
+
+int ws_tensor(const ornith_weights* ws, const std::string& name, int dtype, int64_t numel,
+              const void** out) {
+  const Tensor* t = ws->find(name);
+  ORN_REQUIRE(t, "%s: no such tensor", name.c_str());
+  ORN_REQUIRE(t->dtype == dtype, "%s: dtype %d, expected %d", name.c_str(), t->dtype, dtype);
+  ORN_REQUIRE(t->numel() == numel, "%s: %lld elements, expected %lld", name.c_str(),
+              (long long)t->numel(), (long long)numel);
+  *out = t->d;
+  return ORNITH_OK;
+}
+
+extern "C" {
+
+int ornith_weights_create(ornith_ctx* ctx, ornith_weights** out) {
+  ORN_REQUIRE(ctx && out, "weights_create: null argument");
+  ornith_weights* w = new ornith_weights();
+  w->ctx = ctx;
+  *out = w;
+  return ORNITH_OK;
+}
+
+int ornith_weights_put(ornith_weights* ws, const char* name, int dtype, const int64_t* shape,
+                       int ndim, const void* host_data) {
+  ORN_REQUIRE(ws && name && shape && host_data, "weights_put: null argument");
+  ORN_REQUIRE(ndim >= 1 && ndim <= 8, "weights_put: %s has %d dims", name, ndim);
+  const size_t es = dt_size(dtype);
+  ORN_REQUIRE(es, "weights_put: %s has unknown dtype %d", name, dtype);
+  ORN_REQUIRE(!ws->find(name), "weights_put: %s is already in the store", name);
+  Tensor t;
+  t.dtype = dtype;
+  int64_t n = 1;
+  for (int i = 0; i < ndim; ++i) {
+    ORN_REQUIRE(shape[i] >= 1, "weights_put: %s dim %d is %lld", name, i, (long long)shape[i]);
+    t.shape.push_back(shape[i]);
+    n *= shape[i];
+  }
+  t.bytes = (size_t)n * es;
+  int rc = ornith_alloc(ws->ctx, t.bytes, &t.d);
+  if (rc) return rc;
+  rc = ornith_upload(ws->ctx, t.d, host_data, t.bytes);
+  if (rc) {
+    ornith_free(ws->ctx, t.d);
+    return rc;
+  }
+  ws->total_bytes += t.bytes;
+  ws->t.emplace(name, std::move(t));
+  return ORNITH_OK;
+}
+
+int ornith_weights_destroy(ornith_weights* ws) {
+  if (!ws) return ORNITH_OK;
+  for (auto& kv : ws->t) ornith_free(ws->ctx, kv.second.d);
+  delete ws;
+  return ORNITH_OK;
+}
+
+int ornith_weights_stats(const ornith_weights* ws, int64_t* n_tensors, int64_t* bytes) {
+  ORN_REQUIRE(ws, "weights_stats: null store");
+  if (n_tensors) *n_tensors = (int64_t)ws->t.size();
+  if (bytes) *bytes = (int64_t)ws->total_bytes;
+  return ORNITH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,266 @@
+"""Host-side mirror of the reference's engine objects over the C ABI:
+WeightStore, TextModel (+ caches), FrSpec, MtpHead, generate_step, generate_step_mtp.
+Names and argument meaning follow /root/reference/src/{weights,frspec,generate,
+mtp_generate}.rs and src/model/{qwen3_5,mtp}.rs so tests read like the reference's."""
+import ctypes as C
+
+import numpy as np
+
+from . import (BF16, F32, LinearStruct, OrnithError, _check, _ptr, lib)
+
+DT_F32, DT_BF16, DT_F16, DT_U8, DT_U32, DT_I32 = range(6)
+HISTORY_CYCLE, HISTORY_COMMITTED = 0, 1
+MAX_DEPTH = 8
+
+
+class TextConfig(C.Structure):
+    """TextConfig (src/model/config.rs); defaults are the Qwen3.5-35B-A3B shape."""
+    _fields_ = [(n, C.c_int) for n in (
+        "hidden_size", "num_hidden_layers", "vocab_size", "num_experts", "num_experts_per_tok",
+        "moe_intermediate_size", "shared_expert_intermediate_size", "linear_num_key_heads",
+        "linear_num_value_heads", "linear_key_head_dim", "linear_value_head_dim",
+        "linear_conv_kernel_dim", "num_attention_heads", "num_key_value_heads", "head_dim",
+        "rope_dims", "full_attention_interval", "norm_topk_prob")] + [
+        ("rms_norm_eps", C.c_float), ("rope_theta", C.c_double)]
+
+    @staticmethod
+    def qwen35_35b_a3b(**over):
+        d = dict(hidden_size=2048, num_hidden_layers=40, vocab_size=248320, num_experts=256,
+                 num_experts_per_tok=8, moe_intermediate_size=512, shared_expert_intermediate_size=512,
+                 linear_num_key_heads=16, linear_num_value_heads=32, linear_key_head_dim=128,
+                 linear_value_head_dim=128, linear_conv_kernel_dim=4, num_attention_heads=16,
+                 num_key_value_heads=2, head_dim=256, rope_dims=64, full_attention_interval=4,
+                 norm_topk_prob=1, rms_norm_eps=1e-6, rope_theta=1e7)
+        d.update(over)
+        return TextConfig(**d)
+
+    def key_dim(self):
+        return self.linear_num_key_heads * self.linear_key_head_dim
+
+    def value_dim(self):
+        return self.linear_num_value_heads * self.linear_value_head_dim
+
+    def conv_dim(self):
+        return 2 * self.key_dim() + self.value_dim()
+
+    def is_linear(self, i):
+        return (i + 1) % self.full_attention_interval != 0
+
+
+class Sampler(C.Structure):
+    _fields_ = [("kind", C.c_int), ("temperature", C.c_float), ("top_p", C.c_float),
+                ("top_k", C.c_int), ("seed", C.c_uint64)]
+
+    @staticmethod
+    def greedy():
+        return Sampler(0, 0.0, 1.0, 0, 0)
+
+
+class MtpStats(C.Structure):
+    _fields_ = [("cycles", C.c_size_t), ("drafted", C.c_size_t), ("accepted", C.c_size_t),
+                ("reached_by_depth", C.c_size_t * MAX_DEPTH), ("accepted_by_depth", C.c_size_t * MAX_DEPTH)]
+
+
+_NP_DT = {np.dtype(np.float32): DT_F32, np.dtype(np.float16): DT_F16, np.dtype(np.uint8): DT_U8,
+          np.dtype(np.uint32): DT_U32, np.dtype(np.int32): DT_I32}
+
+TOKEN_CB = C.CFUNCTYPE(C.c_int, C.c_uint32, C.c_void_p)
+PROGRESS_CB = C.CFUNCTYPE(None, C.c_size_t, C.c_size_t, C.c_void_p)
+
+
+class WeightStore:
+    """WeightStore: named tensors on the device."""
+
+    def __init__(self, ctx):
+        self.ctx = ctx
+        h = C.c_void_p()
+        _check(lib().ornith_weights_create(ctx.h, C.byref(h)), "weights_create")
+        self.h = h
+
+    def put(self, name, arr, dtype=None):
+        """dtype: DT_BF16 / DT_F16 for uint16 bit patterns; inferred otherwise."""
+        arr = np.ascontiguousarray(arr)
+        if dtype is None:
+            dtype = _NP_DT[arr.dtype]
+        shape = (C.c_int64 * arr.ndim)(*arr.shape)
+        _check(lib().ornith_weights_put(self.h, name.encode(), dtype, shape, arr.ndim, _ptr(arr)),
+               f"weights_put({name})")
+
+    def stats(self):
+        n, b = C.c_int64(), C.c_int64()
+        _check(lib().ornith_weights_stats(self.h, C.byref(n), C.byref(b)), "weights_stats")
+        return n.value, b.value
+
+    def close(self):
+        if self.h:
+            lib().ornith_weights_destroy(self.h)
+            self.h = None
+
+
+class Caches:
+    def __init__(self, model, capacity, max_window):
+        self.model = model
+        h = C.c_void_p()
+        _check(lib().ornith_caches_create(model.h, capacity, max_window, C.byref(h)), "caches_create")
+        self.h = h
+
+    def reset(self):
+        _check(lib().ornith_caches_reset(self.h), "caches_reset")
+
+    @property
+    def offset(self):
+        o = C.c_int()
+        _check(lib().ornith_caches_offset(self.h, C.byref(o)), "caches_offset")
+        return o.value
+
+    def close(self):
+        if self.h:
+            lib().ornith_caches_destroy(self.h)
+            self.h = None
+
+
+class TextModel:
+    """TextModel::load + forward_hidden / forward_capture / rewind."""
+
+    def __init__(self, ctx, ws, cfg):
+        self.ctx, self.ws, self.cfg = ctx, ws, cfg
+        h = C.c_void_p()
+        _check(lib().ornith_model_load(ctx.h, ws.h, C.byref(cfg), C.byref(h)), "model_load")
+        self.h = h
+
+    def make_cache(self, capacity, max_window=4):
+        return Caches(self, capacity, max_window)
+
+    def forward(self, caches, tokens, capture=False):
+        """tokens: host uint32 array -> post-norm hidden rows as uint16 bf16 bits [T, H]."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+        T, H = len(tokens), self.cfg.hidden_size
+        dt, dh = self.ctx.to_device(tokens), self.ctx.alloc(T * H * 2)
+        try:
+            _check(lib().ornith_model_forward(self.h, caches.h, dt.ptr, T, int(capture), dh.ptr), "model_forward")
+            return dh.download(np.uint16, (T, H))
+        finally:
+            dt.free()
+            dh.free()
+
+    def rewind(self, caches, keep):
+        _check(lib().ornith_model_rewind(self.h, caches.h, keep), "model_rewind")
+
+    def logits(self, hidden):
+        hidden = np.ascontiguousarray(hidden, dtype=np.uint16)
+        T, V = hidden.shape[0], self.cfg.vocab_size
+        dh, dl = self.ctx.to_device(hidden), self.ctx.alloc(T * V * 2)
+        try:
+            _check(lib().ornith_model_logits(self.h, dh.ptr, T, dl.ptr), "model_logits")
+            return dl.download(np.uint16, (T, V))
+        finally:
+            dh.free()
+            dl.free()
+
+    def close(self):
+        if self.h:
+            lib().ornith_model_destroy(self.h)
+            self.h = None
+
+
+class FrSpec:
+    """FrSpec::load / from a list of ids; holds the pruned head."""
+
+    def __init__(self, model, ids=None, path=None):
+        self.model = model
+        h = C.c_void_p()
+        if path is not None:
+            _check(lib().ornith_frspec_load(model.h, str(path).encode(), C.byref(h)), "frspec_load")
+        else:
+            ids = np.ascontiguousarray(ids, dtype=np.uint32)
+            _check(lib().ornith_frspec_from_ids(model.h, _ptr(ids), len(ids), C.byref(h)), "frspec_from_ids")
+        self.h = h
+
+    def head(self):
+        s, n = LinearStruct(), C.c_int()
+        _check(lib().ornith_frspec_head(self.h, C.byref(s), C.byref(n)), "frspec_head")
+        return s, n.value
+
+    def close(self):
+        if self.h:
+            lib().ornith_frspec_destroy(self.h)
+            self.h = None
+
+
+class MtpHead:
+    def __init__(self, model, ws, capacity):
+        self.model = model
+        h = C.c_void_p()
+        _check(lib().ornith_mtp_load(model.h, ws.h, capacity, C.byref(h)), "mtp_load")
+        self.h = h
+
+    def forward(self, trunk_hidden, next_ids, frspec=None, want_logits=True):
+        ctx, cfg = self.model.ctx, self.model.cfg
+        trunk_hidden = np.ascontiguousarray(trunk_hidden, dtype=np.uint16)
+        next_ids = np.ascontiguousarray(next_ids, dtype=np.uint32)
+        T, H = len(next_ids), cfg.hidden_size
+        V = frspec.head()[1] if frspec else cfg.vocab_size
+        dh, di, do = ctx.to_device(trunk_hidden), ctx.to_device(next_ids), ctx.alloc(T * H * 2)
+        dl = ctx.alloc(T * V * 2) if want_logits else None
+        try:
+            _check(lib().ornith_mtp_forward(self.h, frspec.h if frspec else None, dh.ptr, di.ptr, T, do.ptr,
+                                            dl.ptr if dl else None), "mtp_forward")
+            hid = do.download(np.uint16, (T, H))
+            return (dl.download(np.uint16, (T, V)) if dl else None), hid
+        finally:
+            for b in (dh, di, do, dl):
+                if b:
+                    b.free()
+
+    def set_offset(self, off):
+        _check(lib().ornith_mtp_cache_set_offset(self.h, off), "mtp_cache_set_offset")
+
+    @property
+    def offset(self):
+        o = C.c_int()
+        _check(lib().ornith_mtp_cache_offset(self.h, C.byref(o)), "mtp_cache_offset")
+        return o.value
+
+    def close(self):
+        if self.h:
+            lib().ornith_mtp_destroy(self.h)
+            self.h = None
+
+
+def generate_step(model, caches, prompt, max_tokens, sampler=None, prefill_step=2048, on_token=None,
+                  progress=None):
+    """generate::generate_step. Returns the emitted tokens (also handed to on_token one by one;
+    on_token returning False stops)."""
+    prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+    sampler = sampler or Sampler.greedy()
+    out = []
+
+    def _tok(t, _u):
+        out.append(int(t))
+        return 1 if (on_token is None or on_token(int(t))) else 0
+
+    cb = TOKEN_CB(_tok)
+    pcb = PROGRESS_CB((lambda d, t, _u: progress(d, t)) if progress else (lambda d, t, _u: None))
+    _check(lib().ornith_generate(model.h, caches.h, _ptr(prompt), C.c_size_t(len(prompt)), C.byref(sampler),
+                                 C.c_size_t(max_tokens), C.c_size_t(prefill_step), pcb, cb, None), "generate")
+    return out
+
+
+def generate_step_mtp(model, head, frspec, caches, prompt, depth, max_tokens, sampler=None,
+                      prefill_step=2048, policy=HISTORY_COMMITTED, on_token=None, progress=None):
+    """mtp_generate::generate_step_mtp. Returns (tokens, MtpStats)."""
+    prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
+    sampler = sampler or Sampler.greedy()
+    out, stats = [], MtpStats()
+
+    def _tok(t, _u):
+        out.append(int(t))
+        return 1 if (on_token is None or on_token(int(t))) else 0
+
+    cb = TOKEN_CB(_tok)
+    pcb = PROGRESS_CB((lambda d, t, _u: progress(d, t)) if progress else (lambda d, t, _u: None))
+    _check(lib().ornith_mtp_generate(model.h, head.h, frspec.h if frspec else None, caches.h, _ptr(prompt),
+                                     C.c_size_t(len(prompt)), C.byref(sampler), depth, C.c_size_t(max_tokens),
+                                     C.c_size_t(prefill_step), policy, pcb, cb, None, C.byref(stats)),
+           "mtp_generate")
+    return out, stats

@@ -1,0 +1,197 @@
+"""GPU parity at model level on reduced configurations: trunk forward / capture / rewind,
+MTP head, FR-Spec, and both generation loops vs the CPU oracle. Hidden states and logits
+are compared by bf16 bits, tokens and acceptance counters exactly. The reference's own
+release check -- greedy speculative output identical to plain greedy
+(/root/reference/README.md:193-197, tests/mtp.rs:246-349) -- is asserted on both sides."""
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import synth
+import util
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def tiny(orn, ctx):
+    s = synth.SynthModel(synth.TINY, seed=11)
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    yield s, ws, model
+    model.close()
+    ws.close()
+
+
+@pytest.fixture(scope="module")
+def tiny_small_vocab(orn, ctx):
+    """vocab 32: random drafts agree often enough to exercise acceptance and history repair"""
+    s = synth.SynthModel(dict(synth.TINY, vocab_size=32), seed=12)
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    yield s, ws, model
+    model.close()
+    ws.close()
+
+
+def test_forward_capture_rewind_bit_exact(orn, ctx, tiny):
+    s, ws, model = tiny
+    rng = np.random.default_rng(0)
+    toks = rng.integers(0, s.cfg["vocab_size"], 12).astype(np.uint32)
+    caches = model.make_cache(64, 4)
+    orc = synth.OracleRun(s, 64)
+    # a 5-token chunk (prefill width), then single steps, then a captured window
+    for chunk, cap in ((toks[:5], False), (toks[5:6], False), (toks[6:7], False), (toks[7:10], True)):
+        got = model.forward(caches, chunk, capture=cap)
+        want = orc.forward(chunk, capture=cap)
+        assert np.array_equal(got, want), (len(chunk), cap)
+    assert caches.offset == 10 == util.oracle().orc_state_offset(orc.st)
+    # reject two of the three window tokens, then continue: must equal the oracle doing the same,
+    # and must equal a run that never saw the rejected tokens
+    model.rewind(caches, 1)
+    orc.rewind(1)
+    assert caches.offset == 8
+    nxt = model.forward(caches, toks[10:12])
+    assert np.array_equal(nxt, orc.forward(toks[10:12]))
+    fresh = model.make_cache(64, 4)
+    model.forward(fresh, toks[:5]); model.forward(fresh, toks[5:8])
+    assert np.array_equal(model.forward(fresh, toks[10:12]), nxt)
+    # logits and the greedy choice
+    lg = model.logits(nxt)
+    assert np.array_equal(lg, orc.logits(nxt))
+    for c in (caches, fresh): c.close()
+    orc.close()
+
+
+def test_batch_invariance_chunking_does_not_matter(orn, ctx, tiny):
+    """row r of a T-row forward == that row run alone (src/ops/invariant.rs:88-116)."""
+    s, ws, model = tiny
+    toks = np.random.default_rng(1).integers(0, s.cfg["vocab_size"], 9).astype(np.uint32)
+    a, b = model.make_cache(32, 4), model.make_cache(32, 4)
+    whole = np.concatenate([model.forward(a, toks[:4]), model.forward(a, toks[4:9])])
+    single = np.concatenate([model.forward(b, toks[i:i + 1]) for i in range(9)])
+    assert np.array_equal(whole, single)
+    a.close(); b.close()
+
+
+def test_mtp_head_forward_bit_exact(orn, ctx, tiny):
+    s, ws, model = tiny
+    rng = np.random.default_rng(2)
+    head = orn.MtpHead(model, ws, 64)
+    orc = synth.OracleRun(s, 64)
+    hid = util.bf16_normal(rng, (3, s.cfg["hidden_size"]))
+    ids = rng.integers(0, s.cfg["vocab_size"], 3).astype(np.uint32)
+    lg, h1 = head.forward(hid[:1], ids[:1])
+    w1 = orc.mtp_hidden(hid[:1], ids[:1])
+    assert np.array_equal(h1, w1) and np.array_equal(lg, orc.logits(w1))
+    _, h2 = head.forward(hid[1:], ids[1:], want_logits=False)   # two rows at once, cache offset 1
+    assert np.array_equal(h2, orc.mtp_hidden(hid[1:], ids[1:]))
+    assert head.offset == 3
+    head.close(); orc.close()
+
+
+def test_frspec_prune_map_and_file_format(orn, ctx, tiny, tmp_path):
+    s, ws, model = tiny
+    V = s.cfg["vocab_size"]
+    ids = synth.zipf_frspec_ids(V, 256, seed=5)
+    fr = orn.FrSpec(model, ids=ids)
+    head, n = fr.head()
+    assert n == 256
+    # pruned row == original row, exact (tests/q4k.rs:739-767)
+    x = util.bf16_normal(np.random.default_rng(3), (2, s.cfg["hidden_size"]))
+    full = model.logits(x)
+    dx, dy = ctx.to_device(x), ctx.alloc(2 * 256 * 2)
+    lin = orn.Linear(head, [])
+    ctx.linear_matmul(lin, dx, 2, dy)
+    assert np.array_equal(dy.download(np.uint16, (2, 256)), full[:, ids.astype(np.int64)])
+    dx.free(); dy.free(); fr.close()
+    # the file format: u32 n, then n x u32 little endian (src/frspec.rs:101-117)
+    path = tmp_path / "ids.bin"
+    path.write_bytes(struct.pack("<I", len(ids)) + ids.astype("<u4").tobytes())
+    fr = orn.FrSpec(model, path=path)
+    assert fr.head()[1] == 256
+    fr.close()
+    bad = {
+        "empty": struct.pack("<I", 0),
+        "too many": struct.pack("<I", V) + np.arange(V, dtype="<u4").tobytes(),
+        "out of range": struct.pack("<I", 2) + np.array([1, V], "<u4").tobytes(),
+        "listed twice": struct.pack("<I", 3) + np.array([4, 9, 4], "<u4").tobytes(),
+        "holds": struct.pack("<I", 5) + np.array([1, 2], "<u4").tobytes(),
+    }
+    msgs = {"empty": "empty", "too many": "nothing to prune", "out of range": "outside the vocabulary",
+            "listed twice": "listed twice", "holds": "header says"}
+    for k, blob in bad.items():
+        path.write_bytes(blob)
+        with pytest.raises(orn.OrnithError, match=msgs[k]):
+            orn.FrSpec(model, path=path)
+    with pytest.raises(orn.OrnithError, match="cannot open"):
+        orn.FrSpec(model, path=tmp_path / "missing.bin")
+
+
+def _run_loops(orn, ctx, s, ws, model, max_tokens, depths, fr_n):
+    rng = np.random.default_rng(7)
+    V = s.cfg["vocab_size"]
+    prompt = rng.integers(0, V, 11).astype(np.uint32)
+    cap = 11 + max_tokens + 8
+    caches = model.make_cache(cap, 4)
+    ar = orn.generate_step(model, caches, prompt, max_tokens, prefill_step=4)
+    assert len(ar) == max_tokens and caches.offset == 11 + max_tokens
+    orc = synth.OracleRun(s, cap)
+    assert ar == orc.generate(prompt, max_tokens, prefill_step=4), "AR tokens differ from the oracle"
+    orc.close()
+    head = orn.MtpHead(model, ws, cap)
+    fr_ids = synth.zipf_frspec_ids(V, fr_n, seed=1)
+    fr = orn.FrSpec(model, ids=fr_ids)
+    fr_host = synth.prune_head(s.lm_head, fr_ids)
+    total_acc = 0
+    for depth in depths:
+        for policy in (orn.HISTORY_CYCLE, orn.HISTORY_COMMITTED):
+            for use_fr in (False, True):
+                caches.reset()
+                toks, st = orn.generate_step_mtp(model, head, fr if use_fr else None, caches, prompt, depth,
+                                                 max_tokens, prefill_step=4, policy=policy)
+                assert toks == ar, f"depth {depth} policy {policy} frspec {use_fr}: not identical to greedy"
+                assert st.accepted <= st.drafted and len(toks) == max_tokens
+                assert caches.offset == 11 + max_tokens
+                orc = synth.OracleRun(s, cap)
+                otoks, ost = orc.mtp_generate(prompt, depth, max_tokens, fr_ids if use_fr else None,
+                                              fr_host if use_fr else None, policy=policy, prefill_step=4)
+                orc.close()
+                assert otoks == ar
+                assert (st.cycles, st.drafted, st.accepted) == (ost.cycles, ost.drafted, ost.accepted)
+                assert list(st.accepted_by_depth[:depth]) == list(ost.accepted_by[:depth])
+                assert list(st.reached_by_depth[:depth]) == list(ost.reached[:depth])
+                total_acc += st.accepted
+    for o in (fr, head, caches): o.close()
+    return total_acc
+
+
+def test_generation_loops_tiny(orn, ctx, tiny):
+    s, ws, model = tiny
+    _run_loops(orn, ctx, s, ws, model, max_tokens=12, depths=(1, 3), fr_n=512)
+
+
+def test_generation_loops_small_vocab_exercise_acceptance(orn, ctx, tiny_small_vocab):
+    s, ws, model = tiny_small_vocab
+    acc = _run_loops(orn, ctx, s, ws, model, max_tokens=40, depths=(1, 2), fr_n=24)
+    assert acc > 0, "no draft was ever accepted: the acceptance path went untested"
+
+
+def test_stop_callback_and_errors(orn, ctx, tiny):
+    s, ws, model = tiny
+    prompt = np.arange(5, dtype=np.uint32)
+    caches = model.make_cache(32, 2)
+    seen = []
+    orn.generate_step(model, caches, prompt, 10, on_token=lambda t: (seen.append(t), len(seen) < 3)[1])
+    assert len(seen) == 3 and caches.offset == 5 + 3   # the stopping token is in the caches too
+    head = orn.MtpHead(model, ws, 32)
+    caches.reset()
+    with pytest.raises(orn.OrnithError, match="capture window"):
+        orn.generate_step_mtp(model, head, None, caches, prompt, 3, 5)
+    with pytest.raises(orn.OrnithError, match="exceed cache capacity"):
+        model.forward(caches, np.zeros(16, np.uint32)); model.forward(caches, np.zeros(16, np.uint32)); model.forward(caches, np.zeros(1, np.uint32))
+    with pytest.raises(orn.OrnithError, match="greedy"):
+        orn.generate_step(model, caches, prompt, 2, sampler=orn.Sampler(1, 0.8, 0.95, 0, 1))
+    head.close(); caches.close()
