@@ -61,6 +61,13 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
 /* Event timing on the context's stream (the reference sums GPUEndTime -
  * GPUStartTime per command buffer, src/metal/mod.rs:197-285). begin/end record
  * events; elapsed synchronises on the end event and returns milliseconds. */
+/* Behaviour switches (the reference's ORNITH_* flags with their runtime set_* twins,
+ * src/ops/moe.rs:397-414, src/ops/gdn.rs:416-426). Each is also read once from the
+ * environment variable named here; every value gives bit-identical results.
+ *   "fuse_moe"  (ORNITH_FUSE_MOE, default 1): the two fused expert kernels vs. one
+ *               launch per operator
+ *   "fuse_proj" (ORNITH_FUSE_PROJ, default 1): projections sharing an input in one launch */
+ORNITH_API int ornith_set_option(const char* name, int value);
 ORNITH_API int ornith_timer_begin(ornith_ctx* ctx);
 ORNITH_API int ornith_timer_end(ornith_ctx* ctx, float* ms_out);
 
@@ -90,6 +97,13 @@ ORNITH_API int ornith_kq_dequantize(ornith_ctx* ctx, const ornith_kmatrix* w, vo
  * decode/verify shape; larger M loops in groups of four. */
 ORNITH_API int ornith_kq_qmv(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int x_dtype, int M,
                   void* d_y, int y_dtype);
+
+/* n <= 4 kquant::qmv calls over the same activations in one launch (the reference issues
+ * them back to back, src/model/qwen3_5.rs:441-447,493-494). All matrices must share
+ * format and width; d_ys[i] receives [M, ws[i]->O]. Bit-identical to separate calls. */
+ORNITH_API int ornith_kq_qmv_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n,
+                                   const void* d_x, int x_dtype, int M, void* const* d_ys,
+                                   int y_dtype);
 
 /* kquant::gather_qmv (src/ops/kquant.rs:741-770): out[r] = x[lhs[r]] . W[rhs[r]]^T,
  * r < rows; lhs/rhs are device u32 arrays; x has x_rows rows. Indices live on the

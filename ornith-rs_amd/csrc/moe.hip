@@ -12,6 +12,12 @@
 #include "dmath.h"
 #include "rt.h"
 
+// moe_fused.hip
+bool moe_fused_supported(const ornith_moe_weights* w);
+int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                      const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
+                      void* d_out);
+
 namespace {
 
 // One wavefront per token. Lane l holds gates [l*PER, (l+1)*PER).
@@ -196,7 +202,7 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
   const int SI = w->sh_gate.O;
 
   const size_t need = 2 * ((size_t)T * E * 2 + (size_t)T * SI * 3 + (size_t)T * H + T +
-                           (size_t)T * k * (2 * I + I + H + 1)) +
+                           (size_t)(T * k + T) * (2 * I + I + SI + H + 1)) +
                       4 * (size_t)T * k * 3 + 64 * 256;
   void* base = nullptr;
   int rc = ornith_scratch(ctx, need, &base);
@@ -214,7 +220,7 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
   bf16_t* eg = sc.take<bf16_t>((size_t)T);
   bf16_t* xg = sc.take<bf16_t>((size_t)T * k * I);
   bf16_t* xu = sc.take<bf16_t>((size_t)T * k * I);
-  bf16_t* act = sc.take<bf16_t>((size_t)T * k * I);
+  bf16_t* act = sc.take<bf16_t>((size_t)(T * k + T) * (I > SI ? I : SI));
   bf16_t* y = sc.take<bf16_t>((size_t)T * k * H);
 
 #define TRY(e)          \
@@ -222,6 +228,20 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
     rc = (e);           \
     if (rc) return rc;  \
   } while (0)
+  if (ornith_option_fuse_moe() && moe_fused_supported(w)) {
+    // three small launches for the router, then the two expert kernels
+    TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
+    TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
+    TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
+    TRY(moe_fused_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out));
+    if (d_inds_out)
+      ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,
+                             ctx->stream));
+    if (d_scores_out)
+      ORN_HIP(hipMemcpyAsync(d_scores_out, scores, 2 * (size_t)T * k, hipMemcpyDeviceToDevice,
+                             ctx->stream));
+    return ORNITH_OK;
+  }
   TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
   TRY(ornith_linear_matmul(ctx, &w->sh_gate, d_x, T, sg));
   TRY(ornith_linear_matmul(ctx, &w->sh_up, d_x, T, su));

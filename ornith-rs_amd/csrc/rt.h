@@ -63,4 +63,10 @@ int ornith_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2,
                          hipGetErrorString(e__));                                       \
   } while (0)
 
+// Behaviour switches, read once from the environment (ORNITH_FUSE_MOE=0 ...) and
+// settable at run time through ornith_set_option so A/B runs share a process, the way
+// the reference's ORNITH_* flags work (/root/reference/src/ops/moe.rs:397-414).
+int ornith_option_fuse_moe();
+int ornith_option_fuse_proj();
+
 static inline size_t ornith_dtype_size(int dt) { return dt == ORNITH_F32 ? 4 : 2; }

@@ -4,6 +4,8 @@
 // tracker, barrier epochs and command-buffer batching have no counterpart here.
 #include "rt.h"
 
+#include <cstdlib>
+
 static thread_local char g_err[512] = "";
 
 int ornith_fail(int code, const char* fmt, ...) {
@@ -28,7 +30,37 @@ int ornith_scratch(ornith_ctx* ctx, size_t bytes, void** out) {
   return ORNITH_OK;
 }
 
+namespace {
+struct Option {
+  const char* name;
+  const char* env;
+  int value;  // -1: not read yet
+};
+Option g_options[] = {{"fuse_moe", "ORNITH_FUSE_MOE", -1}, {"fuse_proj", "ORNITH_FUSE_PROJ", -1}};
+int option_value(int i) {
+  Option& o = g_options[i];
+  if (o.value < 0) {
+    const char* e = getenv(o.env);
+    o.value = (e && e[0] == '0') ? 0 : 1;
+  }
+  return o.value;
+}
+}  // namespace
+
+int ornith_option_fuse_moe() { return option_value(0); }
+int ornith_option_fuse_proj() { return option_value(1); }
+
 extern "C" {
+
+int ornith_set_option(const char* name, int value) {
+  ORN_REQUIRE(name, "set_option: null name");
+  for (auto& o : g_options)
+    if (!strcmp(o.name, name)) {
+      o.value = value ? 1 : 0;
+      return ORNITH_OK;
+    }
+  return ornith_fail(ORNITH_ERR_INVALID, "set_option: unknown option '%s'", name);
+}
 
 const char* ornith_last_error(void) { return g_err; }
 

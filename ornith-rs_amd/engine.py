@@ -13,6 +13,20 @@ HISTORY_CYCLE, HISTORY_COMMITTED = 0, 1
 MAX_DEPTH = 8
 
 
+def set_option(name, value):
+    """ornith_set_option: 'fuse_moe', 'fuse_proj' (bit-identical either way)."""
+    _check(lib().ornith_set_option(name.encode(), int(value)), f"set_option({name})")
+
+
+def kq_qmv_multi(ctx, ws, x, x_dtype, M, ys, y_dtype):
+    """Several k-quant mat-vecs over the same activations in one launch.
+    ws: list of KMatrix, ys: list of DeviceBuffer."""
+    n = len(ws)
+    wp = (C.c_void_p * n)(*[C.cast(C.pointer(w.s), C.c_void_p) for w in ws])
+    yp = (C.c_void_p * n)(*[y.ptr for y in ys])
+    _check(lib().ornith_kq_qmv_multi(ctx.h, wp, n, x.ptr, x_dtype, M, yp, y_dtype), "kq_qmv_multi")
+
+
 class TextConfig(C.Structure):
     """TextConfig (src/model/config.rs); defaults are the Qwen3.5-35B-A3B shape."""
     _fields_ = [(n, C.c_int) for n in (

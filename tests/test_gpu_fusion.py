@@ -1,0 +1,62 @@
+"""GPU: every fused launch structure gives the same bits as the one-launch-per-operator
+path (the reference holds its own fusions to the same standard, e.g. tests/gdn.rs:176-230,
+tests/q4k.rs:778-822), and as the oracle."""
+import numpy as np
+import pytest
+
+import util
+from util import Q4K, Q6K
+
+pytestmark = pytest.mark.gpu
+
+
+def _block(orn, ctx, moe, dw, xb, T):
+    dx, dout = ctx.to_device(xb), ctx.alloc(T * moe.H * 2)
+    di, ds = ctx.alloc(T * moe.top_k * 4), ctx.alloc(T * moe.top_k * 2)
+    ctx.moe_block(dw, dx, T, dout, di, ds)
+    r = (dout.download(np.uint16, (T, moe.H)), di.download(np.uint32, (T, moe.top_k)), ds.download(np.uint16, (T, moe.top_k)))
+    for b in (dx, dout, di, ds): b.free()
+    return r
+
+
+@pytest.mark.parametrize("H,E,I,gk,dk", [(2048, 256, 512, Q4K, Q6K), (512, 64, 256, Q4K, Q6K),
+                                          (512, 64, 256, Q6K, Q4K), (1024, 64, 512, Q4K, Q4K)])
+def test_moe_fused_equals_unfused_and_oracle(orn, ctx, H, E, I, gk, dk):
+    rng = np.random.default_rng(H + E + I + gk)
+    moe = util.HostMoe(rng, H=H, E=E, I=I, top_k=8, gate_kind=gk, down_kind=dk, router_kind=Q6K)
+    dw = moe.dev(orn, ctx)
+    try:
+        for T in (1, 2, 4, 7):
+            xb = util.bf16_normal(rng, (T, H))
+            orn.set_option("fuse_moe", 1)
+            fused = _block(orn, ctx, moe, dw, xb, T)
+            orn.set_option("fuse_moe", 0)
+            plain = _block(orn, ctx, moe, dw, xb, T)
+            for a, b in zip(fused, plain):
+                assert np.array_equal(a, b), T
+            if T <= 2:
+                want_out, want_inds, want_sc, _ = util.orc_moe_block(moe, xb, T)
+                assert np.array_equal(fused[1], want_inds) and np.array_equal(fused[0], want_out)
+    finally:
+        orn.set_option("fuse_moe", 1)
+        moe.free()
+
+
+def test_multi_matrix_launch_equals_separate(orn, ctx):
+    rng = np.random.default_rng(5)
+    for kind, K in ((Q4K, 2048), (Q6K, 2048), (Q4K, 512), (Q4K, 4096)):
+        Os = (8192, 4096, 40)
+        ts = [util.make_kq(kind, rng, 1, O, K) for O in Os]
+        ws = [orn.KMatrix(ctx, kind, *t, 1, O, K) for t, O in zip(ts, Os)]
+        for M in (1, 2, 4):
+            xb = util.bf16_normal(rng, (M, K))
+            dx = ctx.to_device(xb)
+            ys = [ctx.alloc(M * O * 2) for O in Os]
+            orn.kq_qmv_multi(ctx, ws, dx, orn.BF16, M, ys, orn.BF16)
+            for w, y, O in zip(ws, ys, Os):
+                y1 = ctx.alloc(M * O * 2)
+                ctx.kq_qmv(w, dx, orn.BF16, M, y1, orn.BF16)
+                assert np.array_equal(y.download(np.uint16, (M, O)), y1.download(np.uint16, (M, O))), (kind, K, M, O)
+                y1.free()
+            for b in ys + [dx]: b.free()
+        for w in ws: w.free()
