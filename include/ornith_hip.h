@@ -66,7 +66,9 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  * environment variable named here; every value gives bit-identical results.
  *   "fuse_moe"  (ORNITH_FUSE_MOE, default 1): the two fused expert kernels vs. one
  *               launch per operator
- *   "fuse_proj" (ORNITH_FUSE_PROJ, default 1): projections sharing an input in one launch */
+ *   "fuse_proj" (ORNITH_FUSE_PROJ, default 1): projections sharing an input in one launch
+ *   "moe_up_iters" (ORNITH_MOE_UP_ITERS, default 0 = chosen by shape; 2 or 4): output
+ *               rows per wavefront of the fused gate+up expert kernel, a tuning knob */
 ORNITH_API int ornith_set_option(const char* name, int value);
 ORNITH_API int ornith_timer_begin(ornith_ctx* ctx);
 ORNITH_API int ornith_timer_end(ornith_ctx* ctx, float* ms_out);
@@ -131,6 +133,21 @@ typedef struct ornith_linear {
 ORNITH_API int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_x, int M,
                                     void* d_y);
 
+/* Linear::matmul followed by norm::add_rms_norm (the mixer's output projection and the
+ * post-attention norm, src/model/qwen3_5.rs:374-390): y = x . W^T; h = res + y (bf16);
+ * normed = rms_norm(h, w_norm). One launch for k-quant weights at M <= 4 (the last
+ * workgroup to finish applies the norm), two otherwise; bit-identical either way. */
+ORNITH_API int ornith_linear_matmul_add_rms(ornith_ctx* ctx, const ornith_linear* w, const void* d_x,
+                                            int M, void* d_y, const void* d_res, const void* d_wnorm,
+                                            float eps, void* d_h_out, void* d_normed_out);
+
+/* n Linear::matmul calls over the same activations (in_proj_qkv + in_proj_z, in_proj_a +
+ * in_proj_b, q/k/v projections: src/model/qwen3_5.rs:441-447,493-499). Fused into one
+ * launch where the formats allow (same mode, width and k-quant kind; n <= 4), issued
+ * one by one otherwise. Results are bit-identical either way. */
+ORNITH_API int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, int n,
+                                          const void* d_x, int M, void* const* d_ys);
+
 /* ops::matmul::gather_mv (src/ops/matmul.rs:649-): stacked dense bf16 experts
  * W[E,O,K]; out[r] = x[lhs[r]] . W[rhs[r]]^T. Used by the MTP head's MoE. */
 ORNITH_API int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K,
@@ -178,6 +195,28 @@ typedef struct ornith_moe_weights {
  * d_inds_out (u32 [T,k]) and d_scores_out (bf16 [T,k]) may be null. T <= 64. */
 ORNITH_API int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                                 void* d_out, uint32_t* d_inds_out, void* d_scores_out);
+
+/* sparse_moe_block followed by the decoder layer's closing add and the next layer's
+ * input norm (src/model/qwen3_5.rs:388-396 and the head of the next layer's forward):
+ * out = moe(x); h = res + out; normed = rms_norm(h, w_norm). With the fused expert
+ * kernels and T <= top_k + 1 the last workgroup of the down kernel applies the norm, so
+ * the block ends in the same launch; bit-identical to moe_block + add_rms_norm. */
+ORNITH_API int ornith_moe_block_add_rms(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x,
+                                        int T, void* d_out, const void* d_res, const void* d_wnorm,
+                                        float eps, void* d_h_out, void* d_normed_out);
+
+/* moe::switch_glu_rows + the shared expert + moe::combine (src/ops/moe.rs:256-338,548-596)
+ * given the router's picks: the expert gather-GEMV proper, as two kernels.
+ *   phases & 1: act[(t*k+j)] = swiglu(gate_e(x_t), up_e(x_t)) for every routed pair, and
+ *               act[T*k + t] for the shared expert; act is bf16 [(T*k + T), I] scratch
+ *   phases & 2: out[t] = sum_j w_j * down_e(act) + sigmoid(egate_t) * down_shared(act)
+ * d_inds u32 [T,k], d_scores bf16 [T,k] (router_topk outputs), d_egate bf16 [T]
+ * (shared_expert_gate's output). Needs k-quant routed and shared experts of matching
+ * formats and top_k <= 8 (ORNITH_ERR_UNSUPPORTED otherwise; ornith_moe_block falls back
+ * to one launch per operator by itself). */
+ORNITH_API int ornith_moe_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                                  const uint32_t* d_inds, const void* d_scores, const void* d_egate,
+                                  void* d_act, void* d_out, int phases);
 
 /* ---- norms: src/ops/norm.rs:19-220 (vendored rms_norm.metal:12-81,
  * kernels/ornith_norm.metal:28-183). Rows of n bf16 values, n = 64 * 2^j <= 4096. */

@@ -23,7 +23,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fno-fast-math", "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
+    "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument", "-Wno-pass-failed",
 ]
 
 

@@ -122,18 +122,79 @@ __device__ __forceinline__ float dm_sigmoid_f32(float x) {
 
 // ---- wavefront reductions: v[l] += v[l ^ s], s = 32,16,...,1 ---------------
 // fp32 add commutes, so all 64 lanes finish with identical bits.
+
+// value of lane (l ^ S): DPP quad permutes for 1 and 2 (no LDS traffic, fold into the
+// consuming add), ds_swizzle for 4, 8, 16, the LDS crossbar permute for 32.
+template <int S>
+__device__ __forceinline__ float dm_xor_lane(float v) {
+  int i = __builtin_bit_cast(int, v);
+  if constexpr (S == 1)
+    i = __builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  else if constexpr (S == 2)
+    i = __builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  else if constexpr (S == 4)
+    i = __builtin_amdgcn_ds_swizzle(i, 0x101F);  // bit-mask mode: and 0x1f, xor 4
+  else if constexpr (S == 8)
+    i = __builtin_amdgcn_ds_swizzle(i, 0x201F);
+  else if constexpr (S == 16)
+    i = __builtin_amdgcn_ds_swizzle(i, 0x401F);
+  else
+    i = __shfl_xor(i, 32, 64);
+  return __builtin_bit_cast(float, i);
+}
+
 template <int WIDTH>
 __device__ __forceinline__ float dm_wave_sum(float v) {
-#pragma unroll
-  for (int s = WIDTH / 2; s >= 1; s >>= 1) v = v + __shfl_xor(v, s, 64);
+  if constexpr (WIDTH >= 64) v = v + dm_xor_lane<32>(v);
+  if constexpr (WIDTH >= 32) v = v + dm_xor_lane<16>(v);
+  if constexpr (WIDTH >= 16) v = v + dm_xor_lane<8>(v);
+  if constexpr (WIDTH >= 8) v = v + dm_xor_lane<4>(v);
+  if constexpr (WIDTH >= 4) v = v + dm_xor_lane<2>(v);
+  if constexpr (WIDTH >= 2) v = v + dm_xor_lane<1>(v);
   return v;
 }
 template <int WIDTH>
 __device__ __forceinline__ float dm_wave_max(float v) {
-#pragma unroll
-  for (int s = WIDTH / 2; s >= 1; s >>= 1) {
-    float o = __shfl_xor(v, s, 64);
-    v = o > v ? o : v;
-  }
+  float o;
+  if constexpr (WIDTH >= 64) { o = dm_xor_lane<32>(v); v = o > v ? o : v; }
+  if constexpr (WIDTH >= 32) { o = dm_xor_lane<16>(v); v = o > v ? o : v; }
+  if constexpr (WIDTH >= 16) { o = dm_xor_lane<8>(v); v = o > v ? o : v; }
+  if constexpr (WIDTH >= 8) { o = dm_xor_lane<4>(v); v = o > v ? o : v; }
+  if constexpr (WIDTH >= 4) { o = dm_xor_lane<2>(v); v = o > v ? o : v; }
+  if constexpr (WIDTH >= 2) { o = dm_xor_lane<1>(v); v = o > v ? o : v; }
   return v;
+}
+
+// Four 64-lane butterfly sums for the price of one and a bit: at the 32 and 16 steps
+// each lane sends the value its partner is going to keep, so two sums share a permute.
+// Every addition pairs the same two operands as the plain butterfly, so the bits are
+// those of dm_wave_sum<64>. On return lanes [0,16) hold sum(a), [16,32) sum(c),
+// [32,48) sum(b), [48,64) sum(d).
+__device__ __forceinline__ float dm_wave_sum4(float a, float b, float c, float d, int lane) {
+  const bool h32 = lane & 32, h16 = lane & 16;
+  const float r1 = (h32 ? b : a) + dm_xor_lane<32>(h32 ? a : b);
+  const float r2 = (h32 ? d : c) + dm_xor_lane<32>(h32 ? c : d);
+  float r = (h16 ? r2 : r1) + dm_xor_lane<16>(h16 ? r1 : r2);
+  r = r + dm_xor_lane<8>(r);
+  r = r + dm_xor_lane<4>(r);
+  r = r + dm_xor_lane<2>(r);
+  r = r + dm_xor_lane<1>(r);
+  return r;
+}
+__device__ __forceinline__ float dm_lane_value(float v, int lane) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// byte k of a dword as a float, one instruction (the compiler's own pattern match gives
+// a bit-field extract plus a convert once the operand carries a nibble mask)
+__device__ __forceinline__ float dm_ubyte0(uint32_t w) { float r; asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(r) : "v"(w)); return r; }
+__device__ __forceinline__ float dm_ubyte1(uint32_t w) { float r; asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(r) : "v"(w)); return r; }
+__device__ __forceinline__ float dm_ubyte2(uint32_t w) { float r; asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(r) : "v"(w)); return r; }
+__device__ __forceinline__ float dm_ubyte3(uint32_t w) { float r; asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(r) : "v"(w)); return r; }
+template <int K>
+__device__ __forceinline__ float dm_ubyte(uint32_t w) {
+  if constexpr (K == 0) return dm_ubyte0(w);
+  else if constexpr (K == 1) return dm_ubyte1(w);
+  else if constexpr (K == 2) return dm_ubyte2(w);
+  else return dm_ubyte3(w);
 }

@@ -57,11 +57,16 @@ struct Q4Lane {
   float xl[M][16], xh[M][16], sl[M], sh[M];
   int b, g, h;  // block, 64-group, half
 
-  template <bool XF32>
-  __device__ __forceinline__ void load_x(const void* const (&xrow)[M], int chunk) {
+  // which block / group / half chunk `chunk` of a row is (needed by the row loads)
+  __device__ __forceinline__ void set_chunk(int chunk) {
     b = chunk >> 3;
     g = (chunk & 7) >> 1;
     h = chunk & 1;
+  }
+
+  template <bool XF32>
+  __device__ __forceinline__ void load_x(const void* const (&xrow)[M], int chunk) {
+    set_chunk(chunk);
     const int off = 256 * b + 64 * g + 16 * h;
 #pragma unroll
     for (int t = 0; t < M; ++t) {
@@ -104,14 +109,10 @@ __device__ __forceinline__ void q4_accumulate(const Q4Row& r, const Q4Lane<M>& L
   const int sh16 = (L.g & 1) * 16;
   const uint32_t a = (r.s0 >> sh16) & 0xffffu, b = (r.s1 >> sh16) & 0xffffu,
                  c = (r.s2 >> sh16) & 0xffffu;
-  uint32_t sc16, m16;
-  if (L.g < 2) {
-    sc16 = a & 0x3f3fu;
-    m16 = b & 0x3f3fu;
-  } else {
-    sc16 = (c & 0x0f0fu) | ((a & 0xc0c0u) >> 2);
-    m16 = ((c >> 4) & 0x0f0fu) | ((b & 0xc0c0u) >> 2);
-  }
+  // both field layouts evaluated, one selected: no branch in the row loop
+  const bool low = L.g < 2;
+  const uint32_t sc16 = low ? (a & 0x3f3fu) : ((c & 0x0f0fu) | ((a & 0xc0c0u) >> 2));
+  const uint32_t m16 = low ? (b & 0x3f3fu) : (((c >> 4) & 0x0f0fu) | ((b & 0xc0c0u) >> 2));
   const float s1 = (float)(sc16 & 0xffu), s2 = (float)(sc16 >> 8);
   const float m1 = (float)(m16 & 0xffu), m2 = (float)(m16 >> 8);
   const float d = dm_h2f((f16_t)(r.dmw & 0xffffu)), dmin = dm_h2f((f16_t)(r.dmw >> 16));
@@ -126,15 +127,19 @@ __device__ __forceinline__ void q4_accumulate(const Q4Row& r, const Q4Lane<M>& L
     // high nibbles left in place: 16*n. Scaling by a power of two commutes with
     // every rounding below, so 16*sum == sum of 16*terms bit for bit.
     const uint32_t wh = w[k] & 0xf0f0f0f0u;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float fl = kq_ub(wl, i), fh = kq_ub(wh, i);
-#pragma unroll
-      for (int t = 0; t < M; ++t) {
-        lo[t] = dm_fma(L.xl[t][4 * k + i], fl, lo[t]);
-        hi[t] = dm_fma(L.xh[t][4 * k + i], fh, hi[t]);
-      }
-    }
+#define ORN_Q4_STEP(I)                                              \
+  {                                                                 \
+    const float fl = dm_ubyte<I>(wl), fh = dm_ubyte<I>(wh);         \
+    _Pragma("unroll") for (int t = 0; t < M; ++t) {                 \
+      lo[t] = dm_fma(L.xl[t][4 * k + I], fl, lo[t]);                \
+      hi[t] = dm_fma(L.xh[t][4 * k + I], fh, hi[t]);                \
+    }                                                               \
+  }
+    ORN_Q4_STEP(0)
+    ORN_Q4_STEP(1)
+    ORN_Q4_STEP(2)
+    ORN_Q4_STEP(3)
+#undef ORN_Q4_STEP
   }
 #pragma unroll
   for (int t = 0; t < M; ++t) {
@@ -154,11 +159,15 @@ struct Q6Lane {
   float x[M][4][16];
   int b, n, u;
 
-  template <bool XF32>
-  __device__ __forceinline__ void load_x(const void* const (&xrow)[M], int chunk) {
+  __device__ __forceinline__ void set_chunk(int chunk) {
     b = chunk >> 2;
     n = (chunk & 3) >> 1;
     u = chunk & 1;
+  }
+
+  template <bool XF32>
+  __device__ __forceinline__ void load_x(const void* const (&xrow)[M], int chunk) {
+    set_chunk(chunk);
     const int off = 256 * b + 128 * n + 16 * u;
 #pragma unroll
     for (int t = 0; t < M; ++t)
@@ -203,16 +212,17 @@ __device__ __forceinline__ void q6_accumulate(const Q6Row& r, const Q6Lane<M>& L
     c[1] = (B[k] & 0x0f0f0f0fu) | ((H[k] << 2) & 0x30303030u);
     c[2] = ((A[k] >> 4) & 0x0f0f0f0fu) | (H[k] & 0x30303030u);
     c[3] = ((B[k] >> 4) & 0x0f0f0f0fu) | ((H[k] >> 2) & 0x30303030u);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        // code - 32, exact either as an integer or (as here) as a float subtract
-        const float q = kq_ub(c[g], i) - 32.0f;
-#pragma unroll
-        for (int t = 0; t < M; ++t) s[t][g] = dm_fma(L.x[t][g][4 * k + i], q, s[t][g]);
-      }
-    }
+    // code - 32, exact either as an integer or (as here) as a float subtract
+#define ORN_Q6_STEP(I)                                                                        \
+  _Pragma("unroll") for (int g = 0; g < 4; ++g) {                                             \
+    const float q = dm_ubyte<I>(c[g]) - 32.0f;                                                \
+    _Pragma("unroll") for (int t = 0; t < M; ++t) s[t][g] = dm_fma(L.x[t][g][4 * k + I], q, s[t][g]); \
+  }
+    ORN_Q6_STEP(0)
+    ORN_Q6_STEP(1)
+    ORN_Q6_STEP(2)
+    ORN_Q6_STEP(3)
+#undef ORN_Q6_STEP
   }
   // scales: bytes u, u+2, u+4, u+6 of the half's eight
   const uint32_t lo = r.sc.x >> (8 * L.u), hi = r.sc.y >> (8 * L.u);

@@ -13,6 +13,11 @@
 #include "dmath.h"
 #include "rt.h"
 
+// kquant.hip
+extern "C" int kq_qmv_add_rms(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int M, void* d_y,
+                   const void* d_res, const void* d_wnorm, float eps, void* d_h_out,
+                   void* d_normed_out);
+
 namespace {
 
 // ---- 8-bit affine, group 64 ---------------------------------------------
@@ -50,13 +55,23 @@ __global__ __launch_bounds__(64) void affine8_qmv_kernel(const uint8_t* w, const
 // ---- dense bf16 ------------------------------------------------------------
 // grid.x covers rows four at a time (one per wavefront), grid.y is the
 // activation row; GATHER selects expert / activation row through lhs, rhs.
+// rows [0, O) of w -> y; with w2 != null rows [O, O + O2) come from w2 and go to y2
+// (two small projections of the same activations in one launch)
 template <bool GATHER>
 __global__ __launch_bounds__(256) void dense_gemv_kernel(const bf16_t* w, const bf16_t* x,
                                                          bf16_t* y, int O, int K, int E, int x_rows,
-                                                         const uint32_t* lhs, const uint32_t* rhs) {
+                                                         const uint32_t* lhs, const uint32_t* rhs,
+                                                         const bf16_t* w2 = nullptr,
+                                                         bf16_t* y2 = nullptr, int O2 = 0) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int o = blockIdx.x * 4 + wave;
-  if (o >= O) return;
+  int o = blockIdx.x * 4 + wave;
+  if (o >= O + O2) return;
+  if (o >= O) {
+    o -= O;
+    w = w2;
+    y = y2;
+    O = O2;
+  }
   const int r = blockIdx.y;
   const bf16_t* wr;
   const bf16_t* xr;
@@ -132,6 +147,49 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
     default:
       return ornith_fail(ORNITH_ERR_INVALID, "linear_matmul: unknown mode %d", w->mode);
   }
+}
+
+int ornith_linear_matmul_add_rms(ornith_ctx* ctx, const ornith_linear* w, const void* d_x, int M,
+                                 void* d_y, const void* d_res, const void* d_wnorm, float eps,
+                                 void* d_h_out, void* d_normed_out) {
+  ORN_REQUIRE(ctx && w && d_x && d_y && d_res && d_wnorm && d_h_out && d_normed_out,
+              "linear_matmul_add_rms: null argument");
+  if (ornith_option_fuse_proj() && w->mode == ORNITH_LIN_KQUANT) {
+    const int rc = kq_qmv_add_rms(ctx, &w->km, d_x, M, d_y, d_res, d_wnorm, eps, d_h_out, d_normed_out);
+    if (rc >= 0) return rc;
+  }
+  int rc = ornith_linear_matmul(ctx, w, d_x, M, d_y);
+  if (rc) return rc;
+  return ornith_add_rms_norm(ctx, d_res, d_y, d_wnorm, M, w->O, eps, d_h_out, d_normed_out);
+}
+
+int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, int n,
+                               const void* d_x, int M, void* const* d_ys) {
+  ORN_REQUIRE(ctx && ws && d_x && d_ys && n >= 1, "linear_matmul_multi: bad argument");
+  bool fuse = ornith_option_fuse_proj() && n >= 2 && n <= 4;
+  for (int i = 0; i < n; ++i) {
+    ORN_REQUIRE(ws[i] && d_ys[i], "linear_matmul_multi: null entry %d", i);
+    fuse = fuse && ws[i]->mode == ws[0]->mode && ws[i]->K == ws[0]->K;
+    if (ws[i]->mode == ORNITH_LIN_KQUANT) fuse = fuse && ws[i]->km.kind == ws[0]->km.kind;
+  }
+  if (fuse && ws[0]->mode == ORNITH_LIN_KQUANT) {
+    const ornith_kmatrix* kms[4];
+    for (int i = 0; i < n; ++i) kms[i] = &ws[i]->km;
+    return ornith_kq_qmv_multi(ctx, kms, n, d_x, ORNITH_BF16, M, d_ys, ORNITH_BF16);
+  }
+  if (fuse && ws[0]->mode == ORNITH_LIN_DENSE && n == 2 && ws[0]->K % 8 == 0 && M <= 65535) {
+    hipLaunchKernelGGL(dense_gemv_kernel<false>, dim3((ws[0]->O + ws[1]->O + 3) / 4, M), dim3(256),
+                       0, ctx->stream, (const bf16_t*)ws[0]->d_w, (const bf16_t*)d_x,
+                       (bf16_t*)d_ys[0], ws[0]->O, ws[0]->K, 1, M, nullptr, nullptr,
+                       (const bf16_t*)ws[1]->d_w, (bf16_t*)d_ys[1], ws[1]->O);
+    ORN_LAUNCH_CHECK("dense_gemv_kernel<pair>");
+    return ORNITH_OK;
+  }
+  for (int i = 0; i < n; ++i) {
+    int rc = ornith_linear_matmul(ctx, ws[i], d_x, M, d_ys[i]);
+    if (rc) return rc;
+  }
+  return ORNITH_OK;
 }
 
 int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K, const void* d_x,

@@ -157,23 +157,24 @@ int model_ensure_rope(ornith_model* m, int npos) {
   return ORNITH_OK;
 }
 
-// q/k/v projections, per-head norm + rope + append, attention + gate, o_proj.
-// `sb` provides qg, kx, vx, q_rot, att of at least T rows.
+// q/k/v projections, per-head norm + rope + append, attention + gate; the caller applies
+// o_proj to `att`. qg, kx, vx, q_rot, att hold at least T rows.
 static int attention_block(ornith_model* m, const AttnLayer& a, const void* d_x, int T, void* k_cache,
                            void* v_cache, int offset, int cap, char* qg, char* kx, char* vx,
-                           char* q_rot, char* att, void* d_out) {
+                           char* q_rot, char* att) {
   ornith_ctx* ctx = m->ctx;
   const auto& c = m->cfg;
-  TRY(ornith_linear_matmul(ctx, &a.q_proj, d_x, T, qg));
-  TRY(ornith_linear_matmul(ctx, &a.k_proj, d_x, T, kx));
-  TRY(ornith_linear_matmul(ctx, &a.v_proj, d_x, T, vx));
+  {
+    const ornith_linear* ws[3] = {&a.q_proj, &a.k_proj, &a.v_proj};
+    void* ys[3] = {qg, kx, vx};
+    TRY(ornith_linear_matmul_multi(ctx, ws, 3, d_x, T, ys));
+  }
   TRY(ornith_attn_prep(ctx, qg, kx, vx, a.q_norm, a.k_norm, T, c.num_attention_heads,
                        c.num_key_value_heads, c.head_dim, c.rope_dims, c.rms_norm_eps, m->d_cos,
                        m->d_sin, m->rope_npos, offset, nullptr, cap, q_rot, k_cache, v_cache));
   const float scale = 1.0f / sqrtf((float)c.head_dim);
-  TRY(ornith_sdpa_decode_gated(ctx, q_rot, k_cache, v_cache, qg, T, c.num_attention_heads,
-                               c.num_key_value_heads, c.head_dim, offset, nullptr, cap, scale, att));
-  return ornith_linear_matmul(ctx, &a.o_proj, att, T, d_out);
+  return ornith_sdpa_decode_gated(ctx, q_rot, k_cache, v_cache, qg, T, c.num_attention_heads,
+                                  c.num_key_value_heads, c.head_dim, offset, nullptr, cap, scale, att);
 }
 
 static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_tokens, int T,
@@ -192,25 +193,31 @@ static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_to
     LayerCache& lc = cc->layers[i];
     if (L.linear) {
       const GdnLayer& g = L.gdn;
-      TRY(ornith_linear_matmul(ctx, &g.in_proj_qkv, s.normed, T, s.qkv));
-      TRY(ornith_linear_matmul(ctx, &g.in_proj_z, s.normed, T, s.z));
-      TRY(ornith_linear_matmul(ctx, &g.in_proj_a, s.normed, T, s.a));
-      TRY(ornith_linear_matmul(ctx, &g.in_proj_b, s.normed, T, s.b));
+      {
+        const ornith_linear* big[2] = {&g.in_proj_qkv, &g.in_proj_z};
+        void* ybig[2] = {s.qkv, s.z};
+        TRY(ornith_linear_matmul_multi(ctx, big, 2, s.normed, T, ybig));
+        const ornith_linear* ab[2] = {&g.in_proj_a, &g.in_proj_b};
+        void* yab[2] = {s.a, s.b};
+        TRY(ornith_linear_matmul_multi(ctx, ab, 2, s.normed, T, yab));
+      }
       const char* conv_state = (const char*)lc.conv[cc->conv_cur] + (size_t)cc->conv_off * D * 2;
       TRY(ornith_gdn_front(ctx, conv_state, s.qkv, g.conv1d, s.a, s.b, g.a_log, g.dt_bias, T, K, Hk,
                            Dk, Hv, Dv, 1e-6f, s.q, s.k, s.v, s.beta, s.g, lc.conv[1 - cc->conv_cur]));
       TRY(ornith_gdn_recurrence(ctx, s.q, s.k, s.v, s.g, s.beta, lc.state + (size_t)cc->state_cur * ssz,
                                 T, Hk, Hv, Dk, Dv, s.y, lc.state, capture ? 1 : 0));
       TRY(ornith_rms_norm_gated(ctx, s.y, g.norm, s.z, T * Hv, Dv, c.rms_norm_eps, s.gated));
-      TRY(ornith_linear_matmul(ctx, &g.out_proj, s.gated, T, s.r));
+      TRY(ornith_linear_matmul_add_rms(ctx, &g.out_proj, s.gated, T, s.r, s.x, L.post_ln,
+                                       c.rms_norm_eps, s.h, s.normed2));
     } else {
       TRY(attention_block(m, L.attn, s.normed, T, lc.k, lc.v, cc->offset, cc->capacity, s.qg, s.kx,
-                          s.vx, s.q_rot, s.att, s.r));
+                          s.vx, s.q_rot, s.att));
+      TRY(ornith_linear_matmul_add_rms(ctx, &L.attn.o_proj, s.att, T, s.r, s.x, L.post_ln,
+                                       c.rms_norm_eps, s.h, s.normed2));
     }
-    TRY(ornith_add_rms_norm(ctx, s.x, s.r, L.post_ln, T, H, c.rms_norm_eps, s.h, s.normed2));
-    TRY(ornith_moe_block(ctx, &L.moe, s.normed2, T, s.mo, nullptr, nullptr));
     const void* next_w = (i + 1 < m->layers.size()) ? m->layers[i + 1].input_ln : m->final_norm;
-    TRY(ornith_add_rms_norm(ctx, s.h, s.mo, next_w, T, H, c.rms_norm_eps, s.x, s.normed));
+    TRY(ornith_moe_block_add_rms(ctx, &L.moe, s.normed2, T, s.mo, s.h, next_w, c.rms_norm_eps, s.x,
+                                 s.normed));
   }
   TRY(ornith_copy(ctx, d_hidden_out, s.normed, (size_t)T * H * 2));
   // every layer advanced together
@@ -609,11 +616,12 @@ int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspec, const vo
   }
   TRY(ornith_linear_matmul(ctx, &h->fc, joined, T, x));
   TRY(ornith_rms_norm(ctx, x, h->input_ln, T, (int)H, c.rms_norm_eps, normed));
-  TRY(attention_block(m, h->attn, normed, T, h->k, h->v, h->offset, h->capacity, qg, kx, vx, q_rot, att, r));
-  TRY(ornith_add_rms_norm(ctx, x, r, h->post_ln, T, (int)H, c.rms_norm_eps, hh, normed2));
-  TRY(ornith_moe_block(ctx, &h->moe, normed2, T, mo, nullptr, nullptr));
+  TRY(attention_block(m, h->attn, normed, T, h->k, h->v, h->offset, h->capacity, qg, kx, vx, q_rot, att));
+  TRY(ornith_linear_matmul_add_rms(ctx, &h->attn.o_proj, att, T, r, x, h->post_ln, c.rms_norm_eps, hh,
+                                   normed2));
   // add(h, m) then mtp.norm; the un-normed sum is not needed afterwards
-  TRY(ornith_add_rms_norm(ctx, hh, mo, h->norm, T, (int)H, c.rms_norm_eps, x, d_hidden_out));
+  TRY(ornith_moe_block_add_rms(ctx, &h->moe, normed2, T, mo, hh, h->norm, c.rms_norm_eps, x,
+                               d_hidden_out));
   h->offset += T;
   if (d_logits) {
     const ornith_linear* lm = frspec ? &frspec->head : &m->lm_head;

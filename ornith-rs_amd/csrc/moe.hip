@@ -9,14 +9,17 @@
 //
 // Rounding points are the reference's: gates, probabilities, every expert output
 // and every step of the tail are bf16; sums inside a kernel are fp32.
-#include "dmath.h"
+#include "moe_device.h"
 #include "rt.h"
 
 // moe_fused.hip
 bool moe_fused_supported(const ornith_moe_weights* w);
+bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                      void* d_gates, uint32_t* d_inds, void* d_scores, void* d_egate, int* rc);
+bool moe_fused_tail_supported(const ornith_moe_weights* w, int T);
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
-                      void* d_out);
+                      void* d_out, int phases, const MoeTail* tail);
 
 namespace {
 
@@ -32,65 +35,8 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const bf16_t* gates, in
                                                          bf16_t* probs, uint32_t* lhs_tok,
                                                          uint32_t* lhs_row) {
   const int t = blockIdx.x, lane = threadIdx.x;
-  const bf16_t* g = gates + (size_t)t * E + lane * PER;
-  float v[PER];
-  float m = -DM_INF;
-#pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    v[i] = dm_bf2f(g[i]);
-    m = v[i] > m ? v[i] : m;
-  }
-  m = dm_wave_max<64>(m);
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    v[i] = dm_exp(v[i] - m);
-    s = s + v[i];
-  }
-  const float inv = 1.0f / dm_wave_sum<64>(s);
-#pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    const bf16_t pb = dm_f2bf(v[i] * inv);
-    if (probs) probs[(size_t)t * E + lane * PER + i] = pb;
-    v[i] = dm_bf2f(pb);
-  }
-  for (int r = 0; r < k; ++r) {
-    float best = -DM_INF;
-    int besti = -1;
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      // ascending i, so >= keeps the larger index among equals
-      if (v[i] >= best && !(v[i] != v[i])) {
-        if (v[i] > best || besti < lane * PER + i) {
-          best = v[i];
-          besti = lane * PER + i;
-        }
-      }
-    }
-    const float wm = dm_wave_max<64>(best);
-    int cand = (best == wm) ? besti : -1;
-#pragma unroll
-    for (int sft = 32; sft >= 1; sft >>= 1) {
-      const int o = __shfl_xor(cand, sft, 64);
-      cand = o > cand ? o : cand;
-    }
-    // cand: the winning expert, identical in every lane (never -1: probabilities are
-    // finite and at most k <= E entries are ever removed)
-    const int owner = cand / PER;
-    float wv = 0.f;
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      if (lane == owner && i == cand - owner * PER) {
-        wv = v[i];
-        v[i] = -DM_INF;
-      }
-    }
-    if (lane == owner) {
-      const size_t slot = (size_t)t * k + (k - 1 - r);
-      inds[slot] = (uint32_t)cand;
-      scores[slot] = dm_f2bf(wv);  // already a bf16 value
-    }
-  }
+  router_topk_wave<PER>(gates + (size_t)t * E, k, inds + (size_t)t * k, scores + (size_t)t * k,
+                        probs ? probs + (size_t)t * E : nullptr, lane);
   if (lane < k) {
     if (lhs_tok) lhs_tok[t * k + lane] = t;
     if (lhs_row) lhs_row[t * k + lane] = t * k + lane;
@@ -183,8 +129,10 @@ int ornith_moe_combine(ornith_ctx* ctx, const void* d_scores, const void* d_y, c
   return ORNITH_OK;
 }
 
-int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                     void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
+// The block; with `tail`, followed by h = res + out, normed = rms_norm(h).
+static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                          void* d_out, uint32_t* d_inds_out, void* d_scores_out,
+                          const MoeTail* tail) {
   ORN_REQUIRE(ctx && w && d_x && d_out, "moe_block: null argument");
   const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
   ORN_REQUIRE(T >= 1 && T <= 64, "moe_block: T=%d (decode/verify widths only)", T);
@@ -230,10 +178,19 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
   } while (0)
   if (ornith_option_fuse_moe() && moe_fused_supported(w)) {
     // three small launches for the router, then the two expert kernels
-    TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
-    TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
-    TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
-    TRY(moe_fused_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out));
+    int rrc = ORNITH_OK;
+    if (moe_fused_router(ctx, w, d_x, T, gates, inds, scores, eg, &rrc)) {
+      if (rrc) return rrc;
+    } else {
+      TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
+      TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
+      TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
+    }
+    const bool in_kernel = tail && moe_fused_tail_supported(w, T);
+    TRY(moe_fused_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, 3, in_kernel ? tail : nullptr));
+    if (tail && !in_kernel)
+      TRY(ornith_add_rms_norm(ctx, tail->d_res, d_out, tail->d_wnorm, T, H, tail->eps, tail->d_h_out,
+                              tail->d_normed_out));
     if (d_inds_out)
       ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,
                              ctx->stream));
@@ -265,6 +222,9 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
                              ORNITH_BF16));
   }
   TRY(ornith_moe_combine(ctx, scores, y, eg, sy, T, k, H, w->norm_topk_prob, d_out));
+  if (tail)
+    TRY(ornith_add_rms_norm(ctx, tail->d_res, d_out, tail->d_wnorm, T, H, tail->eps, tail->d_h_out,
+                            tail->d_normed_out));
   if (d_inds_out)
     ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,
                            ctx->stream));
@@ -273,6 +233,19 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
                            ctx->stream));
 #undef TRY
   return ORNITH_OK;
+}
+
+int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                     void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
+  return moe_block_impl(ctx, w, d_x, T, d_out, d_inds_out, d_scores_out, nullptr);
+}
+
+int ornith_moe_block_add_rms(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                             void* d_out, const void* d_res, const void* d_wnorm, float eps,
+                             void* d_h_out, void* d_normed_out) {
+  ORN_REQUIRE(d_res && d_wnorm && d_h_out && d_normed_out, "moe_block_add_rms: null argument");
+  const MoeTail tail{d_res, d_wnorm, eps, d_h_out, d_normed_out};
+  return moe_block_impl(ctx, w, d_x, T, d_out, nullptr, nullptr, &tail);
 }
 
 }  // extern "C"

@@ -1,0 +1,73 @@
+// Device-side router: precise softmax (fp32 inside, bf16 out) and top-k selection for
+// one token by one wavefront. Shared by the stand-alone router kernel and the fused
+// router launch.
+//
+// Restates vendored softmax.h:10-98 and /root/reference/kernels/moe.metal:568-614:
+// p = bf16(exp(g - max) * (1 / sum)); k rounds of selection under "by value, then by
+// larger index"; round r fills slot k-1-r, so the slots are the tail of a stable
+// ascending sort.
+#pragma once
+
+#include "dmath.h"
+
+template <int S>
+__device__ __forceinline__ uint32_t dm_xor_lane_u32(uint32_t v) {
+  return __builtin_bit_cast(uint32_t, dm_xor_lane<S>(__builtin_bit_cast(float, v)));
+}
+__device__ __forceinline__ uint32_t dm_wave_max_u32(uint32_t v) {
+  uint32_t o;
+  o = dm_xor_lane_u32<32>(v); v = o > v ? o : v;
+  o = dm_xor_lane_u32<16>(v); v = o > v ? o : v;
+  o = dm_xor_lane_u32<8>(v); v = o > v ? o : v;
+  o = dm_xor_lane_u32<4>(v); v = o > v ? o : v;
+  o = dm_xor_lane_u32<2>(v); v = o > v ? o : v;
+  o = dm_xor_lane_u32<1>(v); v = o > v ? o : v;
+  return v;
+}
+
+// Lane l holds gates [l*PER, (l+1)*PER) of the row. All 64 lanes must be active.
+// E = 64 * PER <= 1024 so an index fits 10 bits: a candidate is the single integer
+// (bf16 probability bits << 16 | index) + 1, whose order is exactly (value, index) for
+// the non-negative probabilities a softmax produces; 0 marks a taken entry.
+template <int PER>
+__device__ __forceinline__ void router_topk_wave(const bf16_t* gates_row, int k, uint32_t* inds_row,
+                                                 bf16_t* scores_row, bf16_t* probs_row, int lane) {
+  const bf16_t* g = gates_row + lane * PER;
+  float v[PER];
+  float m = -DM_INF;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    v[i] = dm_bf2f(g[i]);
+    m = v[i] > m ? v[i] : m;
+  }
+  m = dm_wave_max<64>(m);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    v[i] = dm_exp(v[i] - m);
+    s = s + v[i];
+  }
+  const float inv = 1.0f / dm_wave_sum<64>(s);
+  uint32_t key[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const bf16_t pb = dm_f2bf(v[i] * inv);
+    if (probs_row) probs_row[lane * PER + i] = pb;
+    // a NaN probability (NaN gates) never wins
+    key[i] = (pb & 0x7fffu) > 0x7f80u ? 0u : ((((uint32_t)(pb & 0x7fffu)) << 16) | (uint32_t)(lane * PER + i)) + 1u;
+  }
+  for (int r = 0; r < k; ++r) {
+    uint32_t best = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) best = key[i] > best ? key[i] : best;
+    const uint32_t win = dm_wave_max_u32(best);
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+      if (key[i] == win) key[i] = 0;
+    if (lane == 0) {
+      const uint32_t w = win - 1u;  // win == 0 only if every entry is NaN / taken: id wraps, clamped by users
+      inds_row[k - 1 - r] = win ? (w & 0xffffu) : 0xffffffffu;
+      scores_row[k - 1 - r] = win ? (bf16_t)(w >> 16) : (bf16_t)0;
+    }
+  }
+}

@@ -19,9 +19,15 @@
 //
 // These two kernels are the expert gather-GEMV: per distinct expert they stream
 // 2 x I x K Q4_K codes and H x I Q6_K codes once, with nothing but the activations
-// and index lists read besides.
+// and index lists read besides. Both are latency-shaped, not throughput-shaped: at
+// verify width 2 a launch moves ~19 MB / ~15 MB, less than the chip can hold in
+// flight, so every wavefront issues ALL of its weight loads first (they depend on
+// nothing but the index list), then the activation loads, and only then computes.
 #include "kq_device.h"
+#include "moe_device.h"
+#include "norm_device.h"
 #include "rt.h"
+#include "sync_device.h"
 
 namespace {
 
@@ -37,7 +43,7 @@ struct UpArgs {
   const bf16_t* x;       // [T, K]
   const uint32_t* inds;  // [T*k]
   bf16_t* act;           // [T*k + T, I]
-  int T, k, E, I, K, iters;
+  int T, k, E, I, K;
 };
 
 __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
@@ -46,8 +52,8 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
   return dm_f2bf(s * ub);
 }
 
-// grid (ceil(I / rows_per_block), T*k + T), 256 threads
-template <int KIND, int LPR>
+// grid (ceil(I / (RPW * 4 * ITERS)), T*k + T), 256 threads
+template <int KIND, int LPR, int ITERS>
 __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
   using KL = KqLane<KIND, 1>;
   constexpr int RPW = 64 / LPR;
@@ -70,25 +76,47 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
     wg = a.sgate;
     wu = a.sup;
   }
-  const void* xrow[1] = {a.x + (size_t)token * a.K};
   typename KL::Lane L;
-  L.template load_x<false>(xrow, c);
-
-  const int rows_per_wave = RPW * a.iters;
-  const int base = (blockIdx.x * 4 + wave) * rows_per_wave;
-#pragma unroll 2
-  for (int it = 0; it < a.iters; ++it) {
+  L.set_chunk(c);
+  const int base = (blockIdx.x * 4 + wave) * (RPW * ITERS);
+  typename KL::Row rg[ITERS], ru[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
     const int o = base + it * RPW + slot;
-    const bool valid = o < a.I;
-    const int64_t row = row0 + (valid ? o : a.I - 1);
-    const typename KL::Row rg = KL::load(wg.qs, wg.scales, wg.dm, row, nb, L);
-    const typename KL::Row ru = KL::load(wu.qs, wu.scales, wu.dm, row, nb, L);
-    float ag[1] = {0.f}, au[1] = {0.f};
-    KL::accumulate(rg, L, ag);
-    KL::accumulate(ru, L, au);
-    const float g = dm_wave_sum<LPR>(ag[0]);
-    const float u = dm_wave_sum<LPR>(au[0]);
-    if (c == 0 && valid) a.act[(size_t)r * a.I + o] = swiglu_bf16(g, u);
+    const int64_t row = row0 + (o < a.I ? o : a.I - 1);
+    rg[it] = KL::load(wg.qs, wg.scales, wg.dm, row, nb, L);
+    ru[it] = KL::load(wu.qs, wu.scales, wu.dm, row, nb, L);
+  }
+  const void* xrow[1] = {a.x + (size_t)token * a.K};
+  L.template load_x<false>(xrow, c);
+  if constexpr (LPR == 64 && ITERS % 2 == 0) {
+    // one row per wavefront pass: reduce two rows' gate and up sums together
+#pragma unroll
+    for (int it = 0; it < ITERS; it += 2) {
+      float g0[1] = {0.f}, u0[1] = {0.f}, g1[1] = {0.f}, u1[1] = {0.f};
+      KL::accumulate(rg[it], L, g0);
+      KL::accumulate(ru[it], L, u0);
+      KL::accumulate(rg[it + 1], L, g1);
+      KL::accumulate(ru[it + 1], L, u1);
+      const float red = dm_wave_sum4(g0[0], u0[0], g1[0], u1[0], lane);
+      // lanes [0,16): gate row it, [32,48): up row it, [16,32): gate row it+1, [48,64): up row it+1
+      const float ga = dm_lane_value(red, 0), ua = dm_lane_value(red, 32);
+      const float gb = dm_lane_value(red, 16), ub = dm_lane_value(red, 48);
+      const int o = base + it;
+      if (lane == 0 && o < a.I) a.act[(size_t)r * a.I + o] = swiglu_bf16(ga, ua);
+      if (lane == 1 && o + 1 < a.I) a.act[(size_t)r * a.I + o + 1] = swiglu_bf16(gb, ub);
+    }
+  } else {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int o = base + it * RPW + slot;
+      float ag[1] = {0.f}, au[1] = {0.f};
+      KL::accumulate(rg[it], L, ag);
+      KL::accumulate(ru[it], L, au);
+      const float g = dm_wave_sum<LPR>(ag[0]);
+      const float u = dm_wave_sum<LPR>(au[0]);
+      if (c == 0 && o < a.I) a.act[(size_t)r * a.I + o] = swiglu_bf16(g, u);
+    }
   }
 }
 
@@ -100,26 +128,42 @@ struct DownArgs {
   const bf16_t* scores;  // [T*k]
   const bf16_t* egate;   // [T]
   bf16_t* out;           // [T, H]
-  int T, k, E, H, I, iters, normalize;
+  int T, k, E, H, I, normalize;
+  AddRmsTail tail;       // tail.counter != null: the last workgroup also applies h = res + out,
+                         // normed = rms_norm(h) to the T rows (needs T <= k + 1)
 };
 
 constexpr int kMaxK = 8;
-constexpr int kMaxCols = 64 * 4;  // RPW * iters upper bound (LPR >= 4, iters <= 16)
 
-// grid (ceil(H / (RPW * iters)), T), 64 * (k + 1) threads
-template <int KIND, int LPR>
+// grid (ceil(H / (RPW * ITERS)), T), 64 * (k + 1) threads
+template <int KIND, int LPR, int ITERS>
 __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) {
   using KL = KqLane<KIND, 1>;
-  constexpr int RPW = 64 / LPR;
+  constexpr int RPW = 64 / LPR, COLS = RPW * ITERS;
   const int lane = threadIdx.x & 63, j = threadIdx.x >> 6;  // j: expert slot, k = shared
   const int slot = lane / LPR, c = lane % LPR;
   const int nb = a.I >> 8;
   const int t = blockIdx.y, k = a.k;
-  const int cols = RPW * a.iters, c0 = blockIdx.x * cols;
+  const int c0 = blockIdx.x * COLS;
 
-  __shared__ float yl[kMaxK + 1][kMaxCols];
+  __shared__ float yl[kMaxK + 1][COLS];
   __shared__ float wj[kMaxK];
   __shared__ float gsig;
+
+  const bool shared = j == k;
+  const int arow = shared ? a.T * k + t : t * k + j;
+  const KqPtr w = shared ? a.sdown : a.down;
+  const int64_t row0 = shared ? 0 : (int64_t)min(a.inds[t * k + j], (uint32_t)(a.E - 1)) * a.H;
+  typename KL::Lane L;
+  L.set_chunk(c);
+  typename KL::Row rr[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int o = c0 + it * RPW + slot;
+    rr[it] = KL::load(w.qs, w.scales, w.dm, row0 + (o < a.H ? o : a.H - 1), nb, L);
+  }
+  const void* xrow[1] = {a.act + (size_t)arow * a.I};
+  L.template load_x<false>(xrow, c);
 
   if (j == 0) {
     // the router weights of this token: denom = ((0+s0)+s1)..., w_j = bf16(s_j / denom)
@@ -130,28 +174,16 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) 
     if (lane < k) wj[lane] = a.normalize ? dm_rb(dm_bf2f(s[lane]) / denom) : dm_bf2f(s[lane]);
     if (lane == 0) gsig = dm_sigmoid_bf16(dm_bf2f(a.egate[t]));
   }
-
-  const bool shared = j == k;
-  const int arow = shared ? a.T * k + t : t * k + j;
-  const KqPtr w = shared ? a.sdown : a.down;
-  const int64_t row0 = shared ? 0 : (int64_t)min(a.inds[t * k + j], (uint32_t)(a.E - 1)) * a.H;
-  const void* xrow[1] = {a.act + (size_t)arow * a.I};
-  typename KL::Lane L;
-  L.template load_x<false>(xrow, c);
-#pragma unroll 2
-  for (int it = 0; it < a.iters; ++it) {
-    const int col = it * RPW + slot;
-    const int o = c0 + col;
-    const bool valid = o < a.H;
-    const typename KL::Row r = KL::load(w.qs, w.scales, w.dm, row0 + (valid ? o : a.H - 1), nb, L);
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
     float acc[1] = {0.f};
-    KL::accumulate(r, L, acc);
+    KL::accumulate(rr[it], L, acc);
     const float v = dm_wave_sum<LPR>(acc[0]);
-    if (c == 0) yl[j][col] = dm_rb(v);  // expert outputs are bf16 in the unfused path
+    if (c == 0) yl[j][it * RPW + slot] = dm_rb(v);  // expert outputs are bf16 in the unfused path
   }
   __syncthreads();
   const int col = threadIdx.x;
-  if (col < cols && c0 + col < a.H) {
+  if (col < COLS && c0 + col < a.H) {
     float acc = 0.f;
     for (int i = 0; i < k; ++i) {
       const float weighted = dm_rb(yl[i][col] * wj[i]);
@@ -159,6 +191,117 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) 
     }
     const float gated = dm_rb(gsig * yl[k][col]);
     a.out[(size_t)t * a.H + c0 + col] = dm_f2bf(acc + gated);
+  }
+  if (a.tail.counter) {
+    if (!last_block_done(a.tail.counter, gridDim.x * gridDim.y)) return;
+    if (j < a.T) add_rms_tail_row(a.tail, a.out + (size_t)j * a.H, j, a.H, lane);
+  }
+}
+
+// ---- router: gates mat-vec, then the last workgroup does softmax + top-k and the
+// shared expert's scalar gate for every token (one wavefront per token) -------------
+struct RouterArgs {
+  KqPtr w;               // router [E, K]
+  const bf16_t* x;       // [M, K]
+  bf16_t* gates;         // [M, E]
+  uint32_t* inds;        // [M, k]
+  bf16_t* scores;        // [M, k]
+  bf16_t* egate;         // [M]
+  const void* eg_w;      // shared_expert_gate weights: affine8 u8[K] or dense bf16[K]
+  const bf16_t* eg_s;    // affine8 scales [K/64]
+  const bf16_t* eg_b;    // affine8 biases [K/64]
+  int eg_affine;
+  unsigned int* counter;
+  int E, K, k;
+};
+
+// one row of the 8-bit affine / dense mat-vec by one wavefront (the order of linear.hip)
+__device__ __forceinline__ float egate_row_dot(const RouterArgs& a, const bf16_t* xr, int lane) {
+  float acc_lane = 0.f;
+  for (int j = lane; j < a.K / 8; j += 64) {
+    const uint4 xv = *reinterpret_cast<const uint4*>(xr + 8 * j);
+    const float xs[8] = {dm_bf2f_lo(xv.x), dm_bf2f_hi(xv.x), dm_bf2f_lo(xv.y), dm_bf2f_hi(xv.y),
+                         dm_bf2f_lo(xv.z), dm_bf2f_hi(xv.z), dm_bf2f_lo(xv.w), dm_bf2f_hi(xv.w)};
+    if (a.eg_affine) {
+      const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint8_t*>(a.eg_w) + 8 * j);
+      const uint32_t qw[2] = {q.x, q.y};
+      float acc = 0.f, sum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float qf = (float)((qw[i >> 2] >> (8 * (i & 3))) & 0xffu);
+        acc = dm_fma(xs[i], qf, acc);
+        sum = sum + xs[i];
+      }
+      float p = dm_bf2f(a.eg_s[j >> 3]) * acc;
+      p = dm_fma(sum, dm_bf2f(a.eg_b[j >> 3]), p);
+      acc_lane = acc_lane + p;
+    } else {
+      const uint4 wv = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(a.eg_w) + 8 * j);
+      acc_lane = dm_fma(dm_bf2f_lo(wv.x), xs[0], acc_lane);
+      acc_lane = dm_fma(dm_bf2f_hi(wv.x), xs[1], acc_lane);
+      acc_lane = dm_fma(dm_bf2f_lo(wv.y), xs[2], acc_lane);
+      acc_lane = dm_fma(dm_bf2f_hi(wv.y), xs[3], acc_lane);
+      acc_lane = dm_fma(dm_bf2f_lo(wv.z), xs[4], acc_lane);
+      acc_lane = dm_fma(dm_bf2f_hi(wv.z), xs[5], acc_lane);
+      acc_lane = dm_fma(dm_bf2f_lo(wv.w), xs[6], acc_lane);
+      acc_lane = dm_fma(dm_bf2f_hi(wv.w), xs[7], acc_lane);
+    }
+  }
+  return dm_wave_sum<64>(acc_lane);
+}
+
+// grid ceil(E / (RPW * 4)), 256 threads, M <= 4 tokens
+template <int KIND, int LPR, int M>
+__global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
+  using KL = KqLane<KIND, M>;
+  constexpr int RPW = 64 / LPR;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int slot = lane / LPR, c = lane % LPR;
+  const int nb = a.K >> 8;
+  typename KL::Lane L;
+  L.set_chunk(c);
+  const int o = (blockIdx.x * 4 + wave) * RPW + slot;
+  const typename KL::Row row = KL::load(a.w.qs, a.w.scales, a.w.dm, o < a.E ? o : a.E - 1, nb, L);
+  const void* xrow[M];
+#pragma unroll
+  for (int t = 0; t < M; ++t) xrow[t] = a.x + (size_t)t * a.K;
+  L.template load_x<false>(xrow, c);
+  float acc[M];
+#pragma unroll
+  for (int t = 0; t < M; ++t) acc[t] = 0.f;
+  KL::accumulate(row, L, acc);
+#pragma unroll
+  for (int t = 0; t < M; ++t) {
+    const float v = dm_wave_sum<LPR>(acc[t]);
+    if (c == 0 && o < a.E) a.gates[(size_t)t * a.E + o] = dm_f2bf(v);
+  }
+  if (!last_block_done(a.counter, gridDim.x)) return;
+  if (wave < M) {
+    const int t = wave;
+    const bf16_t* g = a.gates + (size_t)t * a.E;
+    uint32_t* ir = a.inds + (size_t)t * a.k;
+    bf16_t* sr = a.scores + (size_t)t * a.k;
+    switch (a.E / 64) {
+      case 1: router_topk_wave<1>(g, a.k, ir, sr, nullptr, lane); break;
+      case 2: router_topk_wave<2>(g, a.k, ir, sr, nullptr, lane); break;
+      case 4: router_topk_wave<4>(g, a.k, ir, sr, nullptr, lane); break;
+      case 8: router_topk_wave<8>(g, a.k, ir, sr, nullptr, lane); break;
+      default: router_topk_wave<16>(g, a.k, ir, sr, nullptr, lane); break;
+    }
+    const float e = egate_row_dot(a, a.x + (size_t)t * a.K, lane);
+    if (lane == 0) a.egate[t] = dm_f2bf(e);
+  }
+}
+
+template <int KIND, int LPR>
+void launch_router_fused(ornith_ctx* ctx, const RouterArgs& a, int M) {
+  constexpr int RPW = 64 / LPR;
+  dim3 grid((a.E + RPW * 4 - 1) / (RPW * 4));
+  switch (M) {
+    case 1: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 1>), grid, dim3(256), 0, ctx->stream, a); break;
+    case 2: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 2>), grid, dim3(256), 0, ctx->stream, a); break;
+    case 3: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 3>), grid, dim3(256), 0, ctx->stream, a); break;
+    default: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 4>), grid, dim3(256), 0, ctx->stream, a); break;
   }
 }
 
@@ -168,7 +311,42 @@ KqPtr ptr_of(const ornith_kmatrix& m) {
 
 int chunks_of(const ornith_kmatrix& m) { return (m.K >> 8) * (m.kind == ORNITH_Q4K ? 8 : 4); }
 
+template <int KIND, int LPR>
+void launch_up(ornith_ctx* ctx, const UpArgs& a, int rows_y) {
+  constexpr int RPW = 64 / LPR;
+  // Two rows per wavefront measured faster than four at every decode/verify width (four
+  // rows of gate + up codes in flight cost enough registers to halve the occupancy);
+  // four stays selectable for wider inputs.
+  if (ornith_option_moe_up_iters() == 4) {
+    dim3 grid((a.I + RPW * 4 * 4 - 1) / (RPW * 4 * 4), rows_y);
+    hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4>), grid, dim3(256), 0, ctx->stream, a);
+  } else {
+    dim3 grid((a.I + RPW * 4 * 2 - 1) / (RPW * 4 * 2), rows_y);
+    hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2>), grid, dim3(256), 0, ctx->stream, a);
+  }
+}
+
+template <int KIND, int LPR>
+void launch_down(ornith_ctx* ctx, const DownArgs& a) {
+  constexpr int RPW = 64 / LPR;
+  dim3 block(64 * (a.k + 1));
+  const long groups1 = (long)(a.H + RPW - 1) / RPW * a.T;
+  if (groups1 >= (long)ctx->compute_units * 4) {
+    dim3 grid((a.H + RPW * 2 - 1) / (RPW * 2), a.T);
+    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 2>), grid, block, 0, ctx->stream, a);
+  } else {
+    dim3 grid((a.H + RPW - 1) / RPW, a.T);
+    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 1>), grid, block, 0, ctx->stream, a);
+  }
+}
+
 }  // namespace
+
+// Whether the down kernel can also apply the residual add + norm that follows the block.
+bool moe_fused_tail_supported(const ornith_moe_weights* w, int T) {
+  const int H = w->router.K, per = H / 64;
+  return T <= w->top_k + 1 && H % 64 == 0 && per <= 64 && (per & (per - 1)) == 0;
+}
 
 // Whether the two fused kernels cover this block's shapes and formats.
 bool moe_fused_supported(const ornith_moe_weights* w) {
@@ -186,12 +364,56 @@ bool moe_fused_supported(const ornith_moe_weights* w) {
   return ok(cu) && ok(cd);
 }
 
-// act: scratch bf16 [(T*k + T), I]
+// Router mat-vec + softmax + top-k + shared_expert_gate in one launch. Returns false
+// (nothing launched) when the shapes / formats are outside what the kernel covers.
+bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                      void* d_gates, uint32_t* d_inds, void* d_scores, void* d_egate, int* rc) {
+  *rc = ORNITH_OK;
+  const ornith_linear& r = w->router;
+  const ornith_linear& g = w->sh_egate;
+  if (T > 4 || r.mode != ORNITH_LIN_KQUANT) return false;
+  if (g.mode != ORNITH_LIN_AFFINE8 && g.mode != ORNITH_LIN_DENSE) return false;
+  if (g.K % 64 != 0) return false;
+  const int E = r.O, per = E / 64;
+  if (E % 64 != 0 || !(per == 1 || per == 2 || per == 4 || per == 8 || per == 16)) return false;
+  const int nch = chunks_of(r.km);
+  if (!(nch == 8 || nch == 16 || nch == 32 || nch == 64)) return false;
+  RouterArgs a{};
+  a.w = ptr_of(r.km);
+  a.x = (const bf16_t*)d_x;
+  a.gates = (bf16_t*)d_gates;
+  a.inds = d_inds;
+  a.scores = (bf16_t*)d_scores;
+  a.egate = (bf16_t*)d_egate;
+  a.eg_w = g.d_w;
+  a.eg_s = (const bf16_t*)g.d_scales;
+  a.eg_b = (const bf16_t*)g.d_biases;
+  a.eg_affine = g.mode == ORNITH_LIN_AFFINE8;
+  a.counter = ctx->counters + 0;
+  a.E = E;
+  a.K = r.K;
+  a.k = w->top_k;
+#define R_CASE(KIND, N) \
+  case N:               \
+    launch_router_fused<KIND, N>(ctx, a, T); \
+    break;
+  if (r.km.kind == ORNITH_Q4K) {
+    switch (nch) { R_CASE(ORNITH_Q4K, 8) R_CASE(ORNITH_Q4K, 16) R_CASE(ORNITH_Q4K, 32) R_CASE(ORNITH_Q4K, 64) }
+  } else {
+    switch (nch) { R_CASE(ORNITH_Q6K, 8) R_CASE(ORNITH_Q6K, 16) R_CASE(ORNITH_Q6K, 32) R_CASE(ORNITH_Q6K, 64) }
+  }
+#undef R_CASE
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) *rc = ornith_fail(ORNITH_ERR_HIP, "launch of moe_router_kernel failed: %s", hipGetErrorString(e));
+  return true;
+}
+
+// act: scratch bf16 [(T*k + T), I]. phases: 1 = up, 2 = down, 3 = both.
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
-                      void* d_out) {
+                      void* d_out, int phases, const MoeTail* tail) {
   const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
-  {
+  if (phases & 1) {
     UpArgs a{};
     a.gate = ptr_of(w->ex_gate);
     a.up = ptr_of(w->ex_up);
@@ -205,26 +427,20 @@ int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
     a.E = E;
     a.I = I;
     a.K = H;
-    const int nch = chunks_of(w->ex_gate), rpw = 64 / nch;
-    const int rows_y = T * k + T;
-    // enough workgroups to fill the chip; each wavefront keeps >= 2 row loads in flight
-    int iters = (int)(((long)I * rows_y) / ((long)rpw * 4 * ctx->compute_units * 4));
-    iters = iters < 2 ? 2 : (iters > 8 ? 8 : iters);
-    a.iters = iters;
-    dim3 grid((I + rpw * 4 * iters - 1) / (rpw * 4 * iters), rows_y);
-#define UP_CASE(KIND, N)                                                                     \
-  case N:                                                                                    \
-    hipLaunchKernelGGL((moe_up_kernel<KIND, N>), grid, dim3(256), 0, ctx->stream, a);        \
+    const int nch = chunks_of(w->ex_gate), rows_y = T * k + T;
+#define UP_CASE(KIND, N) \
+  case N:                \
+    launch_up<KIND, N>(ctx, a, rows_y); \
     break;
     if (w->ex_gate.kind == ORNITH_Q4K) {
-      switch (nch) { UP_CASE(ORNITH_Q4K, 4) UP_CASE(ORNITH_Q4K, 8) UP_CASE(ORNITH_Q4K, 16) UP_CASE(ORNITH_Q4K, 32) UP_CASE(ORNITH_Q4K, 64) }
+      switch (nch) { UP_CASE(ORNITH_Q4K, 8) UP_CASE(ORNITH_Q4K, 16) UP_CASE(ORNITH_Q4K, 32) UP_CASE(ORNITH_Q4K, 64) }
     } else {
       switch (nch) { UP_CASE(ORNITH_Q6K, 4) UP_CASE(ORNITH_Q6K, 8) UP_CASE(ORNITH_Q6K, 16) UP_CASE(ORNITH_Q6K, 32) UP_CASE(ORNITH_Q6K, 64) }
     }
 #undef UP_CASE
     ORN_LAUNCH_CHECK("moe_up_kernel");
   }
-  {
+  if (phases & 2) {
     DownArgs a{};
     a.down = ptr_of(w->ex_down);
     a.sdown = ptr_of(w->sh_down.km);
@@ -239,21 +455,21 @@ int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
     a.H = H;
     a.I = I;
     a.normalize = w->norm_topk_prob;
-    const int nch = chunks_of(w->ex_down), rpw = 64 / nch;
-    // columns per workgroup: aim for >= 2 workgroups per CU, at least 2 iterations
-    int iters = (int)(((long)H * T) / ((long)rpw * ctx->compute_units * 2));
-    iters = iters < 1 ? 1 : (iters > 4 ? 4 : iters);
-    while (rpw * iters > kMaxCols) --iters;
-    a.iters = iters;
-    const int cols = rpw * iters;
-    dim3 grid((H + cols - 1) / cols, T);
-    dim3 block(64 * (k + 1));
-#define DOWN_CASE(KIND, N)                                                                   \
-  case N:                                                                                    \
-    hipLaunchKernelGGL((moe_down_kernel<KIND, N>), grid, block, 0, ctx->stream, a);          \
+    if (tail) {
+      a.tail.res = (const bf16_t*)tail->d_res;
+      a.tail.w = (const bf16_t*)tail->d_wnorm;
+      a.tail.h_out = (bf16_t*)tail->d_h_out;
+      a.tail.normed_out = (bf16_t*)tail->d_normed_out;
+      a.tail.eps = tail->eps;
+      a.tail.counter = ctx->counters + 2;
+    }
+    const int nch = chunks_of(w->ex_down);
+#define DOWN_CASE(KIND, N) \
+  case N:                  \
+    launch_down<KIND, N>(ctx, a); \
     break;
     if (w->ex_down.kind == ORNITH_Q4K) {
-      switch (nch) { DOWN_CASE(ORNITH_Q4K, 4) DOWN_CASE(ORNITH_Q4K, 8) DOWN_CASE(ORNITH_Q4K, 16) DOWN_CASE(ORNITH_Q4K, 32) DOWN_CASE(ORNITH_Q4K, 64) }
+      switch (nch) { DOWN_CASE(ORNITH_Q4K, 8) DOWN_CASE(ORNITH_Q4K, 16) DOWN_CASE(ORNITH_Q4K, 32) DOWN_CASE(ORNITH_Q4K, 64) }
     } else {
       switch (nch) { DOWN_CASE(ORNITH_Q6K, 4) DOWN_CASE(ORNITH_Q6K, 8) DOWN_CASE(ORNITH_Q6K, 16) DOWN_CASE(ORNITH_Q6K, 32) DOWN_CASE(ORNITH_Q6K, 64) }
     }
@@ -262,3 +478,20 @@ int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
   }
   return ORNITH_OK;
 }
+
+extern "C" {
+
+int ornith_moe_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
+                       void* d_out, int phases) {
+  ORN_REQUIRE(ctx && w && d_x && d_inds && d_scores && d_egate && d_act && d_out,
+              "moe_experts: null argument");
+  ORN_REQUIRE(T >= 1 && T <= 64 && phases >= 1 && phases <= 3, "moe_experts: T=%d phases=%d", T, phases);
+  if (!moe_fused_supported(w))
+    return ornith_fail(ORNITH_ERR_UNSUPPORTED,
+                       "moe_experts: the fused expert kernels need k-quant routed and shared experts "
+                       "of matching formats and top_k <= %d", kMaxK);
+  return moe_fused_experts(ctx, w, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, phases, nullptr);
+}
+
+}  // extern "C"

@@ -5,105 +5,21 @@
 // (/root/reference/src/ops/norm.rs:19-220; vendored rms_norm.metal:12-81,
 // /root/reference/kernels/ornith_norm.metal:28-183).
 //
-// One wavefront per row. Lane l owns the contiguous piece [l*n/64, (l+1)*n/64),
-// sums its squares with one fma chain, and the 64 lane sums go through the
-// butterfly. Two roundings on the way out, as in the reference:
-//   out = bf16(w * bf16(x * inv)),  inv = 1 / sqrt(sum / n + eps).
+// One wavefront per row (see norm_device.h for the arithmetic and its order).
 // A lane's piece is moved with the widest aligned vector access (16 bytes for
 // pieces of 8 or more values), so a 2048-wide row is four loads per lane.
-#include "dmath.h"
+#include "norm_device.h"
 #include "rt.h"
 
 namespace {
-
-enum { NORM_PLAIN = 0, NORM_ADD = 1, NORM_GATED = 2 };
-
-// PER consecutive bf16 values <-> fp32 registers
-template <int PER>
-__device__ __forceinline__ void load_bf16(const bf16_t* p, float (&v)[PER]) {
-  if constexpr (PER >= 8) {
-#pragma unroll
-    for (int c = 0; c < PER / 8; ++c) {
-      const uint4 w = reinterpret_cast<const uint4*>(p)[c];
-      v[8 * c + 0] = dm_bf2f_lo(w.x);
-      v[8 * c + 1] = dm_bf2f_hi(w.x);
-      v[8 * c + 2] = dm_bf2f_lo(w.y);
-      v[8 * c + 3] = dm_bf2f_hi(w.y);
-      v[8 * c + 4] = dm_bf2f_lo(w.z);
-      v[8 * c + 5] = dm_bf2f_hi(w.z);
-      v[8 * c + 6] = dm_bf2f_lo(w.w);
-      v[8 * c + 7] = dm_bf2f_hi(w.w);
-    }
-  } else if constexpr (PER == 4) {
-    const uint2 w = *reinterpret_cast<const uint2*>(p);
-    v[0] = dm_bf2f_lo(w.x);
-    v[1] = dm_bf2f_hi(w.x);
-    v[2] = dm_bf2f_lo(w.y);
-    v[3] = dm_bf2f_hi(w.y);
-  } else if constexpr (PER == 2) {
-    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
-    v[0] = dm_bf2f_lo(w);
-    v[1] = dm_bf2f_hi(w);
-  } else {
-    v[0] = dm_bf2f(p[0]);
-  }
-}
-
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)dm_f2bf(a) | ((uint32_t)dm_f2bf(b) << 16);
-}
-
-// rounds each value to bf16 and stores
-template <int PER>
-__device__ __forceinline__ void store_bf16(bf16_t* p, const float (&v)[PER]) {
-  if constexpr (PER >= 8) {
-#pragma unroll
-    for (int c = 0; c < PER / 8; ++c)
-      reinterpret_cast<uint4*>(p)[c] =
-          make_uint4(pack2(v[8 * c], v[8 * c + 1]), pack2(v[8 * c + 2], v[8 * c + 3]),
-                     pack2(v[8 * c + 4], v[8 * c + 5]), pack2(v[8 * c + 6], v[8 * c + 7]));
-  } else if constexpr (PER == 4) {
-    *reinterpret_cast<uint2*>(p) = make_uint2(pack2(v[0], v[1]), pack2(v[2], v[3]));
-  } else if constexpr (PER == 2) {
-    *reinterpret_cast<uint32_t*>(p) = pack2(v[0], v[1]);
-  } else {
-    p[0] = dm_f2bf(v[0]);
-  }
-}
 
 template <int PER, int MODE>
 __global__ __launch_bounds__(64) void rms_kernel(const bf16_t* a, const bf16_t* b, const bf16_t* w,
                                                  const bf16_t* z, bf16_t* h_out, bf16_t* out, int n,
                                                  float eps) {
-  const int r = blockIdx.x, lane = threadIdx.x;
-  const size_t base = (size_t)r * n + lane * PER;
-  float x[PER];
-  load_bf16<PER>(a + base, x);
-  if constexpr (MODE == NORM_ADD) {
-    float y[PER];
-    load_bf16<PER>(b + base, y);
-#pragma unroll
-    for (int i = 0; i < PER; ++i) x[i] = dm_rb(x[i] + y[i]);
-    store_bf16<PER>(h_out + base, x);
-  }
-  float acc = 0.f;
-#pragma unroll
-  for (int i = 0; i < PER; ++i) acc = dm_fma(x[i], x[i], acc);
-  const float inv = dm_rsqrt(dm_wave_sum<64>(acc) / (float)n + eps);
-  float wv[PER];
-  if (w) load_bf16<PER>(w + lane * PER, wv);
-#pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    x[i] = dm_rb(x[i] * inv);
-    if (w) x[i] = dm_rb(wv[i] * x[i]);
-  }
-  if constexpr (MODE == NORM_GATED) {
-    float g[PER];
-    load_bf16<PER>(z + base, g);
-#pragma unroll
-    for (int i = 0; i < PER; ++i) x[i] = (g[i] * dm_sigmoid_f32(g[i])) * x[i];
-  }
-  store_bf16<PER>(out + base, x);
+  const size_t off = (size_t)blockIdx.x * n;
+  rms_row<PER, MODE>(a + off, b ? b + off : nullptr, w, z ? z + off : nullptr,
+                     h_out ? h_out + off : nullptr, out + off, n, eps, threadIdx.x);
 }
 
 template <int MODE>

@@ -1,0 +1,128 @@
+// One row of an RMS norm by one wavefront, shared by the norm kernels and by the
+// projection / MoE kernels whose last workgroup applies the following
+// "residual add + norm" itself.
+//
+// Arithmetic of vendored rms_norm.metal:12-81 and
+// /root/reference/kernels/ornith_norm.metal:28-183: lane l owns the contiguous piece
+// [l*PER, (l+1)*PER) of the row, one fma chain of squares per lane, butterfly over the
+// 64 lanes, inv = 1/sqrt(sum/n + eps), out = bf16(w * bf16(x * inv)).
+#pragma once
+
+#include "dmath.h"
+
+// PER consecutive bf16 values <-> fp32 registers, widest aligned access
+template <int PER>
+__device__ __forceinline__ void load_bf16(const bf16_t* p, float (&v)[PER]) {
+  if constexpr (PER >= 8) {
+#pragma unroll
+    for (int c = 0; c < PER / 8; ++c) {
+      const uint4 w = reinterpret_cast<const uint4*>(p)[c];
+      v[8 * c + 0] = dm_bf2f_lo(w.x);
+      v[8 * c + 1] = dm_bf2f_hi(w.x);
+      v[8 * c + 2] = dm_bf2f_lo(w.y);
+      v[8 * c + 3] = dm_bf2f_hi(w.y);
+      v[8 * c + 4] = dm_bf2f_lo(w.z);
+      v[8 * c + 5] = dm_bf2f_hi(w.z);
+      v[8 * c + 6] = dm_bf2f_lo(w.w);
+      v[8 * c + 7] = dm_bf2f_hi(w.w);
+    }
+  } else if constexpr (PER == 4) {
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    v[0] = dm_bf2f_lo(w.x);
+    v[1] = dm_bf2f_hi(w.x);
+    v[2] = dm_bf2f_lo(w.y);
+    v[3] = dm_bf2f_hi(w.y);
+  } else if constexpr (PER == 2) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
+    v[0] = dm_bf2f_lo(w);
+    v[1] = dm_bf2f_hi(w);
+  } else {
+    v[0] = dm_bf2f(p[0]);
+  }
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  return (uint32_t)dm_f2bf(a) | ((uint32_t)dm_f2bf(b) << 16);
+}
+
+// rounds each value to bf16 and stores
+template <int PER>
+__device__ __forceinline__ void store_bf16(bf16_t* p, const float (&v)[PER]) {
+  if constexpr (PER >= 8) {
+#pragma unroll
+    for (int c = 0; c < PER / 8; ++c)
+      reinterpret_cast<uint4*>(p)[c] =
+          make_uint4(pack_bf16x2(v[8 * c], v[8 * c + 1]), pack_bf16x2(v[8 * c + 2], v[8 * c + 3]),
+                     pack_bf16x2(v[8 * c + 4], v[8 * c + 5]), pack_bf16x2(v[8 * c + 6], v[8 * c + 7]));
+  } else if constexpr (PER == 4) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
+  } else if constexpr (PER == 2) {
+    *reinterpret_cast<uint32_t*>(p) = pack_bf16x2(v[0], v[1]);
+  } else {
+    p[0] = dm_f2bf(v[0]);
+  }
+}
+
+enum { NORM_PLAIN = 0, NORM_ADD = 1, NORM_GATED = 2 };
+
+// One row. a (and b for NORM_ADD, z for NORM_GATED) point at the row; w at the weights
+// (may be null for NORM_PLAIN); h_out receives bf16(a + b) for NORM_ADD.
+template <int PER, int MODE>
+__device__ __forceinline__ void rms_row(const bf16_t* a, const bf16_t* b, const bf16_t* w,
+                                        const bf16_t* z, bf16_t* h_out, bf16_t* out, int n,
+                                        float eps, int lane) {
+  const int base = lane * PER;
+  float x[PER], wv[PER];
+  load_bf16<PER>(a + base, x);
+  if (w) load_bf16<PER>(w + base, wv);
+  if constexpr (MODE == NORM_ADD) {
+    float y[PER];
+    load_bf16<PER>(b + base, y);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) x[i] = dm_rb(x[i] + y[i]);
+    store_bf16<PER>(h_out + base, x);
+  }
+  float acc = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) acc = dm_fma(x[i], x[i], acc);
+  const float inv = dm_rsqrt(dm_wave_sum<64>(acc) / (float)n + eps);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    x[i] = dm_rb(x[i] * inv);
+    if (w) x[i] = dm_rb(wv[i] * x[i]);
+  }
+  if constexpr (MODE == NORM_GATED) {
+    float g[PER];
+    load_bf16<PER>(z + base, g);
+#pragma unroll
+    for (int i = 0; i < PER; ++i) x[i] = (g[i] * dm_sigmoid_f32(g[i])) * x[i];
+  }
+  store_bf16<PER>(out + base, x);
+}
+
+// The "residual add + norm" that follows a projection or the MoE block, for one row,
+// dispatched on the row width (n = 64 * PER).
+struct AddRmsTail {
+  const bf16_t* res;   // residual rows [M, n]
+  const bf16_t* w;     // norm weight [n]
+  bf16_t* h_out;       // res + y, [M, n]
+  bf16_t* normed_out;  // [M, n]
+  unsigned int* counter;
+  float eps;
+};
+
+__device__ __forceinline__ void add_rms_tail_row(const AddRmsTail& t, const bf16_t* y_row, int row,
+                                                 int n, int lane) {
+  const bf16_t* a = t.res + (size_t)row * n;
+  bf16_t* h = t.h_out + (size_t)row * n;
+  bf16_t* o = t.normed_out + (size_t)row * n;
+  switch (n / 64) {
+    case 1: rms_row<1, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
+    case 2: rms_row<2, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
+    case 4: rms_row<4, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
+    case 8: rms_row<8, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
+    case 16: rms_row<16, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
+    case 32: rms_row<32, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
+    default: rms_row<64, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
+  }
+}

@@ -34,14 +34,17 @@ namespace {
 struct Option {
   const char* name;
   const char* env;
+  int dflt;
   int value;  // -1: not read yet
 };
-Option g_options[] = {{"fuse_moe", "ORNITH_FUSE_MOE", -1}, {"fuse_proj", "ORNITH_FUSE_PROJ", -1}};
+Option g_options[] = {{"fuse_moe", "ORNITH_FUSE_MOE", 1, -1},
+                      {"fuse_proj", "ORNITH_FUSE_PROJ", 1, -1},
+                      {"moe_up_iters", "ORNITH_MOE_UP_ITERS", 0, -1}};
 int option_value(int i) {
   Option& o = g_options[i];
   if (o.value < 0) {
     const char* e = getenv(o.env);
-    o.value = (e && e[0] == '0') ? 0 : 1;
+    o.value = (e && e[0] >= '0' && e[0] <= '9') ? atoi(e) : o.dflt;
   }
   return o.value;
 }
@@ -49,6 +52,7 @@ int option_value(int i) {
 
 int ornith_option_fuse_moe() { return option_value(0); }
 int ornith_option_fuse_proj() { return option_value(1); }
+int ornith_option_moe_up_iters() { return option_value(2); }
 
 extern "C" {
 
@@ -56,7 +60,7 @@ int ornith_set_option(const char* name, int value) {
   ORN_REQUIRE(name, "set_option: null name");
   for (auto& o : g_options)
     if (!strcmp(o.name, name)) {
-      o.value = value ? 1 : 0;
+      o.value = value < 0 ? 0 : value;
       return ORNITH_OK;
     }
   return ornith_fail(ORNITH_ERR_INVALID, "set_option: unknown option '%s'", name);
@@ -82,6 +86,8 @@ int ornith_ctx_create(int device, ornith_ctx** out) {
   ORN_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   ORN_HIP(hipEventCreate(&c->ev0));
   ORN_HIP(hipEventCreate(&c->ev1));
+  ORN_HIP(hipMalloc((void**)&c->counters, kNumCounters * sizeof(unsigned int)));
+  ORN_HIP(hipMemsetAsync(c->counters, 0, kNumCounters * sizeof(unsigned int), c->stream));
   *out = c;
   return ORNITH_OK;
 }
@@ -90,6 +96,7 @@ int ornith_ctx_destroy(ornith_ctx* ctx) {
   if (!ctx) return ORNITH_OK;
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->scratch) (void)hipFree(ctx->scratch);
+  if (ctx->counters) (void)hipFree(ctx->counters);
   (void)hipEventDestroy(ctx->ev0);
   (void)hipEventDestroy(ctx->ev1);
   (void)hipStreamDestroy(ctx->stream);

@@ -63,19 +63,34 @@ __global__ __launch_bounds__(CH) void argmax_chunk_kernel(const bf16_t* logits, 
   __shared__ float s_lse;
   float lse = 0.f;
   if constexpr (USE_LSE) {
-    // every workgroup repeats the (short, sequential) merge: cheaper than another launch
+    // every workgroup repeats the short merge: cheaper than another launch
     __shared__ float smax[16];
     float m = -DM_INF;
     for (int k = tid; k < nch; k += CH) m = mc[(size_t)r * nch + k] > m ? mc[(size_t)r * nch + k] : m;
     m = dm_wave_max<64>(m);
     if (lane == 0) smax[wave] = m;
     __syncthreads();
+    float M = smax[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) M = smax[w] > M ? smax[w] : M;
+    // the chunk terms are independent and computed by all threads; only the fma chain
+    // over them (ascending chunk order) is sequential
+    __shared__ float s_l[CH], s_e[CH];
+    float L = 0.f;
+    for (int k0 = 0; k0 < nch; k0 += CH) {
+      const int k = k0 + tid;
+      if (k < nch) {
+        s_l[tid] = lc[(size_t)r * nch + k];
+        s_e[tid] = dm_exp(mc[(size_t)r * nch + k] - M);
+      }
+      __syncthreads();
+      if (tid == 0) {
+        const int n = min(CH, nch - k0);
+        for (int q = 0; q < n; ++q) L = dm_fma(s_l[q], s_e[q], L);
+      }
+      __syncthreads();
+    }
     if (tid == 0) {
-      float M = smax[0];
-      for (int w = 1; w < 16; ++w) M = smax[w] > M ? smax[w] : M;
-      float L = 0.f;
-      for (int k = 0; k < nch; ++k)
-        L = dm_fma(lc[(size_t)r * nch + k], dm_exp(mc[(size_t)r * nch + k] - M), L);
       s_lse = dm_rb(dm_log(L) + M);
       if (c == 0 && lse_out) lse_out[r] = dm_f2bf(s_lse);
     }

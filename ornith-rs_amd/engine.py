@@ -27,6 +27,12 @@ def kq_qmv_multi(ctx, ws, x, x_dtype, M, ys, y_dtype):
     _check(lib().ornith_kq_qmv_multi(ctx.h, wp, n, x.ptr, x_dtype, M, yp, y_dtype), "kq_qmv_multi")
 
 
+def moe_experts(ctx, w, x, T, inds, scores, egate, act, out, phases=3):
+    """ornith_moe_experts: the two expert gather-GEMV kernels (1 = up, 2 = down, 3 = both)."""
+    _check(lib().ornith_moe_experts(ctx.h, C.byref(w), x.ptr, T, inds.ptr, scores.ptr, egate.ptr, act.ptr,
+                                    out.ptr, phases), "moe_experts")
+
+
 class TextConfig(C.Structure):
     """TextConfig (src/model/config.rs); defaults are the Qwen3.5-35B-A3B shape."""
     _fields_ = [(n, C.c_int) for n in (
