@@ -68,7 +68,9 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *               launch per operator
  *   "fuse_proj" (ORNITH_FUSE_PROJ, default 1): projections sharing an input in one launch
  *   "moe_up_iters" (ORNITH_MOE_UP_ITERS, default 0 = chosen by shape; 2 or 4): output
- *               rows per wavefront of the fused gate+up expert kernel, a tuning knob */
+ *               rows per wavefront of the fused gate+up expert kernel, a tuning knob
+ *   "kq_iters"  (ORNITH_KQ_ITERS, default 0 = chosen by shape; 1..8): output rows each
+ *               wavefront of the k-quant mat-vec walks, a tuning knob */
 ORNITH_API int ornith_set_option(const char* name, int value);
 ORNITH_API int ornith_timer_begin(ornith_ctx* ctx);
 ORNITH_API int ornith_timer_end(ornith_ctx* ctx, float* ms_out);
@@ -133,14 +135,6 @@ typedef struct ornith_linear {
 ORNITH_API int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_x, int M,
                                     void* d_y);
 
-/* Linear::matmul followed by norm::add_rms_norm (the mixer's output projection and the
- * post-attention norm, src/model/qwen3_5.rs:374-390): y = x . W^T; h = res + y (bf16);
- * normed = rms_norm(h, w_norm). One launch for k-quant weights at M <= 4 (the last
- * workgroup to finish applies the norm), two otherwise; bit-identical either way. */
-ORNITH_API int ornith_linear_matmul_add_rms(ornith_ctx* ctx, const ornith_linear* w, const void* d_x,
-                                            int M, void* d_y, const void* d_res, const void* d_wnorm,
-                                            float eps, void* d_h_out, void* d_normed_out);
-
 /* n Linear::matmul calls over the same activations (in_proj_qkv + in_proj_z, in_proj_a +
  * in_proj_b, q/k/v projections: src/model/qwen3_5.rs:441-447,493-499). Fused into one
  * launch where the formats allow (same mode, width and k-quant kind; n <= 4), issued
@@ -196,14 +190,6 @@ typedef struct ornith_moe_weights {
 ORNITH_API int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                                 void* d_out, uint32_t* d_inds_out, void* d_scores_out);
 
-/* sparse_moe_block followed by the decoder layer's closing add and the next layer's
- * input norm (src/model/qwen3_5.rs:388-396 and the head of the next layer's forward):
- * out = moe(x); h = res + out; normed = rms_norm(h, w_norm). With the fused expert
- * kernels and T <= top_k + 1 the last workgroup of the down kernel applies the norm, so
- * the block ends in the same launch; bit-identical to moe_block + add_rms_norm. */
-ORNITH_API int ornith_moe_block_add_rms(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x,
-                                        int T, void* d_out, const void* d_res, const void* d_wnorm,
-                                        float eps, void* d_h_out, void* d_normed_out);
 
 /* moe::switch_glu_rows + the shared expert + moe::combine (src/ops/moe.rs:256-338,548-596)
  * given the router's picks: the expert gather-GEMV proper, as two kernels.

@@ -275,19 +275,6 @@ def moe_block(self, w, x, T, out, inds=None, scores=None):
            "moe_block")
 
 
-@_ctx_method
-def moe_block_add_rms(self, w, x, T, out, res, wnorm, eps, h_out, normed_out):
-    _check(lib().ornith_moe_block_add_rms(self.h, C.byref(w), x.ptr, T, out.ptr, res.ptr, wnorm.ptr,
-                                          C.c_float(eps), h_out.ptr, normed_out.ptr), "moe_block_add_rms")
-
-
-@_ctx_method
-def linear_matmul_add_rms(self, lin, x, M, y, res, wnorm, eps, h_out, normed_out):
-    _check(lib().ornith_linear_matmul_add_rms(self.h, C.byref(lin.s), x.ptr, M, y.ptr, res.ptr, wnorm.ptr,
-                                              C.c_float(eps), h_out.ptr, normed_out.ptr),
-           "linear_matmul_add_rms")
-
-
 # ---- norms / gated-delta ----------------------------------------------------------
 @_ctx_method
 def rms_norm(self, x, w, rows, n, eps, out):

@@ -4,8 +4,9 @@
 // same on every run and agree with a scalar CPU evaluation, so nothing here
 // calls the device math library: exp/log are written out with fp32 add, mul and
 // fma only, divide and sqrt are the correctly rounded IEEE ones (hipcc's
-// default), and conversions are integer bit moves. The file is compiled with
-// -ffp-contract=off, so the only fused operations are the explicit __builtin_fmaf.
+// default), and conversions are integer bit moves or the hardware's exact / round-to-
+// nearest-even ones. The file is compiled with -ffp-contract=off, so the only fused
+// operations are the explicit __builtin_fmaf.
 //
 // Rounding points follow the reference: activations are bf16 in memory and fp32
 // in registers (/root/reference/kernels/q4k.metal:216-221), bf16 rounding is
@@ -24,11 +25,12 @@ __device__ __forceinline__ float dm_fma(float a, float b, float c) { return __bu
 
 __device__ __forceinline__ float dm_bf2f(bf16_t b) { return __uint_as_float((uint32_t)b << 16); }
 
+// fp32 -> bf16, round to nearest even: gfx950's v_cvt_pk_bf16_f32 (one instruction for
+// two values; subnormals are kept, fp32 denormals being on). Equal to the integer
+// formulation u += 0x7fff + ((u >> 16) & 1) for every non-NaN input.
 __device__ __forceinline__ bf16_t dm_f2bf(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, b);
 }
 // round to bf16 precision, keep as float
 __device__ __forceinline__ float dm_rb(float f) { return dm_bf2f(dm_f2bf(f)); }

@@ -24,9 +24,7 @@
 //   read the same activations (q/k/v projections, in_proj_qkv + in_proj_z): the
 //   grid is the concatenation of their row ranges.
 #include "kq_device.h"
-#include "norm_device.h"
 #include "rt.h"
-#include "sync_device.h"
 
 namespace {
 
@@ -51,16 +49,13 @@ struct KqArgs {
   int E, x_rows;  // gather only: bounds for rhs / lhs (out-of-range ids are clamped)
   int iters;      // row iterations per wavefront
   int y_bf16;     // 1: round outputs to bf16, 0: fp32
-  AddRmsTail tail;  // TAIL kernels only: the residual add + norm that follows this projection
 };
 
 // One kernel for plain and gathered mat-vecs.
 //   KIND  format; LPR lanes per row (4,8,16,32,64); KS wavefronts per row (1,2)
 //   M     activation rows sharing each weight read (1..4); gather uses M == 1
 //   grid.x covers output rows (of all segments), grid.y is the gather row
-//   TAIL  the last workgroup to finish also applies h = res + y, normed = rms_norm(h)
-//         to the M output rows (one wavefront per row); single matrix, bf16 output
-template <int KIND, int LPR, int KS, int M, bool XF32, bool GATHER, bool TAIL = false>
+template <int KIND, int LPR, int KS, int M, bool XF32, bool GATHER>
 __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
   using KL = KqLane<KIND, M>;
   constexpr int RPW = 64 / LPR;  // rows in flight per wavefront
@@ -133,10 +128,6 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
           static_cast<float*>(sg.y)[yi] = v;
       }
     }
-  }
-  if constexpr (TAIL) {
-    if (!last_block_done(a.tail.counter, gridDim.x)) return;
-    if (wave < M) add_rms_tail_row(a.tail, static_cast<const bf16_t*>(sg.y) + (size_t)wave * O, wave, O, lane);
   }
 }
 
@@ -219,38 +210,6 @@ int launch_one(ornith_ctx* ctx, KqArgs& a, int grid_y) {
   return ORNITH_OK;
 }
 
-template <int KIND, int LPR, int KS, int M>
-int launch_one_tail(ornith_ctx* ctx, KqArgs& a) {
-  dim3 grid(layout_segments<LPR, KS>(a), 1, 1);
-  hipLaunchKernelGGL((kq_qmv_kernel<KIND, LPR, KS, M, false, false, true>), grid, dim3(256), 0,
-                     ctx->stream, a);
-  ORN_LAUNCH_CHECK("kq_qmv_kernel<tail>");
-  return ORNITH_OK;
-}
-
-template <int KIND, int M>
-int launch_shape_tail(ornith_ctx* ctx, KqArgs& a) {
-  const int nch = (a.K >> 8) * (KIND == ORNITH_Q4K ? 8 : 4);
-  switch (nch) {
-    case 8: return launch_one_tail<KIND, 8, 1, M>(ctx, a);
-    case 16: return launch_one_tail<KIND, 16, 1, M>(ctx, a);
-    case 32: return launch_one_tail<KIND, 32, 1, M>(ctx, a);
-    case 64: return launch_one_tail<KIND, 64, 1, M>(ctx, a);
-    case 128: return launch_one_tail<KIND, 64, 2, M>(ctx, a);
-    default: return -1;
-  }
-}
-
-template <int KIND>
-int launch_m_tail(ornith_ctx* ctx, KqArgs& a, int M) {
-  switch (M) {
-    case 1: return launch_shape_tail<KIND, 1>(ctx, a);
-    case 2: return launch_shape_tail<KIND, 2>(ctx, a);
-    case 3: return launch_shape_tail<KIND, 3>(ctx, a);
-    default: return launch_shape_tail<KIND, 4>(ctx, a);
-  }
-}
-
 template <int KIND, int M, bool XF32, bool GATHER>
 int launch_shape(ornith_ctx* ctx, KqArgs& a, int grid_y) {
   const int nch = (a.K >> 8) * (KIND == ORNITH_Q4K ? 8 : 4);
@@ -279,15 +238,17 @@ int launch_m(ornith_ctx* ctx, KqArgs& a, int M) {
   }
 }
 
-// rows each wavefront walks: enough blocks to cover the chip several times over
-// while keeping the activation registers amortised.
+// rows each wavefront walks: the kernels are bound by VALU issue and by latency, not by
+// HBM, so the converted activations are amortised over as many rows as still leaves
+// about three workgroups per compute unit (measured optimum on 256 CUs for 0.4..55 MB).
 int pick_iters(const ornith_ctx* ctx, int kind, int K, long total_rows, int grid_y) {
+  if (const int forced = ornith_option_kq_iters()) return forced > 8 ? 8 : forced;
   const int nch = (K >> 8) * (kind == ORNITH_Q4K ? 8 : 4);
   const int lpr = nch >= 64 ? 64 : nch;
   const int ks = nch > 64 ? 2 : 1;
   const int rows_per_pass = (64 / lpr) * (4 / ks);  // rows a block covers per iteration
   const long blocks_at_1 = (total_rows + rows_per_pass - 1) / rows_per_pass * grid_y;
-  const long want = (long)ctx->compute_units * 8;
+  const long want = (long)ctx->compute_units * 3;
   int iters = (int)(blocks_at_1 / want);
   if (iters < 1) iters = 1;
   if (iters > 8) iters = 8;
@@ -387,35 +348,6 @@ int ornith_kq_qmv_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n,
     if (rc) return rc;
   }
   return ORNITH_OK;
-}
-
-// y = x . W^T (bf16) followed by h = res + y, normed = rms_norm(h, w_norm) in the same launch.
-// Returns -1 (nothing launched) if the shape is outside what the tail covers.
-int kq_qmv_add_rms(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int M, void* d_y,
-                   const void* d_res, const void* d_wnorm, float eps, void* d_h_out,
-                   void* d_normed_out) {
-  if (M < 1 || M > 4 || w->E != 1 || w->O % 64 != 0 || w->O > 4096) return -1;
-  const int per = w->O / 64;
-  if (per & (per - 1)) return -1;
-  if (check_matrix(w, "kq_qmv_add_rms")) return -1;
-  KqArgs a{};
-  a.nseg = 1;
-  a.seg[0].qs = (const uint8_t*)w->d_qs;
-  a.seg[0].scales = (const uint8_t*)w->d_scales;
-  a.seg[0].dm = (const uint16_t*)w->d_dm;
-  a.seg[0].O = w->O;
-  a.seg[0].y = d_y;
-  a.x = d_x;
-  a.K = w->K;
-  a.y_bf16 = 1;
-  a.iters = pick_iters(ctx, w->kind, w->K, w->O, 1);
-  a.tail.res = (const bf16_t*)d_res;
-  a.tail.w = (const bf16_t*)d_wnorm;
-  a.tail.h_out = (bf16_t*)d_h_out;
-  a.tail.normed_out = (bf16_t*)d_normed_out;
-  a.tail.counter = ctx->counters + 1;
-  a.tail.eps = eps;
-  return w->kind == ORNITH_Q4K ? launch_m_tail<ORNITH_Q4K>(ctx, a, M) : launch_m_tail<ORNITH_Q6K>(ctx, a, M);
 }
 
 int ornith_kq_qmv(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int x_dtype, int M,

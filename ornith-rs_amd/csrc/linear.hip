@@ -13,11 +13,6 @@
 #include "dmath.h"
 #include "rt.h"
 
-// kquant.hip
-extern "C" int kq_qmv_add_rms(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int M, void* d_y,
-                   const void* d_res, const void* d_wnorm, float eps, void* d_h_out,
-                   void* d_normed_out);
-
 namespace {
 
 // ---- 8-bit affine, group 64 ---------------------------------------------
@@ -147,20 +142,6 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
     default:
       return ornith_fail(ORNITH_ERR_INVALID, "linear_matmul: unknown mode %d", w->mode);
   }
-}
-
-int ornith_linear_matmul_add_rms(ornith_ctx* ctx, const ornith_linear* w, const void* d_x, int M,
-                                 void* d_y, const void* d_res, const void* d_wnorm, float eps,
-                                 void* d_h_out, void* d_normed_out) {
-  ORN_REQUIRE(ctx && w && d_x && d_y && d_res && d_wnorm && d_h_out && d_normed_out,
-              "linear_matmul_add_rms: null argument");
-  if (ornith_option_fuse_proj() && w->mode == ORNITH_LIN_KQUANT) {
-    const int rc = kq_qmv_add_rms(ctx, &w->km, d_x, M, d_y, d_res, d_wnorm, eps, d_h_out, d_normed_out);
-    if (rc >= 0) return rc;
-  }
-  int rc = ornith_linear_matmul(ctx, w, d_x, M, d_y);
-  if (rc) return rc;
-  return ornith_add_rms_norm(ctx, d_res, d_y, d_wnorm, M, w->O, eps, d_h_out, d_normed_out);
 }
 
 int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, int n,

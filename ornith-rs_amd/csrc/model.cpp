@@ -207,17 +207,16 @@ static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_to
       TRY(ornith_gdn_recurrence(ctx, s.q, s.k, s.v, s.g, s.beta, lc.state + (size_t)cc->state_cur * ssz,
                                 T, Hk, Hv, Dk, Dv, s.y, lc.state, capture ? 1 : 0));
       TRY(ornith_rms_norm_gated(ctx, s.y, g.norm, s.z, T * Hv, Dv, c.rms_norm_eps, s.gated));
-      TRY(ornith_linear_matmul_add_rms(ctx, &g.out_proj, s.gated, T, s.r, s.x, L.post_ln,
-                                       c.rms_norm_eps, s.h, s.normed2));
+      TRY(ornith_linear_matmul(ctx, &g.out_proj, s.gated, T, s.r));
     } else {
       TRY(attention_block(m, L.attn, s.normed, T, lc.k, lc.v, cc->offset, cc->capacity, s.qg, s.kx,
                           s.vx, s.q_rot, s.att));
-      TRY(ornith_linear_matmul_add_rms(ctx, &L.attn.o_proj, s.att, T, s.r, s.x, L.post_ln,
-                                       c.rms_norm_eps, s.h, s.normed2));
+      TRY(ornith_linear_matmul(ctx, &L.attn.o_proj, s.att, T, s.r));
     }
+    TRY(ornith_add_rms_norm(ctx, s.x, s.r, L.post_ln, T, H, c.rms_norm_eps, s.h, s.normed2));
     const void* next_w = (i + 1 < m->layers.size()) ? m->layers[i + 1].input_ln : m->final_norm;
-    TRY(ornith_moe_block_add_rms(ctx, &L.moe, s.normed2, T, s.mo, s.h, next_w, c.rms_norm_eps, s.x,
-                                 s.normed));
+    TRY(ornith_moe_block(ctx, &L.moe, s.normed2, T, s.mo, nullptr, nullptr));
+    TRY(ornith_add_rms_norm(ctx, s.h, s.mo, next_w, T, H, c.rms_norm_eps, s.x, s.normed));
   }
   TRY(ornith_copy(ctx, d_hidden_out, s.normed, (size_t)T * H * 2));
   // every layer advanced together
@@ -617,11 +616,11 @@ int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspec, const vo
   TRY(ornith_linear_matmul(ctx, &h->fc, joined, T, x));
   TRY(ornith_rms_norm(ctx, x, h->input_ln, T, (int)H, c.rms_norm_eps, normed));
   TRY(attention_block(m, h->attn, normed, T, h->k, h->v, h->offset, h->capacity, qg, kx, vx, q_rot, att));
-  TRY(ornith_linear_matmul_add_rms(ctx, &h->attn.o_proj, att, T, r, x, h->post_ln, c.rms_norm_eps, hh,
-                                   normed2));
+  TRY(ornith_linear_matmul(ctx, &h->attn.o_proj, att, T, r));
+  TRY(ornith_add_rms_norm(ctx, x, r, h->post_ln, T, (int)H, c.rms_norm_eps, hh, normed2));
   // add(h, m) then mtp.norm; the un-normed sum is not needed afterwards
-  TRY(ornith_moe_block_add_rms(ctx, &h->moe, normed2, T, mo, hh, h->norm, c.rms_norm_eps, x,
-                               d_hidden_out));
+  TRY(ornith_moe_block(ctx, &h->moe, normed2, T, mo, nullptr, nullptr));
+  TRY(ornith_add_rms_norm(ctx, hh, mo, h->norm, T, (int)H, c.rms_norm_eps, x, d_hidden_out));
   h->offset += T;
   if (d_logits) {
     const ornith_linear* lm = frspec ? &frspec->head : &m->lm_head;

@@ -15,11 +15,10 @@
 // moe_fused.hip
 bool moe_fused_supported(const ornith_moe_weights* w);
 bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                      void* d_gates, uint32_t* d_inds, void* d_scores, void* d_egate, int* rc);
-bool moe_fused_tail_supported(const ornith_moe_weights* w, int T);
+                      void* d_gates, void* d_egate, int* rc);
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
-                      void* d_out, int phases, const MoeTail* tail);
+                      void* d_out, int phases);
 
 namespace {
 
@@ -129,10 +128,8 @@ int ornith_moe_combine(ornith_ctx* ctx, const void* d_scores, const void* d_y, c
   return ORNITH_OK;
 }
 
-// The block; with `tail`, followed by h = res + out, normed = rms_norm(h).
-static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                          void* d_out, uint32_t* d_inds_out, void* d_scores_out,
-                          const MoeTail* tail) {
+int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                     void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
   ORN_REQUIRE(ctx && w && d_x && d_out, "moe_block: null argument");
   const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
   ORN_REQUIRE(T >= 1 && T <= 64, "moe_block: T=%d (decode/verify widths only)", T);
@@ -177,20 +174,16 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
     if (rc) return rc;  \
   } while (0)
   if (ornith_option_fuse_moe() && moe_fused_supported(w)) {
-    // three small launches for the router, then the two expert kernels
+    // gates + shared-expert gate, softmax + top-k, then the two expert kernels
     int rrc = ORNITH_OK;
-    if (moe_fused_router(ctx, w, d_x, T, gates, inds, scores, eg, &rrc)) {
+    if (moe_fused_router(ctx, w, d_x, T, gates, eg, &rrc)) {
       if (rrc) return rrc;
     } else {
       TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
       TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
-      TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
     }
-    const bool in_kernel = tail && moe_fused_tail_supported(w, T);
-    TRY(moe_fused_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, 3, in_kernel ? tail : nullptr));
-    if (tail && !in_kernel)
-      TRY(ornith_add_rms_norm(ctx, tail->d_res, d_out, tail->d_wnorm, T, H, tail->eps, tail->d_h_out,
-                              tail->d_normed_out));
+    TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
+    TRY(moe_fused_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, 3));
     if (d_inds_out)
       ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,
                              ctx->stream));
@@ -222,9 +215,6 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
                              ORNITH_BF16));
   }
   TRY(ornith_moe_combine(ctx, scores, y, eg, sy, T, k, H, w->norm_topk_prob, d_out));
-  if (tail)
-    TRY(ornith_add_rms_norm(ctx, tail->d_res, d_out, tail->d_wnorm, T, H, tail->eps, tail->d_h_out,
-                            tail->d_normed_out));
   if (d_inds_out)
     ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,
                            ctx->stream));
@@ -233,19 +223,6 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
                            ctx->stream));
 #undef TRY
   return ORNITH_OK;
-}
-
-int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                     void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
-  return moe_block_impl(ctx, w, d_x, T, d_out, d_inds_out, d_scores_out, nullptr);
-}
-
-int ornith_moe_block_add_rms(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                             void* d_out, const void* d_res, const void* d_wnorm, float eps,
-                             void* d_h_out, void* d_normed_out) {
-  ORN_REQUIRE(d_res && d_wnorm && d_h_out && d_normed_out, "moe_block_add_rms: null argument");
-  const MoeTail tail{d_res, d_wnorm, eps, d_h_out, d_normed_out};
-  return moe_block_impl(ctx, w, d_x, T, d_out, nullptr, nullptr, &tail);
 }
 
 }  // extern "C"

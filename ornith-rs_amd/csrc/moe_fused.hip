@@ -25,9 +25,7 @@
 // nothing but the index list), then the activation loads, and only then computes.
 #include "kq_device.h"
 #include "moe_device.h"
-#include "norm_device.h"
 #include "rt.h"
-#include "sync_device.h"
 
 namespace {
 
@@ -129,8 +127,6 @@ struct DownArgs {
   const bf16_t* egate;   // [T]
   bf16_t* out;           // [T, H]
   int T, k, E, H, I, normalize;
-  AddRmsTail tail;       // tail.counter != null: the last workgroup also applies h = res + out,
-                         // normed = rms_norm(h) to the T rows (needs T <= k + 1)
 };
 
 constexpr int kMaxK = 8;
@@ -192,27 +188,22 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) 
     const float gated = dm_rb(gsig * yl[k][col]);
     a.out[(size_t)t * a.H + c0 + col] = dm_f2bf(acc + gated);
   }
-  if (a.tail.counter) {
-    if (!last_block_done(a.tail.counter, gridDim.x * gridDim.y)) return;
-    if (j < a.T) add_rms_tail_row(a.tail, a.out + (size_t)j * a.H, j, a.H, lane);
-  }
 }
 
-// ---- router: gates mat-vec, then the last workgroup does softmax + top-k and the
-// shared expert's scalar gate for every token (one wavefront per token) -------------
+// ---- router: the gates mat-vec and, in one extra workgroup, the shared expert's scalar
+// gate for every token (one wavefront per token). Softmax + top-k follow in their own
+// small launch: a hand-off inside this one needs device-wide release fences, which on a
+// multi-die part write the L2 back and cost more than the launch they would save. ------
 struct RouterArgs {
   KqPtr w;               // router [E, K]
   const bf16_t* x;       // [M, K]
   bf16_t* gates;         // [M, E]
-  uint32_t* inds;        // [M, k]
-  bf16_t* scores;        // [M, k]
   bf16_t* egate;         // [M]
   const void* eg_w;      // shared_expert_gate weights: affine8 u8[K] or dense bf16[K]
   const bf16_t* eg_s;    // affine8 scales [K/64]
   const bf16_t* eg_b;    // affine8 biases [K/64]
   int eg_affine;
-  unsigned int* counter;
-  int E, K, k;
+  int E, K;
 };
 
 // one row of the 8-bit affine / dense mat-vec by one wavefront (the order of linear.hip)
@@ -250,12 +241,19 @@ __device__ __forceinline__ float egate_row_dot(const RouterArgs& a, const bf16_t
   return dm_wave_sum<64>(acc_lane);
 }
 
-// grid ceil(E / (RPW * 4)), 256 threads, M <= 4 tokens
+// grid ceil(E / (RPW * 4)) + 1, 256 threads, M <= 4 tokens
 template <int KIND, int LPR, int M>
 __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
   using KL = KqLane<KIND, M>;
   constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (blockIdx.x == gridDim.x - 1) {
+    if (wave < M) {
+      const float e = egate_row_dot(a, a.x + (size_t)wave * a.K, lane);
+      if (lane == 0) a.egate[wave] = dm_f2bf(e);
+    }
+    return;
+  }
   const int slot = lane / LPR, c = lane % LPR;
   const int nb = a.K >> 8;
   typename KL::Lane L;
@@ -275,28 +273,12 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
     const float v = dm_wave_sum<LPR>(acc[t]);
     if (c == 0 && o < a.E) a.gates[(size_t)t * a.E + o] = dm_f2bf(v);
   }
-  if (!last_block_done(a.counter, gridDim.x)) return;
-  if (wave < M) {
-    const int t = wave;
-    const bf16_t* g = a.gates + (size_t)t * a.E;
-    uint32_t* ir = a.inds + (size_t)t * a.k;
-    bf16_t* sr = a.scores + (size_t)t * a.k;
-    switch (a.E / 64) {
-      case 1: router_topk_wave<1>(g, a.k, ir, sr, nullptr, lane); break;
-      case 2: router_topk_wave<2>(g, a.k, ir, sr, nullptr, lane); break;
-      case 4: router_topk_wave<4>(g, a.k, ir, sr, nullptr, lane); break;
-      case 8: router_topk_wave<8>(g, a.k, ir, sr, nullptr, lane); break;
-      default: router_topk_wave<16>(g, a.k, ir, sr, nullptr, lane); break;
-    }
-    const float e = egate_row_dot(a, a.x + (size_t)t * a.K, lane);
-    if (lane == 0) a.egate[t] = dm_f2bf(e);
-  }
 }
 
 template <int KIND, int LPR>
 void launch_router_fused(ornith_ctx* ctx, const RouterArgs& a, int M) {
   constexpr int RPW = 64 / LPR;
-  dim3 grid((a.E + RPW * 4 - 1) / (RPW * 4));
+  dim3 grid((a.E + RPW * 4 - 1) / (RPW * 4) + 1);
   switch (M) {
     case 1: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 1>), grid, dim3(256), 0, ctx->stream, a); break;
     case 2: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 2>), grid, dim3(256), 0, ctx->stream, a); break;
@@ -342,12 +324,6 @@ void launch_down(ornith_ctx* ctx, const DownArgs& a) {
 
 }  // namespace
 
-// Whether the down kernel can also apply the residual add + norm that follows the block.
-bool moe_fused_tail_supported(const ornith_moe_weights* w, int T) {
-  const int H = w->router.K, per = H / 64;
-  return T <= w->top_k + 1 && H % 64 == 0 && per <= 64 && (per & (per - 1)) == 0;
-}
-
 // Whether the two fused kernels cover this block's shapes and formats.
 bool moe_fused_supported(const ornith_moe_weights* w) {
   if (w->ex_dense) return false;
@@ -364,35 +340,30 @@ bool moe_fused_supported(const ornith_moe_weights* w) {
   return ok(cu) && ok(cd);
 }
 
-// Router mat-vec + softmax + top-k + shared_expert_gate in one launch. Returns false
-// (nothing launched) when the shapes / formats are outside what the kernel covers.
+// Router mat-vec + shared_expert_gate in one launch. Returns false (nothing launched)
+// when the shapes / formats are outside what the kernel covers.
 bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                      void* d_gates, uint32_t* d_inds, void* d_scores, void* d_egate, int* rc) {
+                      void* d_gates, void* d_egate, int* rc) {
   *rc = ORNITH_OK;
   const ornith_linear& r = w->router;
   const ornith_linear& g = w->sh_egate;
   if (T > 4 || r.mode != ORNITH_LIN_KQUANT) return false;
   if (g.mode != ORNITH_LIN_AFFINE8 && g.mode != ORNITH_LIN_DENSE) return false;
   if (g.K % 64 != 0) return false;
-  const int E = r.O, per = E / 64;
-  if (E % 64 != 0 || !(per == 1 || per == 2 || per == 4 || per == 8 || per == 16)) return false;
+  const int E = r.O;
   const int nch = chunks_of(r.km);
   if (!(nch == 8 || nch == 16 || nch == 32 || nch == 64)) return false;
   RouterArgs a{};
   a.w = ptr_of(r.km);
   a.x = (const bf16_t*)d_x;
   a.gates = (bf16_t*)d_gates;
-  a.inds = d_inds;
-  a.scores = (bf16_t*)d_scores;
   a.egate = (bf16_t*)d_egate;
   a.eg_w = g.d_w;
   a.eg_s = (const bf16_t*)g.d_scales;
   a.eg_b = (const bf16_t*)g.d_biases;
   a.eg_affine = g.mode == ORNITH_LIN_AFFINE8;
-  a.counter = ctx->counters + 0;
   a.E = E;
   a.K = r.K;
-  a.k = w->top_k;
 #define R_CASE(KIND, N) \
   case N:               \
     launch_router_fused<KIND, N>(ctx, a, T); \
@@ -411,7 +382,7 @@ bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
 // act: scratch bf16 [(T*k + T), I]. phases: 1 = up, 2 = down, 3 = both.
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
-                      void* d_out, int phases, const MoeTail* tail) {
+                      void* d_out, int phases) {
   const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
   if (phases & 1) {
     UpArgs a{};
@@ -455,14 +426,6 @@ int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
     a.H = H;
     a.I = I;
     a.normalize = w->norm_topk_prob;
-    if (tail) {
-      a.tail.res = (const bf16_t*)tail->d_res;
-      a.tail.w = (const bf16_t*)tail->d_wnorm;
-      a.tail.h_out = (bf16_t*)tail->d_h_out;
-      a.tail.normed_out = (bf16_t*)tail->d_normed_out;
-      a.tail.eps = tail->eps;
-      a.tail.counter = ctx->counters + 2;
-    }
     const int nch = chunks_of(w->ex_down);
 #define DOWN_CASE(KIND, N) \
   case N:                  \
@@ -491,7 +454,7 @@ int ornith_moe_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void*
     return ornith_fail(ORNITH_ERR_UNSUPPORTED,
                        "moe_experts: the fused expert kernels need k-quant routed and shared experts "
                        "of matching formats and top_k <= %d", kMaxK);
-  return moe_fused_experts(ctx, w, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, phases, nullptr);
+  return moe_fused_experts(ctx, w, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, phases);
 }
 
 }  // extern "C"

@@ -5,9 +5,14 @@
 // (/root/reference/src/ops/norm.rs:19-220; vendored rms_norm.metal:12-81,
 // /root/reference/kernels/ornith_norm.metal:28-183).
 //
-// One wavefront per row (see norm_device.h for the arithmetic and its order).
-// A lane's piece is moved with the widest aligned vector access (16 bytes for
-// pieces of 8 or more values), so a 2048-wide row is four loads per lane.
+// Rows up to 512 wide: one wavefront per row (see norm_device.h for the arithmetic and
+// its order). Wider rows: one workgroup of n/8 threads per row, eight values (16 bytes)
+// per thread, because a single wavefront walking 32 or 64 values per lane through the
+// add / round / scale / round steps is a chain of thousands of dependent instructions.
+// The element-wise steps are spread over the workgroup; only the sum of squares keeps
+// its defined order (lane l of the first wavefront owns [l*PER, (l+1)*PER), one fma
+// chain, butterfly), reading the values from LDS laid out so that lane l's i-th value
+// sits at [i][l].
 #include "norm_device.h"
 #include "rt.h"
 
@@ -20,6 +25,50 @@ __global__ __launch_bounds__(64) void rms_kernel(const bf16_t* a, const bf16_t* 
   const size_t off = (size_t)blockIdx.x * n;
   rms_row<PER, MODE>(a + off, b ? b + off : nullptr, w, z ? z + off : nullptr,
                      h_out ? h_out + off : nullptr, out + off, n, eps, threadIdx.x);
+}
+
+template <int PER, int MODE>
+__global__ __launch_bounds__(PER * 8) void rms_wide_kernel(const bf16_t* a, const bf16_t* b,
+                                                           const bf16_t* w, bf16_t* h_out,
+                                                           bf16_t* out, int n, float eps) {
+  static_assert(PER % 8 == 0 && MODE != NORM_GATED, "wide rows: plain and add only");
+  __shared__ float xs[PER * 64];
+  __shared__ float s_inv;
+  const size_t off = (size_t)blockIdx.x * n;
+  const int tid = threadIdx.x, e0 = tid * 8;
+  float x[8], wv[8];
+  load_bf16<8>(a + off + e0, x);
+  if (w) load_bf16<8>(w + e0, wv);
+  if constexpr (MODE == NORM_ADD) {
+    float y[8];
+    load_bf16<8>(b + off + e0, y);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = dm_rb(x[i] + y[i]);
+    store_bf16<8>(h_out + off + e0, x);
+  }
+  // value e belongs to lane e / PER, position e % PER
+  const int lane_of = e0 / PER, pos0 = e0 % PER;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) xs[(pos0 + i) * 64 + lane_of] = x[i];
+  __syncthreads();
+  if (tid < 64) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const float v = xs[i * 64 + tid];
+      acc = dm_fma(v, v, acc);
+    }
+    const float inv = dm_rsqrt(dm_wave_sum<64>(acc) / (float)n + eps);
+    if (tid == 0) s_inv = inv;
+  }
+  __syncthreads();
+  const float inv = s_inv;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    x[i] = dm_rb(x[i] * inv);
+    if (w) x[i] = dm_rb(wv[i] * x[i]);
+  }
+  store_bf16<8>(out + off + e0, x);
 }
 
 template <int MODE>
@@ -41,6 +90,18 @@ int launch_rms(ornith_ctx* ctx, const void* a, const void* b, const void* w, con
     RMS_CASE(2)
     RMS_CASE(4)
     RMS_CASE(8)
+#undef RMS_CASE
+#define RMS_CASE(P)                                                                              \
+  case P:                                                                                        \
+    if constexpr (MODE == NORM_GATED)                                                            \
+      hipLaunchKernelGGL((rms_kernel<P, MODE>), dim3(rows), dim3(64), 0, ctx->stream,            \
+                         (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)w, (const bf16_t*)z, \
+                         (bf16_t*)h_out, (bf16_t*)out, n, eps);                                  \
+    else                                                                                         \
+      hipLaunchKernelGGL((rms_wide_kernel<P, MODE>), dim3(rows), dim3(P * 8), 0, ctx->stream,    \
+                         (const bf16_t*)a, (const bf16_t*)b, (const bf16_t*)w, (bf16_t*)h_out,   \
+                         (bf16_t*)out, n, eps);                                                  \
+    break;
     RMS_CASE(16)
     RMS_CASE(32)
     RMS_CASE(64)

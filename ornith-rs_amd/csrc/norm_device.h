@@ -1,6 +1,5 @@
-// One row of an RMS norm by one wavefront, shared by the norm kernels and by the
-// projection / MoE kernels whose last workgroup applies the following
-// "residual add + norm" itself.
+// One row of an RMS norm by one wavefront, shared by the norm kernels and by kernels
+// that apply a norm to their own input.
 //
 // Arithmetic of vendored rms_norm.metal:12-81 and
 // /root/reference/kernels/ornith_norm.metal:28-183: lane l owns the contiguous piece
@@ -98,31 +97,4 @@ __device__ __forceinline__ void rms_row(const bf16_t* a, const bf16_t* b, const 
     for (int i = 0; i < PER; ++i) x[i] = (g[i] * dm_sigmoid_f32(g[i])) * x[i];
   }
   store_bf16<PER>(out + base, x);
-}
-
-// The "residual add + norm" that follows a projection or the MoE block, for one row,
-// dispatched on the row width (n = 64 * PER).
-struct AddRmsTail {
-  const bf16_t* res;   // residual rows [M, n]
-  const bf16_t* w;     // norm weight [n]
-  bf16_t* h_out;       // res + y, [M, n]
-  bf16_t* normed_out;  // [M, n]
-  unsigned int* counter;
-  float eps;
-};
-
-__device__ __forceinline__ void add_rms_tail_row(const AddRmsTail& t, const bf16_t* y_row, int row,
-                                                 int n, int lane) {
-  const bf16_t* a = t.res + (size_t)row * n;
-  bf16_t* h = t.h_out + (size_t)row * n;
-  bf16_t* o = t.normed_out + (size_t)row * n;
-  switch (n / 64) {
-    case 1: rms_row<1, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
-    case 2: rms_row<2, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
-    case 4: rms_row<4, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
-    case 8: rms_row<8, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
-    case 16: rms_row<16, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
-    case 32: rms_row<32, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
-    default: rms_row<64, NORM_ADD>(a, y_row, t.w, nullptr, h, o, n, t.eps, lane); break;
-  }
 }

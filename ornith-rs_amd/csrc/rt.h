@@ -19,11 +19,7 @@ struct ornith_ctx {
   // stream order makes reuse by the next operator safe.
   void* scratch = nullptr;
   size_t scratch_cap = 0;
-  // zero-initialised device counters for kernels whose last workgroup runs a tail
-  // (each such kernel leaves its counters at zero again)
-  unsigned int* counters = nullptr;
 };
-constexpr int kNumCounters = 256;
 
 // Returns at least `bytes` of device scratch (256-byte aligned). Growing it
 // synchronises the stream; callers that must not allocate size it once up front.
@@ -72,15 +68,7 @@ int ornith_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2,
 // the reference's ORNITH_* flags work (/root/reference/src/ops/moe.rs:397-414).
 int ornith_option_fuse_moe();
 int ornith_option_fuse_proj();
+int ornith_option_kq_iters();      // output rows per wavefront pass of the mat-vec kernels; 0 = by shape
 int ornith_option_moe_up_iters();  // rows per wavefront of the fused gate+up kernel; 0 = by shape
-
-// The residual add + norm that follows a MoE block, handed to the fused down kernel.
-struct MoeTail {
-  const void* d_res;
-  const void* d_wnorm;
-  float eps;
-  void* d_h_out;
-  void* d_normed_out;
-};
 
 static inline size_t ornith_dtype_size(int dt) { return dt == ORNITH_F32 ? 4 : 2; }

@@ -39,7 +39,8 @@ struct Option {
 };
 Option g_options[] = {{"fuse_moe", "ORNITH_FUSE_MOE", 1, -1},
                       {"fuse_proj", "ORNITH_FUSE_PROJ", 1, -1},
-                      {"moe_up_iters", "ORNITH_MOE_UP_ITERS", 0, -1}};
+                      {"moe_up_iters", "ORNITH_MOE_UP_ITERS", 0, -1},
+                      {"kq_iters", "ORNITH_KQ_ITERS", 0, -1}};
 int option_value(int i) {
   Option& o = g_options[i];
   if (o.value < 0) {
@@ -53,6 +54,7 @@ int option_value(int i) {
 int ornith_option_fuse_moe() { return option_value(0); }
 int ornith_option_fuse_proj() { return option_value(1); }
 int ornith_option_moe_up_iters() { return option_value(2); }
+int ornith_option_kq_iters() { return option_value(3); }
 
 extern "C" {
 
@@ -86,8 +88,6 @@ int ornith_ctx_create(int device, ornith_ctx** out) {
   ORN_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   ORN_HIP(hipEventCreate(&c->ev0));
   ORN_HIP(hipEventCreate(&c->ev1));
-  ORN_HIP(hipMalloc((void**)&c->counters, kNumCounters * sizeof(unsigned int)));
-  ORN_HIP(hipMemsetAsync(c->counters, 0, kNumCounters * sizeof(unsigned int), c->stream));
   *out = c;
   return ORNITH_OK;
 }
@@ -96,7 +96,6 @@ int ornith_ctx_destroy(ornith_ctx* ctx) {
   if (!ctx) return ORNITH_OK;
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->scratch) (void)hipFree(ctx->scratch);
-  if (ctx->counters) (void)hipFree(ctx->counters);
   (void)hipEventDestroy(ctx->ev0);
   (void)hipEventDestroy(ctx->ev1);
   (void)hipStreamDestroy(ctx->stream);

@@ -61,51 +61,3 @@ def test_multi_matrix_launch_equals_separate(orn, ctx):
             for b in ys + [dx]: b.free()
         for w in ws: w.free()
 
-
-def test_projection_with_norm_tail_equals_separate(orn, ctx):
-    """o_proj / out_proj with the residual add + norm applied by the last workgroup ==
-    matmul then add_rms_norm, for every width the model uses (and a repeat, which checks
-    that the hand-off counter is left ready for the next launch)."""
-    rng = np.random.default_rng(11)
-    for kind, O, K in ((Q4K, 2048, 4096), (Q6K, 2048, 4096), (Q4K, 512, 1024), (Q6K, 256, 512), (Q6K, 2048, 8192)):
-        t = util.make_kq(kind, rng, 1, O, K)
-        lin = orn.Linear.kquant(ctx, kind, *t, O, K)
-        wn = ctx.to_device(util.bf16_normal(rng, (O,)))
-        for M in (1, 2, 3, 4, 6, 2):
-            xb, rb = util.bf16_normal(rng, (M, K)), util.bf16_normal(rng, (M, O))
-            dx, dr = ctx.to_device(xb), ctx.to_device(rb)
-            got = [ctx.alloc(M * O * 2) for _ in range(3)]
-            want = [ctx.alloc(M * O * 2) for _ in range(3)]
-            ctx.linear_matmul_add_rms(lin, dx, M, got[0], dr, wn, 1e-6, got[1], got[2])
-            ctx.linear_matmul(lin, dx, M, want[0])
-            ctx.add_rms_norm(dr, want[0], wn, M, O, 1e-6, want[1], want[2])
-            for g, w_ in zip(got, want):
-                assert np.array_equal(g.download(np.uint16, (M, O)), w_.download(np.uint16, (M, O))), (kind, O, K, M)
-            for b in got + want + [dx, dr]: b.free()
-        wn.free(); lin.free()
-
-
-@pytest.mark.parametrize("H,E,I", [(2048, 256, 512), (512, 64, 256)])
-def test_moe_block_with_norm_tail_equals_separate(orn, ctx, H, E, I):
-    rng = np.random.default_rng(H + 1)
-    moe = util.HostMoe(rng, H=H, E=E, I=I, top_k=8, gate_kind=Q4K, down_kind=Q6K, router_kind=Q6K)
-    dw = moe.dev(orn, ctx)
-    wn = ctx.to_device(util.bf16_normal(rng, (H,)))
-    try:
-        for fuse in (1, 0):
-            orn.set_option("fuse_moe", fuse)
-            for T in (1, 2, 4, 9, 12, 2):
-                xb, rb = util.bf16_normal(rng, (T, H)), util.bf16_normal(rng, (T, H))
-                dx, dr = ctx.to_device(xb), ctx.to_device(rb)
-                got = [ctx.alloc(T * H * 2) for _ in range(3)]
-                want = [ctx.alloc(T * H * 2) for _ in range(3)]
-                ctx.moe_block_add_rms(dw, dx, T, got[0], dr, wn, 1e-6, got[1], got[2])
-                ctx.moe_block(dw, dx, T, want[0])
-                ctx.add_rms_norm(dr, want[0], wn, T, H, 1e-6, want[1], want[2])
-                for g, w_ in zip(got, want):
-                    assert np.array_equal(g.download(np.uint16, (T, H)), w_.download(np.uint16, (T, H))), (fuse, T)
-                for b in got + want + [dx, dr]: b.free()
-    finally:
-        orn.set_option("fuse_moe", 1)
-        wn.free()
-        moe.free()

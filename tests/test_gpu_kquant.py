@@ -45,6 +45,16 @@ def test_device_scalar_functions_bit_exact(orn, ctx):
     assert np.array_equal(util.f32_to_bf16(got[fin]), want[fin])
     # rounding and the wavefront butterfly
     assert np.array_equal(util.f32_to_bf16(ctx.selftest_unary(orn.FN_ROUND_BF16, x)), util.f32_to_bf16(x))
+    # ... over every exponent and upper mantissa, with the lower halves that decide rounding
+    # (ties, just above / below, zero) and random ones: subnormals, infinities, both signs
+    lows = np.concatenate([np.array([0, 1, 0x7fff, 0x8000, 0x8001, 0xffff], np.uint32),
+                           rng.integers(0, 65536, 26).astype(np.uint32)])
+    pat = ((np.arange(65536, dtype=np.uint32)[:, None] << 16) | lows[None, :]).reshape(-1)
+    xf = pat.view(np.float32)
+    ok = ~np.isnan(xf)
+    got = ctx.selftest_unary(orn.FN_ROUND_BF16, xf)
+    assert np.array_equal(got[ok].view(np.uint32) >> 16, util.f32_to_bf16(xf[ok]).astype(np.uint32))
+    assert np.all((got[ok].view(np.uint32) & 0xffff) == 0) and np.all(np.isnan(got[~ok]))
     v = (rng.standard_normal(64 * 50) * 10.0 ** rng.integers(-3, 4, 64 * 50)).astype(np.float32)
     got = ctx.selftest_unary(orn.FN_WAVE_SUM, v).reshape(50, 64)
     for i in range(50):
