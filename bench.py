@@ -12,9 +12,10 @@ been consumed (weights, caches and prompt state are resident in HBM) and `value`
 generated tokens per second.
 
 Also measured in the same run and printed on the same JSON line:
-  roofline      the expert gather-GEMV kernel: algorithmic bytes per launch (distinct
-                routed experts x bytes per expert matrix + activations) over the average
-                launch duration from HIP events on the library's stream, against 8 TB/s
+  roofline      the expert gate+up gather-GEMV kernel (the largest share of the step):
+                algorithmic bytes per launch (distinct routed experts + the shared one,
+                two Q4_K matrices each, + activations) over the average launch duration
+                from HIP events on the library's stream, against 8 TB/s
   cpu_baseline  the CPU oracle running the same loop on the host cores (bounded sample)
 """
 import argparse
@@ -36,43 +37,38 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def gather_gemv_roofline(orn, ctx, synth_model, util, np, T, launches=400):
-    """Times the routed gate-projection gather mat-vec (Q4_K [256, 512, 2048]) at verify width T
-    over every layer's weights in turn, so no launch finds its weights in cache."""
+def expert_gemv_roofline(orn, ctx, model, util, np, n_layers, T, launches=800):
+    """Times the expert gate+up gather-GEMV kernel (Q4_K: top-8 of 256 routed experts plus the
+    shared expert, gate and up projections and swiglu in one launch) at verify width T on the
+    model's resident weights, cycling through every layer so no launch finds its experts in
+    cache. Algorithmic bytes per launch: (distinct routed experts + 1) x 2 matrices x 512 x
+    2048 weights x 144/256 bytes, plus the activations read and written."""
     rng = np.random.default_rng(123)
-    kms = []
-    for lay in synth_model.layers:
-        km = lay["moe"]["ex_gate"]
-        kms.append(km)
-    # device copies already live in the weight store; rebuild kmatrix views by uploading again
-    # only the index / activation buffers: the weights are addressed through fresh KMatrix
-    # objects over the SAME host arrays (one extra upload of the gate tensors, 151 MB a layer).
-    devs = [km.dev(orn, ctx) for km in kms]
-    H, O, E, k = 2048, 512, 256, 8
-    rows = T * k
+    H, I, E, k = 2048, 512, 256, 8
+    moes = [model.moe_weights(i) for i in range(n_layers)]
     xb = util.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32))
-    lhs = np.repeat(np.arange(T, dtype=np.uint32), k)
-    rhs = np.concatenate([rng.permutation(E)[:k] for _ in range(T)]).astype(np.uint32)
-    U = len(np.unique(rhs))
-    dx, dl, dr, dy = ctx.to_device(xb), ctx.to_device(lhs), ctx.to_device(rhs), ctx.alloc(rows * O * 2)
-    for d in devs:
-        ctx.kq_gather_qmv(d, dx, orn.BF16, T, dl, dr, rows, dy, orn.BF16)
+    inds = np.concatenate([rng.permutation(E)[:k] for _ in range(T)]).astype(np.uint32)
+    U = len(np.unique(inds))
+    scores = util.f32_to_bf16(rng.random((T, k)).astype(np.float32))
+    eg = util.f32_to_bf16(rng.standard_normal(T).astype(np.float32))
+    dx, di, ds, de = ctx.to_device(xb), ctx.to_device(inds), ctx.to_device(scores), ctx.to_device(eg)
+    act, out = ctx.alloc((T * k + T) * I * 2), ctx.alloc(T * H * 2)
+    for w in moes:
+        orn.moe_experts(ctx, w, dx, T, di, ds, de, act, out, 1)
     ctx.sync()
     ctx.timer_begin()
     for i in range(launches):
-        ctx.kq_gather_qmv(devs[i % len(devs)], dx, orn.BF16, T, dl, dr, rows, dy, orn.BF16)
-    ms = ctx.timer_end()
-    us = ms * 1000.0 / launches
-    bytes_per_launch = U * O * (H // 256) * 144 + T * H * 2 + rows * O * 2
-    for b in (dx, dl, dr, dy):
+        orn.moe_experts(ctx, moes[i % len(moes)], dx, T, di, ds, de, act, out, 1)
+    us = ctx.timer_end() * 1000.0 / launches
+    bytes_per_launch = (U + 1) * 2 * I * (H // 256) * 144 + T * H * 2 + (T * k + T) * I * 2 + T * k * 4
+    for b in (dx, di, ds, de, act, out):
         b.free()
-    for d in devs:
-        d.free()
     achieved = bytes_per_launch / (us * 1e-6) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-            "kernel": "kq_qmv_kernel<Q4_K, 64 lanes/row, gather>", "us_per_launch": round(us, 3),
-            "bytes_per_launch": int(bytes_per_launch), "distinct_experts": int(U), "rows": int(rows)}
+            "kernel": "moe_up_kernel<Q4_K, 64 lanes/row, 2 rows/wavefront> (expert gate+up gather-GEMV + swiglu)",
+            "us_per_launch": round(us, 3), "bytes_per_launch": int(bytes_per_launch),
+            "distinct_experts": int(U), "verify_width": int(T)}
 
 
 def cpu_baseline(synth, synth_model, np, depth, tokens):
@@ -102,6 +98,9 @@ def main():
     ap.add_argument("--layers", type=int, default=40, help="trunk layers (40 = the named config)")
     ap.add_argument("--cpu-tokens", type=int, default=12)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--roofline-only", action="store_true",
+                    help="only the expert-kernel timing loop plus three 256 MiB device copies "
+                         "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (one process, one stream); "
@@ -123,6 +122,14 @@ def main():
     ws = sm.upload(orn, ctx)
     log(f"uploaded in {time.time() - t0:.1f} s")
     model = orn.TextModel(ctx, ws, sm.text_config(orn))
+    if args.roofline_only:
+        roof = expert_gemv_roofline(orn, ctx, model, util, np, args.layers, T=args.depth + 1, launches=200)
+        a, b = ctx.alloc(256 << 20), ctx.alloc(256 << 20)
+        for _ in range(3):
+            ctx.copy(a, b, 256 << 20)
+        ctx.sync()
+        print(json.dumps({"roofline": roof}), flush=True)
+        return
     rng = np.random.default_rng(51)
     prompt = rng.integers(0, cfg["vocab_size"], 51).astype(np.uint32)
     cap = 4096
@@ -164,7 +171,7 @@ def main():
     total_s = sum(times)
     tok_s = args.tokens * len(times) / total_s
 
-    roof = gather_gemv_roofline(orn, ctx, sm, util, np, T=args.depth + 1)
+    roof = expert_gemv_roofline(orn, ctx, model, util, np, args.layers, T=args.depth + 1)
     log("roofline:", roof)
 
     cpu = None

@@ -316,6 +316,11 @@ typedef struct ornith_caches ornith_caches;
 ORNITH_API int ornith_model_load(ornith_ctx* ctx, const ornith_weights* ws,
                                  const ornith_text_config* cfg, ornith_model** out);
 ORNITH_API int ornith_model_destroy(ornith_model* m);
+/* The MoE block of decoder layer `layer` as the model holds it (pointers into the weight
+ * store, valid while the model lives): lets a caller run or time ornith_moe_block /
+ * ornith_moe_experts on the resident weights (the reference reaches them as
+ * model.layers[i].mlp, src/model/qwen3_5.rs:261-283). */
+ORNITH_API int ornith_model_moe_weights(const ornith_model* m, int layer, ornith_moe_weights* out);
 /* make_cache: one KvCache (bf16 [Hkv, capacity, hd] x2) or GdnCache (conv window +
  * fp32 state with max_window snapshot slots) per layer. capacity bounds prompt +
  * generated tokens (the reference grows in steps of 256; here it is fixed up front). */

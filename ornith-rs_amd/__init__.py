@@ -138,6 +138,9 @@ class Ctx:
         arr = np.ascontiguousarray(arr)
         return DeviceBuffer(self, max(arr.nbytes, 1)).upload(arr)
 
+    def copy(self, dst, src, nbytes):
+        _check(lib().ornith_copy(self.h, dst.ptr, src.ptr, nbytes), "copy")
+
     def device_info(self):
         name = C.create_string_buffer(256)
         cus, mem = C.c_int(), C.c_size_t()

@@ -87,21 +87,40 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
     for (int t = 0; t < M; ++t) xrow[t] = static_cast<const char*>(a.x) + (size_t)t * a.K * xsz;
   }
 
+  // Rows kept in flight per wavefront. Cold weights come from HBM with a latency many
+  // times the arithmetic of one row, so every wavefront issues the loads of its first PF
+  // rows before anything else (they depend on nothing), then its activations, and
+  // refills a slot as soon as that row's registers are consumed.
+  constexpr int PF = (KIND == ORNITH_Q4K) ? (M <= 2 ? 4 : 2) : (M <= 2 ? 2 : 1);
   typename KL::Lane L;
-  L.template load_x<XF32>(xrow, c + 64 * ks);
+  L.set_chunk(c + 64 * ks);
 
   __shared__ float part[(KS == 2) ? 2 * M * 64 : 1];
 
   const int rows_per_wave = RPW * a.iters;
   const int base = (((int)blockIdx.x - sg.first_block) * WPB + rw) * rows_per_wave;
-  for (int it = 0; it < a.iters; ++it) {
+  auto row_of = [&](int it) {
+    const int o = base + it * RPW + slot;
+    return row0 + (o < O ? o : O - 1);
+  };
+  typename KL::Row pf[PF];
+#pragma unroll
+  for (int i = 0; i < PF; ++i) pf[i] = KL::load(sg.qs, sg.scales, sg.dm, row_of(i), nb, L);
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  L.template load_x<XF32>(xrow, c + 64 * ks);
+
+  for (int it0 = 0; it0 < a.iters; it0 += PF) {
+#pragma unroll
+   for (int i = 0; i < PF; ++i) {
+    const int it = it0 + i;
+    if (it >= a.iters) break;
     const int o = base + it * RPW + slot;
     const bool valid = o < O;
-    const int64_t row = row0 + (valid ? o : O - 1);
     float acc[M];
 #pragma unroll
     for (int t = 0; t < M; ++t) acc[t] = 0.f;
-    const typename KL::Row r = KL::load(sg.qs, sg.scales, sg.dm, row, nb, L);
+    const typename KL::Row r = pf[i];
+    if (it + PF < a.iters) pf[i] = KL::load(sg.qs, sg.scales, sg.dm, row_of(it + PF), nb, L);
     KL::accumulate(r, L, acc);
     if constexpr (KS == 2) {
       // lane partial = (chunk l) + (chunk l + 64), in that order
@@ -128,6 +147,7 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
           static_cast<float*>(sg.y)[yi] = v;
       }
     }
+   }
   }
 }
 

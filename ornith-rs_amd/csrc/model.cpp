@@ -300,6 +300,14 @@ int ornith_model_load(ornith_ctx* ctx, const ornith_weights* ws, const ornith_te
   return ORNITH_OK;
 }
 
+int ornith_model_moe_weights(const ornith_model* m, int layer, ornith_moe_weights* out) {
+  ORN_REQUIRE(m && out, "model_moe_weights: null argument");
+  ORN_REQUIRE(layer >= 0 && layer < (int)m->layers.size(), "model_moe_weights: layer %d of %zu", layer,
+              m->layers.size());
+  *out = m->layers[layer].moe;
+  return ORNITH_OK;
+}
+
 int ornith_model_destroy(ornith_model* m) {
   if (!m) return ORNITH_OK;
   ornith_free(m->ctx, m->ws_buf);

@@ -85,6 +85,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
     rg[it] = KL::load(wg.qs, wg.scales, wg.dm, row, nb, L);
     ru[it] = KL::load(wu.qs, wu.scales, wu.dm, row, nb, L);
   }
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
   const void* xrow[1] = {a.x + (size_t)token * a.K};
   L.template load_x<false>(xrow, c);
   if constexpr (LPR == 64 && ITERS % 2 == 0) {
@@ -158,6 +159,7 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) 
     const int o = c0 + it * RPW + slot;
     rr[it] = KL::load(w.qs, w.scales, w.dm, row0 + (o < a.H ? o : a.H - 1), nb, L);
   }
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
   const void* xrow[1] = {a.act + (size_t)arow * a.I};
   L.template load_x<false>(xrow, c);
 
@@ -260,6 +262,7 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
   L.set_chunk(c);
   const int o = (blockIdx.x * 4 + wave) * RPW + slot;
   const typename KL::Row row = KL::load(a.w.qs, a.w.scales, a.w.dm, o < a.E ? o : a.E - 1, nb, L);
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
   const void* xrow[M];
 #pragma unroll
   for (int t = 0; t < M; ++t) xrow[t] = a.x + (size_t)t * a.K;

@@ -166,6 +166,13 @@ class TextModel:
     def rewind(self, caches, keep):
         _check(lib().ornith_model_rewind(self.h, caches.h, keep), "model_rewind")
 
+    def moe_weights(self, layer):
+        """The resident MoE block of one decoder layer (valid while the model lives)."""
+        from . import MoeWeightsStruct
+        w = MoeWeightsStruct()
+        _check(lib().ornith_model_moe_weights(self.h, layer, C.byref(w)), "model_moe_weights")
+        return w
+
     def logits(self, hidden):
         hidden = np.ascontiguousarray(hidden, dtype=np.uint16)
         T, V = hidden.shape[0], self.cfg.vocab_size
