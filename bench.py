@@ -32,6 +32,13 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch of the expert gate+up kernel at verify width 2 (17 distinct experts),
+# from two `rocprofv3 --pmc` runs of `bench.py --roofline-only` (FETCH_SIZE, then WRITE_SIZE,
+# KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device copies
+# that run issues: FETCH_SIZE 9870.1 x 2.0 (the copy reads 131,094 for 262,144 KiB),
+# WRITE_SIZE 36.0 x 1.0. Counters cannot be read from inside this script; other widths: null.
+PMC_TRAFFIC_BYTES = {2: int(round((9870.1 * 2.0 + 36.0 * 1.0) * 1024))}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -65,7 +72,8 @@ def expert_gemv_roofline(orn, ctx, model, util, np, n_layers, T, launches=800):
         b.free()
     achieved = bytes_per_launch / (us * 1e-6) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": PMC_TRAFFIC_BYTES.get(T) if U == 16 else None,
             "kernel": "moe_up_kernel<Q4_K, 64 lanes/row, 2 rows/wavefront> (expert gate+up gather-GEMV + swiglu)",
             "us_per_launch": round(us, 3), "bytes_per_launch": int(bytes_per_launch),
             "distinct_experts": int(U), "verify_width": int(T)}
@@ -96,7 +104,7 @@ def main():
     ap.add_argument("--tokens", type=int, default=200)
     ap.add_argument("--depth", type=int, default=1)
     ap.add_argument("--layers", type=int, default=40, help="trunk layers (40 = the named config)")
-    ap.add_argument("--cpu-tokens", type=int, default=12)
+    ap.add_argument("--cpu-tokens", type=int, default=48)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the expert-kernel timing loop plus three 256 MiB device copies "
@@ -188,10 +196,11 @@ def main():
         "metric": "decode tok/s @MTP depth 1 (1 GPU, byte-exact); expert GEMV HBM GB/s vs peak",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(total_s / len(times) * 1e3, 3), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "bf16 activations, fp32 accumulate, Q4_K/Q6_K/int8 weights",
+        "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": f"config4: greedy MTP depth-{args.depth} + FR-Spec(32768) decode of {args.tokens} tokens, "
                                f"51-token prompt, Qwen3.5-35B-A3B shape, {args.layers} layers, KV capacity {cap}",
+                   "arithmetic": "fp32 accumulate over bf16 activations and Q4_K/Q6_K/int8/bf16 weights",
                    "tokens_per_step": args.tokens, "byte_identical_to_greedy": True,
                    "plain_greedy_tok_s": round(len(ar) / ar_s, 2),
                    "cycles": int(stats.cycles), "accepted": int(stats.accepted), "drafted": int(stats.drafted),
