@@ -366,6 +366,39 @@ ORNITH_API int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspe
 ORNITH_API int ornith_mtp_cache_set_offset(ornith_mtp_head* h, int offset);
 ORNITH_API int ornith_mtp_cache_offset(const ornith_mtp_head* h, int* offset_out);
 
+/* ---- the sampled-token path: TopSampler (src/sample.rs:79-225) -------------------------
+ * bf16 throughout except the CDF, as in the reference. Cumulative sums associate in
+ * chunks of 1024 / segments of 64 (see csrc/sampler.hip); sorts are stable. */
+/* random::key / KeySequence::next / random::bits (src/ops/random.rs:16-67; threefry2x32 of
+ * vendored random.metal:5-66). Host functions: the key sequence is 64 bits of integer state. */
+ORNITH_API void ornith_random_key(uint64_t seed, uint32_t key_out[2]);
+ORNITH_API int ornith_random_split(uint32_t key_state[2], uint32_t sub_out[2]);
+ORNITH_API int ornith_random_bits(const uint32_t key[2], int n, uint32_t* out);
+/* ops::sort::argsort_last_axis over one row of bf16 (negate != 0: of the negated values,
+ * as apply_top_k asks): the stable ascending order as u32 indices. */
+ORNITH_API int ornith_argsort_bf16(ornith_ctx* ctx, const void* d_x, int n, int negate,
+                                   uint32_t* d_idx_out);
+/* ops::scan::cumsum_last_axis, inclusive, one row; dtype ORNITH_BF16 accumulates in bf16. */
+ORNITH_API int ornith_cumsum(ornith_ctx* ctx, const void* d_x, int dtype, int n, void* d_out);
+/* apply_top_p (src/sample.rs:79-115), apply_top_k (:117-136): bf16 logprobs [V] -> bf16 [V]
+ * with the dropped entries at -inf. d_out must not alias the input. */
+ORNITH_API int ornith_apply_top_p(ornith_ctx* ctx, const void* d_logprobs, int V, double top_p,
+                                  void* d_out);
+ORNITH_API int ornith_apply_top_k(ornith_ctx* ctx, const void* d_logprobs, int V, int top_k,
+                                  void* d_out);
+/* categorical_sampling (src/sample.rs:138-190) with the raw 32-bit random word given:
+ * writes the drawn index to d_token_out. */
+ORNITH_API int ornith_categorical(ornith_ctx* ctx, const void* d_logprobs, int V, double temp,
+                                  uint32_t raw_bits, uint32_t* d_token_out);
+/* TopSampler (src/sample.rs:192-225): log-softmax of one row of logits, top-p if
+ * 0 < top_p < 1, top-k if top_k > 0, one draw; every sample consumes one split of the key. */
+typedef struct ornith_top_sampler ornith_top_sampler;
+ORNITH_API int ornith_top_sampler_create(ornith_ctx* ctx, double temp, double top_p, int top_k,
+                                         uint64_t seed, int vocab, ornith_top_sampler** out);
+ORNITH_API int ornith_top_sampler_destroy(ornith_top_sampler* s);
+ORNITH_API int ornith_top_sampler_sample(ornith_top_sampler* s, const void* d_logits_row,
+                                         uint32_t* d_token_out);
+
 /* ---- generation loops ---------------------------------------------------------------- */
 /* Sampler (src/generate.rs:36-64, src/sample.rs:205-225). rows_are_independent is
  * true for GREEDY. */

@@ -301,7 +301,37 @@ ORC_API void orc_mtp_hidden(orc_state* s, const orc_mtp_w* w, const bf16_t* trun
 
 ORC_API void orc_mtp_set_offset(orc_state* s, int off) { s->moffset = off; }
 
-/* generate_step with the greedy sampler; returns the number of tokens written */
+/* The sampler the two loops below drive (generate.rs:36-64): greedy unless
+ * orc_set_sampler chose the top-p / top-k / temperature one (sample.rs:192-225). Each
+ * loop call starts from the seed, as a freshly built TopSampler does. */
+static struct {
+  int kind;
+  double temp, top_p;
+  int top_k;
+  uint64_t seed;
+  uint32_t key[2];
+} g_sampler;
+extern void orc_key_from_seed(uint64_t seed, uint32_t key[2]);
+extern uint32_t orc_top_sample(const bf16_t* logits, int V, double temp, double top_p, int top_k,
+                               uint32_t key_state[2]);
+ORC_API void orc_set_sampler(int kind, double temp, double top_p, int top_k, uint64_t seed) {
+  g_sampler.kind = kind;
+  g_sampler.temp = temp;
+  g_sampler.top_p = top_p;
+  g_sampler.top_k = top_k;
+  g_sampler.seed = seed;
+}
+static void sampler_begin(void) { orc_key_from_seed(g_sampler.seed, g_sampler.key); }
+static uint32_t sample_row(const bf16_t* logits, int V) {
+  if (g_sampler.kind == 0) {
+    uint32_t t;
+    orc_greedy_rows(logits, 1, V, &t, NULL);
+    return t;
+  }
+  return orc_top_sample(logits, V, g_sampler.temp, g_sampler.top_p, g_sampler.top_k, g_sampler.key);
+}
+
+/* generate_step; returns the number of tokens written */
 ORC_API int orc_generate(orc_state* s, const uint32_t* prompt, int n_prompt, int max_tokens, int prefill_step,
                          uint32_t* out) {
   const orc_model_w* m = s->m;
@@ -316,14 +346,15 @@ ORC_API int orc_generate(orc_state* s, const uint32_t* prompt, int n_prompt, int
   }
   int rows = n_prompt - processed;
   uint32_t y, next;
+  sampler_begin();
   orc_forward(s, prompt + processed, rows, 0, hid);
   orc_logits(m, hid + (size_t)(rows - 1) * H, 1, logits);
-  orc_greedy_rows(logits, 1, V, &y, NULL);
+  y = sample_row(logits, V);
   int n = 0;
   while (n != max_tokens) {
     orc_forward(s, &y, 1, 0, hid);
     orc_logits(m, hid, 1, logits);
-    orc_greedy_rows(logits, 1, V, &next, NULL);
+    next = sample_row(logits, V);
     out[n++] = y;
     y = next;
   }
@@ -333,7 +364,10 @@ ORC_API int orc_generate(orc_state* s, const uint32_t* prompt, int n_prompt, int
 
 typedef struct orc_mtp_stats { int64_t cycles, drafted, accepted, reached[8], accepted_by[8]; } orc_mtp_stats;
 
-/* generate_step_mtp with the greedy sampler. fr_ids/fr_head: the FR-Spec list and its
+/* generate_step_mtp. With the greedy sampler every row's target is taken at once; with a
+ * sampler whose rows depend on each other (each draw advances the key) the rows are
+ * sampled one by one and only as far as the accept loop asks (mtp_generate.rs:236-279).
+ * fr_ids/fr_head: the FR-Spec list and its
  * pruned head (NULL for the full lm_head). policy: 0 Cycle, 1 Committed. */
 ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* fr_ids, int fr_n,
                              const orc_linear* fr_head, const uint32_t* prompt, int n_prompt, int depth,
@@ -357,8 +391,8 @@ ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* f
   const int rows = n_prompt - processed;
   orc_forward(s, prompt + processed, rows, 0, hid);
   orc_logits(m, hid + (size_t)(rows - 1) * H, 1, vlogits);
-  uint32_t primary;
-  orc_greedy_rows(vlogits, 1, V, &primary, NULL);
+  sampler_begin();
+  uint32_t primary = sample_row(vlogits, V);
   memcpy(h, hid + (size_t)(rows - 1) * H, 2 * (size_t)H);
   int emitted = 0;
   s->moffset = 0;
@@ -389,17 +423,19 @@ ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* f
     const int n_rows = want + 1;
     orc_forward(s, window, n_rows, 1, hid);
     orc_logits(m, hid, n_rows, vlogits);
-    orc_greedy_rows(vlogits, n_rows, V, targets, NULL);
+    const int independent = g_sampler.kind == 0;
+    if (independent) orc_greedy_rows(vlogits, n_rows, V, targets, NULL);
     int k = 0, have = 0;
     uint32_t next_primary = 0;
     while (k < want) {
+      const uint32_t target = independent ? targets[k] : sample_row(vlogits + (size_t)k * V, V);
       stats->reached[k]++;
-      if (targets[k] != window[1 + k]) { next_primary = targets[k]; have = 1; break; }
+      if (target != window[1 + k]) { next_primary = target; have = 1; break; }
       stats->accepted_by[k]++;
       stats->accepted++;
       k++;
     }
-    if (!have) next_primary = targets[k];
+    if (!have) next_primary = independent ? targets[k] : sample_row(vlogits + (size_t)k * V, V);
     orc_rewind(s, k + 1);
     if (policy == 1) {
       s->moffset = cycle_off + 1;

@@ -40,13 +40,31 @@ struct Bufs {
   }
 };
 
-int check_sampler(const ornith_sampler* s) {
-  ORN_REQUIRE(s, "sampler is null");
-  if (s->kind == ORNITH_SAMPLER_GREEDY) return ORNITH_OK;
-  return ornith_fail(ORNITH_ERR_UNSUPPORTED,
-                     "sampler kind %d: only the greedy sampler is built in this library so far",
-                     s->kind);
-}
+// The `Sampler` a loop drives (src/generate.rs:36-64): Greedy, or TopSampler built from
+// the tagged struct. rows_are_independent() is true for Greedy only: every draw of the
+// other advances its key, so rows are sampled one by one and only when asked for.
+struct LoopSampler {
+  ornith_ctx* ctx = nullptr;
+  ornith_top_sampler* top = nullptr;
+  int V = 0;
+  ~LoopSampler() {
+    if (top) ornith_top_sampler_destroy(top);
+  }
+  int init(ornith_ctx* c, const ornith_sampler* s, int vocab) {
+    ORN_REQUIRE(s, "sampler is null");
+    ctx = c;
+    V = vocab;
+    if (s->kind == ORNITH_SAMPLER_GREEDY) return ORNITH_OK;
+    ORN_REQUIRE(s->kind == ORNITH_SAMPLER_TOP_P, "unknown sampler kind %d", s->kind);
+    return ornith_top_sampler_create(c, s->temperature, s->top_p, s->top_k, s->seed, vocab, &top);
+  }
+  bool rows_are_independent() const { return top == nullptr; }
+  // one row of logits -> token on the device
+  int sample(const void* d_logits_row, uint32_t* d_token) {
+    if (top) return ornith_top_sampler_sample(top, d_logits_row, d_token);
+    return ornith_greedy_rows(ctx, d_logits_row, 1, V, d_token, nullptr);
+  }
+};
 
 // prefill (src/generate.rs:90-136): everything but the last token, in chunks
 int prefill(ornith_model* m, ornith_caches* c, const uint32_t* prompt, size_t total, size_t step,
@@ -76,9 +94,10 @@ int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, s
                     ornith_progress_cb progress, ornith_token_cb on_token, void* user) {
   ORN_REQUIRE(m && c && prompt && on_token, "generate: null argument");
   ORN_REQUIRE(n_prompt >= 1, "generate_step needs a prompt");
-  TRY(check_sampler(sampler));
   ornith_ctx* ctx = m->ctx;
   const size_t H = m->cfg.hidden_size, V = m->cfg.vocab_size, R = m->max_rows;
+  LoopSampler smp;
+  TRY(smp.init(ctx, sampler, (int)V));
   Bufs b(ctx);
   uint32_t *d_tok, *d_out;
   void *d_hidden, *d_logits;
@@ -94,7 +113,7 @@ int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, s
     TRY(ornith_upload(ctx, d_tok, toks, n * 4));
     TRY(ornith_model_forward(m, c, d_tok, (int)n, 0, d_hidden));
     TRY(ornith_model_logits(m, (char*)d_hidden + (n - 1) * H * 2, 1, d_logits));
-    TRY(ornith_greedy_rows(ctx, d_logits, 1, (int)V, d_out, nullptr));
+    TRY(smp.sample(d_logits, d_out));
     return ornith_download(ctx, y, d_out, 4);
   };
   uint32_t y = 0;
@@ -126,9 +145,10 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   ORN_REQUIRE(policy == ORNITH_HISTORY_CYCLE || policy == ORNITH_HISTORY_COMMITTED,
               "mtp_generate: unknown history policy %d", policy);
   ORN_REQUIRE(head->m == m && (!frspec || frspec->m == m), "mtp_generate: head / frspec of another model");
-  TRY(check_sampler(sampler));
   ornith_ctx* ctx = m->ctx;
   const size_t H = m->cfg.hidden_size, V = m->cfg.vocab_size, R = m->max_rows;
+  LoopSampler smp;
+  TRY(smp.init(ctx, sampler, (int)V));
   ornith_mtp_stats stats{};
 
   Bufs b(ctx);
@@ -153,7 +173,7 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   TRY(ornith_model_forward(m, c, d_tok, (int)rows, 0, d_hidden));
   if (progress) progress(n_prompt, n_prompt, user);
   TRY(ornith_model_logits(m, (char*)d_hidden + (rows - 1) * H * 2, 1, d_vlogits));
-  TRY(ornith_greedy_rows(ctx, d_vlogits, 1, (int)V, d_targets, nullptr));
+  TRY(smp.sample(d_vlogits, d_targets));
   uint32_t primary = 0;
   TRY(ornith_download(ctx, &primary, d_targets, 4));
   TRY(ornith_copy(ctx, d_h, (char*)d_hidden + (rows - 1) * H * 2, H * 2));
@@ -195,16 +215,29 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
     const int n_rows = want + 1;
     TRY(ornith_model_forward(m, c, d_window, n_rows, 1, d_hidden));
     TRY(ornith_model_logits(m, d_hidden, n_rows, d_vlogits));
-    TRY(ornith_greedy_rows(ctx, d_vlogits, n_rows, (int)V, d_targets, nullptr));
-    TRY(ornith_download(ctx, targets.data(), d_targets, (size_t)n_rows * 4));  // the cycle's one sync
+    const bool independent = smp.rows_are_independent();
+    if (independent) {
+      TRY(ornith_greedy_rows(ctx, d_vlogits, n_rows, (int)V, d_targets, nullptr));
+      TRY(ornith_download(ctx, targets.data(), d_targets, (size_t)n_rows * 4));  // the cycle's one sync
+    }
     TRY(ornith_download(ctx, win.data(), d_window, (size_t)n_rows * 4));
+    // a dependent sampler draws row by row, as far as the accept loop asks
+    auto take = [&](int row, uint32_t* t) -> int {
+      if (independent) {
+        *t = targets[row];
+        return ORNITH_OK;
+      }
+      TRY(smp.sample((const char*)d_vlogits + (size_t)row * V * 2, d_targets + row));
+      return ornith_download(ctx, t, d_targets + row, 4);
+    };
 
     // accept the leading run of agreements
     int k = 0;
     bool have_next = false;
     uint32_t next_primary = 0;
     while (k < want) {
-      const uint32_t target = targets[k];
+      uint32_t target = 0;
+      TRY(take(k, &target));
       stats.reached_by_depth[k] += 1;
       if (target != win[1 + k]) {
         next_primary = target;
@@ -215,7 +248,7 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
       stats.accepted += 1;
       ++k;
     }
-    if (!have_next) next_primary = targets[k];  // the bonus token
+    if (!have_next) TRY(take(k, &next_primary));  // the bonus token
 
     // the window put want+1 tokens into the caches; k+1 of them are committed
     TRY(ornith_model_rewind(m, c, k + 1));

@@ -38,6 +38,11 @@ struct ScratchCursor {
   }
 };
 
+// ornith_greedy_rows with its temporaries taken from the caller's cursor (for operators
+// that hold other scratch buffers at the same time). Needs rows * ceil(V/1024) * 16 + 2048 bytes.
+int ornith_greedy_rows_ws(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens,
+                          void* d_lse, ScratchCursor& sc);
+
 // Records the message for ornith_last_error() and returns `code`.
 int ornith_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 

@@ -141,14 +141,17 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* bv, const
 }
 
 int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens, void* d_lse,
-        bool use_lse, const char* who) {
+        bool use_lse, const char* who, ScratchCursor* ws = nullptr) {
   ORN_REQUIRE(ctx && d_logits && d_tokens, "%s: null argument", who);
   ORN_REQUIRE(rows >= 1 && rows <= 65535 && V >= 1, "%s: rows=%d V=%d", who, rows, V);
   const int nch = (V + CH - 1) / CH;
   void* base = nullptr;
-  int rc = ornith_scratch(ctx, (size_t)rows * nch * 16 + 2048, &base);
-  if (rc) return rc;
-  ScratchCursor sc(base);
+  if (!ws) {
+    int rc = ornith_scratch(ctx, (size_t)rows * nch * 16 + 2048, &base);
+    if (rc) return rc;
+  }
+  ScratchCursor own(base);
+  ScratchCursor& sc = ws ? *ws : own;
   float* mc = sc.take<float>((size_t)rows * nch);
   float* lc = sc.take<float>((size_t)rows * nch);
   float* bv = sc.take<float>((size_t)rows * nch);
@@ -171,6 +174,11 @@ int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_toke
 }
 
 }  // namespace
+
+int ornith_greedy_rows_ws(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens,
+                          void* d_lse, ScratchCursor& sc) {
+  return run(ctx, d_logits, rows, V, d_tokens, d_lse, true, "greedy_rows", &sc);
+}
 
 extern "C" {
 

@@ -291,3 +291,69 @@ def generate_step_mtp(model, head, frspec, caches, prompt, depth, max_tokens, sa
                                      C.c_size_t(prefill_step), policy, pcb, cb, None, C.byref(stats)),
            "mtp_generate")
     return out, stats
+
+
+# ---- the sampled-token path (src/sample.rs, src/ops/random.rs) ----------------------------
+def random_key(seed):
+    k = (C.c_uint32 * 2)()
+    lib().ornith_random_key(C.c_uint64(seed), k)
+    return [k[0], k[1]]
+
+
+def random_split(state):
+    """KeySequence::next: returns (new_state, sub_key)."""
+    st = (C.c_uint32 * 2)(*state)
+    sub = (C.c_uint32 * 2)()
+    _check(lib().ornith_random_split(st, sub), "random_split")
+    return [st[0], st[1]], [sub[0], sub[1]]
+
+
+def random_bits(key, n):
+    k = (C.c_uint32 * 2)(*key)
+    out = (C.c_uint32 * n)()
+    _check(lib().ornith_random_bits(k, n, out), "random_bits")
+    return np.array(list(out), dtype=np.uint32)
+
+
+def argsort_bf16(ctx, x, n, negate, idx_out):
+    _check(lib().ornith_argsort_bf16(ctx.h, x.ptr, n, int(negate), idx_out.ptr), "argsort_bf16")
+
+
+def cumsum(ctx, x, dtype, n, out):
+    _check(lib().ornith_cumsum(ctx.h, x.ptr, dtype, n, out.ptr), "cumsum")
+
+
+def apply_top_p(ctx, lp, V, top_p, out):
+    _check(lib().ornith_apply_top_p(ctx.h, lp.ptr, V, C.c_double(top_p), out.ptr), "apply_top_p")
+
+
+def apply_top_k(ctx, lp, V, top_k, out):
+    _check(lib().ornith_apply_top_k(ctx.h, lp.ptr, V, top_k, out.ptr), "apply_top_k")
+
+
+def categorical(ctx, lp, V, temp, raw_bits, token_out):
+    _check(lib().ornith_categorical(ctx.h, lp.ptr, V, C.c_double(temp), C.c_uint32(raw_bits), token_out.ptr),
+           "categorical")
+
+
+class TopSampler:
+    """TopSampler::new(temp, top_p, top_k, seed) over a vocabulary of `vocab` ids."""
+
+    def __init__(self, ctx, temp, top_p, top_k, seed, vocab):
+        self.ctx, self.vocab = ctx, vocab
+        h = C.c_void_p()
+        _check(lib().ornith_top_sampler_create(ctx.h, C.c_double(temp), C.c_double(top_p), top_k,
+                                               C.c_uint64(seed), vocab, C.byref(h)), "top_sampler_create")
+        self.h = h
+        self._tok = ctx.alloc(4)
+
+    def sample(self, logits_row):
+        """logits_row: DeviceBuffer of bf16 [vocab] -> token id."""
+        _check(lib().ornith_top_sampler_sample(self.h, logits_row.ptr, self._tok.ptr), "top_sampler_sample")
+        return int(self._tok.download(np.uint32, (1,))[0])
+
+    def close(self):
+        if self.h:
+            lib().ornith_top_sampler_destroy(self.h)
+            self.h = None
+            self._tok.free()

@@ -285,6 +285,12 @@ class OracleRun:
         self.o.orc_mtp_hidden(self.st, C.byref(self.mtp), p(trunk_hidden), p(next_ids), len(next_ids), p(out))
         return out
 
+    def set_sampler(self, kind=0, temp=1.0, top_p=1.0, top_k=0, seed=0):
+        """kind 0 greedy, 1 top-p/top-k/temperature; temp and top_p as the float32 values the
+        C struct carries. Process-global in the oracle: reset to greedy when done."""
+        self.o.orc_set_sampler(kind, C.c_double(float(np.float32(temp))), C.c_double(float(np.float32(top_p))),
+                               top_k, C.c_uint64(seed))
+
     def generate(self, prompt, max_tokens, prefill_step=16):
         prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
         out = np.empty(max_tokens, np.uint32)

@@ -1,4 +1,5 @@
 """The C-ABI library loads and exports every function include/*.h declares (no GPU needed)."""
+import numpy as np
 import ctypes
 import glob
 import os
@@ -47,3 +48,22 @@ def test_error_path_reports_message_without_gpu(orn):
     s = orn.KMatrixStruct(orn.Q4K, 1, 4, 512, 1, 1, 1)
     assert orn.lib().ornith_kmatrix_check(ctypes.byref(s), ctypes.c_size_t(4 * 2 * 128), ctypes.c_size_t(4 * 2 * 12), ctypes.c_size_t(4 * 2 * 4)) == 0
     assert orn.lib().ornith_kmatrix_check(ctypes.byref(s), ctypes.c_size_t(4 * 2 * 128), ctypes.c_size_t(4 * 2 * 16), ctypes.c_size_t(4 * 2 * 4)) == 1
+
+
+def test_host_random_functions_match_known_answers():
+    """The key sequence is host code inside the library: threefry2x32-20 against the
+    published Random123 vectors (through bits(), whose first word of a 2-word request is
+    x of hash(key, (0, 1))), and the split against the oracle."""
+    import importlib
+    import util
+    orn = importlib.import_module("ornith-rs_amd")
+    assert orn.random_key(0x0123456789ABCDEF) == [0x01234567, 0x89ABCDEF]
+    for key in ([0, 0], [0xFFFFFFFF, 0xFFFFFFFF], [0x13198A2E, 0x03707344]):
+        for n in (1, 2, 3, 4, 9):
+            assert np.array_equal(orn.random_bits(key, n), util.orc_random_bits(key, n))
+        st, sub = orn.random_split(key)
+        assert (st, sub) == tuple(util.orc_key_next(key))
+    # a direct known answer: counter (0, 1) under key (0, 0) is not in the KAT list, but n = 2 with
+    # key = KAT key and the oracle (itself pinned on the three KATs) covers the layout; and here
+    # the one KAT that bits() can reach directly: n = 1 hashes (0, 0)
+    assert orn.random_bits([0, 0], 1)[0] == 0x6B200159

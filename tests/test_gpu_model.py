@@ -192,6 +192,45 @@ def test_stop_callback_and_errors(orn, ctx, tiny):
         orn.generate_step_mtp(model, head, None, caches, prompt, 3, 5)
     with pytest.raises(orn.OrnithError, match="exceed cache capacity"):
         model.forward(caches, np.zeros(16, np.uint32)); model.forward(caches, np.zeros(16, np.uint32)); model.forward(caches, np.zeros(1, np.uint32))
-    with pytest.raises(orn.OrnithError, match="greedy"):
-        orn.generate_step(model, caches, prompt, 2, sampler=orn.Sampler(1, 0.8, 0.95, 0, 1))
+    with pytest.raises(orn.OrnithError, match="sampler kind"):
+        orn.generate_step(model, caches, prompt, 2, sampler=orn.Sampler(7, 0.8, 0.95, 0, 1))
+    with pytest.raises(orn.OrnithError, match="temp"):
+        orn.generate_step(model, caches, prompt, 2, sampler=orn.Sampler(1, 0.0, 0.95, 0, 1))
     head.close(); caches.close()
+
+
+@pytest.mark.parametrize("temp,top_p,top_k", [(0.8, 0.95, 0), (0.6, 0.95, 20), (1.0, 1.0, 0)])
+def test_sampled_loops_match_oracle(orn, ctx, tiny_small_vocab, temp, top_p, top_k):
+    """Sampled decode (temperature / top-p / top-k, seeded threefry keys): the AR loop and
+    the depth-1..3 MTP loop draw the same tokens, accept the same drafts and leave the caches
+    at the same length as the oracle. Rows are sampled one by one, only as far as the accept
+    loop asks, so the key sequence is part of what is compared."""
+    s, ws, model = tiny_small_vocab
+    V = s.cfg["vocab_size"]
+    rng = np.random.default_rng(3)
+    prompt = rng.integers(0, V, 9).astype(np.uint32)
+    n_tok, cap = 24, 9 + 24 + 8
+    smp = orn.Sampler(1, temp, top_p, top_k, 4242)
+    caches = model.make_cache(cap, 4)
+    head = orn.MtpHead(model, ws, cap)
+    orc = synth.OracleRun(s, cap)
+    try:
+        orc.set_sampler(1, temp, top_p, top_k, 4242)
+        got = orn.generate_step(model, caches, prompt, n_tok, sampler=smp, prefill_step=4)
+        want = orc.generate(prompt, n_tok, prefill_step=4)
+        assert got == want
+        greedy = orn.generate_step(model, model.make_cache(cap, 4), prompt, n_tok, prefill_step=4)
+        assert got != greedy, "the sampled run never left the greedy path: nothing was tested"
+        for depth in (1, 3):
+            caches.reset()
+            toks, st = orn.generate_step_mtp(model, head, None, caches, prompt, depth, n_tok, sampler=smp,
+                                             prefill_step=4, policy=orn.HISTORY_COMMITTED)
+            o2 = synth.OracleRun(s, cap)
+            otoks, ost = o2.mtp_generate(prompt, depth, n_tok, policy=1, prefill_step=4)
+            o2.close()
+            assert toks == otoks, depth
+            assert (st.cycles, st.drafted, st.accepted) == (ost.cycles, ost.drafted, ost.accepted)
+            assert caches.offset == 9 + n_tok
+    finally:
+        orc.set_sampler(0)
+        orc.close(); head.close(); caches.close()

@@ -350,3 +350,82 @@ def orc_sdpa(q_rot, k_cache, v_cache, gate, offset, scale):
     oracle().orc_sdpa_decode_gated(p(q_rot), p(k_cache), p(v_cache), p(gate), T, Hq, Hkv, hd, offset, cap,
                                    C.c_float(scale), p(out))
     return out
+
+
+# ---- sampler oracle wrappers -----------------------------------------------------------
+def orc_threefry(key, count):
+    k = (C.c_uint32 * 2)(*key); c = (C.c_uint32 * 2)(*count); o = (C.c_uint32 * 2)()
+    oracle().orc_threefry2x32(k, c, o)
+    return o[0], o[1]
+
+
+def orc_random_bits(key, n):
+    k = (C.c_uint32 * 2)(*key); out = np.empty(n, np.uint32)
+    oracle().orc_random_bits(k, n, p(out))
+    return out
+
+
+def orc_key_next(state):
+    st = (C.c_uint32 * 2)(*state); sub = (C.c_uint32 * 2)()
+    oracle().orc_key_next(st, sub)
+    return [st[0], st[1]], [sub[0], sub[1]]
+
+
+def orc_uniform_scaled(bits, total):
+    f = oracle().orc_uniform_scaled
+    f.restype = C.c_float
+    return np.float32(f(C.c_uint32(bits), C.c_float(total)))
+
+
+def orc_argsort_bf16(x, negate=False):
+    x = np.ascontiguousarray(x, np.uint16); idx = np.empty(x.size, np.uint32)
+    oracle().orc_argsort_bf16(p(x), x.size, int(negate), p(idx))
+    return idx
+
+
+def orc_cumsum_bf16(x):
+    x = np.ascontiguousarray(x, np.uint16); out = np.empty(x.size, np.uint16)
+    oracle().orc_cumsum_bf16(p(x), x.size, p(out))
+    return out
+
+
+def orc_cumsum_f32(x):
+    x = np.ascontiguousarray(x, np.float32); out = np.empty(x.size, np.float32)
+    f = oracle().orc_cumsum_f32
+    f.restype = C.c_float
+    total = f(p(x), x.size, p(out))
+    return out, np.float32(total)
+
+
+def orc_logprobs_row(logits):
+    logits = np.ascontiguousarray(logits, np.uint16); out = np.empty(logits.size, np.uint16)
+    oracle().orc_logprobs_row(p(logits), logits.size, p(out))
+    return out
+
+
+def orc_apply_top_p(lp, top_p):
+    lp = np.ascontiguousarray(lp, np.uint16); out = np.empty(lp.size, np.uint16)
+    oracle().orc_apply_top_p(p(lp), lp.size, C.c_double(top_p), p(out))
+    return out
+
+
+def orc_apply_top_k(lp, k):
+    lp = np.ascontiguousarray(lp, np.uint16); out = np.empty(lp.size, np.uint16)
+    oracle().orc_apply_top_k(p(lp), lp.size, k, p(out))
+    return out
+
+
+def orc_categorical(lp, temp, bits):
+    lp = np.ascontiguousarray(lp, np.uint16)
+    f = oracle().orc_categorical
+    f.restype = C.c_uint32
+    return int(f(p(lp), lp.size, C.c_double(temp), C.c_uint32(bits)))
+
+
+def orc_top_sample(logits, temp, top_p, top_k, key_state):
+    logits = np.ascontiguousarray(logits, np.uint16)
+    st = (C.c_uint32 * 2)(*key_state)
+    f = oracle().orc_top_sample
+    f.restype = C.c_uint32
+    tok = int(f(p(logits), logits.size, C.c_double(temp), C.c_double(top_p), top_k, st))
+    return tok, [st[0], st[1]]
