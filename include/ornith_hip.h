@@ -117,6 +117,26 @@ ORNITH_API int ornith_kq_gather_qmv(ornith_ctx* ctx, const ornith_kmatrix* w, co
                          int x_rows, const uint32_t* d_lhs, const uint32_t* d_rhs, int rows,
                          void* d_y, int y_dtype);
 
+/* kquant::matmul / qmm_t (src/ops/kquant.rs:783-905; kernels/kquant_mm.h): the prefill-width
+ * GEMM y[M,O] = x[M,K] . W^T, bf16 in and out, on the matrix cores: weight tiles are
+ * dequantized to bf16 on the way into LDS (HBM traffic stays at the quantized size), fp32
+ * accumulate. Agrees with kq_qmv to bf16 rounding of the weights, not bit for bit (prefill
+ * is outside the reference's exact window as well, src/ops/invariant.rs:140-168). */
+ORNITH_API int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int M,
+                                void* d_y);
+/* kquant::gather_matmul / gather_qmm_t (src/ops/kquant.rs:907-1027): the same GEMM over an
+ * expert-stacked matrix, rows grouped by routed expert. d_inds[p] is the expert of pair
+ * p = token * top_k + slot. is_up != 0: pair p reads row p / top_k of x (the token) and
+ * writes row p of y (gate / up projections); is_up == 0: reads row p of x and writes row p
+ * (down projection). d_plan: ornith_kq_gather_plan_bytes(pairs, E) bytes of device memory
+ * holding the expert-sorted pair list; rebuild_plan != 0 recomputes it from d_inds (one
+ * launch), 0 reuses what an earlier call with the same inds left there (gate, up and down
+ * of one MoE block share one plan). */
+ORNITH_API size_t ornith_kq_gather_plan_bytes(int pairs, int E);
+ORNITH_API int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x,
+                                       const uint32_t* d_inds, int pairs, int top_k, int is_up,
+                                       void* d_plan, int rebuild_plan, void* d_y);
+
 /* ---- Linear: ops::linear::Linear (src/ops/linear.rs:23-28), one polymorphic
  * projection. Activations in and out are bf16. -------------------------------- */
 #define ORNITH_LIN_KQUANT 0  /* Linear::K(KMatrix) */

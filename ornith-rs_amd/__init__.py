@@ -138,6 +138,9 @@ class Ctx:
         arr = np.ascontiguousarray(arr)
         return DeviceBuffer(self, max(arr.nbytes, 1)).upload(arr)
 
+    def memset(self, dst, byte, nbytes):
+        _check(lib().ornith_memset(self.h, dst.ptr, byte, C.c_size_t(nbytes)), "memset")
+
     def copy(self, dst, src, nbytes):
         _check(lib().ornith_copy(self.h, dst.ptr, src.ptr, nbytes), "copy")
 

@@ -1,0 +1,371 @@
+// Q4_K / Q6_K tiled GEMM on the matrix cores, for prefill widths.
+//
+// Replaces kquant::{qmm_t, gather_qmm_t, matmul, gather_matmul}
+// (/root/reference/src/ops/kquant.rs:783-1027; kernels/kquant_mm.h): Y[M,O] = X[M,K] . W^T
+// with the weight tile dequantized to bf16 on the way into LDS and fp32 accumulation, and
+// the expert-gathered form where each tile's rows belong to one routed expert.
+//
+// This is the one GEMM-shaped piece of the path (81 % of a prefill chunk in the
+// reference, /root/reference/src/bin/arithmetic.rs:4-7), so it runs on MFMA:
+// v_mfma_f32_32x32x16_bf16, a workgroup tile of BM x 128 outputs over K slabs of 128.
+//   * A (activations, bf16) goes global -> LDS as is.
+//   * B (weights) is read as k-quant codes (the 144 / 210 bytes per 256 weights that HBM
+//     holds), dequantized with the arithmetic of kquant::dequantize (d*sc*q - dmin*m,
+//     resp. d*sc*q) and rounded to bf16 into LDS: HBM traffic stays at the quantized size.
+//   * LDS rows are padded by 8 elements so the 16-byte fragment reads of 32 consecutive
+//     rows spread over the banks.
+//   * Four wavefronts: 2 x 2 of 64 x 64 outputs each for BM = 128, 1 x 4 of 64 x 32 for
+//     BM = 64 (used when an expert's share of the tokens is small).
+//
+// Prefill is exempt from the "row r of a batch == row r alone" rule in the reference too
+// (src/ops/invariant.rs:140-168): results agree with the mat-vec path to bf16 rounding of
+// the weights and the order of the fp32 sums, not bit for bit.
+#include "dmath.h"
+#include "rt.h"
+
+namespace {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+constexpr int BN = 128, BK = 128, LDK = BK + 8;
+
+struct MmArgs {
+  const uint8_t* qs;
+  const uint8_t* scales;
+  const uint16_t* dm;
+  const bf16_t* x;   // [x_rows, K]
+  bf16_t* y;         // [y_rows, O]
+  int M, O, K;
+  // gathered form: tiles over (expert, row range) of an expert-sorted pair list
+  const uint32_t* pair;        // [pairs] expert-sorted pair ids (row of y; row of x is pair / up_div)
+  int up_div;                  // top_k for the gate / up projections (x row = token), 1 for down
+  const uint32_t* tile_expert; // [tiles]
+  const uint32_t* tile_start;  // [tiles] first pair
+  const uint32_t* tile_count;  // [tiles] pairs in the tile (<= BM)
+  const uint32_t* n_tiles;     // device scalar
+};
+
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)dm_f2bf(a) | ((uint32_t)dm_f2bf(b) << 16);
+}
+
+// 64 weights of row `row` (already offset by the expert), 64-group `grp` of super-block
+// `ib`, as bf16 into dst[0..64)
+__device__ __forceinline__ void dequant64_q4k(const MmArgs& a, int64_t row, int nb, int ib, int grp,
+                                              bf16_t* dst) {
+  const int64_t blk = row * nb + ib;
+  const uint8_t* sc = a.scales + blk * 12;
+  const float d = dm_h2f(a.dm[blk * 2]), dmin = dm_h2f(a.dm[blk * 2 + 1]);
+  float dd[2], mm[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int j = 2 * grp + k;
+    uint32_t s, m;
+    if (j < 4) {
+      s = sc[j] & 63;
+      m = sc[j + 4] & 63;
+    } else {
+      s = (sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4);
+      m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4);
+    }
+    dd[k] = d * (float)s;
+    mm[k] = dmin * (float)m;
+  }
+  const uint4* q = reinterpret_cast<const uint4*>(a.qs + blk * 128 + grp * 32);
+  uint32_t* out = reinterpret_cast<uint32_t*>(dst);
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint4 v = q[h];
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t b = w[i];
+      const float l0 = dd[0] * (float)(b & 0xF) - mm[0], l1 = dd[0] * (float)((b >> 8) & 0xF) - mm[0];
+      const float l2 = dd[0] * (float)((b >> 16) & 0xF) - mm[0], l3 = dd[0] * (float)((b >> 24) & 0xF) - mm[0];
+      const float h0 = dd[1] * (float)((b >> 4) & 0xF) - mm[1], h1 = dd[1] * (float)((b >> 12) & 0xF) - mm[1];
+      const float h2 = dd[1] * (float)((b >> 20) & 0xF) - mm[1], h3 = dd[1] * (float)(b >> 28) - mm[1];
+      const int e = 16 * h + 4 * i;  // element index within the low / high run of 32
+      out[(e >> 1)] = pack2(l0, l1);
+      out[(e >> 1) + 1] = pack2(l2, l3);
+      out[16 + (e >> 1)] = pack2(h0, h1);
+      out[16 + (e >> 1) + 1] = pack2(h2, h3);
+    }
+  }
+}
+
+// positions l in [16*j, 16*j + 16) of the 128-half `hh` of super-block `ib`: the four
+// weights l, l+32, l+64, l+96 each, as bf16 into dst[0..128) (dst = start of the half)
+__device__ __forceinline__ void dequant_q6k_part(const MmArgs& a, int64_t row, int nb, int ib, int hh,
+                                                 int j, bf16_t* dst) {
+  const int64_t blk = row * nb + ib;
+  const float d = dm_h2f(a.dm[blk]);
+  const uint8_t* base = a.qs + blk * 192;
+  const uint4 qa = *reinterpret_cast<const uint4*>(base + 64 * hh + 16 * j);
+  const uint4 qb = *reinterpret_cast<const uint4*>(base + 64 * hh + 32 + 16 * j);
+  const uint4 qhv = *reinterpret_cast<const uint4*>(base + 128 + 32 * hh + 16 * j);
+  const int8_t* sc = reinterpret_cast<const int8_t*>(a.scales + blk * 16) + 8 * hh;
+  const float s1 = d * (float)sc[j], s2 = d * (float)sc[j + 2], s3 = d * (float)sc[j + 4],
+              s4 = d * (float)sc[j + 6];
+  const uint32_t la[4] = {qa.x, qa.y, qa.z, qa.w}, lb[4] = {qb.x, qb.y, qb.z, qb.w},
+                 hv[4] = {qhv.x, qhv.y, qhv.z, qhv.w};
+  uint32_t* out = reinterpret_cast<uint32_t*>(dst);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float w1[4], w2[4], w3[4], w4[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const uint32_t a8 = (la[i] >> (8 * b)) & 0xFF, b8 = (lb[i] >> (8 * b)) & 0xFF,
+                     h8 = (hv[i] >> (8 * b)) & 0xFF;
+      w1[b] = s1 * (float)((int)((a8 & 0xF) | ((h8 & 3) << 4)) - 32);
+      w2[b] = s2 * (float)((int)((b8 & 0xF) | (((h8 >> 2) & 3) << 4)) - 32);
+      w3[b] = s3 * (float)((int)((a8 >> 4) | (((h8 >> 4) & 3) << 4)) - 32);
+      w4[b] = s4 * (float)((int)((b8 >> 4) | ((h8 >> 6) << 4)) - 32);
+    }
+    const int e = (16 * j + 4 * i) >> 1;
+    out[e] = pack2(w1[0], w1[1]);
+    out[e + 1] = pack2(w1[2], w1[3]);
+    out[16 + e] = pack2(w2[0], w2[1]);
+    out[16 + e + 1] = pack2(w2[2], w2[3]);
+    out[32 + e] = pack2(w3[0], w3[1]);
+    out[32 + e + 1] = pack2(w3[2], w3[3]);
+    out[48 + e] = pack2(w4[0], w4[1]);
+    out[48 + e + 1] = pack2(w4[2], w4[3]);
+  }
+}
+
+template <int KIND, int BM, bool GATHER>
+__global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
+  constexpr int WN = BM == 128 ? 2 : 4;        // wavefronts along n
+  constexpr int WTN = BN / WN;                 // wave tile width: 64 or 32
+  constexpr int TM = 2, TN = WTN / 32;         // 32x32 MFMA tiles per wavefront
+  __shared__ __attribute__((aligned(16))) bf16_t As[BM][LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[BN][LDK];
+  __shared__ uint32_t s_src[BM], s_dst[BM];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = BM == 128 ? (wave >> 1) : 0, wn = BM == 128 ? (wave & 1) : wave;
+  const int n0 = blockIdx.x * BN;
+  const int nb = a.K >> 8;
+
+  int rows_here, m0 = 0;
+  int64_t wrow0 = 0;  // first weight row of this tile's matrix
+  if constexpr (GATHER) {
+    if (blockIdx.y >= *a.n_tiles) return;
+    const uint32_t e = a.tile_expert[blockIdx.y], st = a.tile_start[blockIdx.y];
+    rows_here = (int)a.tile_count[blockIdx.y];
+    wrow0 = (int64_t)e * a.O;
+    for (int r = tid; r < BM; r += 256) {
+      const uint32_t p = r < rows_here ? a.pair[st + r] : 0u;
+      s_src[r] = p / (uint32_t)a.up_div;
+      s_dst[r] = p;
+    }
+    __syncthreads();
+  } else {
+    m0 = blockIdx.y * BM;
+    rows_here = min(BM, a.M - m0);
+  }
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  for (int k0 = 0; k0 < a.K; k0 += BK) {
+    // ---- A slab: BM rows x 128 bf16
+#pragma unroll
+    for (int i = 0; i < BM * 16 / 256; ++i) {
+      const int idx = tid + 256 * i, r = idx >> 4, c8 = idx & 15;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (r < rows_here) {
+        const int64_t src = GATHER ? (int64_t)s_src[r] : (int64_t)(m0 + r);
+        v = *reinterpret_cast<const uint4*>(a.x + src * a.K + k0 + 8 * c8);
+      }
+      *reinterpret_cast<uint4*>(&As[r][8 * c8]) = v;
+    }
+    // ---- B slab: 128 weight rows x 128 weights, dequantized
+    {
+      const int r = tid >> 1, part = tid & 1;
+      const int o = n0 + r;
+      const int64_t row = wrow0 + (o < a.O ? o : a.O - 1);
+      const int ib = k0 >> 8;
+      if constexpr (KIND == ORNITH_Q4K)
+        dequant64_q4k(a, row, nb, ib, ((k0 & 255) >> 6) + part, &Bs[r][64 * part]);
+      else
+        dequant_q6k_part(a, row, nb, ib, (k0 & 255) >> 7, part, &Bs[r][0]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      const int kc = kk * 16 + 8 * (lane >> 5);
+      bf16x8_t af[TM], bfr[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        af[i] = *reinterpret_cast<const bf16x8_t*>(&As[wm * 64 + i * 32 + (lane & 31)][kc]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        bfr[j] = *reinterpret_cast<const bf16x8_t*>(&Bs[wn * WTN + j * 32 + (lane & 31)][kc]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: D[row = 8*b + 4*(lane/32) + r][col = lane%32] = acc[4*b + r]
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int o = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        if (r < rows_here && o < a.O) {
+          const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
+          a.y[dst * a.O + o] = dm_f2bf(acc[i][j][e]);
+        }
+      }
+    }
+}
+
+// BM == 64 has two 32-row MFMA tiles per wavefront as well (TM = 2), one wavefront column
+static_assert(BN == 128 && BK == 128, "tile constants are baked into the index arithmetic");
+
+// ---- expert-sorted pair list for the gathered form -----------------------------------
+// inds [pairs] (expert of pair p; pair p = token * k + slot). One workgroup:
+// counts per expert, exclusive scan, stable scatter, then the tile list.
+__global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* inds, int pairs, int E,
+                                                              int bm, uint32_t* pair, uint32_t* tile_expert,
+                                                              uint32_t* tile_start, uint32_t* tile_count,
+                                                              uint32_t* n_tiles) {
+  __shared__ uint32_t cnt[1024], start[1025], tiles_before[1025];
+  const int tid = threadIdx.x;
+  if (tid < 1024) cnt[tid] = 0;
+  __syncthreads();
+  for (int p = tid; p < pairs; p += 1024) atomicAdd(&cnt[min(inds[p], (uint32_t)(E - 1))], 1u);
+  __syncthreads();
+  if (tid == 0) {
+    uint32_t s = 0, t = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = s;
+      tiles_before[e] = t;
+      s += cnt[e];
+      t += (cnt[e] + bm - 1) / bm;
+    }
+    start[E] = s;
+    tiles_before[E] = t;
+    *n_tiles = t;
+  }
+  __syncthreads();
+  // stable placement: expert e's pairs in ascending pair order (one thread per expert walks
+  // the list; pairs <= 2048 * 8 and this runs once per layer per chunk)
+  for (int e = tid; e < E; e += 1024) {
+    uint32_t w = start[e];
+    if (cnt[e]) {
+      for (int p = 0; p < pairs; ++p)
+        if (min(inds[p], (uint32_t)(E - 1)) == (uint32_t)e) pair[w++] = (uint32_t)p;
+    }
+    const uint32_t nt = (cnt[e] + bm - 1) / bm;
+    for (uint32_t t = 0; t < nt; ++t) {
+      tile_expert[tiles_before[e] + t] = e;
+      tile_start[tiles_before[e] + t] = start[e] + t * bm;
+      tile_count[tiles_before[e] + t] = min((uint32_t)bm, cnt[e] - t * bm);
+    }
+  }
+}
+
+int check(const ornith_kmatrix* w, const char* who) {
+  ORN_REQUIRE(w && (w->kind == ORNITH_Q4K || w->kind == ORNITH_Q6K), "%s: bad matrix", who);
+  ORN_REQUIRE(w->K >= 256 && w->K % 256 == 0 && w->O >= 1 && w->E >= 1, "%s: bad dims E=%d O=%d K=%d", who,
+              w->E, w->O, w->K);
+  ORN_REQUIRE(w->d_qs && w->d_scales && w->d_dm, "%s: null tensor", who);
+  return ORNITH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int M, void* d_y) {
+  ORN_REQUIRE(ctx && d_x && d_y, "kq_matmul: null argument");
+  int rc = check(w, "kq_matmul");
+  if (rc) return rc;
+  ORN_REQUIRE(w->E == 1, "kq_matmul: stacked matrix (use kq_gather_matmul)");
+  ORN_REQUIRE(M >= 1, "kq_matmul: M=%d", M);
+  ORN_REQUIRE(((uintptr_t)d_x & 15) == 0, "kq_matmul: x must be 16-byte aligned");
+  MmArgs a{};
+  a.qs = (const uint8_t*)w->d_qs;
+  a.scales = (const uint8_t*)w->d_scales;
+  a.dm = (const uint16_t*)w->d_dm;
+  a.x = (const bf16_t*)d_x;
+  a.y = (bf16_t*)d_y;
+  a.M = M;
+  a.O = w->O;
+  a.K = w->K;
+  const dim3 grid((w->O + BN - 1) / BN, (M + 127) / 128);
+  if (w->kind == ORNITH_Q4K)
+    hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 128, false>), grid, dim3(256), 0, ctx->stream, a);
+  else
+    hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q6K, 128, false>), grid, dim3(256), 0, ctx->stream, a);
+  ORN_LAUNCH_CHECK("kq_mm_kernel");
+  return ORNITH_OK;
+}
+
+// gather plan: expert-sorted pairs and the tile list, in caller-provided device memory
+// (ornith_kq_gather_plan_bytes(pairs, E) bytes)
+size_t ornith_kq_gather_plan_bytes(int pairs, int E) {
+  const size_t tiles = (size_t)pairs / 64 + (size_t)E + 1;
+  return ((size_t)pairs + tiles * 3 + 1) * 4 + 5 * 256;
+}
+
+int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x,
+                            const uint32_t* d_inds, int pairs, int top_k, int is_up, void* d_plan,
+                            int rebuild_plan, void* d_y) {
+  ORN_REQUIRE(ctx && d_x && d_inds && d_plan && d_y, "kq_gather_matmul: null argument");
+  int rc = check(w, "kq_gather_matmul");
+  if (rc) return rc;
+  ORN_REQUIRE(pairs >= 1 && top_k >= 1 && pairs % top_k == 0 && w->E <= 1024,
+              "kq_gather_matmul: pairs=%d top_k=%d E=%d", pairs, top_k, w->E);
+  const size_t tiles_max = (size_t)pairs / 64 + (size_t)w->E + 1;
+  ScratchCursor pc(d_plan);
+  uint32_t* pair = pc.take<uint32_t>(pairs);
+  uint32_t* te = pc.take<uint32_t>(tiles_max);
+  uint32_t* ts = pc.take<uint32_t>(tiles_max);
+  uint32_t* tc = pc.take<uint32_t>(tiles_max);
+  uint32_t* nt = pc.take<uint32_t>(1);
+  if (rebuild_plan) {
+    hipLaunchKernelGGL(moe_sort_pairs_kernel, dim3(1), dim3(1024), 0, ctx->stream, d_inds, pairs, w->E,
+                       64, pair, te, ts, tc, nt);
+    ORN_LAUNCH_CHECK("moe_sort_pairs_kernel");
+  }
+  MmArgs a{};
+  a.qs = (const uint8_t*)w->d_qs;
+  a.scales = (const uint8_t*)w->d_scales;
+  a.dm = (const uint16_t*)w->d_dm;
+  a.x = (const bf16_t*)d_x;
+  a.y = (bf16_t*)d_y;
+  a.M = pairs;
+  a.O = w->O;
+  a.K = w->K;
+  a.pair = pair;
+  a.up_div = is_up ? top_k : 1;
+  a.tile_expert = te;
+  a.tile_start = ts;
+  a.tile_count = tc;
+  a.n_tiles = nt;
+  const dim3 grid((w->O + BN - 1) / BN, (unsigned)tiles_max);
+  if (w->kind == ORNITH_Q4K)
+    hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 64, true>), grid, dim3(256), 0, ctx->stream, a);
+  else
+    hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q6K, 64, true>), grid, dim3(256), 0, ctx->stream, a);
+  ORN_LAUNCH_CHECK("kq_mm_kernel<gather>");
+  return ORNITH_OK;
+}
+
+}  // extern "C"

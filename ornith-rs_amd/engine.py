@@ -357,3 +357,19 @@ class TopSampler:
             lib().ornith_top_sampler_destroy(self.h)
             self.h = None
             self._tok.free()
+
+
+# ---- prefill-width k-quant GEMM (src/ops/kquant.rs:783-1027) --------------------------------
+def kq_matmul(ctx, w, x, M, y):
+    _check(lib().ornith_kq_matmul(ctx.h, C.byref(w.s), x.ptr, M, y.ptr), "kq_matmul")
+
+
+def kq_gather_plan_bytes(pairs, E):
+    f = lib().ornith_kq_gather_plan_bytes
+    f.restype = C.c_size_t
+    return int(f(pairs, E))
+
+
+def kq_gather_matmul(ctx, w, x, inds, pairs, top_k, is_up, plan, rebuild, y):
+    _check(lib().ornith_kq_gather_matmul(ctx.h, C.byref(w.s), x.ptr, inds.ptr, pairs, top_k, int(is_up),
+                                         plan.ptr, int(rebuild), y.ptr), "kq_gather_matmul")
