@@ -69,6 +69,10 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *   "fuse_proj" (ORNITH_FUSE_PROJ, default 1): projections sharing an input in one launch
  *   "moe_up_iters" (ORNITH_MOE_UP_ITERS, default 0 = chosen by shape; 2 or 4): output
  *               rows per wavefront of the fused gate+up expert kernel, a tuning knob
+ *   "gemm_rows" (ORNITH_GEMM_ROWS, default 32; 0 = never): activation rows from which the
+ *               k-quant projections and the MoE experts run as matrix-core GEMMs instead of
+ *               exact mat-vecs. The one switch that changes results (to bf16 rounding of the
+ *               weights): prefill is outside the exact window in the reference as well.
  *   "kq_iters"  (ORNITH_KQ_ITERS, default 0 = chosen by shape; 1..8): output rows each
  *               wavefront of the k-quant mat-vec walks, a tuning knob */
 ORNITH_API int ornith_set_option(const char* name, int value);
@@ -336,6 +340,11 @@ typedef struct ornith_caches ornith_caches;
 ORNITH_API int ornith_model_load(ornith_ctx* ctx, const ornith_weights* ws,
                                  const ornith_text_config* cfg, ornith_model** out);
 ORNITH_API int ornith_model_destroy(ornith_model* m);
+/* Rows one forward call may carry (default 16: decode, verify, short prompt chunks). The
+ * reference prefills in chunks of prefill_step_size (2048, src/generate.rs:90-136); raise
+ * this before creating caches to prefill in chunks that wide. From 32 rows up the
+ * k-quant projections and the MoE experts run as matrix-core GEMMs. */
+ORNITH_API int ornith_model_set_max_rows(ornith_model* m, int rows);
 /* The MoE block of decoder layer `layer` as the model holds it (pointers into the weight
  * store, valid while the model lives): lets a caller run or time ornith_moe_block /
  * ornith_moe_experts on the resident weights (the reference reaches them as

@@ -120,6 +120,9 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
   switch (w->mode) {
     case ORNITH_LIN_KQUANT:
       ORN_REQUIRE(w->km.O == w->O && w->km.K == w->K, "linear_matmul: k-quant dims disagree");
+      // kquant::matmul (src/ops/kquant.rs:783-800): rows within the exact window go through
+      // the mat-vec (each row as if alone), prefill widths through the tiled GEMM
+      if (M >= kPrefillRows) return ornith_kq_matmul(ctx, &w->km, d_x, M, d_y);
       return ornith_kq_qmv(ctx, &w->km, d_x, ORNITH_BF16, M, d_y, ORNITH_BF16);
     case ORNITH_LIN_AFFINE8:
       ORN_REQUIRE(w->d_w && w->d_scales && w->d_biases, "linear_matmul: affine tensor missing");
@@ -147,7 +150,7 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
 int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, int n,
                                const void* d_x, int M, void* const* d_ys) {
   ORN_REQUIRE(ctx && ws && d_x && d_ys && n >= 1, "linear_matmul_multi: bad argument");
-  bool fuse = ornith_option_fuse_proj() && n >= 2 && n <= 4;
+  bool fuse = ornith_option_fuse_proj() && n >= 2 && n <= 4 && M < kPrefillRows;
   for (int i = 0; i < n; ++i) {
     ORN_REQUIRE(ws[i] && d_ys[i], "linear_matmul_multi: null entry %d", i);
     fuse = fuse && ws[i]->mode == ws[0]->mode && ws[i]->K == ws[0]->K;

@@ -96,7 +96,7 @@ static size_t step_bytes(const ornith_model* m, int R) {
   const size_t Hv = c.linear_num_value_heads;
   const size_t aq = (size_t)c.num_attention_heads * c.head_dim, akv = (size_t)c.num_key_value_heads * c.head_dim;
   size_t per_row = 2 * (6 * H + D + 3 * Vd + 2 * Kd + 3 * Hv + 2 * aq + 2 * akv + 2 * aq) + 4 * Hv;
-  return per_row * R + 64 * 256 + (size_t)R * c.vocab_size * 2 + (size_t)R * 8;
+  return per_row * R + 64 * 256 + (size_t)(R < kMaxRows ? R : kMaxRows) * c.vocab_size * 2 + (size_t)R * 8;
 }
 
 struct StepBufs {
@@ -137,7 +137,7 @@ static StepBufs carve(const ornith_model* m, void* base, int R) {
   s.vx = sc.take<char>(2 * akv * R);
   s.q_rot = sc.take<char>(2 * aq * R);
   s.att = sc.take<char>(2 * aq * R);
-  s.logits = sc.take<char>((size_t)R * c.vocab_size * 2);
+  s.logits = sc.take<char>((size_t)(R < kMaxRows ? R : kMaxRows) * c.vocab_size * 2);
   s.toks = sc.take<uint32_t>(R);
   return s;
 }
@@ -308,6 +308,21 @@ int ornith_model_moe_weights(const ornith_model* m, int layer, ornith_moe_weight
   return ORNITH_OK;
 }
 
+int ornith_model_set_max_rows(ornith_model* m, int rows) {
+  ORN_REQUIRE(m, "model_set_max_rows: null model");
+  ORN_REQUIRE(rows >= kMaxRows && rows <= 4096, "model_set_max_rows: rows=%d (%d..4096)", rows, kMaxRows);
+  if (rows == m->max_rows) return ORNITH_OK;
+  TRY(ornith_sync(m->ctx));
+  void* buf = nullptr;
+  const size_t bytes = step_bytes(m, rows);
+  TRY(ornith_alloc(m->ctx, bytes, &buf));
+  ornith_free(m->ctx, m->ws_buf);
+  m->ws_buf = buf;
+  m->ws_bytes = bytes;
+  m->max_rows = rows;
+  return ORNITH_OK;
+}
+
 int ornith_model_destroy(ornith_model* m) {
   if (!m) return ORNITH_OK;
   ornith_free(m->ctx, m->ws_buf);
@@ -319,9 +334,9 @@ int ornith_model_destroy(ornith_model* m) {
 
 int ornith_caches_create(ornith_model* m, int capacity, int max_window, ornith_caches** out) {
   ORN_REQUIRE(m && out, "caches_create: null argument");
-  ORN_REQUIRE(capacity >= 1 && max_window >= 1 && max_window <= m->max_rows,
+  ORN_REQUIRE(capacity >= 1 && max_window >= 1 && max_window <= kMaxRows,
               "caches_create: capacity=%d max_window=%d (window at most %d)", capacity, max_window,
-              m->max_rows);
+              kMaxRows);
   const auto& c = m->cfg;
   ornith_caches* cc = new ornith_caches();
   cc->m = m;
@@ -397,6 +412,9 @@ int ornith_model_forward(ornith_model* m, ornith_caches* cc, const uint32_t* d_t
   ORN_REQUIRE(m && cc && d_tokens && d_hidden_out, "model_forward: null argument");
   ORN_REQUIRE(cc->m == m, "model_forward: caches belong to another model");
   ORN_REQUIRE(T >= 1 && T <= m->max_rows, "model_forward: T=%d (1..%d rows a call)", T, m->max_rows);
+  ORN_REQUIRE(m->cfg.linear_conv_kernel_dim - 1 + T <= cc->conv_rows,
+              "model_forward: %d rows, but these caches were created for %d rows a call", T,
+              cc->conv_rows - (m->cfg.linear_conv_kernel_dim - 1));
   ORN_REQUIRE(!capture || T <= cc->max_window, "model_forward: capture of %d rows, window is %d", T,
               cc->max_window);
   ORN_REQUIRE(cc->offset + T <= cc->capacity, "model_forward: %d + %d rows exceed cache capacity %d",

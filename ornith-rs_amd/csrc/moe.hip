@@ -93,6 +93,53 @@ int launch_router(ornith_ctx* ctx, const bf16_t* gates, int T, int E, int k, uin
   return ORNITH_OK;
 }
 
+// Prefill widths: the same block with every projection as a matrix-core GEMM and the routed
+// experts as three expert-grouped GEMMs over one sorted pair list
+// (/root/reference/src/ops/moe.rs:662-741 at T above the exact window; gather_qmm_t).
+int moe_block_prefill(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, void* d_out) {
+  const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k, SI = w->sh_gate.O;
+  const int pairs = T * k;
+  const size_t plan_bytes = ornith_kq_gather_plan_bytes(pairs, E);
+  const size_t need = 2 * ((size_t)T * E + (size_t)T * SI * 3 + (size_t)T * H + T + (size_t)pairs * (3 * I + H) +
+                           (size_t)pairs) + 4 * (size_t)pairs + plan_bytes + 24 * 256;
+  void* base = nullptr;
+  int rc = ornith_scratch(ctx, need, &base);
+  if (rc) return rc;
+  ScratchCursor sc(base);
+  bf16_t* gates = sc.take<bf16_t>((size_t)T * E);
+  uint32_t* inds = sc.take<uint32_t>(pairs);
+  bf16_t* scores = sc.take<bf16_t>(pairs);
+  bf16_t* sg = sc.take<bf16_t>((size_t)T * SI);
+  bf16_t* su = sc.take<bf16_t>((size_t)T * SI);
+  bf16_t* sact = sc.take<bf16_t>((size_t)T * SI);
+  bf16_t* sy = sc.take<bf16_t>((size_t)T * H);
+  bf16_t* eg = sc.take<bf16_t>(T);
+  bf16_t* xg = sc.take<bf16_t>((size_t)pairs * I);
+  bf16_t* xu = sc.take<bf16_t>((size_t)pairs * I);
+  bf16_t* act = sc.take<bf16_t>((size_t)pairs * I);
+  bf16_t* y = sc.take<bf16_t>((size_t)pairs * H);
+  void* plan = sc.take<char>(plan_bytes);
+#define TRY(e)          \
+  do {                  \
+    rc = (e);           \
+    if (rc) return rc;  \
+  } while (0)
+  TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
+  TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
+  TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
+  TRY(ornith_linear_matmul(ctx, &w->sh_gate, d_x, T, sg));
+  TRY(ornith_linear_matmul(ctx, &w->sh_up, d_x, T, su));
+  TRY(ornith_swiglu(ctx, sg, su, (int64_t)T * SI, sact));
+  TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
+  TRY(ornith_kq_gather_matmul(ctx, &w->ex_gate, d_x, inds, pairs, k, 1, plan, 1, xg));
+  TRY(ornith_kq_gather_matmul(ctx, &w->ex_up, d_x, inds, pairs, k, 1, plan, 0, xu));
+  TRY(ornith_swiglu(ctx, xg, xu, (int64_t)pairs * I, act));
+  TRY(ornith_kq_gather_matmul(ctx, &w->ex_down, act, inds, pairs, k, 0, plan, 0, y));
+  TRY(ornith_moe_combine(ctx, scores, y, eg, sy, T, k, H, w->norm_topk_prob, d_out));
+#undef TRY
+  return ORNITH_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -132,7 +179,7 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
                      void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
   ORN_REQUIRE(ctx && w && d_x && d_out, "moe_block: null argument");
   const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
-  ORN_REQUIRE(T >= 1 && T <= 64, "moe_block: T=%d (decode/verify widths only)", T);
+  ORN_REQUIRE(T >= 1 && T <= 8192, "moe_block: T=%d", T);
   ORN_REQUIRE(k >= 1 && k <= 16 && k <= E, "moe_block: top_k=%d of %d", k, E);
   ORN_REQUIRE(w->ex_gate.E == E && w->ex_up.E == E && w->ex_down.E == E,
               "moe_block: expert tensors carry %d/%d/%d experts, router has %d", w->ex_gate.E,
@@ -145,6 +192,11 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
                   w->sh_egate.O == 1,
               "moe_block: shared expert shapes do not chain");
   const int SI = w->sh_gate.O;
+  if (T >= kPrefillRows && !w->ex_dense) {
+    ORN_REQUIRE(!d_inds_out && !d_scores_out, "moe_block: index outputs are a decode-width feature");
+    return moe_block_prefill(ctx, w, d_x, T, d_out);
+  }
+  ORN_REQUIRE(T <= 64, "moe_block: T=%d with dense experts (decode/verify widths only)", T);
 
   const size_t need = 2 * ((size_t)T * E * 2 + (size_t)T * SI * 3 + (size_t)T * H + T +
                            (size_t)(T * k + T) * (2 * I + I + SI + H + 1)) +

@@ -38,6 +38,12 @@ struct ScratchCursor {
   }
 };
 
+// Activation rows from which the k-quant projections and the MoE block switch from the
+// exact mat-vec path (every row as if alone) to the matrix-core GEMM path. The reference
+// draws the same line at its EXACT_WINDOW (src/ops/invariant.rs:88-116).
+int ornith_option_gemm_rows();  // default 32; 0 = never (everything through the exact path)
+#define kPrefillRows (ornith_option_gemm_rows())
+
 // ornith_greedy_rows with its temporaries taken from the caller's cursor (for operators
 // that hold other scratch buffers at the same time). Needs rows * ceil(V/1024) * 16 + 2048 bytes.
 int ornith_greedy_rows_ws(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens,

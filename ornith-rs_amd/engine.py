@@ -166,6 +166,11 @@ class TextModel:
     def rewind(self, caches, keep):
         _check(lib().ornith_model_rewind(self.h, caches.h, keep), "model_rewind")
 
+    def set_max_rows(self, rows):
+        """Rows one forward call may carry (before creating caches); from 32 up the projections
+        and experts run as matrix-core GEMMs."""
+        _check(lib().ornith_model_set_max_rows(self.h, rows), "model_set_max_rows")
+
     def moe_weights(self, layer):
         """The resident MoE block of one decoder layer (valid while the model lives)."""
         from . import MoeWeightsStruct
