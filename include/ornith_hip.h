@@ -286,6 +286,13 @@ ORNITH_API int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, co
                                         const void* d_v_cache, const void* d_qg, int T, int Hq,
                                         int Hkv, int hd, int offset, const int* d_offset, int cap,
                                         float scale, void* d_out);
+/* sdpa_unfused (src/ops/sdpa.rs:386-461) for the rows of a prompt chunk, with the same output
+ * gate: causal flash attention on the matrix cores, head_dim 256. Same arguments as
+ * sdpa_decode_gated (host-side offset only), which forwards to it from 32 rows up; agrees
+ * with the exact kernel to rounding, not bit for bit. */
+ORNITH_API int ornith_sdpa_prefill_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d_k_cache,
+                                         const void* d_v_cache, const void* d_qg, int T, int Hq, int Hkv,
+                                         int hd, int offset, int cap, float scale, void* d_out);
 
 /* ---- greedy selection: src/ops/sample.rs ------------------------------------------ */
 /* greedy_token / the verify rows of generate_step_mtp (src/ops/sample.rs:134-147,

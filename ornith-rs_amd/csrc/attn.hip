@@ -319,6 +319,10 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
                              int offset, const int* d_offset, int cap, float scale, void* d_out) {
   ORN_REQUIRE(ctx && d_q_rot && d_k_cache && d_v_cache && d_qg && d_out, "sdpa_decode: null argument");
   ORN_REQUIRE(hd == 256 || hd == 128, "sdpa_decode: head_dim %d (128 or 256)", hd);
+  // prompt chunks: the matrix-core kernel (outside the exact window, like the projections)
+  if (T >= kPrefillRows && hd == 256 && !d_offset)
+    return ornith_sdpa_prefill_gated(ctx, d_q_rot, d_k_cache, d_v_cache, d_qg, T, Hq, Hkv, hd, offset, cap,
+                                     scale, d_out);
   ORN_REQUIRE(T >= 1 && T <= 64 && Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "sdpa_decode: T=%d Hq=%d Hkv=%d",
               T, Hq, Hkv);
   ORN_REQUIRE(offset >= 0 && offset + T <= cap, "sdpa_decode: rows [%d,%d) exceed capacity %d", offset,

@@ -169,3 +169,29 @@ def test_model_prefill_in_wide_chunks_close_to_exact_chunks(orn, ctx, exact_weig
     with pytest.raises(orn.OrnithError, match="created for"):
         model.forward(narrow, toks[:48])          # caches made before the model was widened
     for o in (narrow, wide, model, ws): o.close()
+
+
+@pytest.mark.parametrize("T,Hq,Hkv,cap,offset", [(64, 16, 2, 512, 0), (100, 4, 1, 1024, 37), (300, 16, 2, 2048, 1000),
+                                                 (33, 2, 2, 256, 200), (512, 8, 2, 1024, 512)])
+def test_prefill_attention_close_to_exact_kernel(orn, ctx, T, Hq, Hkv, cap, offset):
+    """Causal flash attention on the matrix cores vs the oracle's exact attention: every row
+    within 1 % relative L2 (bf16 probabilities into the second GEMM, fp32 sums in block order).
+    Cache rows past the chunk hold NaN patterns: nothing may read them."""
+    from test_gpu_attn import _mk
+    hd, rd = 256, 64
+    rng = np.random.default_rng(T + offset)
+    qg, kx, vx, qw, kw, kc, vc = _mk(rng, T, Hq, Hkv, hd, cap, offset)
+    c, s = util.orc_rope_table(cap, rd, 1e7)
+    wkc, wvc = kc.copy(), vc.copy()
+    wq, wgate = util.orc_attn_prep(qg, kx, vx, qw, kw, rd, c, s, offset, wkc, wvc)
+    want = util.orc_sdpa(wq, wkc, wvc, wgate, offset, hd ** -0.5)
+    dq, dk, dv, dg = ctx.to_device(wq), ctx.to_device(wkc), ctx.to_device(wvc), ctx.to_device(qg)
+    dout = ctx.alloc(T * Hq * hd * 2)
+    ctx.sdpa_decode_gated(dq, dk, dv, dg, T, Hq, Hkv, hd, offset, cap, hd ** -0.5, dout)
+    got = dout.download(np.uint16, want.shape)
+    g = util.bf16_to_f32(got).astype(np.float64).reshape(T * Hq, hd)
+    w = util.bf16_to_f32(want).astype(np.float64).reshape(T * Hq, hd)
+    assert np.isfinite(g).all()
+    rel = np.linalg.norm(g - w, axis=1) / np.linalg.norm(w, axis=1)
+    assert rel.max() < 0.01, float(rel.max())
+    for b in (dq, dk, dv, dg, dout): b.free()
