@@ -96,6 +96,58 @@ def cpu_baseline(synth, synth_model, np, depth, tokens):
                       f"whole call {dt:.1f} s ({int(st.cycles)} cycles, {int(st.accepted)} accepted)"}, toks, prompt
 
 
+def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
+    """BASELINE config 5: sampled speculative decode at depth 3 after a long prefill."""
+    depth, n_prompt, n_gen, cap = 3, 6621, 256, 16384
+    model.set_max_rows(args.prefill_chunk)
+    caches = model.make_cache(cap, depth + 1)
+    head = orn.MtpHead(model, ws, cap)
+    fr_ids = synth.zipf_frspec_ids(cfg["vocab_size"], 32768, seed=1)
+    fr = orn.FrSpec(model, ids=fr_ids)
+    rng = np.random.default_rng(6621)
+    prompt = rng.integers(0, cfg["vocab_size"], n_prompt).astype(np.uint32)
+    smp = orn.Sampler(1, 0.8, 0.95, 0, 2025)
+    res = []
+    for it in range(2):
+        caches.reset()
+        mark = {}
+
+        def progress(done, total):
+            ctx.sync()
+            if done == 0:
+                mark["p0"] = time.perf_counter()
+            if done == total:
+                mark["p1"] = time.perf_counter()
+
+        toks, st = orn.generate_step_mtp(model, head, fr, caches, prompt, depth, n_gen, sampler=smp,
+                                         prefill_step=args.prefill_chunk, policy=orn.HISTORY_COMMITTED,
+                                         progress=progress)
+        ctx.sync()
+        t_end = time.perf_counter()
+        res.append((toks, st, mark["p1"] - mark["p0"], t_end - mark["p1"]))
+        log(f"config5 run {it}: prefill {res[-1][2]:.3f} s ({n_prompt / res[-1][2]:.0f} tok/s), decode "
+            f"{n_gen / res[-1][3]:.1f} tok/s, {int(st.cycles)} cycles, {int(st.accepted)}/{int(st.drafted)} accepted")
+    assert res[0][0] == res[1][0], "same seed, different tokens"
+    toks, st, t_pre, t_dec = res[-1]
+    # active weight bytes per prompt token are read once per chunk; the GEMM work is 2 flops per
+    # active weight per token: projections + router + shared expert + 8 routed experts, 40 layers
+    H, I = 2048, 512
+    per_layer_gdn = H * (8192 + 4096) + 4096 * H
+    per_layer_att = H * (8192 + 512 + 512) + 4096 * H
+    per_layer_moe = H * 256 + 9 * 3 * H * I
+    flops_tok = 2.0 * (30 * per_layer_gdn + 10 * per_layer_att + 40 * per_layer_moe)
+    line = {"workload": f"config5: {n_prompt}-token prefill (chunks of {args.prefill_chunk}) into a {cap}-token context, "
+                        f"then sampled MTP depth-{depth} + FR-Spec decode of {n_gen} tokens (temperature 0.8, top-p 0.95, "
+                        "seeded threefry keys)",
+            "prefill_s": round(t_pre, 4), "prefill_tok_s": round(n_prompt / t_pre, 1),
+            "prefill_gemm_tflops": round(flops_tok * n_prompt / t_pre / 1e12, 2),
+            "prefill_frac_of_bf16_mfma_peak": round(flops_tok * n_prompt / t_pre / 2.5e15, 4),
+            "decode_tok_s": round(n_gen / t_dec, 2), "cycles": int(st.cycles), "drafted": int(st.drafted),
+            "accepted": int(st.accepted), "tokens_per_verify_step": round(n_gen / max(1, int(st.cycles)), 3),
+            "repeatable": True, "device": dev_name, "data": "synthetic"}
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -106,6 +158,11 @@ def main():
     ap.add_argument("--layers", type=int, default=40, help="trunk layers (40 = the named config)")
     ap.add_argument("--cpu-tokens", type=int, default=48)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--config5", action="store_true",
+                    help="instead of the metric's workload: BASELINE config 5 (6621-token prefill into a "
+                         "16384-token context through the matrix-core path, then sampled depth-3 MTP "
+                         "decode of 256 tokens, temperature 0.8, top-p 0.95); prints its own JSON line")
+    ap.add_argument("--prefill-chunk", type=int, default=512)
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the expert-kernel timing loop plus three 256 MiB device copies "
                          "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -138,6 +195,8 @@ def main():
         ctx.sync()
         print(json.dumps({"roofline": roof}), flush=True)
         return
+    if args.config5:
+        return config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name)
     rng = np.random.default_rng(51)
     prompt = rng.integers(0, cfg["vocab_size"], 51).astype(np.uint32)
     cap = 4096

@@ -239,7 +239,7 @@ static_assert(BN == 128 && BK == 128, "tile constants are baked into the index a
 
 // ---- expert-sorted pair list for the gathered form -----------------------------------
 // inds [pairs] (expert of pair p; pair p = token * k + slot). One workgroup:
-// counts per expert, exclusive scan, stable scatter, then the tile list.
+// counts per expert, exclusive scan, scatter, then the tile list.
 __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* inds, int pairs, int E,
                                                               int bm, uint32_t* pair, uint32_t* tile_expert,
                                                               uint32_t* tile_start, uint32_t* tile_count,
@@ -263,14 +263,17 @@ __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* in
     *n_tiles = t;
   }
   __syncthreads();
-  // stable placement: expert e's pairs in ascending pair order (one thread per expert walks
-  // the list; pairs <= 2048 * 8 and this runs once per layer per chunk)
+  // placement: a pair takes the next free place of its expert. The order inside an expert's
+  // run depends on the scheduling of the atomics, the results do not: every output row is one
+  // dot product over k in a fixed order, whichever tile row computes it.
+  __shared__ uint32_t fill[1024];
+  fill[tid] = 0;
+  __syncthreads();
+  for (int p = tid; p < pairs; p += 1024) {
+    const uint32_t e = min(inds[p], (uint32_t)(E - 1));
+    pair[start[e] + atomicAdd(&fill[e], 1u)] = (uint32_t)p;
+  }
   for (int e = tid; e < E; e += 1024) {
-    uint32_t w = start[e];
-    if (cnt[e]) {
-      for (int p = 0; p < pairs; ++p)
-        if (min(inds[p], (uint32_t)(E - 1)) == (uint32_t)e) pair[w++] = (uint32_t)p;
-    }
     const uint32_t nt = (cnt[e] + bm - 1) / bm;
     for (uint32_t t = 0; t < nt; ++t) {
       tile_expert[tiles_before[e] + t] = e;

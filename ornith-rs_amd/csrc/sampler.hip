@@ -84,28 +84,43 @@ __global__ __launch_bounds__(RB) void radix_hist_kernel(const bf16_t* x, int neg
   if (tid < 256) table[(size_t)tid * nblk + blockIdx.x] = h[tid];
 }
 
-// in-place exclusive scan of m counters by one workgroup
+// in-place exclusive scan of m counters by one workgroup, in tiles of 1024 consecutive
+// counters (coalesced). Up to 64 tiles are fetched into registers before the first is
+// scanned, so the walk over the tiles never waits on memory.
 __global__ __launch_bounds__(RB) void radix_scan_kernel(uint32_t* table, int m) {
-  __shared__ uint32_t part[RB];
-  const int tid = threadIdx.x;
-  const int span = (m + RB - 1) / RB;
-  const int lo = tid * span, hi = min(lo + span, m);
-  uint32_t s = 0;
-  for (int j = lo; j < hi; ++j) s += table[j];
-  part[tid] = s;
+  __shared__ uint32_t wtot[RB / 64];
+  __shared__ uint32_t s_carry;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) s_carry = 0;
   __syncthreads();
-  // Hillis-Steele over the 1024 partials (integers: any order gives the same sums)
-  for (int d = 1; d < RB; d <<= 1) {
-    const uint32_t o = tid >= d ? part[tid - d] : 0u;
-    __syncthreads();
-    part[tid] += o;
-    __syncthreads();
-  }
-  uint32_t run = part[tid] - s;  // exclusive
-  for (int j = lo; j < hi; ++j) {
-    const uint32_t c = table[j];
-    table[j] = run;
-    run += c;
+  constexpr int G = 64;
+  for (int t0 = 0; t0 * RB < m; t0 += G) {
+    uint32_t v[G];
+#pragma unroll
+    for (int t = 0; t < G; ++t) {
+      const int j = (t0 + t) * RB + tid;
+      v[t] = j < m ? table[j] : 0u;
+    }
+#pragma unroll
+    for (int t = 0; t < G; ++t) {
+      if ((t0 + t) * RB >= m) break;
+      // inclusive scan inside the wavefront, then across the 16 wavefront totals
+      uint32_t x = v[t];
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t o = __shfl_up(x, d, 64);
+        if (lane >= d) x += o;
+      }
+      if (lane == 63) wtot[wave] = x;
+      __syncthreads();
+      uint32_t before = s_carry;
+      for (int w = 0; w < wave; ++w) before += wtot[w];
+      const int j = (t0 + t) * RB + tid;
+      if (j < m) table[j] = before + x - v[t];
+      __syncthreads();
+      if (tid == RB - 1) s_carry = before + x;
+      __syncthreads();
+    }
   }
 }
 
@@ -213,12 +228,23 @@ __global__ __launch_bounds__(RB) void scan_local_kernel(const float* in, int n, 
 template <bool BF16>
 __device__ __forceinline__ void chunk_base(const float* chunk_tot, int nch, float& base, float& total) {
   __shared__ float s_base, s_total;
-  if (threadIdx.x == 0) {
-    float acc = 0.f, b = 0.f;
-    for (int c = 0; c < nch; ++c) {
-      if (c == (int)blockIdx.x) b = acc;
-      acc = add_r<BF16>(acc, chunk_tot[c]);
+  __shared__ float s_tot[RB];
+  // the totals come in with one coalesced load per 1024 chunks; the left-to-right sum over
+  // them is the only sequential part
+  float acc = 0.f, b = 0.f;
+  for (int c0 = 0; c0 < nch; c0 += RB) {
+    if (c0 + (int)threadIdx.x < nch) s_tot[threadIdx.x] = chunk_tot[c0 + threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const int n = min(RB, nch - c0);
+      for (int c = 0; c < n; ++c) {
+        if (c0 + c == (int)blockIdx.x) b = acc;
+        acc = add_r<BF16>(acc, s_tot[c]);
+      }
     }
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
     s_base = b;
     s_total = acc;
   }
