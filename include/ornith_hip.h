@@ -69,6 +69,8 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *   "fuse_proj" (ORNITH_FUSE_PROJ, default 1): projections sharing an input in one launch
  *   "moe_up_iters" (ORNITH_MOE_UP_ITERS, default 0 = chosen by shape; 2 or 4): output
  *               rows per wavefront of the fused gate+up expert kernel, a tuning knob
+ *   "fuse_gdn"  (ORNITH_FUSE_GDN, default 1): the gated-delta mixer core (a / b projections,
+ *               front, recurrence, gated norm) in one launch at decode / verify widths
  *   "gemm_rows" (ORNITH_GEMM_ROWS, default 32; 0 = never): activation rows from which the
  *               k-quant projections and the MoE experts run as matrix-core GEMMs instead of
  *               exact mat-vecs. The one switch that changes results (to bf16 rounding of the
@@ -263,6 +265,20 @@ ORNITH_API int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const voi
                                      const void* d_v, const float* d_g, const void* d_beta,
                                      const float* d_state_in, int T, int Hk, int Hv, int Dk, int Dv,
                                      void* d_y, float* d_snapshots, int snapshot_every_token);
+
+/* The core of GatedDeltaNet::forward / forward_capture between the big projections
+ * (src/model/qwen3_5.rs:493-560, 650-677) in one launch, T <= 16: in_proj_a / in_proj_b
+ * (dense bf16 weights d_wa / d_wb [Hv, H] applied to d_xn [T, H]; or pass the projections
+ * d_a / d_b [T, Hv] and null weights), gdn_front, the recurrence with its per-token state
+ * snapshots, and rms_norm_gated against d_z -> d_gated_out [T, Hv*Dv]. One workgroup per
+ * value head keeps q, k, v, g, beta and y in LDS. Bit-identical to the separate calls. */
+ORNITH_API int ornith_gdn_step(ornith_ctx* ctx, const void* d_conv_state, const void* d_qkv,
+                               const void* d_cw, const void* d_a, const void* d_b, const void* d_wa,
+                               const void* d_wb, const void* d_xn, int H, const void* d_a_log,
+                               const void* d_dt_bias, int T, int K, int Hk, int Dk, int Hv, int Dv,
+                               float eps, const float* d_state_in, float* d_snapshots,
+                               int snapshot_every_token, const void* d_norm_w, const void* d_z,
+                               float norm_eps, void* d_conv_input, void* d_gated_out);
 
 /* ---- full-attention layer at decode / verify width ------------------------------ */
 /* ops::rope tables (src/ops/rope.rs:6-60): cos/sin f32 [npos, dims/2] for

@@ -18,6 +18,7 @@
 // carries eight rows, and the state after EACH token is written out as a
 // snapshot, so rejecting a draft is a pointer move to snapshot keep-1.
 #include "dmath.h"
+#include "linear_device.h"
 #include "rt.h"
 
 namespace {
@@ -177,9 +178,246 @@ __global__ __launch_bounds__(64) void gdn_recurrence_kernel(RecArgs p) {
   }
 }
 
+// ---- the whole mixer core in one launch, decode / verify widths -------------------------
+// One workgroup per value head (16 wavefronts):
+//   1. every thread issues the loads of its slice of the recurrent state (they depend on
+//      nothing), then
+//   2. the wavefronts share out the head's front-end work: conv + silu (+ norm, scale) of
+//      the head's q, k and v channels for each token, the in_proj_a / in_proj_b dot
+//      products of this head, g and beta -- results stay in LDS;
+//   3. the recurrence runs on the state registers, reading q, k, v, g, beta from LDS,
+//      writing the per-token snapshots and leaving y in LDS;
+//   4. one wavefront per token applies the gated RMS norm to the head's 128 outputs.
+// Arithmetic and its order are those of gdn_front_kernel, dense_gemv, gdn_recurrence_kernel
+// and rms_norm_gated: the fused launch is bit-identical to the four separate ones.
+constexpr int kStepMaxT = 16;
+
+struct StepArgs {
+  FrontArgs f;
+  const bf16_t* wa;      // in_proj_a [Hv, H] dense bf16, or null: f.a_in / f.b_in hold the projections
+  const bf16_t* wb;
+  const bf16_t* xn;      // [T, H] input of the projections
+  int H;
+  const float* state_in;  // [Hv, 128, 128]
+  float* snapshots;       // [T][Hv, 128, 128]
+  int snap_all;
+  const bf16_t* norm_w;   // [128]
+  const bf16_t* z;        // [T, Hv*128]
+  float norm_eps;
+  bf16_t* gated;          // [T, Hv*128]
+};
+
+__global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
+  const FrontArgs& p = a.f;
+  __shared__ float qs[kStepMaxT][128], ks[kStepMaxT][128], vs[kStepMaxT][128], ys[kStepMaxT][128];
+  __shared__ float gs[kStepMaxT], bs[kStepMaxT];
+  __shared__ float ab[2][kStepMaxT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int hv = blockIdx.x, ratio = p.Hv / p.Hk, hk = hv / ratio;
+  const int T = p.T, S = p.K - 1, D = p.D, key_dim = p.Hk * 128;
+
+  // 1. state slice of this thread: row dv = 8*wave + lane/8, columns 32*m + 4*(lane%8) ..+4
+  const int row = lane >> 3, j = lane & 7, dv = wave * 8 + row;
+  const size_t ssz = (size_t)p.Hv * 128 * 128;
+  const size_t roff = ((size_t)hv * 128 + dv) * 128 + 4 * j;
+  float s[16];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const float4 f = *reinterpret_cast<const float4*>(a.state_in + roff + 32 * m);
+    s[4 * m + 0] = f.x;
+    s[4 * m + 1] = f.y;
+    s[4 * m + 2] = f.z;
+    s[4 * m + 3] = f.w;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // 2. front-end tasks: [0, 3T) conv of (q | k | v, token); then the a / b projections
+  const int n_conv = 3 * T, n_ab = a.wa ? 2 * T : 0;
+  for (int task = wave; task < n_conv + n_ab; task += 16) {
+    if (task < n_conv) {
+      const int which = task / T, t = task - which * T;  // 0 q, 1 k, 2 v
+      const int slot = which == 0 ? hk : which == 1 ? p.Hk + hk : 2 * p.Hk + hv;
+      const int c0 = slot * 128 + 2 * lane;
+      float acc0 = 0.f, acc1 = 0.f;
+      for (int i = 0; i < p.K; ++i) {
+        const int jj = t + i;
+        const bf16_t* src = (jj < S) ? (p.conv_state + (size_t)jj * D) : (p.qkv + (size_t)(jj - S) * D);
+        const uint32_t xv = *reinterpret_cast<const uint32_t*>(src + c0);
+        acc0 = dm_fma(dm_bf2f_lo(xv), dm_bf2f(p.cw[(size_t)c0 * p.K + i]), acc0);
+        acc1 = dm_fma(dm_bf2f_hi(xv), dm_bf2f(p.cw[(size_t)(c0 + 1) * p.K + i]), acc1);
+      }
+      const float cv0 = dm_rb(acc0), cv1 = dm_rb(acc1);
+      const float y0 = dm_rb(cv0 * dm_sigmoid_bf16(cv0)), y1 = dm_rb(cv1 * dm_sigmoid_bf16(cv1));
+      // the window: v channels belong to this head alone, q / k channels to the first head of the group
+      if (which == 2 || hv % ratio == 0) {
+        *reinterpret_cast<uint32_t*>(p.conv_input + (size_t)(S + t) * D + c0) =
+            *reinterpret_cast<const uint32_t*>(p.qkv + (size_t)t * D + c0);
+        if (t == 0)
+          for (int r = 0; r < S; ++r)
+            *reinterpret_cast<uint32_t*>(p.conv_input + (size_t)r * D + c0) =
+                *reinterpret_cast<const uint32_t*>(p.conv_state + (size_t)r * D + c0);
+      }
+      if (which < 2) {
+        float ss = dm_fma(y0, y0, 0.f);
+        ss = dm_fma(y1, y1, ss);
+        const float inv = dm_rsqrt(dm_wave_sum<64>(ss) / 128.0f + p.eps);
+        const float sc = which == 0 ? p.q_scale : p.k_scale;
+        float* dst = which == 0 ? qs[t] : ks[t];
+        dst[2 * lane] = dm_rb(sc * dm_rb(y0 * inv));
+        dst[2 * lane + 1] = dm_rb(sc * dm_rb(y1 * inv));
+      } else {
+        vs[t][2 * lane] = y0;
+        vs[t][2 * lane + 1] = y1;
+      }
+    } else {
+      const int u = task - n_conv, which = u / T, t = u - which * T;  // 0 a, 1 b
+      const bf16_t* wr = (which == 0 ? a.wa : a.wb) + (size_t)hv * a.H;
+      const float v = dense_row_dot(wr, a.xn + (size_t)t * a.H, a.H, lane);
+      if (lane == 0) ab[which][t] = dm_rb(v);
+    }
+  }
+  __syncthreads();
+  if (tid < T) {
+    const int t = tid, i = t * p.Hv + hv;
+    const float av = a.wa ? ab[0][t] : dm_bf2f(p.a_in[i]);
+    const float bv = a.wa ? ab[1][t] : dm_bf2f(p.b_in[i]);
+    const float sp = softplus_bf16(dm_rb(av + dm_bf2f(p.dt_bias[hv])));
+    const float decay = dm_exp(dm_bf2f(p.a_log[hv]));
+    gs[t] = dm_exp(-decay * sp);
+    bs[t] = dm_rb(dm_sigmoid_bf16(bv));
+  }
+  __syncthreads();
+
+  // 3. recurrence (gdn_recurrence_kernel, operands from LDS)
+  for (int t = 0; t < T; ++t) {
+    float kf[16], qf[16];
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const float4 kv4 = *reinterpret_cast<const float4*>(&ks[t][32 * m + 4 * j]);
+      const float4 qv4 = *reinterpret_cast<const float4*>(&qs[t][32 * m + 4 * j]);
+      kf[4 * m + 0] = kv4.x; kf[4 * m + 1] = kv4.y; kf[4 * m + 2] = kv4.z; kf[4 * m + 3] = kv4.w;
+      qf[4 * m + 0] = qv4.x; qf[4 * m + 1] = qv4.y; qf[4 * m + 2] = qv4.z; qf[4 * m + 3] = qv4.w;
+    }
+    const float gt = gs[t], bt = bs[t], vt = vs[t][dv];
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      s[e] = s[e] * gt;
+      acc = dm_fma(s[e], kf[e], acc);
+    }
+    const float kv = dm_wave_sum<8>(acc);
+    const float delta = (vt - kv) * bt;
+    float o = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      s[e] = dm_fma(kf[e], delta, s[e]);
+      o = dm_fma(s[e], qf[e], o);
+    }
+    o = dm_wave_sum<8>(o);
+    if (j == 0) ys[t][dv] = dm_rb(o);
+    if (a.snap_all || t + 1 == T) {
+      float* snap = a.snapshots + (a.snap_all ? (size_t)t * ssz : 0) + roff;
+#pragma unroll
+      for (int m = 0; m < 4; ++m)
+        *reinterpret_cast<float4*>(snap + 32 * m) =
+            make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+    }
+  }
+  __syncthreads();
+
+  // 4. gated norm of the head's 128 outputs, one wavefront per token (rms_norm_gated, two
+  //    values per lane)
+  for (int t = wave; t < T; t += 16) {
+    float x0 = ys[t][2 * lane], x1 = ys[t][2 * lane + 1];
+    float acc = dm_fma(x0, x0, 0.f);
+    acc = dm_fma(x1, x1, acc);
+    const float inv = dm_rsqrt(dm_wave_sum<64>(acc) / 128.0f + a.norm_eps);
+    const uint32_t wv = *reinterpret_cast<const uint32_t*>(a.norm_w + 2 * lane);
+    const size_t off = ((size_t)t * p.Hv + hv) * 128 + 2 * lane;
+    const uint32_t zv = *reinterpret_cast<const uint32_t*>(a.z + off);
+    x0 = dm_rb(dm_bf2f_lo(wv) * dm_rb(x0 * inv));
+    x1 = dm_rb(dm_bf2f_hi(wv) * dm_rb(x1 * inv));
+    const float g0 = dm_bf2f_lo(zv), g1 = dm_bf2f_hi(zv);
+    x0 = (g0 * dm_sigmoid_f32(g0)) * x0;
+    x1 = (g1 * dm_sigmoid_f32(g1)) * x1;
+    *reinterpret_cast<uint32_t*>(a.gated + off) = (uint32_t)dm_f2bf(x0) | ((uint32_t)dm_f2bf(x1) << 16);
+  }
+}
+
 }  // namespace
 
+// fills the front-end part of the arguments (shared by gdn_front and gdn_step)
+static void fill_front(FrontArgs& p, const void* d_conv_state, const void* d_qkv, const void* d_cw,
+                       const void* d_a, const void* d_b, const void* d_a_log, const void* d_dt_bias, int T,
+                       int K, int Hk, int Dk, int Hv, float eps, void* d_q, void* d_k, void* d_v,
+                       void* d_beta, float* d_g, void* d_conv_input) {
+  p.conv_state = (const bf16_t*)d_conv_state;
+  p.qkv = (const bf16_t*)d_qkv;
+  p.cw = (const bf16_t*)d_cw;
+  p.a_in = (const bf16_t*)d_a;
+  p.b_in = (const bf16_t*)d_b;
+  p.a_log = (const bf16_t*)d_a_log;
+  p.dt_bias = (const bf16_t*)d_dt_bias;
+  p.q = (bf16_t*)d_q;
+  p.k = (bf16_t*)d_k;
+  p.v = (bf16_t*)d_v;
+  p.beta = (bf16_t*)d_beta;
+  p.g = d_g;
+  p.conv_input = (bf16_t*)d_conv_input;
+  p.T = T;
+  p.K = K;
+  p.Hk = Hk;
+  p.Hv = Hv;
+  p.D = 2 * Hk * 128 + Hv * 128;
+  const float inv_scale = 1.0f / sqrtf((float)Dk);
+  // both scales are applied as bf16 values (the reference casts them to T)
+  uint32_t u;
+  float f = inv_scale * inv_scale;
+  memcpy(&u, &f, 4);
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+  memcpy(&p.q_scale, &u, 4);
+  f = inv_scale;
+  memcpy(&u, &f, 4);
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+  memcpy(&p.k_scale, &u, 4);
+  p.eps = eps;
+}
+
 extern "C" {
+
+int ornith_gdn_step(ornith_ctx* ctx, const void* d_conv_state, const void* d_qkv, const void* d_cw,
+                    const void* d_a, const void* d_b, const void* d_wa, const void* d_wb, const void* d_xn,
+                    int H, const void* d_a_log, const void* d_dt_bias, int T, int K, int Hk, int Dk, int Hv,
+                    int Dv, float eps, const float* d_state_in, float* d_snapshots, int snapshot_every_token,
+                    const void* d_norm_w, const void* d_z, float norm_eps, void* d_conv_input,
+                    void* d_gated_out) {
+  ORN_REQUIRE(ctx && d_conv_state && d_qkv && d_cw && d_a_log && d_dt_bias && d_state_in && d_snapshots &&
+                  d_norm_w && d_z && d_conv_input && d_gated_out,
+              "gdn_step: null argument");
+  ORN_REQUIRE((d_wa && d_wb && d_xn && H >= 8 && H % 8 == 0) || (!d_wa && !d_wb && d_a && d_b),
+              "gdn_step: give either the a / b projections or their weights and input");
+  ORN_REQUIRE(Dk == 128 && Dv == 128, "gdn_step: head dims %d/%d (128 only)", Dk, Dv);
+  ORN_REQUIRE(T >= 1 && T <= kStepMaxT && K >= 2 && K <= 8 && Hk >= 1 && Hv >= Hk && Hv % Hk == 0,
+              "gdn_step: T=%d (1..%d) K=%d Hk=%d Hv=%d", T, kStepMaxT, K, Hk, Hv);
+  ORN_REQUIRE(d_conv_input != d_conv_state, "gdn_step: conv_input must not alias conv_state");
+  StepArgs a{};
+  fill_front(a.f, d_conv_state, d_qkv, d_cw, d_a, d_b, d_a_log, d_dt_bias, T, K, Hk, Dk, Hv, eps, nullptr,
+             nullptr, nullptr, nullptr, nullptr, d_conv_input);
+  a.wa = (const bf16_t*)d_wa;
+  a.wb = (const bf16_t*)d_wb;
+  a.xn = (const bf16_t*)d_xn;
+  a.H = H;
+  a.state_in = d_state_in;
+  a.snapshots = d_snapshots;
+  a.snap_all = snapshot_every_token ? 1 : 0;
+  a.norm_w = (const bf16_t*)d_norm_w;
+  a.z = (const bf16_t*)d_z;
+  a.norm_eps = norm_eps;
+  a.gated = (bf16_t*)d_gated_out;
+  hipLaunchKernelGGL(gdn_step_kernel, dim3(Hv), dim3(1024), 0, ctx->stream, a);
+  ORN_LAUNCH_CHECK("gdn_step_kernel");
+  return ORNITH_OK;
+}
 
 int ornith_gdn_front(ornith_ctx* ctx, const void* d_conv_state, const void* d_qkv, const void* d_cw,
                      const void* d_a, const void* d_b, const void* d_a_log, const void* d_dt_bias,

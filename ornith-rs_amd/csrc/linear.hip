@@ -11,6 +11,7 @@
 // through the butterfly. These matrices are small (router-sized or the MTP
 // head), so the layout favours a fixed summation order over tuning.
 #include "dmath.h"
+#include "linear_device.h"
 #include "rt.h"
 
 namespace {
@@ -79,20 +80,7 @@ __global__ __launch_bounds__(256) void dense_gemv_kernel(const bf16_t* w, const 
     wr = w + (size_t)o * K;
     xr = x + (size_t)r * K;
   }
-  float a = 0.f;
-  for (int j = lane; j < K / 8; j += 64) {
-    const uint4 wv = *reinterpret_cast<const uint4*>(wr + 8 * j);
-    const uint4 xv = *reinterpret_cast<const uint4*>(xr + 8 * j);
-    a = dm_fma(dm_bf2f_lo(wv.x), dm_bf2f_lo(xv.x), a);
-    a = dm_fma(dm_bf2f_hi(wv.x), dm_bf2f_hi(xv.x), a);
-    a = dm_fma(dm_bf2f_lo(wv.y), dm_bf2f_lo(xv.y), a);
-    a = dm_fma(dm_bf2f_hi(wv.y), dm_bf2f_hi(xv.y), a);
-    a = dm_fma(dm_bf2f_lo(wv.z), dm_bf2f_lo(xv.z), a);
-    a = dm_fma(dm_bf2f_hi(wv.z), dm_bf2f_hi(xv.z), a);
-    a = dm_fma(dm_bf2f_lo(wv.w), dm_bf2f_lo(xv.w), a);
-    a = dm_fma(dm_bf2f_hi(wv.w), dm_bf2f_hi(xv.w), a);
-  }
-  const float v = dm_wave_sum<64>(a);
+  const float v = dense_row_dot(wr, xr, K, lane);
   if (lane == 0) y[(size_t)r * O + o] = dm_f2bf(v);
 }
 

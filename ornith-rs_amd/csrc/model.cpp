@@ -193,20 +193,31 @@ static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_to
     LayerCache& lc = cc->layers[i];
     if (L.linear) {
       const GdnLayer& g = L.gdn;
-      {
-        const ornith_linear* big[2] = {&g.in_proj_qkv, &g.in_proj_z};
-        void* ybig[2] = {s.qkv, s.z};
-        TRY(ornith_linear_matmul_multi(ctx, big, 2, s.normed, T, ybig));
+      const ornith_linear* big[2] = {&g.in_proj_qkv, &g.in_proj_z};
+      void* ybig[2] = {s.qkv, s.z};
+      TRY(ornith_linear_matmul_multi(ctx, big, 2, s.normed, T, ybig));
+      const char* conv_state = (const char*)lc.conv[cc->conv_cur] + (size_t)cc->conv_off * D * 2;
+      const float* state_in = lc.state + (size_t)cc->state_cur * ssz;
+      const bool dense_ab = g.in_proj_a.mode == ORNITH_LIN_DENSE && g.in_proj_b.mode == ORNITH_LIN_DENSE;
+      const bool fused = T <= 16 && Dk == 128 && Dv == 128 && ornith_option_fuse_gdn();
+      if (!(fused && dense_ab)) {
         const ornith_linear* ab[2] = {&g.in_proj_a, &g.in_proj_b};
         void* yab[2] = {s.a, s.b};
         TRY(ornith_linear_matmul_multi(ctx, ab, 2, s.normed, T, yab));
       }
-      const char* conv_state = (const char*)lc.conv[cc->conv_cur] + (size_t)cc->conv_off * D * 2;
-      TRY(ornith_gdn_front(ctx, conv_state, s.qkv, g.conv1d, s.a, s.b, g.a_log, g.dt_bias, T, K, Hk,
-                           Dk, Hv, Dv, 1e-6f, s.q, s.k, s.v, s.beta, s.g, lc.conv[1 - cc->conv_cur]));
-      TRY(ornith_gdn_recurrence(ctx, s.q, s.k, s.v, s.g, s.beta, lc.state + (size_t)cc->state_cur * ssz,
-                                T, Hk, Hv, Dk, Dv, s.y, lc.state, capture ? 1 : 0));
-      TRY(ornith_rms_norm_gated(ctx, s.y, g.norm, s.z, T * Hv, Dv, c.rms_norm_eps, s.gated));
+      if (fused) {
+        TRY(ornith_gdn_step(ctx, conv_state, s.qkv, g.conv1d, dense_ab ? nullptr : s.a,
+                            dense_ab ? nullptr : s.b, dense_ab ? g.in_proj_a.d_w : nullptr,
+                            dense_ab ? g.in_proj_b.d_w : nullptr, dense_ab ? s.normed : nullptr, H, g.a_log,
+                            g.dt_bias, T, K, Hk, Dk, Hv, Dv, 1e-6f, state_in, lc.state, capture ? 1 : 0,
+                            g.norm, s.z, c.rms_norm_eps, lc.conv[1 - cc->conv_cur], s.gated));
+      } else {
+        TRY(ornith_gdn_front(ctx, conv_state, s.qkv, g.conv1d, s.a, s.b, g.a_log, g.dt_bias, T, K, Hk,
+                             Dk, Hv, Dv, 1e-6f, s.q, s.k, s.v, s.beta, s.g, lc.conv[1 - cc->conv_cur]));
+        TRY(ornith_gdn_recurrence(ctx, s.q, s.k, s.v, s.g, s.beta, state_in, T, Hk, Hv, Dk, Dv, s.y,
+                                  lc.state, capture ? 1 : 0));
+        TRY(ornith_rms_norm_gated(ctx, s.y, g.norm, s.z, T * Hv, Dv, c.rms_norm_eps, s.gated));
+      }
       TRY(ornith_linear_matmul(ctx, &g.out_proj, s.gated, T, s.r));
     } else {
       TRY(attention_block(m, L.attn, s.normed, T, lc.k, lc.v, cc->offset, cc->capacity, s.qg, s.kx,

@@ -61,3 +61,36 @@ def test_multi_matrix_launch_equals_separate(orn, ctx):
             for b in ys + [dx]: b.free()
         for w in ws: w.free()
 
+
+
+def test_gdn_step_fused_equals_separate_launches(orn, ctx):
+    """The gated-delta mixer core in one launch (a / b projections, front, recurrence with
+    snapshots, gated norm) against the four separate launches: same hidden rows, and after a
+    rewind the same continuation, for verify widths 1..4 and a 16-row prompt chunk."""
+    import synth
+    s = synth.SynthModel(synth.TINY, seed=21, with_mtp=False)
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    rng = np.random.default_rng(2)
+    toks = rng.integers(0, s.cfg["vocab_size"], 40).astype(np.uint32)
+
+    def run(fuse):
+        orn.set_option("fuse_gdn", fuse)
+        c = model.make_cache(64, 4)
+        out = [model.forward(c, toks[:16])]
+        pos = 16
+        for T, keep in ((4, 2), (1, 1), (3, 3), (2, 1), (4, 4)):
+            out.append(model.forward(c, toks[pos:pos + T], capture=True))
+            model.rewind(c, keep)
+            pos += keep
+        out.append(model.forward(c, toks[pos:pos + 5]))
+        c.close()
+        return out
+
+    try:
+        a, b = run(1), run(0)
+        for x, y in zip(a, b):
+            assert np.array_equal(x, y)
+    finally:
+        orn.set_option("fuse_gdn", 1)
+        model.close(); ws.close()
