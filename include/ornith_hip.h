@@ -71,6 +71,8 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *               rows per wavefront of the fused gate+up expert kernel, a tuning knob
  *   "fuse_gdn"  (ORNITH_FUSE_GDN, default 1): the gated-delta mixer core (a / b projections,
  *               front, recurrence, gated norm) in one launch at decode / verify widths
+ *   "fuse_norm" (ORNITH_FUSE_NORM, default 1): the residual add + RMS norm in front of a
+ *               group of k-quant projections / the router is computed inside their launch
  *   "gemm_rows" (ORNITH_GEMM_ROWS, default 32; 0 = never): activation rows from which the
  *               k-quant projections and the MoE experts run as matrix-core GEMMs instead of
  *               exact mat-vecs. The one switch that changes results (to bf16 rounding of the
@@ -168,6 +170,18 @@ ORNITH_API int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, con
 ORNITH_API int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, int n,
                                           const void* d_x, int M, void* const* d_ys);
 
+/* norm::add_rms_norm followed by the projections that read its output (the closing add of a
+ * decoder layer, the next layer's input norm and its in_proj_qkv + in_proj_z or q/k/v
+ * projections: src/model/qwen3_5.rs:374-396, 441-447, 493-499): h = res + y (bf16),
+ * normed = rms_norm(h, w_norm), ys[i] = normed . W_i^T. For k-quant projections of width 2048
+ * at M <= 4 the norm is made inside the projections' launch (every workgroup computes it while
+ * its weight loads are in flight; one of them stores h and normed); otherwise add_rms_norm and
+ * linear_matmul_multi are issued. Bit-identical either way. */
+ORNITH_API int ornith_add_rms_linear_multi(ornith_ctx* ctx, const ornith_linear* const* ws, int n,
+                                           const void* d_res, const void* d_y, const void* d_wnorm,
+                                           float eps, int M, void* d_h_out, void* d_normed_out,
+                                           void* const* d_ys);
+
 /* ops::matmul::gather_mv (src/ops/matmul.rs:649-): stacked dense bf16 experts
  * W[E,O,K]; out[r] = x[lhs[r]] . W[rhs[r]]^T. Used by the MTP head's MoE. */
 ORNITH_API int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K,
@@ -215,6 +229,15 @@ typedef struct ornith_moe_weights {
  * d_inds_out (u32 [T,k]) and d_scores_out (bf16 [T,k]) may be null. T <= 64. */
 ORNITH_API int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                                 void* d_out, uint32_t* d_inds_out, void* d_scores_out);
+
+/* norm::add_rms_norm followed by sparse_moe_block on its output (the post-attention norm and
+ * the MLP of a decoder layer, src/model/qwen3_5.rs:384-392): h = res + y, normed =
+ * rms_norm(h, w_norm), out = moe(normed). With the fused expert kernels, hidden size 2048 and
+ * T <= 4 the norm is made inside the router's launch; otherwise add_rms_norm is issued first.
+ * Bit-identical either way. */
+ORNITH_API int ornith_add_rms_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_res,
+                                        const void* d_y, const void* d_wnorm, float eps, int T,
+                                        void* d_h_out, void* d_normed_out, void* d_out);
 
 
 /* moe::switch_glu_rows + the shared expert + moe::combine (src/ops/moe.rs:256-338,548-596)

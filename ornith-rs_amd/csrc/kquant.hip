@@ -24,6 +24,7 @@
 //   read the same activations (q/k/v projections, in_proj_qkv + in_proj_z): the
 //   grid is the concatenation of their row ranges.
 #include "kq_device.h"
+#include "norm_device.h"
 #include "rt.h"
 
 namespace {
@@ -49,13 +50,17 @@ struct KqArgs {
   int E, x_rows;  // gather only: bounds for rhs / lhs (out-of-range ids are clamped)
   int iters;      // row iterations per wavefront
   int y_bf16;     // 1: round outputs to bf16, 0: fp32
+  PreNorm pre;    // PRE kernels: the activations are rms_norm(res + y) computed by every workgroup
 };
 
 // One kernel for plain and gathered mat-vecs.
 //   KIND  format; LPR lanes per row (4,8,16,32,64); KS wavefronts per row (1,2)
 //   M     activation rows sharing each weight read (1..4); gather uses M == 1
 //   grid.x covers output rows (of all segments), grid.y is the gather row
-template <int KIND, int LPR, int KS, int M, bool XF32, bool GATHER>
+//   PRE   the activation rows are not read but made: every workgroup computes
+//         h = res + y, x = rms_norm(h) of the M rows (K == 2048) into LDS while its weight
+//         loads are in flight; workgroup 0 also stores h and x for later consumers
+template <int KIND, int LPR, int KS, int M, bool XF32, bool GATHER, bool PRE = false>
 __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
   using KL = KqLane<KIND, M>;
   constexpr int RPW = 64 / LPR;  // rows in flight per wavefront
@@ -107,6 +112,12 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
 #pragma unroll
   for (int i = 0; i < PF; ++i) pf[i] = KL::load(sg.qs, sg.scales, sg.dm, row_of(i), nb, L);
   __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  if constexpr (PRE) {
+    __shared__ PreNormLds<M> pn;
+    prenorm_rows<M>(a.pre, blockIdx.x == 0, pn);
+#pragma unroll
+    for (int t = 0; t < M; ++t) xrow[t] = &pn.xn[t][0];
+  }
   L.template load_x<XF32>(xrow, c + 64 * ks);
 
   for (int it0 = 0; it0 < a.iters; it0 += PF) {
@@ -248,6 +259,23 @@ int launch_shape(ornith_ctx* ctx, KqArgs& a, int grid_y) {
   }
 }
 
+template <int KIND, int LPR, int M>
+int launch_pre(ornith_ctx* ctx, KqArgs& a) {
+  dim3 grid(layout_segments<LPR, 1>(a), 1, 1);
+  hipLaunchKernelGGL((kq_qmv_kernel<KIND, LPR, 1, M, false, false, true>), grid, dim3(256), 0, ctx->stream, a);
+  ORN_LAUNCH_CHECK("kq_qmv_kernel<pre-norm>");
+  return ORNITH_OK;
+}
+template <int KIND, int LPR>
+int launch_pre_m(ornith_ctx* ctx, KqArgs& a, int M) {
+  switch (M) {
+    case 1: return launch_pre<KIND, LPR, 1>(ctx, a);
+    case 2: return launch_pre<KIND, LPR, 2>(ctx, a);
+    case 3: return launch_pre<KIND, LPR, 3>(ctx, a);
+    default: return launch_pre<KIND, LPR, 4>(ctx, a);
+  }
+}
+
 template <int KIND, bool XF32>
 int launch_m(ornith_ctx* ctx, KqArgs& a, int M) {
   switch (M) {
@@ -323,6 +351,36 @@ int ornith_kq_dequantize(ornith_ctx* ctx, const ornith_kmatrix* w, void* d_out, 
                        (const uint16_t*)w->d_dm, blocks, d_out, out_dtype == ORNITH_BF16);
   ORN_LAUNCH_CHECK("kq_dequant_kernel");
   return ORNITH_OK;
+}
+
+// ys[i] = rms_norm(res + y, w_norm) . W_i^T with the norm made inside the launch.
+// Returns -1 (nothing launched) when the shapes are outside what the kernel covers.
+int kq_qmv_multi_prenorm(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n, const void* d_res,
+                         const void* d_y, const void* d_wnorm, float eps, int M, void* d_h_out,
+                         void* d_normed_out, void* const* d_ys) {
+  if (n < 1 || n > kMaxSeg || M < 1 || M > 4 || ws[0]->K != kPreN) return -1;
+  long total = 0;
+  for (int s = 0; s < n; ++s) {
+    if (check_matrix(ws[s], "kq_qmv_prenorm")) return -1;
+    if (ws[s]->E != 1 || ws[s]->kind != ws[0]->kind || ws[s]->K != ws[0]->K || !d_ys[s]) return -1;
+    total += ws[s]->O;
+  }
+  KqArgs a{};
+  a.nseg = n;
+  a.K = kPreN;
+  a.y_bf16 = 1;
+  a.iters = pick_iters(ctx, ws[0]->kind, kPreN, total, 1);
+  for (int s = 0; s < n; ++s) {
+    a.seg[s].qs = (const uint8_t*)ws[s]->d_qs;
+    a.seg[s].scales = (const uint8_t*)ws[s]->d_scales;
+    a.seg[s].dm = (const uint16_t*)ws[s]->d_dm;
+    a.seg[s].O = ws[s]->O;
+    a.seg[s].y = d_ys[s];
+  }
+  a.pre = PreNorm{(const bf16_t*)d_res, (const bf16_t*)d_y, (const bf16_t*)d_wnorm, (bf16_t*)d_h_out,
+                  (bf16_t*)d_normed_out, eps};
+  return ws[0]->kind == ORNITH_Q4K ? launch_pre_m<ORNITH_Q4K, 64>(ctx, a, M)
+                                   : launch_pre_m<ORNITH_Q6K, 32>(ctx, a, M);
 }
 
 int ornith_kq_qmv_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n, const void* d_x,

@@ -14,6 +14,11 @@
 #include "linear_device.h"
 #include "rt.h"
 
+// kquant.hip
+extern "C" int kq_qmv_multi_prenorm(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n,
+                                    const void* d_res, const void* d_y, const void* d_wnorm, float eps,
+                                    int M, void* d_h_out, void* d_normed_out, void* const* d_ys);
+
 namespace {
 
 // ---- 8-bit affine, group 64 ---------------------------------------------
@@ -162,6 +167,26 @@ int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, 
     if (rc) return rc;
   }
   return ORNITH_OK;
+}
+
+int ornith_add_rms_linear_multi(ornith_ctx* ctx, const ornith_linear* const* ws, int n,
+                                const void* d_res, const void* d_y, const void* d_wnorm, float eps, int M,
+                                void* d_h_out, void* d_normed_out, void* const* d_ys) {
+  ORN_REQUIRE(ctx && ws && d_res && d_y && d_wnorm && d_h_out && d_normed_out && d_ys && n >= 1,
+              "add_rms_linear_multi: bad argument");
+  bool fuse = ornith_option_fuse_norm() && n <= 4 && M <= 4;
+  const ornith_kmatrix* kms[4];
+  for (int i = 0; i < n && fuse; ++i) {
+    fuse = ws[i] && ws[i]->mode == ORNITH_LIN_KQUANT && ws[i]->K == 2048;
+    if (fuse) kms[i] = &ws[i]->km;
+  }
+  if (fuse) {
+    const int rc = kq_qmv_multi_prenorm(ctx, kms, n, d_res, d_y, d_wnorm, eps, M, d_h_out, d_normed_out, d_ys);
+    if (rc >= 0) return rc;
+  }
+  int rc = ornith_add_rms_norm(ctx, d_res, d_y, d_wnorm, M, ws[0]->K, eps, d_h_out, d_normed_out);
+  if (rc) return rc;
+  return ornith_linear_matmul_multi(ctx, ws, n, d_normed_out, M, d_ys);
 }
 
 int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K, const void* d_x,

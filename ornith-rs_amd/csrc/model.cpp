@@ -159,15 +159,25 @@ int model_ensure_rope(ornith_model* m, int npos) {
 
 // q/k/v projections, per-head norm + rope + append, attention + gate; the caller applies
 // o_proj to `att`. qg, kx, vx, q_rot, att hold at least T rows.
-static int attention_block(ornith_model* m, const AttnLayer& a, const void* d_x, int T, void* k_cache,
+// With `pend`, d_x is not ready yet: it is rms_norm(pend->res + pend->y) and the q/k/v launch
+// makes it (and stores it to d_x, and the sum to pend->h_out).
+struct PendingNorm {
+  const void *res, *y, *w;
+  void* h_out;
+};
+static int attention_block(ornith_model* m, const AttnLayer& a, void* d_x, int T, void* k_cache,
                            void* v_cache, int offset, int cap, char* qg, char* kx, char* vx,
-                           char* q_rot, char* att) {
+                           char* q_rot, char* att, const PendingNorm* pend) {
   ornith_ctx* ctx = m->ctx;
   const auto& c = m->cfg;
   {
     const ornith_linear* ws[3] = {&a.q_proj, &a.k_proj, &a.v_proj};
     void* ys[3] = {qg, kx, vx};
-    TRY(ornith_linear_matmul_multi(ctx, ws, 3, d_x, T, ys));
+    if (pend)
+      TRY(ornith_add_rms_linear_multi(ctx, ws, 3, pend->res, pend->y, pend->w, c.rms_norm_eps, T,
+                                      pend->h_out, d_x, ys));
+    else
+      TRY(ornith_linear_matmul_multi(ctx, ws, 3, d_x, T, ys));
   }
   TRY(ornith_attn_prep(ctx, qg, kx, vx, a.q_norm, a.k_norm, T, c.num_attention_heads,
                        c.num_key_value_heads, c.head_dim, c.rope_dims, c.rms_norm_eps, m->d_cos,
@@ -191,11 +201,19 @@ static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_to
   for (size_t i = 0; i < m->layers.size(); ++i) {
     const Layer& L = m->layers[i];
     LayerCache& lc = cc->layers[i];
+    // From the second layer on the layer's input norm is still owed: x = h + mo of the layer
+    // before, normed = rms_norm(x, input_ln). The first projections of the mixer make it.
+    const PendingNorm pend{s.h, s.mo, L.input_ln, s.x};
+    const PendingNorm* pp = i > 0 ? &pend : nullptr;
     if (L.linear) {
       const GdnLayer& g = L.gdn;
       const ornith_linear* big[2] = {&g.in_proj_qkv, &g.in_proj_z};
       void* ybig[2] = {s.qkv, s.z};
-      TRY(ornith_linear_matmul_multi(ctx, big, 2, s.normed, T, ybig));
+      if (pp)
+        TRY(ornith_add_rms_linear_multi(ctx, big, 2, pp->res, pp->y, pp->w, c.rms_norm_eps, T, pp->h_out,
+                                        s.normed, ybig));
+      else
+        TRY(ornith_linear_matmul_multi(ctx, big, 2, s.normed, T, ybig));
       const char* conv_state = (const char*)lc.conv[cc->conv_cur] + (size_t)cc->conv_off * D * 2;
       const float* state_in = lc.state + (size_t)cc->state_cur * ssz;
       const bool dense_ab = g.in_proj_a.mode == ORNITH_LIN_DENSE && g.in_proj_b.mode == ORNITH_LIN_DENSE;
@@ -221,14 +239,13 @@ static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_to
       TRY(ornith_linear_matmul(ctx, &g.out_proj, s.gated, T, s.r));
     } else {
       TRY(attention_block(m, L.attn, s.normed, T, lc.k, lc.v, cc->offset, cc->capacity, s.qg, s.kx,
-                          s.vx, s.q_rot, s.att));
+                          s.vx, s.q_rot, s.att, pp));
       TRY(ornith_linear_matmul(ctx, &L.attn.o_proj, s.att, T, s.r));
     }
-    TRY(ornith_add_rms_norm(ctx, s.x, s.r, L.post_ln, T, H, c.rms_norm_eps, s.h, s.normed2));
-    const void* next_w = (i + 1 < m->layers.size()) ? m->layers[i + 1].input_ln : m->final_norm;
-    TRY(ornith_moe_block(ctx, &L.moe, s.normed2, T, s.mo, nullptr, nullptr));
-    TRY(ornith_add_rms_norm(ctx, s.h, s.mo, next_w, T, H, c.rms_norm_eps, s.x, s.normed));
+    TRY(ornith_add_rms_moe_block(ctx, &L.moe, s.x, s.r, L.post_ln, c.rms_norm_eps, T, s.h, s.normed2, s.mo));
   }
+  // the last layer's closing add and the model's final norm
+  TRY(ornith_add_rms_norm(ctx, s.h, s.mo, m->final_norm, T, H, c.rms_norm_eps, s.x, s.normed));
   TRY(ornith_copy(ctx, d_hidden_out, s.normed, (size_t)T * H * 2));
   // every layer advanced together
   cc->conv_cur = 1 - cc->conv_cur;
@@ -652,7 +669,8 @@ int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspec, const vo
   }
   TRY(ornith_linear_matmul(ctx, &h->fc, joined, T, x));
   TRY(ornith_rms_norm(ctx, x, h->input_ln, T, (int)H, c.rms_norm_eps, normed));
-  TRY(attention_block(m, h->attn, normed, T, h->k, h->v, h->offset, h->capacity, qg, kx, vx, q_rot, att));
+  TRY(attention_block(m, h->attn, normed, T, h->k, h->v, h->offset, h->capacity, qg, kx, vx, q_rot, att,
+                      nullptr));
   TRY(ornith_linear_matmul(ctx, &h->attn.o_proj, att, T, r));
   TRY(ornith_add_rms_norm(ctx, x, r, h->post_ln, T, (int)H, c.rms_norm_eps, hh, normed2));
   // add(h, m) then mtp.norm; the un-normed sum is not needed afterwards

@@ -10,12 +10,13 @@
 // Rounding points are the reference's: gates, probabilities, every expert output
 // and every step of the tail are bf16; sums inside a kernel are fp32.
 #include "moe_device.h"
+#include "norm_device.h"
 #include "rt.h"
 
 // moe_fused.hip
 bool moe_fused_supported(const ornith_moe_weights* w);
 bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                      void* d_gates, void* d_egate, int* rc);
+                      void* d_gates, void* d_egate, int* rc, const PreNorm* pre);
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
                       void* d_out, int phases);
@@ -175,8 +176,11 @@ int ornith_moe_combine(ornith_ctx* ctx, const void* d_scores, const void* d_y, c
   return ORNITH_OK;
 }
 
-int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                     void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
+// The block. With `pre`, x is rms_norm(pre->res + pre->y): made inside the router launch when
+// the fused kernels cover the shapes (d_x then is where the normed rows get stored, and read
+// back by the expert kernels), by a separate add_rms_norm otherwise.
+static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                          void* d_out, uint32_t* d_inds_out, void* d_scores_out, const PreNorm* pre) {
   ORN_REQUIRE(ctx && w && d_x && d_out, "moe_block: null argument");
   const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
   ORN_REQUIRE(T >= 1 && T <= 8192, "moe_block: T=%d", T);
@@ -192,6 +196,14 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
                   w->sh_egate.O == 1,
               "moe_block: shared expert shapes do not chain");
   const int SI = w->sh_gate.O;
+  const bool pre_in_kernel = pre && T <= 4 && H == kPreN && ornith_option_fuse_norm() &&
+                             ornith_option_fuse_moe() && moe_fused_supported(w) &&
+                             w->router.mode == ORNITH_LIN_KQUANT;
+  if (pre && !pre_in_kernel) {
+    int rcn = ornith_add_rms_norm(ctx, pre->res, pre->y, pre->w, T, H, pre->eps, pre->h_out, pre->normed_out);
+    if (rcn) return rcn;
+    pre = nullptr;
+  }
   if (T >= kPrefillRows && !w->ex_dense) {
     ORN_REQUIRE(!d_inds_out && !d_scores_out, "moe_block: index outputs are a decode-width feature");
     return moe_block_prefill(ctx, w, d_x, T, d_out);
@@ -228,9 +240,10 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
   if (ornith_option_fuse_moe() && moe_fused_supported(w)) {
     // gates + shared-expert gate, softmax + top-k, then the two expert kernels
     int rrc = ORNITH_OK;
-    if (moe_fused_router(ctx, w, d_x, T, gates, eg, &rrc)) {
+    if (moe_fused_router(ctx, w, d_x, T, gates, eg, &rrc, pre)) {
       if (rrc) return rrc;
     } else {
+      if (pre) TRY(ornith_add_rms_norm(ctx, pre->res, pre->y, pre->w, T, H, pre->eps, pre->h_out, pre->normed_out));
       TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
       TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
     }
@@ -275,6 +288,20 @@ int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d
                            ctx->stream));
 #undef TRY
   return ORNITH_OK;
+}
+
+int ornith_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                     void* d_out, uint32_t* d_inds_out, void* d_scores_out) {
+  return moe_block_impl(ctx, w, d_x, T, d_out, d_inds_out, d_scores_out, nullptr);
+}
+
+int ornith_add_rms_moe_block(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_res,
+                             const void* d_y, const void* d_wnorm, float eps, int T, void* d_h_out,
+                             void* d_normed_out, void* d_out) {
+  ORN_REQUIRE(d_res && d_y && d_wnorm && d_h_out && d_normed_out, "add_rms_moe_block: null argument");
+  const PreNorm pre{(const bf16_t*)d_res, (const bf16_t*)d_y, (const bf16_t*)d_wnorm, (bf16_t*)d_h_out,
+                    (bf16_t*)d_normed_out, eps};
+  return moe_block_impl(ctx, w, d_normed_out, T, d_out, nullptr, nullptr, &pre);
 }
 
 }  // extern "C"

@@ -25,6 +25,7 @@
 // nothing but the index list), then the activation loads, and only then computes.
 #include "kq_device.h"
 #include "moe_device.h"
+#include "norm_device.h"
 #include "rt.h"
 
 namespace {
@@ -206,6 +207,8 @@ struct RouterArgs {
   const bf16_t* eg_b;    // affine8 biases [K/64]
   int eg_affine;
   int E, K;
+  PreNorm pre;           // pre.res != null: x is not read but made, x = rms_norm(res + y) (K == 2048),
+                         // by every workgroup; workgroup 0 stores h and x
 };
 
 // one row of the 8-bit affine / dense mat-vec by one wavefront (the order of linear.hip)
@@ -249,9 +252,12 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
   using KL = KqLane<KIND, M>;
   constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ PreNormLds<M> pn;
+  const bool pre = a.pre.res != nullptr;
   if (blockIdx.x == gridDim.x - 1) {
+    if (pre) prenorm_rows<M>(a.pre, false, pn);
     if (wave < M) {
-      const float e = egate_row_dot(a, a.x + (size_t)wave * a.K, lane);
+      const float e = egate_row_dot(a, pre ? &pn.xn[wave][0] : a.x + (size_t)wave * a.K, lane);
       if (lane == 0) a.egate[wave] = dm_f2bf(e);
     }
     return;
@@ -263,9 +269,10 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
   const int o = (blockIdx.x * 4 + wave) * RPW + slot;
   const typename KL::Row row = KL::load(a.w.qs, a.w.scales, a.w.dm, o < a.E ? o : a.E - 1, nb, L);
   __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  if (pre) prenorm_rows<M>(a.pre, blockIdx.x == 0, pn);
   const void* xrow[M];
 #pragma unroll
-  for (int t = 0; t < M; ++t) xrow[t] = a.x + (size_t)t * a.K;
+  for (int t = 0; t < M; ++t) xrow[t] = pre ? (const void*)&pn.xn[t][0] : (const void*)(a.x + (size_t)t * a.K);
   L.template load_x<false>(xrow, c);
   float acc[M];
 #pragma unroll
@@ -346,7 +353,7 @@ bool moe_fused_supported(const ornith_moe_weights* w) {
 // Router mat-vec + shared_expert_gate in one launch. Returns false (nothing launched)
 // when the shapes / formats are outside what the kernel covers.
 bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
-                      void* d_gates, void* d_egate, int* rc) {
+                      void* d_gates, void* d_egate, int* rc, const PreNorm* pre) {
   *rc = ORNITH_OK;
   const ornith_linear& r = w->router;
   const ornith_linear& g = w->sh_egate;
@@ -367,6 +374,10 @@ bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
   a.eg_affine = g.mode == ORNITH_LIN_AFFINE8;
   a.E = E;
   a.K = r.K;
+  if (pre) {
+    if (r.K != kPreN) return false;
+    a.pre = *pre;
+  }
 #define R_CASE(KIND, N) \
   case N:               \
     launch_router_fused<KIND, N>(ctx, a, T); \

@@ -98,3 +98,69 @@ __device__ __forceinline__ void rms_row(const bf16_t* a, const bf16_t* b, const 
   }
   store_bf16<PER>(out + base, x);
 }
+
+// Residual add + RMS norm of T <= 4 rows of 2048 values by one 256-thread workgroup, for
+// kernels that consume the normed rows themselves: h = bf16(res + y),
+// normed = bf16(w * bf16(h * inv)). The rows land in LDS (xn); the workgroup for which
+// `write_global` holds also stores h and normed for later consumers. Same arithmetic and
+// order as rms_wide_kernel<32, NORM_ADD> (wavefront t sums row t), so a consumer that
+// recomputes the norm per workgroup sees the bits the stand-alone kernel would have written.
+struct PreNorm {
+  const bf16_t* res;     // [T, 2048]
+  const bf16_t* y;       // [T, 2048]
+  const bf16_t* w;       // [2048]
+  bf16_t* h_out;         // [T, 2048]
+  bf16_t* normed_out;    // [T, 2048]
+  float eps;
+};
+
+constexpr int kPreN = 2048;
+
+template <int T>
+struct PreNormLds {
+  float xs[T * kPreN];
+  __attribute__((aligned(16))) bf16_t xn[T][kPreN];
+  float inv[4];
+};
+
+template <int T>
+__device__ __forceinline__ void prenorm_rows(const PreNorm& p, bool write_global, PreNormLds<T>& s) {
+  static_assert(T >= 1 && T <= 4, "one wavefront per row");
+  constexpr int PER = kPreN / 64;
+  const int tid = threadIdx.x, e0 = tid * 8, lane = tid & 63, wave = tid >> 6;
+  const int lane_of = e0 / PER, pos0 = e0 % PER;
+  float x[T][8], wv[8];
+  load_bf16<8>(p.w + e0, wv);
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    float yv[8];
+    load_bf16<8>(p.res + (size_t)t * kPreN + e0, x[t]);
+    load_bf16<8>(p.y + (size_t)t * kPreN + e0, yv);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[t][i] = dm_rb(x[t][i] + yv[i]);
+    if (write_global) store_bf16<8>(p.h_out + (size_t)t * kPreN + e0, x[t]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s.xs[t * kPreN + (pos0 + i) * 64 + lane_of] = x[t][i];
+  }
+  __syncthreads();
+  if (wave < T) {
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const float v = s.xs[wave * kPreN + i * 64 + lane];
+      acc = dm_fma(v, v, acc);
+    }
+    const float inv = dm_rsqrt(dm_wave_sum<64>(acc) / (float)kPreN + p.eps);
+    if (lane == 0) s.inv[wave] = inv;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const float inv = s.inv[t];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[t][i] = dm_rb(wv[i] * dm_rb(x[t][i] * inv));
+    store_bf16<8>(&s.xn[t][e0], x[t]);
+    if (write_global) store_bf16<8>(p.normed_out + (size_t)t * kPreN + e0, x[t]);
+  }
+  __syncthreads();
+}

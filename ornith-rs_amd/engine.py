@@ -378,3 +378,17 @@ def kq_gather_plan_bytes(pairs, E):
 def kq_gather_matmul(ctx, w, x, inds, pairs, top_k, is_up, plan, rebuild, y):
     _check(lib().ornith_kq_gather_matmul(ctx.h, C.byref(w.s), x.ptr, inds.ptr, pairs, top_k, int(is_up),
                                          plan.ptr, int(rebuild), y.ptr), "kq_gather_matmul")
+
+
+# ---- norm folded into its consumers -----------------------------------------------------------
+def add_rms_linear_multi(ctx, lins, res, y, wnorm, eps, M, h_out, normed_out, ys):
+    n = len(lins)
+    wp = (C.c_void_p * n)(*[C.cast(C.pointer(l.s), C.c_void_p) for l in lins])
+    yp = (C.c_void_p * n)(*[b.ptr for b in ys])
+    _check(lib().ornith_add_rms_linear_multi(ctx.h, wp, n, res.ptr, y.ptr, wnorm.ptr, C.c_float(eps), M,
+                                             h_out.ptr, normed_out.ptr, yp), "add_rms_linear_multi")
+
+
+def add_rms_moe_block(ctx, w, res, y, wnorm, eps, T, h_out, normed_out, out):
+    _check(lib().ornith_add_rms_moe_block(ctx.h, C.byref(w), res.ptr, y.ptr, wnorm.ptr, C.c_float(eps), T,
+                                          h_out.ptr, normed_out.ptr, out.ptr), "add_rms_moe_block")

@@ -94,3 +94,56 @@ def test_gdn_step_fused_equals_separate_launches(orn, ctx):
     finally:
         orn.set_option("fuse_gdn", 1)
         model.close(); ws.close()
+
+
+@pytest.mark.parametrize("kind,Os", [(Q4K, (8192, 4096)), (Q6K, (8192, 512, 512)), (Q4K, (40,))])
+def test_norm_inside_projection_launch_equals_separate(orn, ctx, kind, Os):
+    """add_rms_norm made inside the launch of the projections that read it (every workgroup
+    recomputes it, one stores it) == add_rms_norm, then the projections: h, normed and every
+    projection output, at M = 1..4, plus the M = 6 and fuse_norm = 0 fall-backs."""
+    rng = np.random.default_rng(sum(Os) + kind)
+    H = 2048
+    lins = [orn.Linear.kquant(ctx, kind, *util.make_kq(kind, rng, 1, O, H), O, H) for O in Os]
+    wn = ctx.to_device(util.bf16_normal(rng, (H,)))
+    try:
+        for M, fuse in ((1, 1), (2, 1), (3, 1), (4, 1), (6, 1), (2, 0), (2, 1)):
+            orn.set_option("fuse_norm", fuse)
+            res, y = ctx.to_device(util.bf16_normal(rng, (M, H))), ctx.to_device(util.bf16_normal(rng, (M, H)))
+            h1, n1, h2, n2 = (ctx.alloc(M * H * 2) for _ in range(4))
+            ys1 = [ctx.alloc(M * O * 2) for O in Os]
+            ys2 = [ctx.alloc(M * O * 2) for O in Os]
+            orn.add_rms_linear_multi(ctx, lins, res, y, wn, 1e-6, M, h1, n1, ys1)
+            ctx.add_rms_norm(res, y, wn, M, H, 1e-6, h2, n2)
+            for l, yy in zip(lins, ys2):
+                ctx.linear_matmul(l, n2, M, yy)
+            assert np.array_equal(h1.download(np.uint16, (M, H)), h2.download(np.uint16, (M, H))), (M, fuse)
+            assert np.array_equal(n1.download(np.uint16, (M, H)), n2.download(np.uint16, (M, H))), (M, fuse)
+            for a, b, O in zip(ys1, ys2, Os):
+                assert np.array_equal(a.download(np.uint16, (M, O)), b.download(np.uint16, (M, O))), (M, fuse, O)
+            for b in [res, y, h1, n1, h2, n2] + ys1 + ys2: b.free()
+    finally:
+        orn.set_option("fuse_norm", 1)
+        wn.free()
+        for l in lins: l.free()
+
+
+def test_norm_inside_router_launch_equals_separate(orn, ctx):
+    rng = np.random.default_rng(77)
+    H = 2048
+    moe = util.HostMoe(rng, H=H, E=256, I=512, top_k=8, gate_kind=Q4K, down_kind=Q6K, router_kind=Q6K)
+    dw = moe.dev(orn, ctx)
+    wn = ctx.to_device(util.bf16_normal(rng, (H,)))
+    try:
+        for T, fuse in ((1, 1), (2, 1), (4, 1), (7, 1), (2, 0)):
+            orn.set_option("fuse_norm", fuse)
+            res, y = ctx.to_device(util.bf16_normal(rng, (T, H))), ctx.to_device(util.bf16_normal(rng, (T, H)))
+            h1, n1, o1, h2, n2, o2 = (ctx.alloc(T * H * 2) for _ in range(6))
+            orn.add_rms_moe_block(ctx, dw, res, y, wn, 1e-6, T, h1, n1, o1)
+            ctx.add_rms_norm(res, y, wn, T, H, 1e-6, h2, n2)
+            ctx.moe_block(dw, n2, T, o2)
+            for a, b in ((h1, h2), (n1, n2), (o1, o2)):
+                assert np.array_equal(a.download(np.uint16, (T, H)), b.download(np.uint16, (T, H))), (T, fuse)
+            for b in (res, y, h1, n1, o1, h2, n2, o2): b.free()
+    finally:
+        orn.set_option("fuse_norm", 1)
+        wn.free(); moe.free()
