@@ -19,7 +19,7 @@ bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
                       void* d_gates, void* d_egate, int* rc, const PreNorm* pre);
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
-                      void* d_out, int phases);
+                      void* d_out, int phases, const void* d_gates);
 
 namespace {
 
@@ -247,8 +247,11 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
       TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
       TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
     }
-    TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
-    TRY(moe_fused_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, 3));
+    // softmax + top-k ride in the head of the up kernel (the reference folds its routing
+    // tail the same way, ORNITH_FUSE_MOE_TAIL); E must be one of the wavefront layouts
+    const bool topk_in_up = E % 64 == 0 && E <= 1024 && ((E / 64) & (E / 64 - 1)) == 0 && k <= 16;
+    if (!topk_in_up) TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
+    TRY(moe_fused_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, 3, topk_in_up ? gates : nullptr));
     if (d_inds_out)
       ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice,
                              ctx->stream));

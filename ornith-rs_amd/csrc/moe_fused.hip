@@ -43,6 +43,12 @@ struct UpArgs {
   const uint32_t* inds;  // [T*k]
   bf16_t* act;           // [T*k + T, I]
   int T, k, E, I, K;
+  // gates != null: the routing is not read but made -- every workgroup of a routed row runs
+  // softmax + top-k over its token's gates (one wavefront, ~400 instructions) and the first
+  // workgroup of each token stores inds / scores for the down kernel
+  const bf16_t* gates;   // [T, E]
+  uint32_t* inds_out;    // [T*k]
+  bf16_t* scores_out;    // [T*k]
 };
 
 __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
@@ -66,7 +72,30 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
   KqPtr wg, wu;
   if (r < routed) {
     token = r / a.k;
-    row0 = (int64_t)min(a.inds[r], (uint32_t)(a.E - 1)) * a.I;
+    uint32_t e;
+    if (a.gates) {
+      __shared__ uint32_t s_inds[16];
+      __shared__ bf16_t s_scores[16];
+      if (wave == 0) {
+        const bf16_t* g = a.gates + (size_t)token * a.E;
+        switch (a.E / 64) {
+          case 1: router_topk_wave<1>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+          case 2: router_topk_wave<2>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+          case 4: router_topk_wave<4>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+          case 8: router_topk_wave<8>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+          default: router_topk_wave<16>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+        }
+      }
+      __syncthreads();
+      e = s_inds[r - token * a.k];
+      if (blockIdx.x == 0 && r == token * a.k && threadIdx.x < a.k) {
+        a.inds_out[r + threadIdx.x] = s_inds[threadIdx.x];
+        a.scores_out[r + threadIdx.x] = s_scores[threadIdx.x];
+      }
+    } else {
+      e = a.inds[r];
+    }
+    row0 = (int64_t)min(e, (uint32_t)(a.E - 1)) * a.I;
     wg = a.gate;
     wu = a.up;
   } else {
@@ -394,9 +423,11 @@ bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
 }
 
 // act: scratch bf16 [(T*k + T), I]. phases: 1 = up, 2 = down, 3 = both.
+// d_gates != null (phases & 1): the up kernel makes the routing from the gates and stores it
+// to d_inds / d_scores (which then are outputs).
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
-                      void* d_out, int phases) {
+                      void* d_out, int phases, const void* d_gates) {
   const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
   if (phases & 1) {
     UpArgs a{};
@@ -412,6 +443,9 @@ int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
     a.E = E;
     a.I = I;
     a.K = H;
+    a.gates = (const bf16_t*)d_gates;
+    a.inds_out = const_cast<uint32_t*>(d_inds);
+    a.scores_out = (bf16_t*)const_cast<void*>(d_scores);
     const int nch = chunks_of(w->ex_gate), rows_y = T * k + T;
 #define UP_CASE(KIND, N) \
   case N:                \
@@ -468,7 +502,7 @@ int ornith_moe_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void*
     return ornith_fail(ORNITH_ERR_UNSUPPORTED,
                        "moe_experts: the fused expert kernels need k-quant routed and shared experts "
                        "of matching formats and top_k <= %d", kMaxK);
-  return moe_fused_experts(ctx, w, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, phases);
+  return moe_fused_experts(ctx, w, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, phases, nullptr);
 }
 
 }  // extern "C"
