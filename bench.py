@@ -162,7 +162,7 @@ def main():
                     help="instead of the metric's workload: BASELINE config 5 (6621-token prefill into a "
                          "16384-token context through the matrix-core path, then sampled depth-3 MTP "
                          "decode of 256 tokens, temperature 0.8, top-p 0.95); prints its own JSON line")
-    ap.add_argument("--prefill-chunk", type=int, default=512)
+    ap.add_argument("--prefill-chunk", type=int, default=2048)
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the expert-kernel timing loop plus three 256 MiB device copies "
                          "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")

@@ -50,13 +50,39 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
   return (uint32_t)dm_f2bf(a) | ((uint32_t)dm_f2bf(b) << 16);
 }
 
-// 64 weights of row `row` (already offset by the expert), 64-group `grp` of super-block
-// `ib`, as bf16 into dst[0..64)
-__device__ __forceinline__ void dequant64_q4k(const MmArgs& a, int64_t row, int nb, int ib, int grp,
-                                              bf16_t* dst) {
+// ---- weight slab pieces: loaded as codes into registers (so the loads of the next slab can
+// be in flight while the matrix cores work on this one), dequantized on the way into LDS ----
+struct BRegsQ4 {
+  uint4 q0, q1;
+  uint32_t s0, s1, s2, dmw;
+};
+struct BRegsQ6 {
+  uint4 qa, qb, qh;
+  uint2 sc;
+  uint32_t d;
+};
+
+// 64-group `grp` of super-block `ib` of weight row `row`
+__device__ __forceinline__ BRegsQ4 load_q4k(const MmArgs& a, int64_t row, int nb, int ib, int grp) {
   const int64_t blk = row * nb + ib;
-  const uint8_t* sc = a.scales + blk * 12;
-  const float d = dm_h2f(a.dm[blk * 2]), dmin = dm_h2f(a.dm[blk * 2 + 1]);
+  BRegsQ4 r;
+  const uint4* q = reinterpret_cast<const uint4*>(a.qs + blk * 128 + grp * 32);
+  r.q0 = q[0];
+  r.q1 = q[1];
+  const uint32_t* sc = reinterpret_cast<const uint32_t*>(a.scales + blk * 12);
+  r.s0 = sc[0];
+  r.s1 = sc[1];
+  r.s2 = sc[2];
+  r.dmw = *reinterpret_cast<const uint32_t*>(a.dm + blk * 2);
+  return r;
+}
+
+// 64 weights as bf16 into dst[0..64): d*sc*q - dmin*m (kquant::dequantize, q4k.metal:64-96)
+__device__ __forceinline__ void dequant_q4k(const BRegsQ4& r, int grp, bf16_t* dst) {
+  const uint8_t sc[12] = {(uint8_t)r.s0, (uint8_t)(r.s0 >> 8), (uint8_t)(r.s0 >> 16), (uint8_t)(r.s0 >> 24),
+                          (uint8_t)r.s1, (uint8_t)(r.s1 >> 8), (uint8_t)(r.s1 >> 16), (uint8_t)(r.s1 >> 24),
+                          (uint8_t)r.s2, (uint8_t)(r.s2 >> 8), (uint8_t)(r.s2 >> 16), (uint8_t)(r.s2 >> 24)};
+  const float d = dm_h2f((f16_t)(r.dmw & 0xffffu)), dmin = dm_h2f((f16_t)(r.dmw >> 16));
   float dd[2], mm[2];
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
@@ -72,43 +98,44 @@ __device__ __forceinline__ void dequant64_q4k(const MmArgs& a, int64_t row, int 
     dd[k] = d * (float)s;
     mm[k] = dmin * (float)m;
   }
-  const uint4* q = reinterpret_cast<const uint4*>(a.qs + blk * 128 + grp * 32);
   uint32_t* out = reinterpret_cast<uint32_t*>(dst);
+  const uint32_t w[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const uint4 v = q[h];
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t b = w[i];
-      const float l0 = dd[0] * (float)(b & 0xF) - mm[0], l1 = dd[0] * (float)((b >> 8) & 0xF) - mm[0];
-      const float l2 = dd[0] * (float)((b >> 16) & 0xF) - mm[0], l3 = dd[0] * (float)((b >> 24) & 0xF) - mm[0];
-      const float h0 = dd[1] * (float)((b >> 4) & 0xF) - mm[1], h1 = dd[1] * (float)((b >> 12) & 0xF) - mm[1];
-      const float h2 = dd[1] * (float)((b >> 20) & 0xF) - mm[1], h3 = dd[1] * (float)(b >> 28) - mm[1];
-      const int e = 16 * h + 4 * i;  // element index within the low / high run of 32
-      out[(e >> 1)] = pack2(l0, l1);
-      out[(e >> 1) + 1] = pack2(l2, l3);
-      out[16 + (e >> 1)] = pack2(h0, h1);
-      out[16 + (e >> 1) + 1] = pack2(h2, h3);
-    }
+  for (int i = 0; i < 8; ++i) {
+    const uint32_t b = w[i];
+    const float l0 = dd[0] * (float)(b & 0xF) - mm[0], l1 = dd[0] * (float)((b >> 8) & 0xF) - mm[0];
+    const float l2 = dd[0] * (float)((b >> 16) & 0xF) - mm[0], l3 = dd[0] * (float)((b >> 24) & 0xF) - mm[0];
+    const float h0 = dd[1] * (float)((b >> 4) & 0xF) - mm[1], h1 = dd[1] * (float)((b >> 12) & 0xF) - mm[1];
+    const float h2 = dd[1] * (float)((b >> 20) & 0xF) - mm[1], h3 = dd[1] * (float)(b >> 28) - mm[1];
+    out[2 * i] = pack2(l0, l1);          // low nibbles: weights 4i .. 4i+3
+    out[2 * i + 1] = pack2(l2, l3);
+    out[16 + 2 * i] = pack2(h0, h1);     // high nibbles: the same + 32
+    out[16 + 2 * i + 1] = pack2(h2, h3);
   }
 }
 
-// positions l in [16*j, 16*j + 16) of the 128-half `hh` of super-block `ib`: the four
-// weights l, l+32, l+64, l+96 each, as bf16 into dst[0..128) (dst = start of the half)
-__device__ __forceinline__ void dequant_q6k_part(const MmArgs& a, int64_t row, int nb, int ib, int hh,
-                                                 int j, bf16_t* dst) {
+// positions l in [16*j, 16*j + 16) of the 128-half `hh` of super-block `ib`
+__device__ __forceinline__ BRegsQ6 load_q6k(const MmArgs& a, int64_t row, int nb, int ib, int hh, int j) {
   const int64_t blk = row * nb + ib;
-  const float d = dm_h2f(a.dm[blk]);
   const uint8_t* base = a.qs + blk * 192;
-  const uint4 qa = *reinterpret_cast<const uint4*>(base + 64 * hh + 16 * j);
-  const uint4 qb = *reinterpret_cast<const uint4*>(base + 64 * hh + 32 + 16 * j);
-  const uint4 qhv = *reinterpret_cast<const uint4*>(base + 128 + 32 * hh + 16 * j);
-  const int8_t* sc = reinterpret_cast<const int8_t*>(a.scales + blk * 16) + 8 * hh;
-  const float s1 = d * (float)sc[j], s2 = d * (float)sc[j + 2], s3 = d * (float)sc[j + 4],
-              s4 = d * (float)sc[j + 6];
-  const uint32_t la[4] = {qa.x, qa.y, qa.z, qa.w}, lb[4] = {qb.x, qb.y, qb.z, qb.w},
-                 hv[4] = {qhv.x, qhv.y, qhv.z, qhv.w};
+  BRegsQ6 r;
+  r.qa = *reinterpret_cast<const uint4*>(base + 64 * hh + 16 * j);
+  r.qb = *reinterpret_cast<const uint4*>(base + 64 * hh + 32 + 16 * j);
+  r.qh = *reinterpret_cast<const uint4*>(base + 128 + 32 * hh + 16 * j);
+  r.sc = *reinterpret_cast<const uint2*>(a.scales + blk * 16 + 8 * hh);
+  r.d = a.dm[blk];
+  return r;
+}
+
+// the four weights l, l+32, l+64, l+96 of each position, d*sc*q (q6k.metal:47-77), as bf16
+// into dst[0..128) (dst = start of the half)
+__device__ __forceinline__ void dequant_q6k(const BRegsQ6& r, int j, bf16_t* dst) {
+  const float d = dm_h2f((f16_t)r.d);
+  const uint32_t scw[2] = {r.sc.x, r.sc.y};
+  auto scale = [&](int i) { return (float)(int)(int8_t)((scw[i >> 2] >> (8 * (i & 3))) & 0xffu); };
+  const float s1 = d * scale(j), s2 = d * scale(j + 2), s3 = d * scale(j + 4), s4 = d * scale(j + 6);
+  const uint32_t la[4] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w}, lb[4] = {r.qb.x, r.qb.y, r.qb.z, r.qb.w},
+                 hv[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
   uint32_t* out = reinterpret_cast<uint32_t*>(dst);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -134,17 +161,24 @@ __device__ __forceinline__ void dequant_q6k_part(const MmArgs& a, int64_t row, i
   }
 }
 
+template <int KIND>
+struct BRegsOf { typedef BRegsQ4 type; };
+template <>
+struct BRegsOf<ORNITH_Q6K> { typedef BRegsQ6 type; };
+
+// BM = 256: 2 x 2 wavefronts of 128 x 64; BM = 128: 2 x 2 of 64 x 64; BM = 64: 1 x 4 of 64 x 32
 template <int KIND, int BM, bool GATHER>
 __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
-  constexpr int WN = BM == 128 ? 2 : 4;        // wavefronts along n
-  constexpr int WTN = BN / WN;                 // wave tile width: 64 or 32
-  constexpr int TM = 2, TN = WTN / 32;         // 32x32 MFMA tiles per wavefront
+  constexpr int WM = BM >= 128 ? 2 : 1, WN = 4 / WM;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int NA = BM * 16 / 256;  // 16-byte pieces of the activation slab per thread
   __shared__ __attribute__((aligned(16))) bf16_t As[BM][LDK];
   __shared__ __attribute__((aligned(16))) bf16_t Bs[BN][LDK];
   __shared__ uint32_t s_src[BM], s_dst[BM];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = BM == 128 ? (wave >> 1) : 0, wn = BM == 128 ? (wave & 1) : wave;
+  const int wm = wave / WN, wn = wave % WN;
   const int n0 = blockIdx.x * BN;
   const int nb = a.K >> 8;
 
@@ -166,6 +200,28 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
     rows_here = min(BM, a.M - m0);
   }
 
+  // this thread's pieces of a slab: NA activation pieces and one weight piece
+  const int br = tid >> 1, bpart = tid & 1;
+  const int64_t brow = wrow0 + min(n0 + br, a.O - 1);
+  const bf16_t* asrc[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int idx = tid + 256 * i, r = idx >> 4, c8 = idx & 15;
+    const int64_t src = r < rows_here ? (GATHER ? (int64_t)s_src[r] : (int64_t)(m0 + r)) : -1;
+    asrc[i] = src >= 0 ? a.x + src * a.K + 8 * c8 : nullptr;
+  }
+  uint4 areg[NA];
+  typename BRegsOf<KIND>::type breg;
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+      areg[i] = asrc[i] ? *reinterpret_cast<const uint4*>(asrc[i] + k0) : make_uint4(0, 0, 0, 0);
+    if constexpr (KIND == ORNITH_Q4K)
+      breg = load_q4k(a, brow, nb, k0 >> 8, ((k0 & 255) >> 6) + bpart);
+    else
+      breg = load_q6k(a, brow, nb, k0 >> 8, (k0 & 255) >> 7, bpart);
+  };
+
   f32x16_t acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -174,37 +230,26 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+  fetch(0);
   for (int k0 = 0; k0 < a.K; k0 += BK) {
-    // ---- A slab: BM rows x 128 bf16
 #pragma unroll
-    for (int i = 0; i < BM * 16 / 256; ++i) {
-      const int idx = tid + 256 * i, r = idx >> 4, c8 = idx & 15;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (r < rows_here) {
-        const int64_t src = GATHER ? (int64_t)s_src[r] : (int64_t)(m0 + r);
-        v = *reinterpret_cast<const uint4*>(a.x + src * a.K + k0 + 8 * c8);
-      }
-      *reinterpret_cast<uint4*>(&As[r][8 * c8]) = v;
+    for (int i = 0; i < NA; ++i) {
+      const int idx = tid + 256 * i;
+      *reinterpret_cast<uint4*>(&As[idx >> 4][8 * (idx & 15)]) = areg[i];
     }
-    // ---- B slab: 128 weight rows x 128 weights, dequantized
-    {
-      const int r = tid >> 1, part = tid & 1;
-      const int o = n0 + r;
-      const int64_t row = wrow0 + (o < a.O ? o : a.O - 1);
-      const int ib = k0 >> 8;
-      if constexpr (KIND == ORNITH_Q4K)
-        dequant64_q4k(a, row, nb, ib, ((k0 & 255) >> 6) + part, &Bs[r][64 * part]);
-      else
-        dequant_q6k_part(a, row, nb, ib, (k0 & 255) >> 7, part, &Bs[r][0]);
-    }
+    if constexpr (KIND == ORNITH_Q4K)
+      dequant_q4k(breg, ((k0 & 255) >> 6) + bpart, &Bs[br][64 * bpart]);
+    else
+      dequant_q6k(breg, bpart, &Bs[br][0]);
     __syncthreads();
+    if (k0 + BK < a.K) fetch(k0 + BK);  // in flight while the matrix cores run
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
       const int kc = kk * 16 + 8 * (lane >> 5);
       bf16x8_t af[TM], bfr[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        af[i] = *reinterpret_cast<const bf16x8_t*>(&As[wm * 64 + i * 32 + (lane & 31)][kc]);
+        af[i] = *reinterpret_cast<const bf16x8_t*>(&As[wm * WTM + i * 32 + (lane & 31)][kc]);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
         bfr[j] = *reinterpret_cast<const bf16x8_t*>(&Bs[wn * WTN + j * 32 + (lane & 31)][kc]);
@@ -225,7 +270,7 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
       const int o = n0 + wn * WTN + j * 32 + (lane & 31);
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const int r = wm * 64 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        const int r = wm * WTM + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
         if (r < rows_here && o < a.O) {
           const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
           a.y[dst * a.O + o] = dm_f2bf(acc[i][j][e]);
@@ -311,11 +356,22 @@ int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, 
   a.M = M;
   a.O = w->O;
   a.K = w->K;
-  const dim3 grid((w->O + BN - 1) / BN, (M + 127) / 128);
-  if (w->kind == ORNITH_Q4K)
-    hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 128, false>), grid, dim3(256), 0, ctx->stream, a);
-  else
-    hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q6K, 128, false>), grid, dim3(256), 0, ctx->stream, a);
+  // 256-row tiles dequantize every weight tile half as often; 128-row tiles when that is what
+  // it takes to give every compute unit a workgroup
+  const int nx = (w->O + BN - 1) / BN;
+  const bool big = M >= 256 && (long)nx * ((M + 255) / 256) >= ctx->compute_units;
+  const dim3 grid(nx, big ? (M + 255) / 256 : (M + 127) / 128);
+  if (w->kind == ORNITH_Q4K) {
+    if (big)
+      hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 256, false>), grid, dim3(256), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 128, false>), grid, dim3(256), 0, ctx->stream, a);
+  } else {
+    if (big)
+      hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q6K, 256, false>), grid, dim3(256), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q6K, 128, false>), grid, dim3(256), 0, ctx->stream, a);
+  }
   ORN_LAUNCH_CHECK("kq_mm_kernel");
   return ORNITH_OK;
 }

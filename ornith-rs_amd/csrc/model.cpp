@@ -89,26 +89,16 @@ static int load_attn(const ornith_weights* ws, const std::string& p, const ornit
   return ORNITH_OK;
 }
 
-// bytes of step buffers for R rows (trunk)
-static size_t step_bytes(const ornith_model* m, int R) {
-  const auto& c = m->cfg;
-  const size_t H = c.hidden_size, D = m->conv_dim(), Vd = m->value_dim(), Kd = m->key_dim();
-  const size_t Hv = c.linear_num_value_heads;
-  const size_t aq = (size_t)c.num_attention_heads * c.head_dim, akv = (size_t)c.num_key_value_heads * c.head_dim;
-  size_t per_row = 2 * (6 * H + D + 3 * Vd + 2 * Kd + 3 * Hv + 2 * aq + 2 * akv + 2 * aq) + 4 * Hv;
-  return per_row * R + 64 * 256 + (size_t)(R < kMaxRows ? R : kMaxRows) * c.vocab_size * 2 + (size_t)R * 8;
-}
-
 struct StepBufs {
   char *x, *normed, *r, *h, *normed2, *mo;
   char *qkv, *z, *a, *b, *q, *k, *v, *beta, *y, *gated;
   float* g;
   char *qg, *kx, *vx, *q_rot, *att;
-  char* logits;
-  uint32_t* toks;
 };
 
-static StepBufs carve(const ornith_model* m, void* base, int R) {
+// Lays the step buffers for R rows out from `base`; *total receives the bytes used, so the
+// allocation is sized by the very layout it has to hold.
+static StepBufs carve(const ornith_model* m, void* base, int R, size_t* total = nullptr) {
   const auto& c = m->cfg;
   const size_t H = c.hidden_size, D = m->conv_dim(), Vd = m->value_dim(), Kd = m->key_dim();
   const size_t Hv = c.linear_num_value_heads;
@@ -137,9 +127,15 @@ static StepBufs carve(const ornith_model* m, void* base, int R) {
   s.vx = sc.take<char>(2 * akv * R);
   s.q_rot = sc.take<char>(2 * aq * R);
   s.att = sc.take<char>(2 * aq * R);
-  s.logits = sc.take<char>((size_t)(R < kMaxRows ? R : kMaxRows) * c.vocab_size * 2);
-  s.toks = sc.take<uint32_t>(R);
+  if (total) *total = sc.off;
   return s;
+}
+
+// bytes of step buffers for R rows (trunk)
+static size_t step_bytes(const ornith_model* m, int R) {
+  size_t n = 0;
+  carve(m, nullptr, R, &n);
+  return n + 256;
 }
 
 int model_ensure_rope(ornith_model* m, int npos) {

@@ -195,3 +195,25 @@ def test_prefill_attention_close_to_exact_kernel(orn, ctx, T, Hq, Hkv, cap, offs
     rel = np.linalg.norm(g - w, axis=1) / np.linalg.norm(w, axis=1)
     assert rel.max() < 0.01, float(rel.max())
     for b in (dq, dk, dv, dg, dout): b.free()
+
+
+def test_model_forward_at_the_reference_chunk_width(orn, ctx):
+    """2048 rows in one call (the reference's prefill_step_size): the step buffers are sized by
+    the layout they hold, so every row lands inside them; with bf16-exact weights the result
+    agrees with four 512-row calls to summation-order noise."""
+    import synth
+    s = synth.SynthModel(synth.TINY, seed=8, with_mtp=False)
+    _make_weights_bf16_exact(s)
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    model.set_max_rows(2048)
+    toks = np.random.default_rng(1).integers(0, s.cfg["vocab_size"], 2048).astype(np.uint32)
+    a, b = model.make_cache(2100, 2), model.make_cache(2100, 2)
+    h1 = model.forward(a, toks)
+    h4 = np.concatenate([model.forward(b, toks[i:i + 512]) for i in range(0, 2048, 512)])
+    assert a.offset == b.offset == 2048
+    g = util.bf16_to_f32(h1).astype(np.float64); w = util.bf16_to_f32(h4).astype(np.float64)
+    assert np.isfinite(g).all()
+    rel = np.linalg.norm(g - w, axis=1) / np.linalg.norm(w, axis=1)
+    assert np.median(rel) < 0.003 and (rel <= 0.02).mean() >= 0.95, (float(np.median(rel)), float(rel.max()))
+    for o in (a, b, model, ws): o.close()
