@@ -354,15 +354,37 @@ __global__ __launch_bounds__(RB) void cat_search_kernel(const float* vloc, const
   float base, total;
   chunk_base<false>(chunk_tot, nch, base, total);
   const int i = blockIdx.x * RB + threadIdx.x;
-  if (i >= n) return;
   float u = (float)bits / 4294967296.0f;
   const float upper = __uint_as_float(0x3f7fffffu);
   u = u < upper ? u : upper;
   u = 1.0f * u + 0.0f;
   u = u * total;
-  const float c = cum_at<false>(vloc, segoff, base, i);
-  if (c > u) atomicMin(&first_last[0], (uint32_t)i);
-  if (w[i] > 0.f) atomicMax(&first_last[1], (uint32_t)i);
+  uint32_t first = 0xffffffffu, last = 0u;
+  if (i < n) {
+    if (cum_at<false>(vloc, segoff, base, i) > u) first = (uint32_t)i;
+    if (w[i] > 0.f) last = (uint32_t)i;
+  }
+  // one atomic per workgroup, not per element: half the vocabulary lies above u
+  __shared__ uint32_t s_first[RB / 64], s_last[RB / 64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) {
+    first = min(first, (uint32_t)__shfl_xor((int)first, d, 64));
+    last = max(last, (uint32_t)__shfl_xor((int)last, d, 64));
+  }
+  if (lane == 0) {
+    s_first[wave] = first;
+    s_last[wave] = last;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w2 = 1; w2 < RB / 64; ++w2) {
+      first = min(first, s_first[w2]);
+      last = max(last, s_last[w2]);
+    }
+    if (first != 0xffffffffu) atomicMin(&first_last[0], first);
+    if (last != 0u) atomicMax(&first_last[1], last);
+  }
 }
 
 __global__ void cat_init_kernel(uint32_t* first_last) {
