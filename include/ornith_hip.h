@@ -357,6 +357,14 @@ ORNITH_API int ornith_argmax_rows(ornith_ctx* ctx, const void* d_logits, int row
 #define ORNITH_DT_U8 3
 #define ORNITH_DT_U32 4
 #define ORNITH_DT_I32 5
+/* dtypes a safetensors header may name besides those above; no kernel consumes them */
+#define ORNITH_DT_I8 6
+#define ORNITH_DT_I16 7
+#define ORNITH_DT_U16 8
+#define ORNITH_DT_I64 9
+#define ORNITH_DT_U64 10
+#define ORNITH_DT_F64 11
+#define ORNITH_DT_BOOL 12
 typedef struct ornith_weights ornith_weights;
 ORNITH_API int ornith_weights_create(ornith_ctx* ctx, ornith_weights** out);
 /* WeightStore::tensor: copies host_data to the device and records it under `name`. */
@@ -365,6 +373,55 @@ ORNITH_API int ornith_weights_put(ornith_weights* ws, const char* name, int dtyp
 ORNITH_API int ornith_weights_destroy(ornith_weights* ws);
 /* number of tensors held and their total bytes (the loader's report, src/main.rs:483-488) */
 ORNITH_API int ornith_weights_stats(const ornith_weights* ws, int64_t* n_tensors, int64_t* bytes);
+
+/* ---- artifact files: SafeTensors (src/safetensors.rs:196-310) ---------------------
+ * Host only: maps each shard read-only, parses and validates its JSON header (dtype,
+ * shape, data_offsets against the file length). `data` pointers stay valid until close. */
+typedef struct ornith_safetensors ornith_safetensors;
+/* SafeTensors::open_many (src/safetensors.rs:204-210): later files win a repeated name. */
+ORNITH_API int ornith_safetensors_open(const char* const* paths, int n_paths,
+                                       ornith_safetensors** out);
+/* shards_from_index (src/safetensors.rs:296-310): the shards model.safetensors.index.json's
+ * weight_map names, sorted and de-duplicated, then `extra` (the MTP sidecar file). */
+ORNITH_API int ornith_safetensors_open_model(const char* model_dir, const char* const* extra,
+                                             int n_extra, ornith_safetensors** out);
+ORNITH_API int ornith_safetensors_close(ornith_safetensors* st);
+ORNITH_API int ornith_safetensors_count(const ornith_safetensors* st, int64_t* n_tensors,
+                                        int64_t* n_files);
+/* SafeTensors::names (src/safetensors.rs:283-285), in sorted order */
+ORNITH_API int ornith_safetensors_name(const ornith_safetensors* st, int64_t i, const char** name);
+/* SafeTensors::{get, bytes} (src/safetensors.rs:275-281); shape has room for 8 dims */
+ORNITH_API int ornith_safetensors_info(const ornith_safetensors* st, const char* name, int* dtype,
+                                       int64_t* shape, int* ndim, const void** data,
+                                       size_t* nbytes);
+
+/* config.json's `quantization` block (src/weights.rs:46-80): top-level group_size / bits /
+ * mode (absent mode = affine) with per-module overrides; mode strings as
+ * QuantMode::from_config (src/ops/quantized.rs:60-75). nvfp4 / mxfp4 / mxfp8 are
+ * ORNITH_ERR_UNSUPPORTED. */
+#define ORNITH_QM_AFFINE 0
+#define ORNITH_QM_Q4K 1
+#define ORNITH_QM_Q6K 2
+/* WeightStore::quant_config (src/weights.rs:96-98) straight from <model_dir>/config.json */
+ORNITH_API int ornith_quant_config_load(const char* model_dir, const char* module_path,
+                                        int* group_size, int* bits, int* mode);
+/* WeightStore::open (src/weights.rs:41-80): the indexed shards plus `extra` files and the
+ * quantization block. Tensors are copied to the device the first time a loader asks for
+ * them (WeightStore::tensor, src/weights.rs:101-108), so only what the model uses is
+ * resident. With a quantization block present, ornith_model_load / ornith_mtp_load check
+ * each module's tensors against its configured mode (src/weights.rs:132-150, 199-220). The
+ * MTP head's numbered experts.N.* tensors are stacked on load (stacked_experts,
+ * src/weights.rs:237-279). */
+ORNITH_API int ornith_weights_open(ornith_ctx* ctx, const char* model_dir,
+                                   const char* const* extra, int n_extra, ornith_weights** out);
+ORNITH_API int ornith_weights_quant_config(const ornith_weights* ws, const char* module_path,
+                                           int* group_size, int* bits, int* mode);
+/* WeightStore::has (src/weights.rs:82-84): 1 if resident or in a mapped shard, else 0 */
+ORNITH_API int ornith_weights_has(const ornith_weights* ws, const char* name);
+/* WeightStore::tensor followed by a copy back: dtype / shape of `name` and, when host_out is
+ * not NULL, its bytes (host_bytes must equal the tensor's size). */
+ORNITH_API int ornith_weights_fetch(const ornith_weights* ws, const char* name, int* dtype,
+                                    int64_t* shape, int* ndim, void* host_out, size_t host_bytes);
 
 /* TextConfig (src/model/config.rs:46-134), the fields this path reads. */
 typedef struct ornith_text_config {
@@ -385,6 +442,11 @@ typedef struct ornith_caches ornith_caches;
 /* TextModel::load: resolves every tensor by name; the store must outlive the model. */
 ORNITH_API int ornith_model_load(ornith_ctx* ctx, const ornith_weights* ws,
                                  const ornith_text_config* cfg, ornith_model** out);
+/* TextConfig::load (src/model/config.rs:46-133): <model_dir>/config.json, keys under
+ * `text_config` when present; rope settings from `rope_parameters`; mtp_layers (may be NULL)
+ * receives num_nextn_predict_layers. Host only. */
+ORNITH_API int ornith_text_config_load(const char* model_dir, ornith_text_config* out,
+                                       int* mtp_layers);
 ORNITH_API int ornith_model_destroy(ornith_model* m);
 /* Rows one forward call may carry (default 16: decode, verify, short prompt chunks). The
  * reference prefills in chunks of prefill_step_size (2048, src/generate.rs:90-136); raise

@@ -48,9 +48,18 @@ static int load_moe(const ornith_weights* ws, const std::string& mlp, const orni
   if (dense_experts) {
     const int64_t n = (int64_t)E * I * H;
     w->ex_dense = 1;
-    TRY(ws_tensor(ws, mlp + "switch_mlp.gate_proj.weight", ORNITH_DT_BF16, n, &w->d_ex_gate));
-    TRY(ws_tensor(ws, mlp + "switch_mlp.up_proj.weight", ORNITH_DT_BF16, n, &w->d_ex_up));
-    TRY(ws_tensor(ws, mlp + "switch_mlp.down_proj.weight", ORNITH_DT_BF16, n, &w->d_ex_down));
+    if (ornith_weights_has(ws, (mlp + "switch_mlp.gate_proj.weight").c_str())) {
+      TRY(ws_tensor(ws, mlp + "switch_mlp.gate_proj.weight", ORNITH_DT_BF16, n, &w->d_ex_gate));
+      TRY(ws_tensor(ws, mlp + "switch_mlp.up_proj.weight", ORNITH_DT_BF16, n, &w->d_ex_up));
+      TRY(ws_tensor(ws, mlp + "switch_mlp.down_proj.weight", ORNITH_DT_BF16, n, &w->d_ex_down));
+    } else {
+      // the sidecar file keeps the experts as numbered tensors
+      // (/root/reference/src/model/mtp.rs:118-135)
+      const std::string ex = mlp + "experts";
+      TRY(ws_stacked(ws, ex, "gate_proj.weight", E, ORNITH_DT_BF16, n, &w->d_ex_gate));
+      TRY(ws_stacked(ws, ex, "up_proj.weight", E, ORNITH_DT_BF16, n, &w->d_ex_up));
+      TRY(ws_stacked(ws, ex, "down_proj.weight", E, ORNITH_DT_BF16, n, &w->d_ex_down));
+    }
     w->ex_gate.E = w->ex_up.E = w->ex_down.E = E;
     w->ex_gate.O = w->ex_up.O = I;
     w->ex_gate.K = w->ex_up.K = H;
@@ -592,7 +601,7 @@ int ornith_mtp_load(ornith_model* m, const ornith_weights* ws, int capacity, orn
   MTRY(ws_tensor(ws, "mtp.layers.0.post_attention_layernorm.weight", ORNITH_DT_BF16, H, &h->post_ln));
   MTRY(ws_tensor(ws, "mtp.norm.weight", ORNITH_DT_BF16, H, &h->norm));
   MTRY(load_attn(ws, "mtp.layers.0.self_attn.", c, &h->attn));
-  MTRY(load_moe(ws, "mtp.layers.0.mlp.", c, ws->find("mtp.layers.0.mlp.switch_mlp.gate_proj.dm") == nullptr, &h->moe));
+  MTRY(load_moe(ws, "mtp.layers.0.mlp.", c, !ornith_weights_has(ws, "mtp.layers.0.mlp.switch_mlp.gate_proj.dm"), &h->moe));
   h->capacity = capacity;
   h->max_rows = m->max_rows;
   const size_t kv = (size_t)c.num_key_value_heads * capacity * c.head_dim * 2;

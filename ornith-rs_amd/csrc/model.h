@@ -25,13 +25,40 @@ struct Tensor {
   }
 };
 
+// One module's entry in config.json's `quantization` block
+// (/root/reference/src/weights.rs:31-37).
+struct QuantSpec {
+  int group_size = 0, bits = 0, mode = ORNITH_QM_AFFINE;
+};
+struct QuantTable {
+  bool loaded = false;
+  QuantSpec def;
+  std::map<std::string, QuantSpec> per_module;
+  // per-module override, else the top-level default (/root/reference/src/weights.rs:96-98)
+  QuantSpec lookup(const std::string& path) const {
+    auto it = per_module.find(path);
+    return it == per_module.end() ? def : it->second;
+  }
+};
+int quant_table_load(const std::string& model_dir, QuantTable* qt);
+
+struct ornith_weights_files;  // the mapped shards behind a store opened from a directory
+struct ornith_weights;
+const Tensor* ws_fault_in(const ornith_weights* ws, const std::string& name);
+void ws_release_files(ornith_weights* ws);
+
 struct ornith_weights {
   ornith_ctx* ctx = nullptr;
-  std::map<std::string, Tensor> t;
-  size_t total_bytes = 0;
+  // resident tensors; a store opened from a directory copies each one in on first use
+  // (WeightStore::tensor, /root/reference/src/weights.rs:101-108), hence mutable
+  mutable std::map<std::string, Tensor> t;
+  mutable size_t total_bytes = 0;
+  ornith_weights_files* files = nullptr;
+  QuantTable quant;
   const Tensor* find(const std::string& name) const {
     auto it = t.find(name);
-    return it == t.end() ? nullptr : &it->second;
+    if (it != t.end()) return &it->second;
+    return files ? ws_fault_in(this, name) : nullptr;
   }
 };
 
@@ -42,6 +69,11 @@ int ws_kmatrix(const ornith_weights* ws, const std::string& path, ornith_kmatrix
 // A plain tensor with an expected element count and dtype.
 int ws_tensor(const ornith_weights* ws, const std::string& name, int dtype, int64_t numel,
               const void** out);
+// <prefix>.<e>.<suffix> for e in 0..experts copied into one [experts, ...] tensor, kept under
+// "<prefix>.*.<suffix>" (WeightStore::stacked_experts, /root/reference/src/weights.rs:237-279).
+int ws_stacked(const ornith_weights* ws, const std::string& prefix, const std::string& suffix,
+               int experts, int dtype, int64_t numel, const void** out);
+size_t ornith_dt_size(int dt);
 
 struct GdnLayer {
   ornith_linear in_proj_qkv, in_proj_z, out_proj, in_proj_a, in_proj_b;

@@ -7,13 +7,30 @@
 // with the tensor shapes of /root/reference/src/ops/kquant.rs:20-26.
 #include "model.h"
 
-static size_t dt_size(int dt) {
-  switch (dt) {
-    case ORNITH_DT_F32: case ORNITH_DT_U32: case ORNITH_DT_I32: return 4;
-    case ORNITH_DT_BF16: case ORNITH_DT_F16: return 2;
-    case ORNITH_DT_U8: return 1;
-    default: return 0;
+// config.json's mode for a module must agree with the tensors the artifact holds for it
+// (/root/reference/src/weights.rs:132-150, 199-220); stores filled by ornith_weights_put carry
+// no config and resolve by the tensors alone.
+static int check_mode(const ornith_weights* ws, const std::string& path, bool is_k, int kind) {
+  if (!ws->quant.loaded) return ORNITH_OK;
+  const QuantSpec s = ws->quant.lookup(path);
+  const bool says_k = s.mode == ORNITH_QM_Q4K || s.mode == ORNITH_QM_Q6K;
+  if (is_k) {
+    ORN_REQUIRE(says_k, "%s holds a .dm tensor but config.json's quantization block says affine",
+                path.c_str());
+    ORN_REQUIRE(s.group_size == 256, "%s: a k-quant's super-block is 256 weights, not %d",
+                path.c_str(), s.group_size);
+    ORN_REQUIRE((s.mode == ORNITH_QM_Q4K) == (kind == ORNITH_Q4K),
+                "%s: config.json says %s but the scales are laid out as %s", path.c_str(),
+                s.mode == ORNITH_QM_Q4K ? "q4k" : "q6k", kind == ORNITH_Q4K ? "q4k" : "q6k");
+    ORN_REQUIRE(!ornith_weights_has(ws, (path + ".biases").c_str()) &&
+                    !ornith_weights_has(ws, (path + ".global_scale").c_str()),
+                "%s is a k-quant but the artifact has a .biases or .global_scale for it",
+                path.c_str());
+  } else {
+    ORN_REQUIRE(!says_k, "%s is a k-quant in config.json but the artifact has no %s.dm",
+                path.c_str(), path.c_str());
   }
+  return ORNITH_OK;
 }
 
 static int kq_from(const ornith_weights* ws, const std::string& path, bool routed,
@@ -40,6 +57,8 @@ static int kq_from(const ornith_weights* ws, const std::string& path, bool route
   out->d_qs = w->d;
   out->d_scales = s->d;
   out->d_dm = d->d;
+  int rc = check_mode(ws, path, true, out->kind);
+  if (rc) return rc;
   return ornith_kmatrix_check(out, w->bytes, s->bytes, d->bytes);
 }
 
@@ -51,7 +70,7 @@ int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* 
   memset(out, 0, sizeof *out);
   const Tensor* w = ws->find(path + ".weight");
   ORN_REQUIRE(w, "%s.weight: no such tensor", path.c_str());
-  if (ws->find(path + ".dm")) {
+  if (ornith_weights_has(ws, (path + ".dm").c_str())) {
     out->mode = ORNITH_LIN_KQUANT;
     int rc = kq_from(ws, path, false, &out->km);
     if (rc) return rc;
@@ -59,8 +78,16 @@ int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* 
     out->K = out->km.K;
     return ORNITH_OK;
   }
+  int rc = check_mode(ws, path, false, 0);
+  if (rc) return rc;
   if (const Tensor* b = ws->find(path + ".biases")) {
     const Tensor* s = ws->find(path + ".scales");
+    if (ws->quant.loaded) {
+      const QuantSpec q = ws->quant.lookup(path);
+      ORN_REQUIRE(q.bits == 8 && q.group_size == 64,
+                  "%s: affine %d-bit group %d is not carried (8-bit group 64 only)", path.c_str(),
+                  q.bits, q.group_size);
+    }
     ORN_REQUIRE(s, "%s: affine module needs .scales", path.c_str());
     ORN_REQUIRE(s->dtype == ORNITH_DT_BF16 && b->dtype == ORNITH_DT_BF16,
                 "%s: affine scales/biases must be bfloat16", path.c_str());
@@ -113,7 +140,7 @@ int ornith_weights_put(ornith_weights* ws, const char* name, int dtype, const in
                        int ndim, const void* host_data) {
   ORN_REQUIRE(ws && name && shape && host_data, "weights_put: null argument");
   ORN_REQUIRE(ndim >= 1 && ndim <= 8, "weights_put: %s has %d dims", name, ndim);
-  const size_t es = dt_size(dtype);
+  const size_t es = ornith_dt_size(dtype);
   ORN_REQUIRE(es, "weights_put: %s has unknown dtype %d", name, dtype);
   ORN_REQUIRE(!ws->find(name), "weights_put: %s is already in the store", name);
   Tensor t;
@@ -140,6 +167,7 @@ int ornith_weights_put(ornith_weights* ws, const char* name, int dtype, const in
 int ornith_weights_destroy(ornith_weights* ws) {
   if (!ws) return ORNITH_OK;
   for (auto& kv : ws->t) ornith_free(ws->ctx, kv.second.d);
+  ws_release_files(ws);
   delete ws;
   return ORNITH_OK;
 }

@@ -3,12 +3,17 @@ WeightStore, TextModel (+ caches), FrSpec, MtpHead, generate_step, generate_step
 Names and argument meaning follow /root/reference/src/{weights,frspec,generate,
 mtp_generate}.rs and src/model/{qwen3_5,mtp}.rs so tests read like the reference's."""
 import ctypes as C
+import os
 
 import numpy as np
 
 from . import (BF16, F32, LinearStruct, OrnithError, _check, _ptr, lib)
 
 DT_F32, DT_BF16, DT_F16, DT_U8, DT_U32, DT_I32 = range(6)
+DT_I8, DT_I16, DT_U16, DT_I64, DT_U64, DT_F64, DT_BOOL = range(6, 13)
+DT_SIZE = {DT_F32: 4, DT_BF16: 2, DT_F16: 2, DT_U8: 1, DT_U32: 4, DT_I32: 4, DT_I8: 1, DT_I16: 2,
+           DT_U16: 2, DT_I64: 8, DT_U64: 8, DT_F64: 8, DT_BOOL: 1}
+QM_AFFINE, QM_Q4K, QM_Q6K = range(3)
 HISTORY_CYCLE, HISTORY_COMMITTED = 0, 1
 MAX_DEPTH = 8
 
@@ -54,6 +59,14 @@ class TextConfig(C.Structure):
         d.update(over)
         return TextConfig(**d)
 
+    @staticmethod
+    def load(model_dir):
+        """TextConfig::load: (config, mtp_layers) from <model_dir>/config.json."""
+        cfg, mtp = TextConfig(), C.c_int()
+        _check(lib().ornith_text_config_load(os.fsencode(model_dir), C.byref(cfg), C.byref(mtp)),
+               f"text_config_load({model_dir})")
+        return cfg, mtp.value
+
     def key_dim(self):
         return self.linear_num_key_heads * self.linear_key_head_dim
 
@@ -91,12 +104,6 @@ PROGRESS_CB = C.CFUNCTYPE(None, C.c_size_t, C.c_size_t, C.c_void_p)
 class WeightStore:
     """WeightStore: named tensors on the device."""
 
-    def __init__(self, ctx):
-        self.ctx = ctx
-        h = C.c_void_p()
-        _check(lib().ornith_weights_create(ctx.h, C.byref(h)), "weights_create")
-        self.h = h
-
     def put(self, name, arr, dtype=None):
         """dtype: DT_BF16 / DT_F16 for uint16 bit patterns; inferred otherwise."""
         arr = np.ascontiguousarray(arr)
@@ -105,6 +112,45 @@ class WeightStore:
         shape = (C.c_int64 * arr.ndim)(*arr.shape)
         _check(lib().ornith_weights_put(self.h, name.encode(), dtype, shape, arr.ndim, _ptr(arr)),
                f"weights_put({name})")
+
+    def __init__(self, ctx, _handle=None):
+        self.ctx = ctx
+        if _handle is None:
+            _handle = C.c_void_p()
+            _check(lib().ornith_weights_create(ctx.h, C.byref(_handle)), "weights_create")
+        self.h = _handle
+
+    @staticmethod
+    def open(ctx, model_dir, extra=()):
+        """WeightStore::open: the shards the index names plus `extra` files (the MTP sidecar)
+        and config.json's quantization block; tensors reach the device on first use."""
+        h = C.c_void_p()
+        ex = (C.c_char_p * max(len(extra), 1))(*[os.fsencode(p) for p in extra])
+        _check(lib().ornith_weights_open(ctx.h, os.fsencode(model_dir), ex, len(extra), C.byref(h)),
+               f"weights_open({model_dir})")
+        return WeightStore(ctx, h)
+
+    def has(self, name):
+        return bool(lib().ornith_weights_has(self.h, name.encode()))
+
+    def quant_config(self, path):
+        g, b, m = C.c_int(), C.c_int(), C.c_int()
+        _check(lib().ornith_weights_quant_config(self.h, path.encode(), C.byref(g), C.byref(b),
+                                                 C.byref(m)), f"quant_config({path})")
+        return g.value, b.value, m.value
+
+    def fetch(self, name):
+        """(dtype code, shape, raw bytes as uint8) of a tensor, copied back from the device."""
+        dt, nd = C.c_int(), C.c_int()
+        shape = (C.c_int64 * 8)()
+        fn = lib().ornith_weights_fetch
+        fn.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                       C.c_size_t]
+        _check(fn(self.h, name.encode(), C.byref(dt), shape, C.byref(nd), None, 0), f"fetch({name})")
+        shp = tuple(shape[i] for i in range(nd.value))
+        out = np.empty(int(np.prod(shp)) * DT_SIZE[dt.value], np.uint8)
+        _check(fn(self.h, name.encode(), None, None, None, _ptr(out), out.nbytes), f"fetch({name})")
+        return dt.value, shp, out
 
     def stats(self):
         n, b = C.c_int64(), C.c_int64()
@@ -115,6 +161,56 @@ class WeightStore:
         if self.h:
             lib().ornith_weights_destroy(self.h)
             self.h = None
+
+
+class SafeTensors:
+    """SafeTensors::open_many / shards_from_index: mapped shards, host only."""
+
+    def __init__(self, paths=None, model_dir=None, extra=()):
+        h = C.c_void_p()
+        if model_dir is not None:
+            ex = (C.c_char_p * max(len(extra), 1))(*[os.fsencode(p) for p in extra])
+            _check(lib().ornith_safetensors_open_model(os.fsencode(model_dir), ex, len(extra), C.byref(h)),
+                   f"safetensors_open_model({model_dir})")
+        else:
+            ps = (C.c_char_p * max(len(paths), 1))(*[os.fsencode(p) for p in paths])
+            _check(lib().ornith_safetensors_open(ps, len(paths), C.byref(h)), "safetensors_open")
+        self.h = h
+
+    def counts(self):
+        n, f = C.c_int64(), C.c_int64()
+        _check(lib().ornith_safetensors_count(self.h, C.byref(n), C.byref(f)), "safetensors_count")
+        return n.value, f.value
+
+    def names(self):
+        out = []
+        for i in range(self.counts()[0]):
+            s = C.c_char_p()
+            _check(lib().ornith_safetensors_name(self.h, C.c_int64(i), C.byref(s)), "safetensors_name")
+            out.append(s.value.decode())
+        return out
+
+    def info(self, name):
+        """(dtype code, shape, bytes as a uint8 copy)"""
+        dt, nd, data, nb = C.c_int(), C.c_int(), C.c_void_p(), C.c_size_t()
+        shape = (C.c_int64 * 8)()
+        _check(lib().ornith_safetensors_info(self.h, name.encode(), C.byref(dt), shape, C.byref(nd),
+                                             C.byref(data), C.byref(nb)), f"safetensors_info({name})")
+        raw = np.frombuffer(C.string_at(data.value, nb.value), np.uint8) if nb.value else np.empty(0, np.uint8)
+        return dt.value, tuple(shape[i] for i in range(nd.value)), raw
+
+    def close(self):
+        if self.h:
+            lib().ornith_safetensors_close(self.h)
+            self.h = None
+
+
+def quant_config_load(model_dir, path):
+    """(group_size, bits, mode) of a module from <model_dir>/config.json's quantization block."""
+    g, b, m = C.c_int(), C.c_int(), C.c_int()
+    _check(lib().ornith_quant_config_load(os.fsencode(model_dir), path.encode(), C.byref(g), C.byref(b),
+                                          C.byref(m)), f"quant_config_load({path})")
+    return g.value, b.value, m.value
 
 
 class Caches:

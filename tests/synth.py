@@ -326,3 +326,88 @@ def zipf_frspec_ids(vocab, n, seed=0, a=1.1):
     rng = np.random.default_rng(seed)
     perm = rng.permutation(vocab)
     return perm[:n].astype(np.uint32)
+
+
+# ---- artifact files --------------------------------------------------------------------------
+_ST_NAMES = {DT_F32: "F32", DT_BF16: "BF16", DT_F16: "F16", DT_U8: "U8", DT_U32: "U32", 5: "I32"}
+
+
+def write_safetensors(path, tensors, metadata=None, header_pad=0):
+    """tensors: name -> (array, dtype code). Bytes are packed back to back in the given order
+    behind `u64 header_len` + JSON, as the safetensors format has it; header_pad appends spaces
+    to the header so the data section can start on any byte offset."""
+    import json
+    head, blobs, off = {}, [], 0
+    if metadata is not None:
+        head["__metadata__"] = metadata
+    for name, (arr, dt) in tensors.items():
+        raw = np.ascontiguousarray(arr).view(np.uint8).reshape(-1).tobytes()
+        head[name] = {"dtype": _ST_NAMES[dt], "shape": list(arr.shape), "data_offsets": [off, off + len(raw)]}
+        off += len(raw)
+        blobs.append(raw)
+    hj = json.dumps(head, separators=(",", ":")).encode() + b" " * header_pad
+    with open(path, "wb") as f:
+        f.write(len(hj).to_bytes(8, "little"))
+        f.write(hj)
+        for b in blobs:
+            f.write(b)
+
+
+def write_artifact(synth, model_dir, shards=3, nested=True):
+    """The synthetic model as the files the loader reads: sharded safetensors + index,
+    config.json (text config, quantization block with per-module overrides) and the MTP
+    sidecar mtp/weights.safetensors with its experts as numbered tensors. Returns the
+    sidecar's path (None without an MTP head)."""
+    import json
+    import os
+    os.makedirs(model_dir, exist_ok=True)
+    trunk = {n: t for n, t in synth.tensors.items() if not n.startswith("mtp.")}
+    names = list(trunk)
+    per = (len(names) + shards - 1) // shards
+    weight_map = {}
+    for s in range(shards):
+        fn = f"model-{s + 1:05d}-of-{shards:05d}.safetensors"
+        part = {n: trunk[n] for n in names[s * per:(s + 1) * per]}
+        write_safetensors(os.path.join(model_dir, fn), part, metadata={"format": "mlx"}, header_pad=s)
+        for n in part:
+            weight_map[n] = fn
+    with open(os.path.join(model_dir, "model.safetensors.index.json"), "w") as f:
+        json.dump({"metadata": {"total_size": synth.total_bytes()}, "weight_map": weight_map}, f)
+
+    quant = {"group_size": 64, "bits": 8, "mode": "affine"}
+    for n, (arr, dt) in synth.tensors.items():
+        if n.endswith(".dm"):
+            q4 = synth.tensors[n[:-3] + ".scales"][0].shape[-1] == 12
+            quant[n[:-3]] = {"group_size": 256, "bits": 4 if q4 else 6, "mode": "q4k" if q4 else "q6k"}
+    c = synth.cfg
+    text = {k: c[k] for k in c if k not in ("rope_dims", "rope_theta", "norm_topk_prob", "rms_norm_eps")}
+    text["rms_norm_eps"] = c["rms_norm_eps"]
+    text["norm_topk_prob"] = bool(c["norm_topk_prob"])
+    text["rope_parameters"] = {"rope_theta": c["rope_theta"], "rope_type": "default",
+                               "partial_rotary_factor": c["rope_dims"] / c["head_dim"]}
+    text["model_type"] = "qwen3_5_moe_text"
+    cfg = {"model_type": "qwen3_5_moe", "quantization": quant,
+           "num_nextn_predict_layers": 1 if synth.mtp else 0}
+    if nested:
+        cfg["text_config"] = text
+    else:
+        cfg.update(text)
+    with open(os.path.join(model_dir, "config.json"), "w") as f:
+        json.dump(cfg, f, indent=1)
+
+    if not synth.mtp:
+        return None
+    side = {}
+    for n, (arr, dt) in synth.tensors.items():
+        if not n.startswith("mtp."):
+            continue
+        if ".switch_mlp." in n:
+            pre, suf = n.split(".switch_mlp.")
+            for e in range(arr.shape[0]):
+                side[f"{pre}.experts.{e}.{suf}"] = (arr[e], dt)
+        else:
+            side[n] = (arr, dt)
+    os.makedirs(os.path.join(model_dir, "mtp"), exist_ok=True)
+    sp = os.path.join(model_dir, "mtp", "weights.safetensors")
+    write_safetensors(sp, side, header_pad=5)
+    return sp
