@@ -116,106 +116,144 @@ struct SdpaArgs {
   float scale;
 };
 
-// grid (nblk, Hq / G, T), 256 threads: G consecutive query heads (of one kv head) per
-// workgroup. Small G spreads the arithmetic over more workgroups (each re-reads its key
-// block from L2); the sums do not depend on G.
-template <int G, int HD>
-__global__ __launch_bounds__(256) void sdpa_partial_kernel(SdpaArgs p) {
-  const int b = blockIdx.x, hq0 = blockIdx.y * G, t = blockIdx.z, tid = threadIdx.x;
+// grid (nblk, Hq, T), 1024 threads: one query head against one block of ATT_KB keys.
+//
+// The arithmetic is small (a chain of HD fmas per key, one of up to ATT_KB per channel) and a
+// trip to memory is long, so the whole block -- every key row and every value row -- is
+// requested by the 16 wavefronts at once, in 16-byte pieces with eight lanes to a 128-byte
+// line, before anything is computed. The rows then pass through LDS: keys in chunks of 64
+// channels (rows padded by 16 bytes to spread the banks), values in trips of 64 keys. Thread
+// `tid` < ATT_KB owns key `tid` for the scores and thread `tid` < HD owns channel `tid` for
+// the values; the sums and their order are those of one thread walking its row. Rows past the
+// last valid key are read from the last one (in bounds) and never added.
+constexpr int SDPA_NT = 1024;
+
+// A native vector, not HIP's uint4 struct: arrays of the struct copied to LDS through casts are
+// left in scratch memory by the compiler, arrays of this type stay in registers.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int HD>
+__global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sdpa_partial_kernel(SdpaArgs p) {
+  const int b = blockIdx.x, hq = blockIdx.y, t = blockIdx.z, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int offset = p.d_offset ? *p.d_offset : p.offset;
   const int last = min(offset + t, p.cap - 1);
   if (b * ATT_KB > last) return;
-  const int gqa = p.Hq / p.Hkv;
-  const int hk = hq0 / gqa;
+  const int hk = hq / (p.Hq / p.Hkv);
 
-  __shared__ float qs[G][HD];
-  __shared__ float pr[G][ATT_KB];
-  __shared__ float red[G][4];
+  constexpr int PPR = HD / 8;                    // 16-byte pieces per row
+  constexpr int RPU = SDPA_NT / PPR;             // rows covered by one load per thread
+  constexpr int NLD = ATT_KB / RPU;              // loads per thread for the block
+  constexpr int KC = 64, NKC = HD / KC, KROW = KC * 2 + 16;
+  constexpr int VB = 64, NVT = ATT_KB / VB, UPT = VB / RPU;
+  static_assert(SDPA_NT % PPR == 0 && VB % RPU == 0 && ATT_KB % RPU == 0, "piece mapping");
+  static_assert(KC == 64 && VB == 64, "one query value / probability per lane of a wavefront");
+  constexpr int STAGE = ATT_KB * KROW > VB * HD * 2 ? ATT_KB * KROW : VB * HD * 2;
+  __shared__ __align__(16) unsigned char stage[STAGE];
+  __shared__ __align__(16) float qs[HD];
+  __shared__ float pr[ATT_KB];
+  __shared__ float red[4];
 
-  const int key = b * ATT_KB + tid;
-  const bool valid = key <= last;
   const int nvalid = min(ATT_KB, last - b * ATT_KB + 1);
-  const bf16_t* krow = p.k_cache + ((size_t)hk * p.cap + (valid ? key : last)) * HD;
+  const bool valid = tid < nvalid;
+  const int row0 = tid / PPR, piece = tid - row0 * PPR;  // this thread's piece column; rows row0 + RPU*u
+  const bf16_t* kbase = p.k_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD;
+  const bf16_t* vblk = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + 8 * piece;
+  // keys: per chunk every thread holds KPC pieces (row krow0 + KRS*i, piece column kpc), so a
+  // chunk is written to LDS by all lanes at once
+  constexpr int KPC = ATT_KB * (KC / 8) / SDPA_NT, KRS = SDPA_NT / (KC / 8);
+  static_assert(KPC * NKC == NLD, "key pieces per thread");
+  const int krow0 = tid / (KC / 8), kpc = tid % (KC / 8);
+  u32x4 kreg[NLD], vreg[NLD];
+#pragma unroll
+  for (int c = 0; c < NKC; ++c)
+#pragma unroll
+    for (int i = 0; i < KPC; ++i)
+      kreg[c * KPC + i] = *reinterpret_cast<const u32x4*>(
+          kbase + (size_t)min(krow0 + KRS * i, nvalid - 1) * HD + c * KC + 8 * kpc);
+#pragma unroll
+  for (int u = 0; u < NLD; ++u)
+    vreg[u] = *reinterpret_cast<const u32x4*>(vblk + (size_t)min(row0 + RPU * u, nvalid - 1) * HD);
+  if (tid < HD) qs[tid] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq) * HD + tid]);
 
-  for (int i = tid; i < G * HD; i += 256) {
-    const int g = i / HD, d = i - g * HD;
-    qs[g][d] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq0 + g) * HD + d]);
-  }
-  __syncthreads();
-  float acc[G];
+  // scores: key `tid`, channels ascending
+  float acc = 0.f;
 #pragma unroll
-  for (int g = 0; g < G; ++g) acc[g] = 0.f;
-#pragma unroll 4
-  for (int dc = 0; dc < HD / 8; ++dc) {
-    const uint4 kw = *reinterpret_cast<const uint4*>(krow + 8 * dc);
-    const float kf[8] = {dm_bf2f_lo(kw.x), dm_bf2f_hi(kw.x), dm_bf2f_lo(kw.y), dm_bf2f_hi(kw.y),
-                         dm_bf2f_lo(kw.z), dm_bf2f_hi(kw.z), dm_bf2f_lo(kw.w), dm_bf2f_hi(kw.w)};
+  for (int c = 0; c < NKC; ++c) {
+    if (c) __syncthreads();  // the previous chunk has been used
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float4 q0 = *reinterpret_cast<const float4*>(&qs[g][8 * dc]);
-      const float4 q1 = *reinterpret_cast<const float4*>(&qs[g][8 * dc + 4]);
-      float a = acc[g];
-      a = dm_fma(q0.x, kf[0], a);
-      a = dm_fma(q0.y, kf[1], a);
-      a = dm_fma(q0.z, kf[2], a);
-      a = dm_fma(q0.w, kf[3], a);
-      a = dm_fma(q1.x, kf[4], a);
-      a = dm_fma(q1.y, kf[5], a);
-      a = dm_fma(q1.z, kf[6], a);
-      a = dm_fma(q1.w, kf[7], a);
-      acc[g] = a;
+    for (int i = 0; i < KPC; ++i)
+      *reinterpret_cast<u32x4*>(stage + (krow0 + KRS * i) * KROW + 16 * kpc) = kreg[c * KPC + i];
+    __syncthreads();  // also orders the query staging before its first use
+    if (tid < ATT_KB) {
+      u32x4 kws[KC / 8];
+#pragma unroll
+      for (int i = 0; i < KC / 8; ++i) kws[i] = *reinterpret_cast<const u32x4*>(stage + tid * KROW + 16 * i);
+      // the chunk's 64 query values: one per lane, handed out through scalar registers (a
+      // broadcast read from LDS per value would cost a trip to LDS each)
+      const int qv = __float_as_int(qs[c * KC + lane]);
+#pragma unroll
+      for (int i = 0; i < KC / 8; ++i) {
+        const u32x4 kw = kws[i];
+        const float kf[8] = {dm_bf2f_lo(kw.x), dm_bf2f_hi(kw.x), dm_bf2f_lo(kw.y), dm_bf2f_hi(kw.y),
+                             dm_bf2f_lo(kw.z), dm_bf2f_hi(kw.z), dm_bf2f_lo(kw.w), dm_bf2f_hi(kw.w)};
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          acc = dm_fma(__int_as_float(__builtin_amdgcn_readlane(qv, 8 * i + e)), kf[e], acc);
+      }
     }
   }
-  // block max per head
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float m = dm_wave_max<64>(valid ? acc[g] : -DM_INF);
-    if (lane == 0) red[g][wave] = m;
+  // block max, probabilities, their sum (the first four wavefronts hold the keys)
+  if (tid < ATT_KB) {
+    const float m = dm_wave_max<64>(valid ? acc : -DM_INF);
+    if (lane == 0) red[wave] = m;
   }
   __syncthreads();
-  float mg[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float m = red[g][0];
-    m = red[g][1] > m ? red[g][1] : m;
-    m = red[g][2] > m ? red[g][2] : m;
-    m = red[g][3] > m ? red[g][3] : m;
-    mg[g] = m;
-  }
+  float mg = red[0];
+  mg = red[1] > mg ? red[1] : mg;
+  mg = red[2] > mg ? red[2] : mg;
+  mg = red[3] > mg ? red[3] : mg;
   __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float pv = valid ? dm_exp(acc[g] - mg[g]) : 0.f;
-    pr[g][tid] = pv;
+  if (tid < ATT_KB) {
+    const float pv = valid ? dm_exp(acc - mg) : 0.f;
+    pr[tid] = pv;
     const float ws = dm_wave_sum<64>(pv);
-    if (lane == 0) red[g][wave] = ws;
+    if (lane == 0) red[wave] = ws;
   }
-  __syncthreads();
-  // values: thread = channel, keys ascending
-  float o[G];
+  __syncthreads();  // the last key chunk has been used as well: the stage is free for values
+  // values: channel `tid`, keys ascending
+  float o = 0.f;
+  bf16_t (*vst)[HD] = reinterpret_cast<bf16_t (*)[HD]>(stage);
 #pragma unroll
-  for (int g = 0; g < G; ++g) o[g] = 0.f;
-  if (tid < HD) {
-    const bf16_t* vcol = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + tid;
-#pragma unroll 8
-    for (int i = 0; i < nvalid; ++i) {
-      const float v = dm_bf2f(vcol[(size_t)i * HD]);
+  for (int tr = 0; tr < NVT; ++tr) {
+    const int i0 = tr * VB;
+    if (i0 < nvalid) {  // uniform
+      if (tr) __syncthreads();  // the previous rows have been added
 #pragma unroll
-      for (int g = 0; g < G; ++g) o[g] = dm_fma(pr[g][i], v, o[g]);
+      for (int uu = 0; uu < UPT; ++uu)
+        *reinterpret_cast<u32x4*>(&vst[row0 + RPU * uu][8 * piece]) = vreg[tr * UPT + uu];
+      __syncthreads();
+      if (tid < HD) {
+        const int prv = __float_as_int(pr[i0 + lane]);  // one probability per lane, as above
+        bf16_t vv[VB];
+#pragma unroll
+        for (int j = 0; j < VB; ++j) vv[j] = vst[j][tid];
+#pragma unroll
+        for (int j = 0; j < VB; ++j) {
+          const float next = dm_fma(__int_as_float(__builtin_amdgcn_readlane(prv, j)), dm_bf2f(vv[j]), o);
+          o = i0 + j < nvalid ? next : o;
+        }
+      }
     }
   }
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const size_t pi = ((size_t)t * p.Hq + hq0 + g) * p.nblk + b;
-    if (tid < HD) p.part_o[pi * HD + tid] = o[g];
-    if (tid == 0) {
-      float l = red[g][0] + red[g][1];
-      l = l + red[g][2];
-      l = l + red[g][3];
-      p.part_m[pi] = mg[g];
-      p.part_l[pi] = l;
-    }
+  const size_t pi = ((size_t)t * p.Hq + hq) * p.nblk + b;
+  if (tid < HD) p.part_o[pi * HD + tid] = o;
+  if (tid == 0) {
+    float l = red[0] + red[1];
+    l = l + red[2];
+    l = l + red[3];
+    p.part_m[pi] = mg;
+    p.part_l[pi] = l;
   }
 }
 
@@ -355,7 +393,7 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   // bounds a block, so spreading heads over workgroups beats sharing the key loads
   dim3 grid(nblk, Hq, T);
 #define SDPA_LAUNCH(G, HD)                                                                  \
-  hipLaunchKernelGGL((sdpa_partial_kernel<G, HD>), grid, dim3(256), 0, ctx->stream, p)
+  hipLaunchKernelGGL((sdpa_partial_kernel<HD>), grid, dim3(SDPA_NT), 0, ctx->stream, p)
   if (hd == 256)
     SDPA_LAUNCH(1, 256);
   else

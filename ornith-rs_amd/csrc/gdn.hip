@@ -214,7 +214,7 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
   __shared__ float ab[2][kStepMaxT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hv = blockIdx.x, ratio = p.Hv / p.Hk, hk = hv / ratio;
-  const int T = p.T, S = p.K - 1, D = p.D, key_dim = p.Hk * 128;
+  const int T = p.T, S = p.K - 1, D = p.D;
 
   // 1. state slice of this thread: row dv = 8*wave + lane/8, columns 32*m + 4*(lane%8) ..+4
   const int row = lane >> 3, j = lane & 7, dv = wave * 8 + row;
@@ -229,6 +229,19 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     s[4 * m + 2] = f.z;
     s[4 * m + 3] = f.w;
   }
+  // operands of the later phases that depend on nothing computed here: requested now, so that
+  // no phase starts with a trip to memory of its own
+  uint32_t wv_pre = 0, zv_pre = 0;
+  if (wave < T) {
+    wv_pre = *reinterpret_cast<const uint32_t*>(a.norm_w + 2 * lane);
+    zv_pre = *reinterpret_cast<const uint32_t*>(a.z + ((size_t)wave * p.Hv + hv) * 128 + 2 * lane);
+  }
+  const bf16_t dtb_pre = p.dt_bias[hv], alog_pre = p.a_log[hv];
+  bf16_t ain_pre = 0, bin_pre = 0;
+  if (!a.wa && tid < T) {
+    ain_pre = p.a_in[tid * p.Hv + hv];
+    bin_pre = p.b_in[tid * p.Hv + hv];
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   // 2. front-end tasks: [0, 3T) conv of (q | k | v, token); then the a / b projections
@@ -239,12 +252,33 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
       const int slot = which == 0 ? hk : which == 1 ? p.Hk + hk : 2 * p.Hk + hv;
       const int c0 = slot * 128 + 2 * lane;
       float acc0 = 0.f, acc1 = 0.f;
-      for (int i = 0; i < p.K; ++i) {
-        const int jj = t + i;
-        const bf16_t* src = (jj < S) ? (p.conv_state + (size_t)jj * D) : (p.qkv + (size_t)(jj - S) * D);
-        const uint32_t xv = *reinterpret_cast<const uint32_t*>(src + c0);
-        acc0 = dm_fma(dm_bf2f_lo(xv), dm_bf2f(p.cw[(size_t)c0 * p.K + i]), acc0);
-        acc1 = dm_fma(dm_bf2f_hi(xv), dm_bf2f(p.cw[(size_t)(c0 + 1) * p.K + i]), acc1);
+      if (p.K == 4) {
+        // the usual window: the four taps of both channels are one 16-byte load, and the four
+        // input rows are requested together
+        const uint4 w8 = *reinterpret_cast<const uint4*>(p.cw + (size_t)c0 * 4);
+        uint32_t xv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int jj = t + i;
+          const bf16_t* src = (jj < S) ? (p.conv_state + (size_t)jj * D) : (p.qkv + (size_t)(jj - S) * D);
+          xv[i] = *reinterpret_cast<const uint32_t*>(src + c0);
+        }
+        acc0 = dm_fma(dm_bf2f_lo(xv[0]), dm_bf2f_lo(w8.x), acc0);
+        acc0 = dm_fma(dm_bf2f_lo(xv[1]), dm_bf2f_hi(w8.x), acc0);
+        acc0 = dm_fma(dm_bf2f_lo(xv[2]), dm_bf2f_lo(w8.y), acc0);
+        acc0 = dm_fma(dm_bf2f_lo(xv[3]), dm_bf2f_hi(w8.y), acc0);
+        acc1 = dm_fma(dm_bf2f_hi(xv[0]), dm_bf2f_lo(w8.z), acc1);
+        acc1 = dm_fma(dm_bf2f_hi(xv[1]), dm_bf2f_hi(w8.z), acc1);
+        acc1 = dm_fma(dm_bf2f_hi(xv[2]), dm_bf2f_lo(w8.w), acc1);
+        acc1 = dm_fma(dm_bf2f_hi(xv[3]), dm_bf2f_hi(w8.w), acc1);
+      } else {
+        for (int i = 0; i < p.K; ++i) {
+          const int jj = t + i;
+          const bf16_t* src = (jj < S) ? (p.conv_state + (size_t)jj * D) : (p.qkv + (size_t)(jj - S) * D);
+          const uint32_t xv = *reinterpret_cast<const uint32_t*>(src + c0);
+          acc0 = dm_fma(dm_bf2f_lo(xv), dm_bf2f(p.cw[(size_t)c0 * p.K + i]), acc0);
+          acc1 = dm_fma(dm_bf2f_hi(xv), dm_bf2f(p.cw[(size_t)(c0 + 1) * p.K + i]), acc1);
+        }
       }
       const float cv0 = dm_rb(acc0), cv1 = dm_rb(acc1);
       const float y0 = dm_rb(cv0 * dm_sigmoid_bf16(cv0)), y1 = dm_rb(cv1 * dm_sigmoid_bf16(cv1));
@@ -278,11 +312,11 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
   }
   __syncthreads();
   if (tid < T) {
-    const int t = tid, i = t * p.Hv + hv;
-    const float av = a.wa ? ab[0][t] : dm_bf2f(p.a_in[i]);
-    const float bv = a.wa ? ab[1][t] : dm_bf2f(p.b_in[i]);
-    const float sp = softplus_bf16(dm_rb(av + dm_bf2f(p.dt_bias[hv])));
-    const float decay = dm_exp(dm_bf2f(p.a_log[hv]));
+    const int t = tid;
+    const float av = a.wa ? ab[0][t] : dm_bf2f(ain_pre);
+    const float bv = a.wa ? ab[1][t] : dm_bf2f(bin_pre);
+    const float sp = softplus_bf16(dm_rb(av + dm_bf2f(dtb_pre)));
+    const float decay = dm_exp(dm_bf2f(alog_pre));
     gs[t] = dm_exp(-decay * sp);
     bs[t] = dm_rb(dm_sigmoid_bf16(bv));
   }
@@ -332,9 +366,8 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     float acc = dm_fma(x0, x0, 0.f);
     acc = dm_fma(x1, x1, acc);
     const float inv = dm_rsqrt(dm_wave_sum<64>(acc) / 128.0f + a.norm_eps);
-    const uint32_t wv = *reinterpret_cast<const uint32_t*>(a.norm_w + 2 * lane);
+    const uint32_t wv = wv_pre, zv = zv_pre;  // t == wave: T never exceeds the wavefront count
     const size_t off = ((size_t)t * p.Hv + hv) * 128 + 2 * lane;
-    const uint32_t zv = *reinterpret_cast<const uint32_t*>(a.z + off);
     x0 = dm_rb(dm_bf2f_lo(wv) * dm_rb(x0 * inv));
     x1 = dm_rb(dm_bf2f_hi(wv) * dm_rb(x1 * inv));
     const float g0 = dm_bf2f_lo(zv), g1 = dm_bf2f_hi(zv);
