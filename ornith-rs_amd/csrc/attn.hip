@@ -257,6 +257,111 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
   }
 }
 
+// The same partial sums when there are many blocks to work through (long contexts): 256
+// threads a block, several blocks resident per compute unit hide each other's trips to memory.
+// grid (nblk, Hq / G, T), 256 threads: G consecutive query heads (of one kv head) per
+// workgroup. Small G spreads the arithmetic over more workgroups (each re-reads its key
+// block from L2); the sums do not depend on G.
+template <int G, int HD>
+__global__ __launch_bounds__(256) void sdpa_partial_many_kernel(SdpaArgs p) {
+  const int b = blockIdx.x, hq0 = blockIdx.y * G, t = blockIdx.z, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int offset = p.d_offset ? *p.d_offset : p.offset;
+  const int last = min(offset + t, p.cap - 1);
+  if (b * ATT_KB > last) return;
+  const int gqa = p.Hq / p.Hkv;
+  const int hk = hq0 / gqa;
+
+  __shared__ float qs[G][HD];
+  __shared__ float pr[G][ATT_KB];
+  __shared__ float red[G][4];
+
+  const int key = b * ATT_KB + tid;
+  const bool valid = key <= last;
+  const int nvalid = min(ATT_KB, last - b * ATT_KB + 1);
+  const bf16_t* krow = p.k_cache + ((size_t)hk * p.cap + (valid ? key : last)) * HD;
+
+  for (int i = tid; i < G * HD; i += 256) {
+    const int g = i / HD, d = i - g * HD;
+    qs[g][d] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq0 + g) * HD + d]);
+  }
+  __syncthreads();
+  float acc[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) acc[g] = 0.f;
+#pragma unroll 4
+  for (int dc = 0; dc < HD / 8; ++dc) {
+    const uint4 kw = *reinterpret_cast<const uint4*>(krow + 8 * dc);
+    const float kf[8] = {dm_bf2f_lo(kw.x), dm_bf2f_hi(kw.x), dm_bf2f_lo(kw.y), dm_bf2f_hi(kw.y),
+                         dm_bf2f_lo(kw.z), dm_bf2f_hi(kw.z), dm_bf2f_lo(kw.w), dm_bf2f_hi(kw.w)};
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      const float4 q0 = *reinterpret_cast<const float4*>(&qs[g][8 * dc]);
+      const float4 q1 = *reinterpret_cast<const float4*>(&qs[g][8 * dc + 4]);
+      float a = acc[g];
+      a = dm_fma(q0.x, kf[0], a);
+      a = dm_fma(q0.y, kf[1], a);
+      a = dm_fma(q0.z, kf[2], a);
+      a = dm_fma(q0.w, kf[3], a);
+      a = dm_fma(q1.x, kf[4], a);
+      a = dm_fma(q1.y, kf[5], a);
+      a = dm_fma(q1.z, kf[6], a);
+      a = dm_fma(q1.w, kf[7], a);
+      acc[g] = a;
+    }
+  }
+  // block max per head
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const float m = dm_wave_max<64>(valid ? acc[g] : -DM_INF);
+    if (lane == 0) red[g][wave] = m;
+  }
+  __syncthreads();
+  float mg[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    float m = red[g][0];
+    m = red[g][1] > m ? red[g][1] : m;
+    m = red[g][2] > m ? red[g][2] : m;
+    m = red[g][3] > m ? red[g][3] : m;
+    mg[g] = m;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const float pv = valid ? dm_exp(acc[g] - mg[g]) : 0.f;
+    pr[g][tid] = pv;
+    const float ws = dm_wave_sum<64>(pv);
+    if (lane == 0) red[g][wave] = ws;
+  }
+  __syncthreads();
+  // values: thread = channel, keys ascending
+  float o[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) o[g] = 0.f;
+  if (tid < HD) {
+    const bf16_t* vcol = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + tid;
+#pragma unroll 8
+    for (int i = 0; i < nvalid; ++i) {
+      const float v = dm_bf2f(vcol[(size_t)i * HD]);
+#pragma unroll
+      for (int g = 0; g < G; ++g) o[g] = dm_fma(pr[g][i], v, o[g]);
+    }
+  }
+#pragma unroll
+  for (int g = 0; g < G; ++g) {
+    const size_t pi = ((size_t)t * p.Hq + hq0 + g) * p.nblk + b;
+    if (tid < HD) p.part_o[pi * HD + tid] = o[g];
+    if (tid == 0) {
+      float l = red[g][0] + red[g][1];
+      l = l + red[g][2];
+      l = l + red[g][3];
+      p.part_m[pi] = mg[g];
+      p.part_l[pi] = l;
+    }
+  }
+}
+
 // grid (Hq, T), HD threads: merge blocks ascending, divide, gate
 template <int HD>
 __global__ __launch_bounds__(HD) void sdpa_merge_kernel(SdpaArgs p) {
@@ -392,13 +497,21 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   // one query head per workgroup: the arithmetic (256 keys x head_dim fmas per head) is what
   // bounds a block, so spreading heads over workgroups beats sharing the key loads
   dim3 grid(nblk, Hq, T);
-#define SDPA_LAUNCH(G, HD)                                                                  \
-  hipLaunchKernelGGL((sdpa_partial_kernel<HD>), grid, dim3(SDPA_NT), 0, ctx->stream, p)
-  if (hd == 256)
-    SDPA_LAUNCH(1, 256);
-  else
-    SDPA_LAUNCH(1, 128);
-#undef SDPA_LAUNCH
+  // few live blocks (short contexts): one 1024-thread block per (key block, head) finishes
+  // soonest; many: the 256-thread form keeps more blocks in flight. Same sums either way.
+  const int last_max = (d_offset ? cap - 1 : (offset + T - 1 < cap - 1 ? offset + T - 1 : cap - 1));
+  const long live = (long)(last_max / ATT_KB + 1) * Hq * T;
+  if (live <= 2L * ctx->compute_units) {
+    if (hd == 256)
+      hipLaunchKernelGGL((sdpa_partial_kernel<256>), grid, dim3(SDPA_NT), 0, ctx->stream, p);
+    else
+      hipLaunchKernelGGL((sdpa_partial_kernel<128>), grid, dim3(SDPA_NT), 0, ctx->stream, p);
+  } else {
+    if (hd == 256)
+      hipLaunchKernelGGL((sdpa_partial_many_kernel<1, 256>), grid, dim3(256), 0, ctx->stream, p);
+    else
+      hipLaunchKernelGGL((sdpa_partial_many_kernel<1, 128>), grid, dim3(256), 0, ctx->stream, p);
+  }
   ORN_LAUNCH_CHECK("sdpa_partial_kernel");
   if (hd == 256)
     hipLaunchKernelGGL(sdpa_merge_kernel<256>, dim3(Hq, T), dim3(256), 0, ctx->stream, p);

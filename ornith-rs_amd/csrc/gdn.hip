@@ -133,47 +133,86 @@ __global__ __launch_bounds__(64) void gdn_recurrence_kernel(RecArgs p) {
     s[4 * m + 2] = f.z;
     s[4 * m + 3] = f.w;
   }
-  for (int t = 0; t < p.T; ++t) {
-    float kf[16], qf[16];
-    const bf16_t* kp = p.k + ((size_t)t * p.Hk + hk) * 128 + 4 * j;
-    const bf16_t* qp = p.q + ((size_t)t * p.Hk + hk) * 128 + 4 * j;
+  // Each token's step is a short dependent chain, far shorter than a trip to L2 for its
+  // operands: the operands of the next GP tokens are requested while this group is worked
+  // through (token indices past the end are clamped and their loads unused).
+  constexpr int GP = 4;
+  typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+  u32x2 kw[GP][4], qw[GP][4];
+  float gg[GP], bb[GP], vv[GP];
+  auto fetch = [&](int t, u32x2 (&kd)[4], u32x2 (&qd)[4], float& gd, float& bd, float& vd) {
+    const int tc = t < p.T ? t : p.T - 1;
+    const bf16_t* kp = p.k + ((size_t)tc * p.Hk + hk) * 128 + 4 * j;
+    const bf16_t* qp = p.q + ((size_t)tc * p.Hk + hk) * 128 + 4 * j;
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
-      const uint2 kw = *reinterpret_cast<const uint2*>(kp + 32 * m);
-      const uint2 qw = *reinterpret_cast<const uint2*>(qp + 32 * m);
-      kf[4 * m + 0] = dm_bf2f_lo(kw.x);
-      kf[4 * m + 1] = dm_bf2f_hi(kw.x);
-      kf[4 * m + 2] = dm_bf2f_lo(kw.y);
-      kf[4 * m + 3] = dm_bf2f_hi(kw.y);
-      qf[4 * m + 0] = dm_bf2f_lo(qw.x);
-      qf[4 * m + 1] = dm_bf2f_hi(qw.x);
-      qf[4 * m + 2] = dm_bf2f_lo(qw.y);
-      qf[4 * m + 3] = dm_bf2f_hi(qw.y);
+      kd[m] = *reinterpret_cast<const u32x2*>(kp + 32 * m);
+      qd[m] = *reinterpret_cast<const u32x2*>(qp + 32 * m);
     }
-    const float gt = p.g[t * p.Hv + hv], bt = dm_bf2f(p.beta[t * p.Hv + hv]);
-    const float vt = dm_bf2f(p.v[((size_t)t * p.Hv + hv) * p.Dv + dv]);
-    float a = 0.f;
+    gd = p.g[tc * p.Hv + hv];
+    bd = dm_bf2f(p.beta[tc * p.Hv + hv]);
+    vd = dm_bf2f(p.v[((size_t)tc * p.Hv + hv) * p.Dv + dv]);
+  };
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      s[e] = s[e] * gt;
-      a = dm_fma(s[e], kf[e], a);
+  for (int i = 0; i < GP; ++i) fetch(i, kw[i], qw[i], gg[i], bb[i], vv[i]);
+  for (int t0 = 0; t0 < p.T; t0 += GP) {
+    u32x2 kwn[GP][4], qwn[GP][4];
+    float ggn[GP], bbn[GP], vvn[GP];
+#pragma unroll
+    for (int i = 0; i < GP; ++i) fetch(t0 + GP + i, kwn[i], qwn[i], ggn[i], bbn[i], vvn[i]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < GP; ++i) {
+      const int t = t0 + i;
+      if (t < p.T) {
+        float kf[16], qf[16];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          kf[4 * m + 0] = dm_bf2f_lo(kw[i][m].x);
+          kf[4 * m + 1] = dm_bf2f_hi(kw[i][m].x);
+          kf[4 * m + 2] = dm_bf2f_lo(kw[i][m].y);
+          kf[4 * m + 3] = dm_bf2f_hi(kw[i][m].y);
+          qf[4 * m + 0] = dm_bf2f_lo(qw[i][m].x);
+          qf[4 * m + 1] = dm_bf2f_hi(qw[i][m].x);
+          qf[4 * m + 2] = dm_bf2f_lo(qw[i][m].y);
+          qf[4 * m + 3] = dm_bf2f_hi(qw[i][m].y);
+        }
+        const float gt = gg[i], bt = bb[i], vt = vv[i];
+        float a = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          s[e] = s[e] * gt;
+          a = dm_fma(s[e], kf[e], a);
+        }
+        const float kv = dm_wave_sum<8>(a);
+        const float delta = (vt - kv) * bt;
+        float o = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          s[e] = dm_fma(kf[e], delta, s[e]);
+          o = dm_fma(s[e], qf[e], o);
+        }
+        o = dm_wave_sum<8>(o);
+        if (j == 0) p.y[((size_t)t * p.Hv + hv) * p.Dv + dv] = dm_f2bf(o);
+        if (p.snap_all || t + 1 == p.T) {
+          float* snap = p.snapshots + (p.snap_all ? (size_t)t * ssz : 0) + roff;
+#pragma unroll
+          for (int m = 0; m < 4; ++m)
+            *reinterpret_cast<float4*>(snap + 32 * m) =
+                make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+        }
+      }
     }
-    const float kv = dm_wave_sum<8>(a);
-    const float delta = (vt - kv) * bt;
-    float o = 0.f;
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      s[e] = dm_fma(kf[e], delta, s[e]);
-      o = dm_fma(s[e], qf[e], o);
-    }
-    o = dm_wave_sum<8>(o);
-    if (j == 0) p.y[((size_t)t * p.Hv + hv) * p.Dv + dv] = dm_f2bf(o);
-    if (p.snap_all || t + 1 == p.T) {
-      float* snap = p.snapshots + (p.snap_all ? (size_t)t * ssz : 0) + roff;
+    for (int i = 0; i < GP; ++i) {
 #pragma unroll
-      for (int m = 0; m < 4; ++m)
-        *reinterpret_cast<float4*>(snap + 32 * m) =
-            make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+      for (int m = 0; m < 4; ++m) {
+        kw[i][m] = kwn[i][m];
+        qw[i][m] = qwn[i][m];
+      }
+      gg[i] = ggn[i];
+      bb[i] = bbn[i];
+      vv[i] = vvn[i];
     }
   }
 }
