@@ -27,6 +27,10 @@ FLAGS = [
 ]
 
 
+# extra compiler flags for one-off builds (e.g. -DORN_TIMING: per-workgroup time stamps)
+FLAGS += os.environ.get("ORN_EXTRA_FLAGS", "").split()
+
+
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith((".hip", ".cpp")))
 

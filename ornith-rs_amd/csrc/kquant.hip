@@ -53,6 +53,17 @@ struct KqArgs {
   PreNorm pre;    // PRE kernels: the activations are rms_norm(res + y) computed by every workgroup
 };
 
+#ifdef ORN_TIMING
+// debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch
+__device__ long long g_marks[4096][8];
+#define ORN_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x < 4096 && blockIdx.y == 0) g_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks(long long* out, int blocks) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_marks), sizeof(long long) * 8 * blocks);
+}
+#else
+#define ORN_MARK(i)
+#endif
+
 // One kernel for plain and gathered mat-vecs.
 //   KIND  format; LPR lanes per row (4,8,16,32,64); KS wavefronts per row (1,2)
 //   M     activation rows sharing each weight read (1..4); gather uses M == 1
@@ -62,6 +73,7 @@ struct KqArgs {
 //         loads are in flight; workgroup 0 also stores h and x for later consumers
 template <int KIND, int LPR, int KS, int M, bool XF32, bool GATHER, bool PRE = false>
 __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
+  ORN_MARK(0);
   using KL = KqLane<KIND, M>;
   constexpr int RPW = 64 / LPR;  // rows in flight per wavefront
   constexpr int WPB = 4 / KS;    // row-wavefronts per block
@@ -71,9 +83,32 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
   const int rw = (KS == 1) ? wave : (wave >> 1);
   const int nb = a.K >> 8;
 
-  int s = 0;
-  while (s + 1 < a.nseg && (int)blockIdx.x >= a.seg[s + 1].first_block) ++s;
-  const KqSeg sg = a.seg[s];
+  // every segment's fields are fetched at once and one is selected: indexing the argument
+  // array with a computed value would put a second scalar memory trip ahead of the first
+  // weight load
+  KqSeg sg = a.seg[0];
+  {
+    KqSeg all[kMaxSeg];
+    int nseg = a.nseg;
+#pragma unroll
+    for (int i = 0; i < kMaxSeg; ++i) {
+      all[i] = a.seg[i];
+      // pins the values (not their addresses) in scalar registers here, so that all the
+      // argument loads above are issued together and waited for once
+      uint64_t q = (uint64_t)all[i].qs, sc = (uint64_t)all[i].scales, d = (uint64_t)all[i].dm,
+               y = (uint64_t)all[i].y;
+      asm volatile("" : "+s"(q), "+s"(sc), "+s"(d), "+s"(y), "+s"(all[i].O), "+s"(all[i].first_block));
+      all[i].qs = (const uint8_t*)q;
+      all[i].scales = (const uint8_t*)sc;
+      all[i].dm = (const uint16_t*)d;
+      all[i].y = (void*)y;
+    }
+    asm volatile("" : "+s"(nseg));
+    sg = all[0];
+#pragma unroll
+    for (int i = 1; i < kMaxSeg; ++i)
+      if (i < nseg && (int)blockIdx.x >= all[i].first_block) sg = all[i];
+  }
   const int O = sg.O;
 
   const size_t xsz = XF32 ? 4 : 2;
@@ -112,13 +147,16 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
 #pragma unroll
   for (int i = 0; i < PF; ++i) pf[i] = KL::load(sg.qs, sg.scales, sg.dm, row_of(i), nb, L);
   __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  ORN_MARK(1);
   if constexpr (PRE) {
     __shared__ PreNormLds<M> pn;
     prenorm_rows<M>(a.pre, blockIdx.x == 0, pn);
 #pragma unroll
     for (int t = 0; t < M; ++t) xrow[t] = &pn.xn[t][0];
   }
+  ORN_MARK(2);
   L.template load_x<XF32>(xrow, c + 64 * ks);
+  ORN_MARK(3);
 
   for (int it0 = 0; it0 < a.iters; it0 += PF) {
 #pragma unroll
@@ -133,6 +171,7 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
     const typename KL::Row r = pf[i];
     if (it + PF < a.iters) pf[i] = KL::load(sg.qs, sg.scales, sg.dm, row_of(it + PF), nb, L);
     KL::accumulate(r, L, acc);
+    if (it == 0) ORN_MARK(4);
     if constexpr (KS == 2) {
       // lane partial = (chunk l) + (chunk l + 64), in that order
       float* mine = part + rw * M * 64;
@@ -160,6 +199,7 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
     }
    }
   }
+  ORN_MARK(5);
 }
 
 // one thread per 256-weight block, the shape of the reference loop
