@@ -93,6 +93,15 @@ ORC_API void orc_attn_prep(const bf16_t* qg, const bf16_t* kx, const bf16_t* vx,
   }
 }
 
+/* n = 1, 2, 4 or 8 values added pairwise: (p0 + p1) + (p2 + p3), ... */
+static float pair_tree(const float* p, int n) {
+  float t[8];
+  for (int i = 0; i < n; ++i) t[i] = p[i];
+  for (int w = n; w > 1; w /= 2)
+    for (int i = 0; i < w / 2; ++i) t[i] = t[2 * i] + t[2 * i + 1];
+  return t[0];
+}
+
 /*
  * q_rot [T, Hq, hd], caches [Hkv, cap, hd] holding offset+T rows, gate [T, Hq, hd]
  * -> out [T, Hq*hd] = bf16(sigmoid_bf16(gate) * bf16(attn)). hd <= 512.
@@ -122,8 +131,15 @@ ORC_API void orc_sdpa_decode_gated(const bf16_t* q_rot, const bf16_t* k_cache,
             continue;
           }
           const bf16_t* kr = k_cache + ((size_t)hk * cap + key) * hd;
-          float a = 0.f;
-          for (int d = 0; d < hd; ++d) a = fmaf(qs[d], orc_bf16_to_f32(kr[d]), a);
+          /* one chain per 64 channels, the chains added pairwise */
+          float part[8];
+          const int nch = hd / 64;
+          for (int c = 0; c < nch; ++c) {
+            float a = 0.f;
+            for (int d = 64 * c; d < 64 * c + 64; ++d) a = fmaf(qs[d], orc_bf16_to_f32(kr[d]), a);
+            part[c] = a;
+          }
+          const float a = pair_tree(part, nch);
           s[i] = a;
           m = a > m ? a : m;
         }
@@ -134,13 +150,19 @@ ORC_API void orc_sdpa_decode_gated(const bf16_t* q_rot, const bf16_t* k_cache,
         l = l + orc_tree64(pr + 128);
         l = l + orc_tree64(pr + 192);
         for (int d = 0; d < hd; ++d) {
-          float a = 0.f;
-          for (int i = 0; i < ATT_KB; ++i) {
-            const int key = b * ATT_KB + i;
-            if (key > last) break; /* p = 0 beyond: fma(0, v, a) == a */
-            a = fmaf(pr[i], orc_bf16_to_f32(v_cache[((size_t)hk * cap + key) * hd + d]), a);
+          /* one chain per 64 keys (keys past the last visible one are not added), the four
+           * chains added pairwise */
+          float part[ATT_KB / 64];
+          for (int c = 0; c < ATT_KB / 64; ++c) {
+            float a = 0.f;
+            for (int i = 64 * c; i < 64 * c + 64; ++i) {
+              const int key = b * ATT_KB + i;
+              if (key > last) break;
+              a = fmaf(pr[i], orc_bf16_to_f32(v_cache[((size_t)hk * cap + key) * hd + d]), a);
+            }
+            part[c] = a;
           }
-          ob[(size_t)b * hd + d] = a;
+          ob[(size_t)b * hd + d] = pair_tree(part, ATT_KB / 64);
         }
         mb[b] = m;
         lb[b] = l;

@@ -118,19 +118,41 @@ struct SdpaArgs {
 
 // grid (nblk, Hq, T), 1024 threads: one query head against one block of ATT_KB keys.
 //
-// The arithmetic is small (a chain of HD fmas per key, one of up to ATT_KB per channel) and a
-// trip to memory is long, so the whole block -- every key row and every value row -- is
-// requested by the 16 wavefronts at once, in 16-byte pieces with eight lanes to a 128-byte
-// line, before anything is computed. The rows then pass through LDS: keys in chunks of 64
-// channels (rows padded by 16 bytes to spread the banks), values in trips of 64 keys. Thread
-// `tid` < ATT_KB owns key `tid` for the scores and thread `tid` < HD owns channel `tid` for
-// the values; the sums and their order are those of one thread walking its row. Rows past the
-// last valid key are read from the last one (in bounds) and never added.
+// The sums: a key's score is one fma chain per 64 channels, the chains added pairwise
+// ((c0 + c1) + (c2 + c3)); a channel's output over the block is one chain per 64 keys, added
+// the same way. That gives every one of the 1024 threads a chain of 64 in both phases.
+//
+// The arithmetic is small and a trip to memory is long, so the whole block -- every key row
+// and every value row -- is requested by the 16 wavefronts at once, in 16-byte pieces with
+// eight lanes to a 128-byte line, before anything is computed. The rows then pass through
+// LDS (keys as 64-channel panels with rows padded by 16 bytes to spread the banks; the values
+// take the same memory over once the scores are done). Rows past the last valid key are read
+// from the last one (in bounds) and never added.
 constexpr int SDPA_NT = 1024;
+constexpr int SDPA_KROW = 64 * 2 + 16;  // bytes of a staged 64-channel key row
 
 // A native vector, not HIP's uint4 struct: arrays of the struct copied to LDS through casts are
 // left in scratch memory by the compiler, arrays of this type stay in registers.
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <int HD>
+constexpr int sdpa_stage_bytes() {
+  constexpr int k = (HD / 64) * ATT_KB * SDPA_KROW, v = ATT_KB * HD * 2;
+  return k > v ? k : v;
+}
+
+// (p0 + p1) + (p2 + p3) for N = 4, p0 + p1 for N = 2
+template <int N>
+__device__ __forceinline__ float sdpa_pair_tree(const float* p, int stride) {
+  float t[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) t[i] = p[i * stride];
+#pragma unroll
+  for (int w = N; w > 1; w /= 2)
+#pragma unroll
+    for (int i = 0; i < w / 2; ++i) t[i] = t[2 * i] + t[2 * i + 1];
+  return t[0];
+}
 
 template <int HD>
 __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sdpa_partial_kernel(SdpaArgs p) {
@@ -142,28 +164,24 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
   const int hk = hq / (p.Hq / p.Hkv);
 
   constexpr int PPR = HD / 8;                    // 16-byte pieces per row
-  constexpr int RPU = SDPA_NT / PPR;             // rows covered by one load per thread
-  constexpr int NLD = ATT_KB / RPU;              // loads per thread for the block
-  constexpr int KC = 64, NKC = HD / KC, KROW = KC * 2 + 16;
-  constexpr int VB = 64, NVT = ATT_KB / VB, UPT = VB / RPU;
-  static_assert(SDPA_NT % PPR == 0 && VB % RPU == 0 && ATT_KB % RPU == 0, "piece mapping");
-  static_assert(KC == 64 && VB == 64, "one query value / probability per lane of a wavefront");
-  constexpr int STAGE = ATT_KB * KROW > VB * HD * 2 ? ATT_KB * KROW : VB * HD * 2;
-  __shared__ __align__(16) unsigned char stage[STAGE];
+  constexpr int RPU = SDPA_NT / PPR;             // value rows covered by one load per thread
+  constexpr int NLD = ATT_KB / RPU;              // loads per thread for the block (keys: same count)
+  constexpr int KC = 64, NKC = HD / KC, KROW = SDPA_KROW;
+  constexpr int KPC = ATT_KB * (KC / 8) / SDPA_NT, KRS = SDPA_NT / (KC / 8);
+  constexpr int VB = 64, NVB = ATT_KB / VB;
+  static_assert(SDPA_NT % PPR == 0 && ATT_KB % RPU == 0 && KPC * NKC == NLD, "piece mapping");
+  static_assert(ATT_KB == 256 && NKC <= 4 && NVB == 4 && HD <= 256, "chains of 64, four wavefronts a chain group");
+  extern __shared__ __align__(16) unsigned char stage[];
   __shared__ __align__(16) float qs[HD];
   __shared__ float pr[ATT_KB];
   __shared__ float red[4];
+  __shared__ float part[4 * 256];  // chain results: [panel][key], later [key group][channel]
 
   const int nvalid = min(ATT_KB, last - b * ATT_KB + 1);
-  const bool valid = tid < nvalid;
-  const int row0 = tid / PPR, piece = tid - row0 * PPR;  // this thread's piece column; rows row0 + RPU*u
+  const int row0 = tid / PPR, piece = tid - row0 * PPR;    // values: rows row0 + RPU*u, piece column
+  const int krow0 = tid / (KC / 8), kpc = tid % (KC / 8);  // keys: rows krow0 + KRS*i of every panel
   const bf16_t* kbase = p.k_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD;
   const bf16_t* vblk = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + 8 * piece;
-  // keys: per chunk every thread holds KPC pieces (row krow0 + KRS*i, piece column kpc), so a
-  // chunk is written to LDS by all lanes at once
-  constexpr int KPC = ATT_KB * (KC / 8) / SDPA_NT, KRS = SDPA_NT / (KC / 8);
-  static_assert(KPC * NKC == NLD, "key pieces per thread");
-  const int krow0 = tid / (KC / 8), kpc = tid % (KC / 8);
   u32x4 kreg[NLD], vreg[NLD];
 #pragma unroll
   for (int c = 0; c < NKC; ++c)
@@ -176,36 +194,41 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
     vreg[u] = *reinterpret_cast<const u32x4*>(vblk + (size_t)min(row0 + RPU * u, nvalid - 1) * HD);
   if (tid < HD) qs[tid] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq) * HD + tid]);
 
-  // scores: key `tid`, channels ascending
-  float acc = 0.f;
+  // scores: thread (key, panel) runs the chain over the panel's 64 channels
 #pragma unroll
-  for (int c = 0; c < NKC; ++c) {
-    if (c) __syncthreads();  // the previous chunk has been used
+  for (int c = 0; c < NKC; ++c)
 #pragma unroll
     for (int i = 0; i < KPC; ++i)
-      *reinterpret_cast<u32x4*>(stage + (krow0 + KRS * i) * KROW + 16 * kpc) = kreg[c * KPC + i];
-    __syncthreads();  // also orders the query staging before its first use
-    if (tid < ATT_KB) {
-      u32x4 kws[KC / 8];
+      *reinterpret_cast<u32x4*>(stage + c * (ATT_KB * KROW) + (krow0 + KRS * i) * KROW + 16 * kpc) =
+          kreg[c * KPC + i];
+  __syncthreads();
+  const int key = tid & (ATT_KB - 1), grp = tid >> 8;  // four wavefronts a group
+  if (grp < NKC) {
+    u32x4 kws[KC / 8];
 #pragma unroll
-      for (int i = 0; i < KC / 8; ++i) kws[i] = *reinterpret_cast<const u32x4*>(stage + tid * KROW + 16 * i);
-      // the chunk's 64 query values: one per lane, handed out through scalar registers (a
-      // broadcast read from LDS per value would cost a trip to LDS each)
-      const int qv = __float_as_int(qs[c * KC + lane]);
+    for (int i = 0; i < KC / 8; ++i)
+      kws[i] = *reinterpret_cast<const u32x4*>(stage + grp * (ATT_KB * KROW) + key * KROW + 16 * i);
+    // the panel's 64 query values: one per lane, handed out through scalar registers
+    const int qv = __float_as_int(qs[grp * KC + lane]);
+    float acc = 0.f;
 #pragma unroll
-      for (int i = 0; i < KC / 8; ++i) {
-        const u32x4 kw = kws[i];
-        const float kf[8] = {dm_bf2f_lo(kw.x), dm_bf2f_hi(kw.x), dm_bf2f_lo(kw.y), dm_bf2f_hi(kw.y),
-                             dm_bf2f_lo(kw.z), dm_bf2f_hi(kw.z), dm_bf2f_lo(kw.w), dm_bf2f_hi(kw.w)};
+    for (int i = 0; i < KC / 8; ++i) {
+      const u32x4 kw = kws[i];
+      const float kf[8] = {dm_bf2f_lo(kw.x), dm_bf2f_hi(kw.x), dm_bf2f_lo(kw.y), dm_bf2f_hi(kw.y),
+                           dm_bf2f_lo(kw.z), dm_bf2f_hi(kw.z), dm_bf2f_lo(kw.w), dm_bf2f_hi(kw.w)};
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          acc = dm_fma(__int_as_float(__builtin_amdgcn_readlane(qv, 8 * i + e)), kf[e], acc);
-      }
+      for (int e = 0; e < 8; ++e)
+        acc = dm_fma(__int_as_float(__builtin_amdgcn_readlane(qv, 8 * i + e)), kf[e], acc);
     }
+    part[grp * ATT_KB + key] = acc;
   }
+  __syncthreads();
   // block max, probabilities, their sum (the first four wavefronts hold the keys)
+  const bool valid = tid < nvalid;
+  float sc = 0.f;
   if (tid < ATT_KB) {
-    const float m = dm_wave_max<64>(valid ? acc : -DM_INF);
+    sc = sdpa_pair_tree<NKC>(part + tid, ATT_KB);
+    const float m = dm_wave_max<64>(valid ? sc : -DM_INF);
     if (lane == 0) red[wave] = m;
   }
   __syncthreads();
@@ -215,39 +238,33 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
   mg = red[3] > mg ? red[3] : mg;
   __syncthreads();
   if (tid < ATT_KB) {
-    const float pv = valid ? dm_exp(acc - mg) : 0.f;
+    const float pv = valid ? dm_exp(sc - mg) : 0.f;
     pr[tid] = pv;
     const float ws = dm_wave_sum<64>(pv);
     if (lane == 0) red[wave] = ws;
   }
-  __syncthreads();  // the last key chunk has been used as well: the stage is free for values
-  // values: channel `tid`, keys ascending
-  float o = 0.f;
+  // values: thread (channel, group of 64 keys) runs the chain over the group's valid keys
   bf16_t (*vst)[HD] = reinterpret_cast<bf16_t (*)[HD]>(stage);
 #pragma unroll
-  for (int tr = 0; tr < NVT; ++tr) {
-    const int i0 = tr * VB;
-    if (i0 < nvalid) {  // uniform
-      if (tr) __syncthreads();  // the previous rows have been added
+  for (int u = 0; u < NLD; ++u) *reinterpret_cast<u32x4*>(&vst[row0 + RPU * u][8 * piece]) = vreg[u];
+  __syncthreads();  // probabilities and value rows in place (the key panels were last read two barriers ago)
+  const int ch = tid % HD, vg = tid / HD;
+  if (vg < NVB) {
+    const int prv = __float_as_int(pr[VB * vg + lane]);
+    bf16_t vv[VB];
 #pragma unroll
-      for (int uu = 0; uu < UPT; ++uu)
-        *reinterpret_cast<u32x4*>(&vst[row0 + RPU * uu][8 * piece]) = vreg[tr * UPT + uu];
-      __syncthreads();
-      if (tid < HD) {
-        const int prv = __float_as_int(pr[i0 + lane]);  // one probability per lane, as above
-        bf16_t vv[VB];
+    for (int j = 0; j < VB; ++j) vv[j] = vst[VB * vg + j][ch];
+    float o = 0.f;
 #pragma unroll
-        for (int j = 0; j < VB; ++j) vv[j] = vst[j][tid];
-#pragma unroll
-        for (int j = 0; j < VB; ++j) {
-          const float next = dm_fma(__int_as_float(__builtin_amdgcn_readlane(prv, j)), dm_bf2f(vv[j]), o);
-          o = i0 + j < nvalid ? next : o;
-        }
-      }
+    for (int j = 0; j < VB; ++j) {
+      const float next = dm_fma(__int_as_float(__builtin_amdgcn_readlane(prv, j)), dm_bf2f(vv[j]), o);
+      o = VB * vg + j < nvalid ? next : o;
     }
+    part[vg * HD + ch] = o;
   }
+  __syncthreads();
   const size_t pi = ((size_t)t * p.Hq + hq) * p.nblk + b;
-  if (tid < HD) p.part_o[pi * HD + tid] = o;
+  if (tid < HD) p.part_o[pi * HD + tid] = sdpa_pair_tree<NVB>(part + tid, HD);
   if (tid == 0) {
     float l = red[0] + red[1];
     l = l + red[2];
@@ -258,107 +275,91 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
 }
 
 // The same partial sums when there are many blocks to work through (long contexts): 256
-// threads a block, several blocks resident per compute unit hide each other's trips to memory.
-// grid (nblk, Hq / G, T), 256 threads: G consecutive query heads (of one kv head) per
-// workgroup. Small G spreads the arithmetic over more workgroups (each re-reads its key
-// block from L2); the sums do not depend on G.
-template <int G, int HD>
+// threads and little LDS a block, so that several blocks are resident per compute unit and
+// hide each other's trips to memory. Thread `tid` owns key `tid` for the scores and channel
+// `tid` for the values and runs the chains of 64 one after the other.
+// grid (nblk, Hq, T), 256 threads.
+template <int HD>
 __global__ __launch_bounds__(256) void sdpa_partial_many_kernel(SdpaArgs p) {
-  const int b = blockIdx.x, hq0 = blockIdx.y * G, t = blockIdx.z, tid = threadIdx.x;
+  const int b = blockIdx.x, hq = blockIdx.y, t = blockIdx.z, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int offset = p.d_offset ? *p.d_offset : p.offset;
   const int last = min(offset + t, p.cap - 1);
   if (b * ATT_KB > last) return;
-  const int gqa = p.Hq / p.Hkv;
-  const int hk = hq0 / gqa;
+  const int hk = hq / (p.Hq / p.Hkv);
+  constexpr int NKC = HD / 64, NVB = ATT_KB / 64;
 
-  __shared__ float qs[G][HD];
-  __shared__ float pr[G][ATT_KB];
-  __shared__ float red[G][4];
+  __shared__ __align__(16) float qs[HD];
+  __shared__ float pr[ATT_KB];
+  __shared__ float red[4];
 
   const int key = b * ATT_KB + tid;
   const bool valid = key <= last;
   const int nvalid = min(ATT_KB, last - b * ATT_KB + 1);
   const bf16_t* krow = p.k_cache + ((size_t)hk * p.cap + (valid ? key : last)) * HD;
 
-  for (int i = tid; i < G * HD; i += 256) {
-    const int g = i / HD, d = i - g * HD;
-    qs[g][d] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq0 + g) * HD + d]);
-  }
+  for (int d = tid; d < HD; d += 256) qs[d] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq) * HD + d]);
   __syncthreads();
-  float acc[G];
+  float cpart[NKC];
 #pragma unroll
-  for (int g = 0; g < G; ++g) acc[g] = 0.f;
+  for (int c = 0; c < NKC; ++c) {
+    float a = 0.f;
 #pragma unroll 4
-  for (int dc = 0; dc < HD / 8; ++dc) {
-    const uint4 kw = *reinterpret_cast<const uint4*>(krow + 8 * dc);
-    const float kf[8] = {dm_bf2f_lo(kw.x), dm_bf2f_hi(kw.x), dm_bf2f_lo(kw.y), dm_bf2f_hi(kw.y),
-                         dm_bf2f_lo(kw.z), dm_bf2f_hi(kw.z), dm_bf2f_lo(kw.w), dm_bf2f_hi(kw.w)};
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const float4 q0 = *reinterpret_cast<const float4*>(&qs[g][8 * dc]);
-      const float4 q1 = *reinterpret_cast<const float4*>(&qs[g][8 * dc + 4]);
-      float a = acc[g];
-      a = dm_fma(q0.x, kf[0], a);
-      a = dm_fma(q0.y, kf[1], a);
-      a = dm_fma(q0.z, kf[2], a);
-      a = dm_fma(q0.w, kf[3], a);
-      a = dm_fma(q1.x, kf[4], a);
-      a = dm_fma(q1.y, kf[5], a);
-      a = dm_fma(q1.z, kf[6], a);
-      a = dm_fma(q1.w, kf[7], a);
-      acc[g] = a;
+    for (int dc = 8 * c; dc < 8 * c + 8; ++dc) {
+      const uint4 kw = *reinterpret_cast<const uint4*>(krow + 8 * dc);
+      const float4 q0 = *reinterpret_cast<const float4*>(&qs[8 * dc]);
+      const float4 q1 = *reinterpret_cast<const float4*>(&qs[8 * dc + 4]);
+      a = dm_fma(q0.x, dm_bf2f_lo(kw.x), a);
+      a = dm_fma(q0.y, dm_bf2f_hi(kw.x), a);
+      a = dm_fma(q0.z, dm_bf2f_lo(kw.y), a);
+      a = dm_fma(q0.w, dm_bf2f_hi(kw.y), a);
+      a = dm_fma(q1.x, dm_bf2f_lo(kw.z), a);
+      a = dm_fma(q1.y, dm_bf2f_hi(kw.z), a);
+      a = dm_fma(q1.z, dm_bf2f_lo(kw.w), a);
+      a = dm_fma(q1.w, dm_bf2f_hi(kw.w), a);
     }
+    cpart[c] = a;
   }
-  // block max per head
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float m = dm_wave_max<64>(valid ? acc[g] : -DM_INF);
-    if (lane == 0) red[g][wave] = m;
-  }
-  __syncthreads();
-  float mg[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float m = red[g][0];
-    m = red[g][1] > m ? red[g][1] : m;
-    m = red[g][2] > m ? red[g][2] : m;
-    m = red[g][3] > m ? red[g][3] : m;
-    mg[g] = m;
+  const float sc = sdpa_pair_tree<NKC>(cpart, 1);
+  // block max
+  {
+    const float m = dm_wave_max<64>(valid ? sc : -DM_INF);
+    if (lane == 0) red[wave] = m;
   }
   __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const float pv = valid ? dm_exp(acc[g] - mg[g]) : 0.f;
-    pr[g][tid] = pv;
+  float mg = red[0];
+  mg = red[1] > mg ? red[1] : mg;
+  mg = red[2] > mg ? red[2] : mg;
+  mg = red[3] > mg ? red[3] : mg;
+  __syncthreads();
+  {
+    const float pv = valid ? dm_exp(sc - mg) : 0.f;
+    pr[tid] = pv;
     const float ws = dm_wave_sum<64>(pv);
-    if (lane == 0) red[g][wave] = ws;
+    if (lane == 0) red[wave] = ws;
   }
   __syncthreads();
-  // values: thread = channel, keys ascending
-  float o[G];
-#pragma unroll
-  for (int g = 0; g < G; ++g) o[g] = 0.f;
+  // values: channel `tid`, one chain per 64 keys
+  const size_t pi = ((size_t)t * p.Hq + hq) * p.nblk + b;
   if (tid < HD) {
     const bf16_t* vcol = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + tid;
+    float opart[NVB];
+#pragma unroll
+    for (int g = 0; g < NVB; ++g) {
+      float o = 0.f;
+      const int end = min(64 * g + 64, nvalid);
 #pragma unroll 8
-    for (int i = 0; i < nvalid; ++i) {
-      const float v = dm_bf2f(vcol[(size_t)i * HD]);
-#pragma unroll
-      for (int g = 0; g < G; ++g) o[g] = dm_fma(pr[g][i], v, o[g]);
+      for (int i = 64 * g; i < end; ++i) o = dm_fma(pr[i], dm_bf2f(vcol[(size_t)i * HD]), o);
+      opart[g] = o;
     }
+    p.part_o[pi * HD + tid] = sdpa_pair_tree<NVB>(opart, 1);
   }
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    const size_t pi = ((size_t)t * p.Hq + hq0 + g) * p.nblk + b;
-    if (tid < HD) p.part_o[pi * HD + tid] = o[g];
-    if (tid == 0) {
-      float l = red[g][0] + red[g][1];
-      l = l + red[g][2];
-      l = l + red[g][3];
-      p.part_m[pi] = mg[g];
-      p.part_l[pi] = l;
-    }
+  if (tid == 0) {
+    float l = red[0] + red[1];
+    l = l + red[2];
+    l = l + red[3];
+    p.part_m[pi] = mg;
+    p.part_l[pi] = l;
   }
 }
 
@@ -501,16 +502,28 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   // soonest; many: the 256-thread form keeps more blocks in flight. Same sums either way.
   const int last_max = (d_offset ? cap - 1 : (offset + T - 1 < cap - 1 ? offset + T - 1 : cap - 1));
   const long live = (long)(last_max / ATT_KB + 1) * Hq * T;
-  if (live <= 2L * ctx->compute_units) {
+  if (live > 2L * ctx->compute_units) {
     if (hd == 256)
-      hipLaunchKernelGGL((sdpa_partial_kernel<256>), grid, dim3(SDPA_NT), 0, ctx->stream, p);
+      hipLaunchKernelGGL((sdpa_partial_many_kernel<256>), grid, dim3(256), 0, ctx->stream, p);
     else
-      hipLaunchKernelGGL((sdpa_partial_kernel<128>), grid, dim3(SDPA_NT), 0, ctx->stream, p);
+      hipLaunchKernelGGL((sdpa_partial_many_kernel<128>), grid, dim3(256), 0, ctx->stream, p);
+  } else if (hd == 256) {
+    // 150 KB of LDS a block (the whole key block staged at once): asked for once per kernel
+    static bool lds_set = false;
+    if (!lds_set) {
+      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<256>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<256>()));
+      lds_set = true;
+    }
+    hipLaunchKernelGGL((sdpa_partial_kernel<256>), grid, dim3(SDPA_NT), sdpa_stage_bytes<256>(), ctx->stream, p);
   } else {
-    if (hd == 256)
-      hipLaunchKernelGGL((sdpa_partial_many_kernel<1, 256>), grid, dim3(256), 0, ctx->stream, p);
-    else
-      hipLaunchKernelGGL((sdpa_partial_many_kernel<1, 128>), grid, dim3(256), 0, ctx->stream, p);
+    static bool lds_set = false;
+    if (!lds_set) {
+      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<128>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<128>()));
+      lds_set = true;
+    }
+    hipLaunchKernelGGL((sdpa_partial_kernel<128>), grid, dim3(SDPA_NT), sdpa_stage_bytes<128>(), ctx->stream, p);
   }
   ORN_LAUNCH_CHECK("sdpa_partial_kernel");
   if (hd == 256)

@@ -58,7 +58,8 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
 }
 
 // grid (ceil(I / (RPW * 4 * ITERS)), T*k + T), 256 threads
-template <int KIND, int LPR, int ITERS>
+// ROUTE: the routing is made in the head of the launch (a.gates) instead of read (a.inds)
+template <int KIND, int LPR, int ITERS, bool ROUTE>
 __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
   using KL = KqLane<KIND, 1>;
   constexpr int RPW = 64 / LPR;
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
   if (r < routed) {
     token = r / a.k;
     uint32_t e;
-    if (a.gates) {
+    if constexpr (ROUTE) {
       __shared__ uint32_t s_inds[16];
       __shared__ bf16_t s_scores[16];
       if (wave == 0) {
@@ -340,10 +341,16 @@ void launch_up(ornith_ctx* ctx, const UpArgs& a, int rows_y) {
   // four stays selectable for wider inputs.
   if (ornith_option_moe_up_iters() == 4) {
     dim3 grid((a.I + RPW * 4 * 4 - 1) / (RPW * 4 * 4), rows_y);
-    hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4>), grid, dim3(256), 0, ctx->stream, a);
+    if (a.gates)
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4, true>), grid, dim3(256), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4, false>), grid, dim3(256), 0, ctx->stream, a);
   } else {
     dim3 grid((a.I + RPW * 4 * 2 - 1) / (RPW * 4 * 2), rows_y);
-    hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2>), grid, dim3(256), 0, ctx->stream, a);
+    if (a.gates)
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2, true>), grid, dim3(256), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2, false>), grid, dim3(256), 0, ctx->stream, a);
   }
 }
 
