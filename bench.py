@@ -35,9 +35,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the expert gate+up kernel at verify width 2 (17 distinct experts),
 # from two `rocprofv3 --pmc` runs of `bench.py --roofline-only` (FETCH_SIZE, then WRITE_SIZE,
 # KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device copies
-# that run issues: FETCH_SIZE 9870.1 x 2.0 (the copy reads 131,094 for 262,144 KiB),
+# that run issues: FETCH_SIZE 9886.1 x 2.0 (the copy reads 131,086 for 262,144 KiB),
 # WRITE_SIZE 36.0 x 1.0. Counters cannot be read from inside this script; other widths: null.
-PMC_TRAFFIC_BYTES = {2: int(round((9870.1 * 2.0 + 36.0 * 1.0) * 1024))}
+PMC_TRAFFIC_BYTES = {2: int(round((9886.1 * 2.0 + 36.0 * 1.0) * 1024))}
 
 
 def log(*a):
@@ -74,7 +74,7 @@ def expert_gemv_roofline(orn, ctx, model, util, np, n_layers, T, launches=800):
     return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": PMC_TRAFFIC_BYTES.get(T) if U == 16 else None,
-            "kernel": "moe_up_kernel<Q4_K, 64 lanes/row, 2 rows/wavefront> (expert gate+up gather-GEMV + swiglu)",
+            "kernel": "moe_up_kernel<0, 64, 2, false> (Q4_K expert gate+up gather-GEMV + swiglu, expert ids given)",
             "us_per_launch": round(us, 3), "bytes_per_launch": int(bytes_per_launch),
             "distinct_experts": int(U), "verify_width": int(T)}
 
