@@ -108,22 +108,25 @@ int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, s
 
   size_t processed = 0;
   TRY(prefill(m, c, prompt, n_prompt, prefill_step, d_tok, d_hidden, progress, user, &processed));
-  // step(): run the remaining prompt tokens and sample from the last position
-  auto step = [&](const uint32_t* toks, size_t n, uint32_t* y) -> int {
-    TRY(ornith_upload(ctx, d_tok, toks, n * 4));
+  // step(): run the n tokens in d_tok and sample from the last position; the one wait of the
+  // step is the read-back of the sampled id
+  auto step = [&](size_t n, uint32_t* y) -> int {
     TRY(ornith_model_forward(m, c, d_tok, (int)n, 0, d_hidden));
     TRY(ornith_model_logits(m, (char*)d_hidden + (n - 1) * H * 2, 1, d_logits));
     TRY(smp.sample(d_logits, d_out));
     return ornith_download(ctx, y, d_out, 4);
   };
   uint32_t y = 0;
-  TRY(step(prompt + processed, n_prompt - processed, &y));
+  TRY(ornith_upload(ctx, d_tok, prompt + processed, (n_prompt - processed) * 4));
+  TRY(step(n_prompt - processed, &y));
   if (progress) progress(n_prompt, n_prompt, user);
   size_t n = 0;
   for (;;) {
     if (n == max_tokens) return ORNITH_OK;
     uint32_t next = 0;
-    TRY(step(&y, 1, &next));
+    // the token just sampled is fed back from where it lies on the device
+    TRY(ornith_copy(ctx, d_tok, d_out, 4));
+    TRY(step(1, &next));
     if (!on_token(y, user)) return ORNITH_OK;
     y = next;
     ++n;
@@ -156,8 +159,8 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   void *d_hidden, *d_h, *d_vlogits, *d_dlogits, *d_mh, *d_scratch_h;
   const size_t W = (size_t)depth + 1;
   TRY(b.get(R * 4, (void**)&d_tok));
-  TRY(b.get(W * 4, (void**)&d_window));
-  TRY(b.get(W * 4, (void**)&d_targets));
+  TRY(b.get(2 * W * 4, (void**)&d_window));  // window, then the targets: one read-back a cycle
+  d_targets = d_window + W;
   TRY(b.get(4, (void**)&d_local));
   TRY(b.get(R * H * 2, &d_hidden));
   TRY(b.get(H * 2, &d_h));
@@ -181,17 +184,19 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   size_t emitted = 0;
   TRY(ornith_mtp_cache_set_offset(head, 0));  // make_mtp_cache()
   const int draft_vocab = frspec ? frspec->n : (int)V;
-  std::vector<uint32_t> win(W), targets(W);
+  std::vector<uint32_t> wt(2 * W);
+  uint32_t* const win = wt.data();
+  uint32_t* const targets = wt.data() + W;
+  // the token every cycle starts from lies on the device where it was sampled
+  TRY(ornith_copy(ctx, d_window, d_targets, 4));
   for (;;) {
     if (policy == ORNITH_HISTORY_CYCLE) TRY(ornith_mtp_cache_set_offset(head, 0));
     const int cycle_mtp_offset = head->offset;
     const size_t left = max_tokens > emitted + 1 ? max_tokens - (emitted + 1) : 0;
     const int want = (int)std::min<size_t>((size_t)depth, left);
 
-    // draft(): `want` chained head forwards, entirely on the device
-    std::fill(win.begin(), win.end(), 0u);
-    win[0] = primary;
-    TRY(ornith_upload(ctx, d_window, win.data(), W * 4));
+    // draft(): `want` chained head forwards, entirely on the device (d_window[0] holds the
+    // primary token; the chain fills the entries after it)
     const void* hcur = d_h;
     for (int i = 0; i < want; ++i) {
       void* hid = (char*)d_mh + (size_t)i * H * 2;
@@ -218,9 +223,10 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
     const bool independent = smp.rows_are_independent();
     if (independent) {
       TRY(ornith_greedy_rows(ctx, d_vlogits, n_rows, (int)V, d_targets, nullptr));
-      TRY(ornith_download(ctx, targets.data(), d_targets, (size_t)n_rows * 4));  // the cycle's one sync
+      TRY(ornith_download(ctx, wt.data(), d_window, 2 * W * 4));  // the cycle's one wait
+    } else {
+      TRY(ornith_download(ctx, win, d_window, (size_t)n_rows * 4));
     }
-    TRY(ornith_download(ctx, win.data(), d_window, (size_t)n_rows * 4));
     // a dependent sampler draws row by row, as far as the accept loop asks
     auto take = [&](int row, uint32_t* t) -> int {
       if (independent) {
@@ -259,6 +265,8 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
       if (k > 0) TRY(ornith_mtp_forward(head, nullptr, d_hidden, d_window + 1, k, d_scratch_h, nullptr));
     }
     TRY(ornith_copy(ctx, d_h, (char*)d_hidden + (size_t)k * H * 2, H * 2));
+    // next cycle's primary token: row k's target (the correction or the bonus token)
+    TRY(ornith_copy(ctx, d_window, d_targets + k, 4));
 
     for (int i = 0; i <= k; ++i) {
       const uint32_t t = i == 0 ? primary : win[i];

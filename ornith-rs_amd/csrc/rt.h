@@ -19,6 +19,10 @@ struct ornith_ctx {
   // stream order makes reuse by the next operator safe.
   void* scratch = nullptr;
   size_t scratch_cap = 0;
+  // pinned host staging for the few bytes a decode loop reads back per step (token ids):
+  // a copy into pinned memory completes without the runtime's pageable detour
+  void* pinned = nullptr;
+  static constexpr size_t kPinnedBytes = 4096;
 };
 
 // Returns at least `bytes` of device scratch (256-byte aligned). Growing it

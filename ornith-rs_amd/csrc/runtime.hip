@@ -97,6 +97,7 @@ int ornith_ctx_create(int device, ornith_ctx** out) {
   ORN_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
   ORN_HIP(hipEventCreate(&c->ev0));
   ORN_HIP(hipEventCreate(&c->ev1));
+  ORN_HIP(hipHostMalloc(&c->pinned, ornith_ctx::kPinnedBytes, hipHostMallocDefault));
   *out = c;
   return ORNITH_OK;
 }
@@ -105,6 +106,7 @@ int ornith_ctx_destroy(ornith_ctx* ctx) {
   if (!ctx) return ORNITH_OK;
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->scratch) (void)hipFree(ctx->scratch);
+  if (ctx->pinned) (void)hipHostFree(ctx->pinned);
   (void)hipEventDestroy(ctx->ev0);
   (void)hipEventDestroy(ctx->ev1);
   (void)hipStreamDestroy(ctx->stream);
@@ -147,6 +149,12 @@ int ornith_upload(ornith_ctx* ctx, void* d_dst, const void* host, size_t bytes) 
 int ornith_download(ornith_ctx* ctx, void* host, const void* d_src, size_t bytes) {
   ORN_REQUIRE(ctx && (bytes == 0 || (d_src && host)), "ornith_download: null argument");
   if (bytes == 0) return ORNITH_OK;
+  if (bytes <= ornith_ctx::kPinnedBytes && ctx->pinned) {
+    ORN_HIP(hipMemcpyAsync(ctx->pinned, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    ORN_HIP(hipStreamSynchronize(ctx->stream));
+    memcpy(host, ctx->pinned, bytes);
+    return ORNITH_OK;
+  }
   ORN_HIP(hipMemcpyAsync(host, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
   ORN_HIP(hipStreamSynchronize(ctx->stream));
   return ORNITH_OK;
