@@ -246,11 +246,19 @@ struct StepArgs {
   bf16_t* gated;          // [T, Hv*128]
 };
 
+#ifdef ORN_TIMING
+// debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch
+__device__ long long g_gdn_marks[64][8];
+#define GDN_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x < 64) g_gdn_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+#else
+#define GDN_MARK(i)
+#endif
+
 __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
+  GDN_MARK(0);
   const FrontArgs& p = a.f;
   __shared__ float qs[kStepMaxT][128], ks[kStepMaxT][128], vs[kStepMaxT][128], ys[kStepMaxT][128];
   __shared__ float gs[kStepMaxT], bs[kStepMaxT];
-  __shared__ float ab[2][kStepMaxT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hv = blockIdx.x, ratio = p.Hv / p.Hk, hk = hv / ratio;
   const int T = p.T, S = p.K - 1, D = p.D;
@@ -282,6 +290,7 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     bin_pre = p.b_in[tid * p.Hv + hv];
   }
   __builtin_amdgcn_sched_barrier(0);
+  const float decay_pre = dm_exp(dm_bf2f(alog_pre));  // needs only a parameter: made under the loads
 
   // 2. front-end tasks: [0, 3T) conv of (q | k | v, token); then the a / b projections
   const int n_conv = 3 * T, n_ab = a.wa ? 2 * T : 0;
@@ -345,21 +354,29 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     } else {
       const int u = task - n_conv, which = u / T, t = u - which * T;  // 0 a, 1 b
       const bf16_t* wr = (which == 0 ? a.wa : a.wb) + (size_t)hv * a.H;
-      const float v = dense_row_dot(wr, a.xn + (size_t)t * a.H, a.H, lane);
-      if (lane == 0) ab[which][t] = dm_rb(v);
+      const float v = dm_rb(dense_row_dot(wr, a.xn + (size_t)t * a.H, a.H, lane));
+      // the wavefront that made the projection turns it into the token's decay / beta at
+      // once: the two chains of exp / log run side by side in different wavefronts instead of
+      // one after the other behind a barrier
+      if (which == 0) {
+        const float sp = softplus_bf16(dm_rb(v + dm_bf2f(dtb_pre)));
+        const float g = dm_exp(-decay_pre * sp);
+        if (lane == 0) gs[t] = g;
+      } else {
+        const float bt = dm_rb(dm_sigmoid_bf16(v));
+        if (lane == 0) bs[t] = bt;
+      }
     }
   }
-  __syncthreads();
-  if (tid < T) {
-    const int t = tid;
-    const float av = a.wa ? ab[0][t] : dm_bf2f(ain_pre);
-    const float bv = a.wa ? ab[1][t] : dm_bf2f(bin_pre);
-    const float sp = softplus_bf16(dm_rb(av + dm_bf2f(dtb_pre)));
-    const float decay = dm_exp(dm_bf2f(alog_pre));
-    gs[t] = dm_exp(-decay * sp);
-    bs[t] = dm_rb(dm_sigmoid_bf16(bv));
+  if (!a.wa && tid < T) {
+    // projections given: decay and beta of token `tid`
+    const float sp = softplus_bf16(dm_rb(dm_bf2f(ain_pre) + dm_bf2f(dtb_pre)));
+    gs[tid] = dm_exp(-decay_pre * sp);
+    bs[tid] = dm_rb(dm_sigmoid_bf16(dm_bf2f(bin_pre)));
   }
   __syncthreads();
+  GDN_MARK(1);
+  GDN_MARK(2);
 
   // 3. recurrence (gdn_recurrence_kernel, operands from LDS)
   for (int t = 0; t < T; ++t) {
@@ -397,6 +414,7 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     }
   }
   __syncthreads();
+  GDN_MARK(3);
 
   // 4. gated norm of the head's 128 outputs, one wavefront per token (rms_norm_gated, two
   //    values per lane)
@@ -414,9 +432,16 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     x1 = (g1 * dm_sigmoid_f32(g1)) * x1;
     *reinterpret_cast<uint32_t*>(a.gated + off) = (uint32_t)dm_f2bf(x0) | ((uint32_t)dm_f2bf(x1) << 16);
   }
+  GDN_MARK(5);
 }
 
 }  // namespace
+
+#ifdef ORN_TIMING
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_gdn(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_gdn_marks), sizeof(long long) * 64 * 8);
+}
+#endif
 
 // fills the front-end part of the arguments (shared by gdn_front and gdn_step)
 static void fill_front(FrontArgs& p, const void* d_conv_state, const void* d_qkv, const void* d_cw,
