@@ -10,11 +10,12 @@
 // and sigmoid_gate (kernels/ornith_elementwise.metal).
 //
 // Attention is split over keys in blocks of 256 by absolute position, one
-// workgroup per (block, kv head, query row): scores are thread-per-key (one fma
-// chain over the head dimension), values are thread-per-channel (one fma chain
-// over the block's keys), so neither needs a cross-lane reduction per key. The
-// partial (max, sum, values) of each block go to scratch and a second kernel
-// merges them in ascending block order and applies the sigmoid output gate.
+// workgroup per (block, query head, query row): a key's score is one fma chain per
+// 64 channels with the chains added pairwise, a channel's output one fma chain per
+// 64 keys of the block added the same way, so neither needs a cross-lane reduction
+// per key. The partial (max, sum, values) of each block go to scratch and a second
+// kernel merges them in ascending block order and applies the sigmoid output gate;
+// when every row has a single block the partial kernel does that itself.
 // A query row only ever sees keys at or before its own position, and blocks are
 // aligned to absolute positions, so row r of a T-row verify call is bit-identical
 // to a one-row call at that position.
@@ -114,6 +115,8 @@ struct SdpaArgs {
   bf16_t* out;           // [T, Hq*HD]
   int T, Hq, Hkv, offset, cap, nblk;
   float scale;
+  int finish;  // 1: every row has a single key block, the partial kernel applies the merge's
+               //    arithmetic itself and writes `out` (no merge launch follows)
 };
 
 // grid (nblk, Hq, T), 1024 threads: one query head against one block of ATT_KB keys.
@@ -192,6 +195,9 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
 #pragma unroll
   for (int u = 0; u < NLD; ++u)
     vreg[u] = *reinterpret_cast<const u32x4*>(vblk + (size_t)min(row0 + RPU * u, nvalid - 1) * HD);
+  // the output gate of a finishing block is requested with everything else
+  bf16_t gate_pre = 0;
+  if (p.finish && tid < HD) gate_pre = p.qg[((size_t)t * p.Hq + hq) * 2 * HD + HD + tid];
   if (tid < HD) qs[tid] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq) * HD + tid]);
 
   // scores: thread (key, panel) runs the chain over the panel's 64 channels
@@ -264,11 +270,23 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
   }
   __syncthreads();
   const size_t pi = ((size_t)t * p.Hq + hq) * p.nblk + b;
+  float l = red[0] + red[1];
+  l = l + red[2];
+  l = l + red[3];
+  if (p.finish) {
+    // the merge over one block, operation for operation (sdpa_merge_kernel with nb == 1)
+    if (tid < HD) {
+      const float w = dm_exp(mg - mg);
+      const float L = dm_fma(l, w, 0.f);
+      const float O = dm_fma(sdpa_pair_tree<NVB>(part + tid, HD), w, 0.f);
+      const float att = dm_rb(O / L);
+      const float g = dm_sigmoid_bf16(dm_bf2f(gate_pre));
+      p.out[((size_t)t * p.Hq + hq) * HD + tid] = dm_f2bf(g * att);
+    }
+    return;
+  }
   if (tid < HD) p.part_o[pi * HD + tid] = sdpa_pair_tree<NVB>(part + tid, HD);
   if (tid == 0) {
-    float l = red[0] + red[1];
-    l = l + red[2];
-    l = l + red[3];
     p.part_m[pi] = mg;
     p.part_l[pi] = l;
   }
@@ -502,6 +520,8 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   // soonest; many: the 256-thread form keeps more blocks in flight. Same sums either way.
   const int last_max = (d_offset ? cap - 1 : (offset + T - 1 < cap - 1 ? offset + T - 1 : cap - 1));
   const long live = (long)(last_max / ATT_KB + 1) * Hq * T;
+  // one key block for every row (and the kernel form that knows how): no merge launch
+  p.finish = (last_max < ATT_KB && live <= 2L * ctx->compute_units) ? 1 : 0;
   if (live > 2L * ctx->compute_units) {
     if (hd == 256)
       hipLaunchKernelGGL((sdpa_partial_many_kernel<256>), grid, dim3(256), 0, ctx->stream, p);
@@ -526,6 +546,7 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
     hipLaunchKernelGGL((sdpa_partial_kernel<128>), grid, dim3(SDPA_NT), sdpa_stage_bytes<128>(), ctx->stream, p);
   }
   ORN_LAUNCH_CHECK("sdpa_partial_kernel");
+  if (p.finish) return ORNITH_OK;
   if (hd == 256)
     hipLaunchKernelGGL(sdpa_merge_kernel<256>, dim3(Hq, T), dim3(256), 0, ctx->stream, p);
   else
