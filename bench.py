@@ -98,7 +98,7 @@ def cpu_baseline(synth, synth_model, np, depth, tokens):
 
 def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
     """BASELINE config 5: sampled speculative decode at depth 3 after a long prefill."""
-    depth, n_prompt, n_gen, cap = 3, 6621, 256, 16384
+    depth, n_prompt, n_gen, cap = 3, 6621, (1 if args.prefill_only else 256), 16384
     model.set_max_rows(args.prefill_chunk)
     caches = model.make_cache(cap, depth + 1)
     head = orn.MtpHead(model, ws, cap)
@@ -163,6 +163,9 @@ def main():
                          "16384-token context through the matrix-core path, then sampled depth-3 MTP "
                          "decode of 256 tokens, temperature 0.8, top-p 0.95); prints its own JSON line")
     ap.add_argument("--prefill-chunk", type=int, default=2048)
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="with --config5: stop after the first generated token (a short run for "
+                         "profiling the matrix-core prefill kernels)")
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the expert-kernel timing loop plus three 256 MiB device copies "
                          "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")

@@ -475,11 +475,15 @@ int ornith_model_logits(ornith_model* m, const void* d_hidden, int T, void* d_lo
 
 static int gather_rows_dev(ornith_ctx* ctx, const void* src, size_t row_bytes, const std::vector<uint32_t>& ids,
                            void** out) {
-  TRY(ornith_alloc(ctx, row_bytes * ids.size(), out));
-  // FrSpec::prune is a load-time row gather (src/frspec.rs:67-93): plain device copies
-  for (size_t r = 0; r < ids.size(); ++r)
-    TRY(ornith_copy(ctx, (char*)*out + r * row_bytes, (const char*)src + (size_t)ids[r] * row_bytes, row_bytes));
-  return ornith_sync(ctx);
+  // FrSpec::prune is a load-time row gather (src/frspec.rs:67-93): one launch per tensor
+  void* d_ids = nullptr;
+  TRY(ornith_alloc(ctx, ids.size() * 4, &d_ids));
+  int rc = ornith_upload(ctx, d_ids, ids.data(), ids.size() * 4);
+  if (!rc) rc = ornith_alloc(ctx, row_bytes * ids.size(), out);
+  if (!rc) rc = ornith_gather_rows(ctx, src, row_bytes, (const uint32_t*)d_ids, (int)ids.size(), *out);
+  if (!rc) rc = ornith_sync(ctx);
+  ornith_free(ctx, d_ids);
+  return rc;
 }
 
 int ornith_frspec_from_ids(ornith_model* m, const uint32_t* ids, int n, ornith_frspec** out) {

@@ -29,6 +29,10 @@ struct ornith_ctx {
 // synchronises the stream; callers that must not allocate size it once up front.
 int ornith_scratch(ornith_ctx* ctx, size_t bytes, void** out);
 
+// d_dst[r] = d_src[d_ids[r]] for n rows of row_bytes (a multiple of 4) each, one launch.
+int ornith_gather_rows(ornith_ctx* ctx, const void* d_src, size_t row_bytes, const uint32_t* d_ids,
+                       int n, void* d_dst);
+
 // bump allocator over a scratch block
 struct ScratchCursor {
   char* base;

@@ -65,6 +65,27 @@ int ornith_option_gemm_rows() {
   return v <= 0 ? 1 << 30 : v;
 }
 
+namespace {
+// one workgroup per gathered row, 4-byte words
+__global__ __launch_bounds__(256) void gather_rows_kernel(const uint32_t* __restrict__ src, size_t row_words,
+                                                          const uint32_t* __restrict__ ids,
+                                                          uint32_t* __restrict__ dst) {
+  const uint32_t* s = src + (size_t)ids[blockIdx.x] * row_words;
+  uint32_t* d = dst + (size_t)blockIdx.x * row_words;
+  for (size_t i = threadIdx.x; i < row_words; i += 256) d[i] = s[i];
+}
+}  // namespace
+
+int ornith_gather_rows(ornith_ctx* ctx, const void* d_src, size_t row_bytes, const uint32_t* d_ids,
+                       int n, void* d_dst) {
+  ORN_REQUIRE(ctx && d_src && d_ids && d_dst && n >= 1, "gather_rows: null argument");
+  ORN_REQUIRE(row_bytes >= 4 && row_bytes % 4 == 0, "gather_rows: rows of %zu bytes", row_bytes);
+  hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, ctx->stream, (const uint32_t*)d_src,
+                     row_bytes / 4, d_ids, (uint32_t*)d_dst);
+  ORN_LAUNCH_CHECK("gather_rows_kernel");
+  return ORNITH_OK;
+}
+
 extern "C" {
 
 int ornith_set_option(const char* name, int value) {
