@@ -58,9 +58,18 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
 }
 
 // grid (ceil(I / (RPW * 4 * ITERS)), T*k + T), 256 threads
+#ifdef ORN_TIMING
+// debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch
+__device__ long long g_up_marks[2048][8];
+#define UP_MARK(i) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if (threadIdx.x == 0 && bl__ < 2048) g_up_marks[bl__][i] = wall_clock64(); } while (0)
+#else
+#define UP_MARK(i)
+#endif
+
 // ROUTE: the routing is made in the head of the launch (a.gates) instead of read (a.inds)
 template <int KIND, int LPR, int ITERS, bool ROUTE>
 __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
+  UP_MARK(0);
   using KL = KqLane<KIND, 1>;
   constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -117,8 +126,10 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
     ru[it] = KL::load(wu.qs, wu.scales, wu.dm, row, nb, L);
   }
   __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  UP_MARK(1);
   const void* xrow[1] = {a.x + (size_t)token * a.K};
   L.template load_x<false>(xrow, c);
+  UP_MARK(2);
   if constexpr (LPR == 64 && ITERS % 2 == 0) {
     // one row per wavefront pass: reduce two rows' gate and up sums together
 #pragma unroll
@@ -135,6 +146,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
       const int o = base + it;
       if (lane == 0 && o < a.I) a.act[(size_t)r * a.I + o] = swiglu_bf16(ga, ua);
       if (lane == 1 && o + 1 < a.I) a.act[(size_t)r * a.I + o + 1] = swiglu_bf16(gb, ub);
+      if (it == 0) UP_MARK(3);
     }
   } else {
 #pragma unroll
@@ -148,6 +160,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
       if (c == 0 && o < a.I) a.act[(size_t)r * a.I + o] = swiglu_bf16(g, u);
     }
   }
+  UP_MARK(4);
 }
 
 struct DownArgs {
@@ -369,6 +382,12 @@ void launch_down(ornith_ctx* ctx, const DownArgs& a) {
 }
 
 }  // namespace
+
+#ifdef ORN_TIMING
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_up(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_up_marks), sizeof(long long) * 2048 * 8);
+}
+#endif
 
 // Whether the two fused kernels cover this block's shapes and formats.
 bool moe_fused_supported(const ornith_moe_weights* w) {
