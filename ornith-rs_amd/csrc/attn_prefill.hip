@@ -87,26 +87,43 @@ __global__ __launch_bounds__(256) void sdpa_prefill_kernel(FaArgs p) {
 
   const bf16_t* kbase = p.k_cache + (size_t)hk * p.cap * HD;
   const bf16_t* vbase = p.v_cache + (size_t)hk * p.cap * HD;
+  // A key block travels in registers one block ahead of its use. Keys: thread = (key tid/32 + 8i,
+  // 8-channel piece tid%32), stored as they are. Values: thread = (8 keys 8*(lane%8).., piece
+  // tid/8), an 8 x 8 tile that is transposed in registers, so each channel's 8 keys go to LDS as
+  // one 16-byte store.
+  constexpr int NPC = BKV * HD / 8 / 256;  // 8 pieces of each kind per thread
+  static_assert(NPC == 8, "one 8 x 8 value tile per thread");
+  typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+  const int vkg = lane & 7, vc8 = tid >> 3;
+  u32x4_t kr[NPC], vr[NPC];
+  auto fetch = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < NPC; ++i) {
+      const int kkey = kb * BKV + (tid >> 5) + 8 * i, vkey = kb * BKV + 8 * vkg + i;
+      kr[i] = u32x4_t{0, 0, 0, 0};
+      vr[i] = u32x4_t{0, 0, 0, 0};
+      if (kkey < n_keys) kr[i] = *reinterpret_cast<const u32x4_t*>(kbase + (size_t)kkey * HD + 8 * (tid & 31));
+      if (vkey < n_keys) vr[i] = *reinterpret_cast<const u32x4_t*>(vbase + (size_t)vkey * HD + 8 * vc8);
+    }
+  };
+  fetch(0);
   for (int kb = 0; kb < n_kb; ++kb) {
     // ---- K block as is, V block transposed
 #pragma unroll
-    for (int i = 0; i < BKV * HD / 8 / 256; ++i) {
-      const int idx = tid + 256 * i, key = idx >> 5, c8 = idx & 31;
-      const int kpos = kb * BKV + key;
-      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (kpos < n_keys) {
-        kv = *reinterpret_cast<const uint4*>(kbase + (size_t)kpos * HD + 8 * c8);
-        vv = *reinterpret_cast<const uint4*>(vbase + (size_t)kpos * HD + 8 * c8);
-      }
-      *reinterpret_cast<uint4*>(&Ks[key][8 * c8]) = kv;
-      const uint32_t w[4] = {vv.x, vv.y, vv.z, vv.w};
+    for (int i = 0; i < NPC; ++i)
+      *reinterpret_cast<u32x4_t*>(&Ks[(tid >> 5) + 8 * i][8 * (tid & 31)]) = kr[i];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        Vt[8 * c8 + 2 * e][key] = (bf16_t)(w[e] & 0xffffu);
-        Vt[8 * c8 + 2 * e + 1][key] = (bf16_t)(w[e] >> 16);
-      }
+    for (int ch = 0; ch < 8; ++ch) {
+      const int w = ch >> 1;
+      const unsigned sel = (ch & 1) ? 0x07060302u : 0x05040100u;  // high / low halves of a word pair
+      u32x4_t col;
+#pragma unroll
+      for (int kp = 0; kp < 4; ++kp)
+        col[kp] = __builtin_amdgcn_perm(vr[2 * kp + 1][w], vr[2 * kp][w], sel);
+      *reinterpret_cast<u32x4_t*>(&Vt[8 * vc8 + ch][8 * vkg]) = col;
     }
     __syncthreads();
+    if (kb + 1 < n_kb) fetch(kb + 1);  // in flight under this block's matrix work
 
     // ---- S = Q K^T
     f32x4_t s[BKV / 16];
