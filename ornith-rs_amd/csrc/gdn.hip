@@ -161,6 +161,51 @@ __global__ __launch_bounds__(64) void gdn_recurrence_kernel(RecArgs p) {
 #pragma unroll
     for (int i = 0; i < GP; ++i) fetch(t0 + GP + i, kwn[i], qwn[i], ggn[i], bbn[i], vvn[i]);
     __builtin_amdgcn_sched_barrier(0);
+    // a full group with only the final state wanted runs as straight-line code: the output
+    // chain of one token and the k-chain of the next do not depend on each other, and without
+    // branches between them the scheduler interleaves the two
+    const bool straight = t0 + GP <= p.T && !p.snap_all;
+    if (straight) {
+#pragma unroll
+      for (int i = 0; i < GP; ++i) {
+        float kf[16], qf[16];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          kf[4 * m + 0] = dm_bf2f_lo(kw[i][m].x);
+          kf[4 * m + 1] = dm_bf2f_hi(kw[i][m].x);
+          kf[4 * m + 2] = dm_bf2f_lo(kw[i][m].y);
+          kf[4 * m + 3] = dm_bf2f_hi(kw[i][m].y);
+          qf[4 * m + 0] = dm_bf2f_lo(qw[i][m].x);
+          qf[4 * m + 1] = dm_bf2f_hi(qw[i][m].x);
+          qf[4 * m + 2] = dm_bf2f_lo(qw[i][m].y);
+          qf[4 * m + 3] = dm_bf2f_hi(qw[i][m].y);
+        }
+        const float gt = gg[i], bt = bb[i], vt = vv[i];
+        float a = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          s[e] = s[e] * gt;
+          a = dm_fma(s[e], kf[e], a);
+        }
+        const float kv = dm_wave_sum<8>(a);
+        const float delta = (vt - kv) * bt;
+        float o = 0.f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          s[e] = dm_fma(kf[e], delta, s[e]);
+          o = dm_fma(s[e], qf[e], o);
+        }
+        o = dm_wave_sum<8>(o);
+        if (j == 0) p.y[((size_t)(t0 + i) * p.Hv + hv) * p.Dv + dv] = dm_f2bf(o);
+      }
+      if (t0 + GP == p.T) {
+        float* snap = p.snapshots + roff;
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+          *reinterpret_cast<float4*>(snap + 32 * m) =
+              make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+      }
+    } else
 #pragma unroll
     for (int i = 0; i < GP; ++i) {
       const int t = t0 + i;
