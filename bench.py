@@ -162,7 +162,8 @@ def main():
                     help="instead of the metric's workload: BASELINE config 5 (6621-token prefill into a "
                          "16384-token context through the matrix-core path, then sampled depth-3 MTP "
                          "decode of 256 tokens, temperature 0.8, top-p 0.95); prints its own JSON line")
-    ap.add_argument("--prefill-chunk", type=int, default=2048)
+    ap.add_argument("--prefill-chunk", type=int, default=4096,
+                    help="rows per prefill call with --config5 (the reference's prefill_step_size is 2048; up to 4096 here)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="with --config5: stop after the first generated token (a short run for "
                          "profiling the matrix-core prefill kernels)")

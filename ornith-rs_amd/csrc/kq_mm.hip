@@ -398,9 +398,13 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   uint32_t* ts = pc.take<uint32_t>(tiles_max);
   uint32_t* tc = pc.take<uint32_t>(tiles_max);
   uint32_t* nt = pc.take<uint32_t>(1);
+  // rows per tile: an expert's weight tile is dequantized once per tile, so with about 96 or
+  // more rows an expert on average the 128-row tile halves that work (the choice depends only
+  // on pairs and E, so the calls sharing a plan agree on it)
+  const int tile_rows = pairs / w->E >= 96 ? 128 : 64;
   if (rebuild_plan) {
     hipLaunchKernelGGL(moe_sort_pairs_kernel, dim3(1), dim3(1024), 0, ctx->stream, d_inds, pairs, w->E,
-                       64, pair, te, ts, tc, nt);
+                       tile_rows, pair, te, ts, tc, nt);
     ORN_LAUNCH_CHECK("moe_sort_pairs_kernel");
   }
   MmArgs a{};
@@ -419,7 +423,12 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   a.tile_count = tc;
   a.n_tiles = nt;
   const dim3 grid((w->O + BN - 1) / BN, (unsigned)tiles_max);
-  if (w->kind == ORNITH_Q4K)
+  if (tile_rows == 128) {
+    if (w->kind == ORNITH_Q4K)
+      hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 128, true>), grid, dim3(256), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q6K, 128, true>), grid, dim3(256), 0, ctx->stream, a);
+  } else if (w->kind == ORNITH_Q4K)
     hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 64, true>), grid, dim3(256), 0, ctx->stream, a);
   else
     hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q6K, 64, true>), grid, dim3(256), 0, ctx->stream, a);

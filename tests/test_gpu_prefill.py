@@ -52,7 +52,9 @@ def test_kq_matmul_vs_float64(orn, ctx, kind, O, K, M):
 
 
 @pytest.mark.parametrize("kind,E,O,K,T,k", [(Q4K, 8, 256, 512, 40, 2), (Q4K, 256, 512, 2048, 300, 8),
-                                             (Q6K, 256, 2048, 512, 300, 8), (Q6K, 16, 128, 256, 5, 4)])
+                                             (Q6K, 256, 2048, 512, 300, 8), (Q6K, 16, 128, 256, 5, 4),
+                                             # about 100 rows an expert and more: 128-row tiles
+                                             (Q4K, 8, 256, 512, 400, 2), (Q6K, 16, 128, 256, 500, 4)])
 def test_kq_gather_matmul_vs_float64(orn, ctx, kind, E, O, K, T, k):
     rng = np.random.default_rng(E + O + K + T)
     t = util.make_kq(kind, rng, E, O, K)
