@@ -125,8 +125,25 @@ __device__ __forceinline__ float dm_sigmoid_f32(float x) {
 // ---- wavefront reductions: v[l] += v[l ^ s], s = 32,16,...,1 ---------------
 // fp32 add commutes, so all 64 lanes finish with identical bits.
 
-// value of lane (l ^ S): DPP quad permutes for 1 and 2 (no LDS traffic, fold into the
-// consuming add), ds_swizzle for 4, 8, 16, the LDS crossbar permute for 32.
+// Everything here stays in the vector ALU: a trip through the LDS crossbar (ds_swizzle,
+// ds_bpermute) costs an LDS round trip each, and a 64-lane sum would take four of them in series.
+
+// The halves of a wavefront (ROWS = 32) or the 16-lane rows of each half (ROWS = 16) trade
+// places: given v in both operands, on return a holds the even rows' values in every row pair
+// and b the odd rows' (v_permlane32_swap / v_permlane16_swap exchange the odd rows of the
+// first operand with the even rows of the second).
+template <int ROWS>
+__device__ __forceinline__ void dm_row_swap(float v, float& a, float& b) {
+  a = v;
+  b = v;
+  if constexpr (ROWS == 32)
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  else
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+
+// value of lane (l ^ S): DPP quad permutes for 1 and 2 and a row rotate for 8 (they fold
+// into the consuming add), two bank-masked row shifts for 4, a row swap and a select for 16, 32.
 template <int S>
 __device__ __forceinline__ float dm_xor_lane(float v) {
   int i = __builtin_bit_cast(int, v);
@@ -134,23 +151,33 @@ __device__ __forceinline__ float dm_xor_lane(float v) {
     i = __builtin_amdgcn_mov_dpp(i, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
   else if constexpr (S == 2)
     i = __builtin_amdgcn_mov_dpp(i, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
-  else if constexpr (S == 4)
-    i = __builtin_amdgcn_ds_swizzle(i, 0x101F);  // bit-mask mode: and 0x1f, xor 4
-  else if constexpr (S == 8)
-    i = __builtin_amdgcn_ds_swizzle(i, 0x201F);
-  else if constexpr (S == 16)
-    i = __builtin_amdgcn_ds_swizzle(i, 0x401F);
-  else
-    i = __shfl_xor(i, 32, 64);
+  else if constexpr (S == 4) {
+    const int up = __builtin_amdgcn_update_dpp(i, i, 0x104, 0xF, 0x5, false);  // row_shl:4 into lanes 0-3, 8-11
+    i = __builtin_amdgcn_update_dpp(up, i, 0x114, 0xF, 0xA, false);            // row_shr:4 into lanes 4-7, 12-15
+  } else if constexpr (S == 8)
+    i = __builtin_amdgcn_update_dpp(0, i, 0x128, 0xF, 0xF, false);  // row_ror:8 (every lane has a source)
+  else {
+    float a, b;
+    dm_row_swap<S>(v, a, b);
+    return (__lane_id() & S) ? a : b;
+  }
   return __builtin_bit_cast(float, i);
 }
 
 template <int WIDTH>
 __device__ __forceinline__ float dm_wave_sum(float v) {
-  if constexpr (WIDTH >= 64) v = v + dm_xor_lane<32>(v);
-  if constexpr (WIDTH >= 32) v = v + dm_xor_lane<16>(v);
-  if constexpr (WIDTH >= 16) v = v + dm_xor_lane<8>(v);
-  if constexpr (WIDTH >= 8) v = v + dm_xor_lane<4>(v);
+  // a + b after a row swap is v[l] + v[l ^ ROWS] with the operands in one order for both
+  // partners, which is the same bits
+  if constexpr (WIDTH >= 64) { float a, b; dm_row_swap<32>(v, a, b); v = a + b; }
+  if constexpr (WIDTH >= 32) { float a, b; dm_row_swap<16>(v, a, b); v = a + b; }
+  if constexpr (WIDTH >= 16) {
+    v = v + dm_xor_lane<8>(v);
+    // v now repeats every 8 lanes, so the lane 4 further round the row holds the bits of lane
+    // l ^ 4: one rotate that folds into the add
+    v = v + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xF, 0xF, false));
+  } else if constexpr (WIDTH >= 8) {
+    v = v + dm_xor_lane<4>(v);
+  }
   if constexpr (WIDTH >= 4) v = v + dm_xor_lane<2>(v);
   if constexpr (WIDTH >= 2) v = v + dm_xor_lane<1>(v);
   return v;
@@ -158,8 +185,8 @@ __device__ __forceinline__ float dm_wave_sum(float v) {
 template <int WIDTH>
 __device__ __forceinline__ float dm_wave_max(float v) {
   float o;
-  if constexpr (WIDTH >= 64) { o = dm_xor_lane<32>(v); v = o > v ? o : v; }
-  if constexpr (WIDTH >= 32) { o = dm_xor_lane<16>(v); v = o > v ? o : v; }
+  if constexpr (WIDTH >= 64) { float a, b; dm_row_swap<32>(v, a, b); v = b > a ? b : a; }
+  if constexpr (WIDTH >= 32) { float a, b; dm_row_swap<16>(v, a, b); v = b > a ? b : a; }
   if constexpr (WIDTH >= 16) { o = dm_xor_lane<8>(v); v = o > v ? o : v; }
   if constexpr (WIDTH >= 8) { o = dm_xor_lane<4>(v); v = o > v ? o : v; }
   if constexpr (WIDTH >= 4) { o = dm_xor_lane<2>(v); v = o > v ? o : v; }

@@ -262,6 +262,136 @@ __global__ __launch_bounds__(64) void gdn_recurrence_kernel(RecArgs p) {
   }
 }
 
+// ---- the recurrence at prefill widths ---------------------------------------------------
+// A long prompt chunk is a chain of T dependent steps per state row; what a step costs is the
+// instructions a wavefront issues for it and the memory trips that are not hidden. Like every
+// prefill kernel this one agrees with the exact kernel above to rounding, not bit for bit,
+// which frees the order of the sums: 16 lanes share a state row (8 columns a lane), each
+// lane's dot products run as two chains of four, and only the final state is written. Keys
+// and queries of 32 tokens are converted to f32 once and parked in LDS while the next 32
+// tokens' loads are in flight, so no step waits on memory. grid (Dv / 4, Hv), 64 threads.
+__global__ __launch_bounds__(64) void gdn_recurrence_wide_kernel(RecArgs p) {
+  constexpr int C = 32;                          // tokens staged at a time
+  __shared__ __align__(16) float kq[C + 1][2][128];  // k then q of a token, f32
+  __shared__ __align__(16) float gbv[C + 1][8];      // g, beta, -, -, v of the four rows
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x, row = lane >> 4, j = lane & 15;
+  const int hv = blockIdx.y, dv0 = blockIdx.x * 4, dv = dv0 + row;
+  const int hk = hv / (p.Hv / p.Hk);
+  const size_t roff = ((size_t)hv * p.Dv + dv) * 128 + 4 * j;  // columns 64*m + 4*j .. +4
+
+  float s[8];
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    const float4 f = *reinterpret_cast<const float4*>(p.state_in + roff + 64 * m);
+    s[4 * m + 0] = f.x;
+    s[4 * m + 1] = f.y;
+    s[4 * m + 2] = f.z;
+    s[4 * m + 3] = f.w;
+  }
+  // a lane's share of 32 tokens: eight columns (8*j ..) of tokens 4*i + row, i < 8; g and beta
+  // of token lane (lanes below 32); v of tokens lane/4 and 16 + lane/4, row lane%4
+  u32x4 kr[C / 4], qr[C / 4];
+  float gr = 1.f, br = 0.f, vr[2];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < C / 4; ++i) {
+      const int t = min(t0 + 4 * i + row, p.T - 1);
+      const size_t o = ((size_t)t * p.Hk + hk) * 128 + 8 * j;
+      kr[i] = *reinterpret_cast<const u32x4*>(p.k + o);
+      qr[i] = *reinterpret_cast<const u32x4*>(p.q + o);
+    }
+    const int tg = min(t0 + (lane & 31), p.T - 1);
+    gr = p.g[tg * p.Hv + hv];
+    br = dm_bf2f(p.beta[tg * p.Hv + hv]);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int tv = min(t0 + 16 * h + (lane >> 2), p.T - 1);
+      vr[h] = dm_bf2f(p.v[((size_t)tv * p.Hv + hv) * p.Dv + dv0 + (lane & 3)]);
+    }
+  };
+  auto park = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < C / 4; ++i) {
+      float* kd = &kq[4 * i + row][0][8 * j];
+      float* qd = &kq[4 * i + row][1][8 * j];
+      *reinterpret_cast<float4*>(kd) = make_float4(dm_bf2f_lo(kr[i].x), dm_bf2f_hi(kr[i].x), dm_bf2f_lo(kr[i].y), dm_bf2f_hi(kr[i].y));
+      *reinterpret_cast<float4*>(kd + 4) = make_float4(dm_bf2f_lo(kr[i].z), dm_bf2f_hi(kr[i].z), dm_bf2f_lo(kr[i].w), dm_bf2f_hi(kr[i].w));
+      *reinterpret_cast<float4*>(qd) = make_float4(dm_bf2f_lo(qr[i].x), dm_bf2f_hi(qr[i].x), dm_bf2f_lo(qr[i].y), dm_bf2f_hi(qr[i].y));
+      *reinterpret_cast<float4*>(qd + 4) = make_float4(dm_bf2f_lo(qr[i].z), dm_bf2f_hi(qr[i].z), dm_bf2f_lo(qr[i].w), dm_bf2f_hi(qr[i].w));
+    }
+    if (lane < 32) {
+      // tokens past the end of the call leave the state alone: g = 1, beta = 0
+      const bool live = t0 + lane < p.T;
+      *reinterpret_cast<float2*>(&gbv[lane][0]) = make_float2(live ? gr : 1.f, live ? br : 0.f);
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) gbv[16 * h + (lane >> 2)][4 + (lane & 3)] = vr[h];
+  };
+
+  struct Tok {
+    float4 k0, k1, q0, q1;
+    float2 gb;
+    float vt;
+  };
+  auto token = [&](int i) {
+    Tok t;
+    t.k0 = *reinterpret_cast<const float4*>(&kq[i][0][4 * j]);
+    t.k1 = *reinterpret_cast<const float4*>(&kq[i][0][64 + 4 * j]);
+    t.q0 = *reinterpret_cast<const float4*>(&kq[i][1][4 * j]);
+    t.q1 = *reinterpret_cast<const float4*>(&kq[i][1][64 + 4 * j]);
+    t.gb = *reinterpret_cast<const float2*>(&gbv[i][0]);
+    t.vt = gbv[i][4 + row];
+    return t;
+  };
+
+  fetch(0);
+  for (int t0 = 0; t0 < p.T; t0 += C) {
+    __syncthreads();  // the steps before have read their tokens
+    park(t0);
+    __syncthreads();
+    if (t0 + C < p.T) fetch(t0 + C);
+    Tok cur = token(0);
+    for (int h = 0; h < 2; ++h) {
+      float yo = 0.f;
+#pragma unroll 8
+      for (int ii = 0; ii < 16; ++ii) {
+        // the next token's operands leave LDS while this one computes (row C is padding)
+        const Tok nxt = token(16 * h + ii + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        const float kf[8] = {cur.k0.x, cur.k0.y, cur.k0.z, cur.k0.w, cur.k1.x, cur.k1.y, cur.k1.z, cur.k1.w};
+        const float qf[8] = {cur.q0.x, cur.q0.y, cur.q0.z, cur.q0.w, cur.q1.x, cur.q1.y, cur.q1.z, cur.q1.w};
+        const float gt = cur.gb.x, bt = cur.gb.y;
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a0 = dm_fma(s[e], kf[e], a0);
+          a1 = dm_fma(s[4 + e], kf[4 + e], a1);
+        }
+        const float kv = gt * dm_wave_sum<16>(a0 + a1);  // sum_e (g s_e) k_e
+        const float delta = (cur.vt - kv) * bt;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[e] = dm_fma(s[e], gt, kf[e] * delta);
+        float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o0 = dm_fma(s[e], qf[e], o0);
+          o1 = dm_fma(s[4 + e], qf[4 + e], o1);
+        }
+        const float o = dm_wave_sum<16>(o0 + o1);
+        yo = j == ii ? o : yo;  // lane j of a row keeps token j of these sixteen
+        cur = nxt;
+      }
+      const int t = t0 + 16 * h + j;
+      if (t < p.T) p.y[((size_t)t * p.Hv + hv) * p.Dv + dv] = dm_f2bf(yo);
+    }
+  }
+  float* snap = p.snapshots + roff;
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+    *reinterpret_cast<float4*>(snap + 64 * m) = make_float4(s[4 * m + 0], s[4 * m + 1], s[4 * m + 2], s[4 * m + 3]);
+}
+
 // ---- the whole mixer core in one launch, decode / verify widths -------------------------
 // One workgroup per value head (16 wavefronts):
 //   1. every thread issues the loads of its slice of the recurrent state (they depend on
@@ -620,6 +750,12 @@ int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, con
   RecArgs p{(const bf16_t*)d_q, (const bf16_t*)d_k, (const bf16_t*)d_v, d_g, (const bf16_t*)d_beta,
             d_state_in,         (bf16_t*)d_y,       d_snapshots,        T,   Hk, Hv, Dv,
             snapshot_every_token ? 1 : 0};
+  if (T >= kPrefillRows && !snapshot_every_token) {
+    // prompt chunks: the form with the short dependent chain (agrees to rounding)
+    hipLaunchKernelGGL(gdn_recurrence_wide_kernel, dim3(Dv / 4, Hv), dim3(64), 0, ctx->stream, p);
+    ORN_LAUNCH_CHECK("gdn_recurrence_wide_kernel");
+    return ORNITH_OK;
+  }
   hipLaunchKernelGGL(gdn_recurrence_kernel, dim3(Dv / 8, Hv), dim3(64), 0, ctx->stream, p);
   ORN_LAUNCH_CHECK("gdn_recurrence_kernel");
   return ORNITH_OK;

@@ -16,8 +16,11 @@ __device__ __forceinline__ uint32_t dm_xor_lane_u32(uint32_t v) {
 }
 __device__ __forceinline__ uint32_t dm_wave_max_u32(uint32_t v) {
   uint32_t o;
-  o = dm_xor_lane_u32<32>(v); v = o > v ? o : v;
-  o = dm_xor_lane_u32<16>(v); v = o > v ? o : v;
+  float a, b;
+  dm_row_swap<32>(__builtin_bit_cast(float, v), a, b);
+  v = max(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b));
+  dm_row_swap<16>(__builtin_bit_cast(float, v), a, b);
+  v = max(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b));
   o = dm_xor_lane_u32<8>(v); v = o > v ? o : v;
   o = dm_xor_lane_u32<4>(v); v = o > v ? o : v;
   o = dm_xor_lane_u32<2>(v); v = o > v ? o : v;
