@@ -21,6 +21,14 @@ typedef uint16_t f16_t;   // raw bits
 
 #define DM_INF (__builtin_inff())
 
+// A pointer rebuilt from an integer that is known to address device memory. Going through the
+// global address space lets the compiler use global loads (counted by vmcnt alone, so a kernel
+// can wait for its loads one by one) where a bare integer-to-pointer cast gives flat loads.
+template <class T>
+__device__ __forceinline__ T* dm_global_ptr(uint64_t bits) {
+  return (T*)(__attribute__((address_space(1))) T*)bits;
+}
+
 __device__ __forceinline__ float dm_fma(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
 
 __device__ __forceinline__ float dm_bf2f(bf16_t b) { return __uint_as_float((uint32_t)b << 16); }

@@ -98,10 +98,10 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
       uint64_t q = (uint64_t)all[i].qs, sc = (uint64_t)all[i].scales, d = (uint64_t)all[i].dm,
                y = (uint64_t)all[i].y;
       asm volatile("" : "+s"(q), "+s"(sc), "+s"(d), "+s"(y), "+s"(all[i].O), "+s"(all[i].first_block));
-      all[i].qs = (const uint8_t*)q;
-      all[i].scales = (const uint8_t*)sc;
-      all[i].dm = (const uint16_t*)d;
-      all[i].y = (void*)y;
+      all[i].qs = dm_global_ptr<const uint8_t>(q);
+      all[i].scales = dm_global_ptr<const uint8_t>(sc);
+      all[i].dm = dm_global_ptr<const uint16_t>(d);
+      all[i].y = dm_global_ptr<void>(y);
     }
     asm volatile("" : "+s"(nseg));
     sg = all[0];

@@ -80,6 +80,17 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
   int token;
   int64_t row0;
   KqPtr wg, wu;
+  // both sets of weight pointers as values in scalar registers before the choice is made:
+  // chosen by address instead, the pointers would be loaded in a second trip after the first
+  KqPtr pin[4] = {a.gate, a.up, a.sgate, a.sup};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint64_t q = (uint64_t)pin[i].qs, sc = (uint64_t)pin[i].scales, d = (uint64_t)pin[i].dm;
+    asm volatile("" : "+s"(q), "+s"(sc), "+s"(d));
+    pin[i].qs = dm_global_ptr<const uint8_t>(q);
+    pin[i].scales = dm_global_ptr<const uint8_t>(sc);
+    pin[i].dm = dm_global_ptr<const uint16_t>(d);
+  }
   if (r < routed) {
     token = r / a.k;
     uint32_t e;
@@ -106,13 +117,13 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
       e = a.inds[r];
     }
     row0 = (int64_t)min(e, (uint32_t)(a.E - 1)) * a.I;
-    wg = a.gate;
-    wu = a.up;
+    wg = pin[0];
+    wu = pin[1];
   } else {
     token = r - routed;
     row0 = 0;
-    wg = a.sgate;
-    wu = a.sup;
+    wg = pin[2];
+    wu = pin[3];
   }
   typename KL::Lane L;
   L.set_chunk(c);
@@ -140,12 +151,13 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
       KL::accumulate(rg[it + 1], L, g1);
       KL::accumulate(ru[it + 1], L, u1);
       const float red = dm_wave_sum4(g0[0], u0[0], g1[0], u1[0], lane);
-      // lanes [0,16): gate row it, [32,48): up row it, [16,32): gate row it+1, [48,64): up row it+1
-      const float ga = dm_lane_value(red, 0), ua = dm_lane_value(red, 32);
-      const float gb = dm_lane_value(red, 16), ub = dm_lane_value(red, 48);
-      const int o = base + it;
-      if (lane == 0 && o < a.I) a.act[(size_t)r * a.I + o] = swiglu_bf16(ga, ua);
-      if (lane == 1 && o + 1 < a.I) a.act[(size_t)r * a.I + o + 1] = swiglu_bf16(gb, ub);
+      // lanes [0,16): gate row it, [32,48): up row it, [16,32): gate row it+1, [48,64): up row it+1;
+      // after the halves trade places every lane holds a row's gate and up sums, and lanes 0
+      // and 16 finish the two rows in one pass over the swiglu code
+      float gsum, usum;
+      dm_row_swap<32>(red, gsum, usum);
+      const int o = base + it + ((lane >> 4) & 1);
+      if ((lane & 47) == 0 && o < a.I) a.act[(size_t)r * a.I + o] = swiglu_bf16(gsum, usum);
       if (it == 0) UP_MARK(3);
     }
   } else {
