@@ -35,9 +35,9 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the expert gate+up kernel at verify width 2 (17 distinct experts),
 # from two `rocprofv3 --pmc` runs of `bench.py --roofline-only` (FETCH_SIZE, then WRITE_SIZE,
 # KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device copies
-# that run issues: FETCH_SIZE 9870.1 x 2.0 (the copy reads 131,086 for 262,144 KiB),
+# that run issues: FETCH_SIZE 9866.6 x 2.0 (the copy reads 131,086 for 262,144 KiB),
 # WRITE_SIZE 36.0 x 1.0. Counters cannot be read from inside this script; other widths: null.
-PMC_TRAFFIC_BYTES = {2: int(round((9870.1 * 2.0 + 36.0 * 1.0) * 1024))}
+PMC_TRAFFIC_BYTES = {2: int(round((9866.6 * 2.0 + 36.0 * 1.0) * 1024))}
 
 
 def log(*a):
