@@ -590,6 +590,8 @@ ORNITH_API int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const
 #define ORNITH_FN_RECIP 6
 #define ORNITH_FN_ROUND_BF16 7
 #define ORNITH_FN_WAVE_SUM 8
+/* 9 + i: the value of lane (l xor 2^i) of the 64-lane wavefront, i = 0..5 (n a multiple of 64) */
+#define ORNITH_FN_XOR_LANE 9
 ORNITH_API int ornith_selftest_unary(ornith_ctx* ctx, int fn, const float* d_in, float* d_out, int64_t n);
 
 #ifdef __cplusplus

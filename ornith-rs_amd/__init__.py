@@ -183,6 +183,7 @@ class Ctx:
 
 
 FN_EXP, FN_LOG, FN_LOG1P, FN_SIGMOID_BF16, FN_SIGMOID_F32, FN_RSQRT, FN_RECIP, FN_ROUND_BF16, FN_WAVE_SUM = range(9)
+FN_XOR_LANE = 9  # + i: value of lane l ^ 2**i, i = 0..5
 
 
 # ---- Linear / MoE ---------------------------------------------------------------

@@ -19,6 +19,12 @@ __global__ void unary_kernel(int op, const float* in, float* out, int64_t n) {
     case ORNITH_FN_RECIP: y = 1.0f / x; break;
     case ORNITH_FN_ROUND_BF16: y = dm_rb(x); break;
     case ORNITH_FN_WAVE_SUM: y = dm_wave_sum<64>(x); break;
+    case ORNITH_FN_XOR_LANE + 0: y = dm_xor_lane<1>(x); break;
+    case ORNITH_FN_XOR_LANE + 1: y = dm_xor_lane<2>(x); break;
+    case ORNITH_FN_XOR_LANE + 2: y = dm_xor_lane<4>(x); break;
+    case ORNITH_FN_XOR_LANE + 3: y = dm_xor_lane<8>(x); break;
+    case ORNITH_FN_XOR_LANE + 4: y = dm_xor_lane<16>(x); break;
+    case ORNITH_FN_XOR_LANE + 5: y = dm_xor_lane<32>(x); break;
     default: y = x;
   }
   out[i] = y;
@@ -28,8 +34,9 @@ __global__ void unary_kernel(int op, const float* in, float* out, int64_t n) {
 extern "C" int ornith_selftest_unary(ornith_ctx* ctx, int fn, const float* d_in, float* d_out,
                                      int64_t n) {
   ORN_REQUIRE(ctx && d_in && d_out && n >= 0, "selftest_unary: bad argument");
-  ORN_REQUIRE(fn >= 0 && fn <= ORNITH_FN_WAVE_SUM, "selftest_unary: unknown function %d", fn);
-  ORN_REQUIRE(fn != ORNITH_FN_WAVE_SUM || n % 64 == 0, "selftest_unary: wave_sum needs n %% 64 == 0");
+  ORN_REQUIRE(fn >= 0 && fn <= ORNITH_FN_XOR_LANE + 5, "selftest_unary: unknown function %d", fn);
+  // the lane-crossing functions need whole wavefronts: n a multiple of the 256-thread block
+  ORN_REQUIRE(fn < ORNITH_FN_WAVE_SUM || n % 256 == 0, "selftest_unary: function %d needs n %% 256 == 0", fn);
   if (n == 0) return ORNITH_OK;
   hipLaunchKernelGGL(unary_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream, fn,
                      d_in, d_out, n);

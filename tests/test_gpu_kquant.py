@@ -55,9 +55,13 @@ def test_device_scalar_functions_bit_exact(orn, ctx):
     got = ctx.selftest_unary(orn.FN_ROUND_BF16, xf)
     assert np.array_equal(got[ok].view(np.uint32) >> 16, util.f32_to_bf16(xf[ok]).astype(np.uint32))
     assert np.all((got[ok].view(np.uint32) & 0xffff) == 0) and np.all(np.isnan(got[~ok]))
-    v = (rng.standard_normal(64 * 50) * 10.0 ** rng.integers(-3, 4, 64 * 50)).astype(np.float32)
-    got = ctx.selftest_unary(orn.FN_WAVE_SUM, v).reshape(50, 64)
-    for i in range(50):
+    v = (rng.standard_normal(64 * 52) * 10.0 ** rng.integers(-3, 4, 64 * 52)).astype(np.float32)
+    # the lane exchanges every reduction is built from: out[l] = in[l ^ 2**i]
+    for i in range(6):
+        got = ctx.selftest_unary(orn.FN_XOR_LANE + i, v).reshape(52, 64)
+        assert np.array_equal(got.view(np.uint32), v.reshape(52, 64)[:, np.arange(64) ^ (1 << i)].view(np.uint32)), i
+    got = ctx.selftest_unary(orn.FN_WAVE_SUM, v).reshape(52, 64)
+    for i in range(52):
         want_s = o.orc_tree64_export(util.p(np.ascontiguousarray(v[64 * i:64 * i + 64])))
         assert np.all(got[i] == np.float32(want_s))
 
