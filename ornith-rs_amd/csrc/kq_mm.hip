@@ -27,6 +27,8 @@ namespace {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
+// (a native vector: arrays of HIP's uint4 struct that are stored to LDS through casts are left in scratch memory)
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int BN = 128, BK = 128, LDK = BK + 8;
 
@@ -77,40 +79,28 @@ __device__ __forceinline__ BRegsQ4 load_q4k(const MmArgs& a, int64_t row, int nb
   return r;
 }
 
-// 64 weights as bf16 into dst[0..64): d*sc*q - dmin*m (kquant::dequantize, q4k.metal:64-96)
+// 64 weights as bf16 into dst[0..64): d*sc*q - dmin*m (kquant::dequantize, q4k.metal:64-96).
+// About three vector instructions a weight (byte -> float, one fma, half a bf16 pack): the
+// dequantization shares the wavefront with the MFMAs it feeds, so its length is GEMM time.
 __device__ __forceinline__ void dequant_q4k(const BRegsQ4& r, int grp, bf16_t* dst) {
-  const uint8_t sc[12] = {(uint8_t)r.s0, (uint8_t)(r.s0 >> 8), (uint8_t)(r.s0 >> 16), (uint8_t)(r.s0 >> 24),
-                          (uint8_t)r.s1, (uint8_t)(r.s1 >> 8), (uint8_t)(r.s1 >> 16), (uint8_t)(r.s1 >> 24),
-                          (uint8_t)r.s2, (uint8_t)(r.s2 >> 8), (uint8_t)(r.s2 >> 16), (uint8_t)(r.s2 >> 24)};
+  // the 6-bit scale and min of sub-blocks 2*grp and 2*grp + 1, two bytes each way
+  const int sh16 = (grp & 1) * 16;
+  const uint32_t a = r.s0 >> sh16, b = r.s1 >> sh16, c = r.s2 >> sh16;
+  const bool low = grp < 2;
+  const uint32_t sc16 = low ? (a & 0x3f3fu) : ((c & 0x0f0fu) | ((a & 0xc0c0u) >> 2));
+  const uint32_t m16 = low ? (b & 0x3f3fu) : (((c >> 4) & 0x0f0fu) | ((b & 0xc0c0u) >> 2));
   const float d = dm_h2f((f16_t)(r.dmw & 0xffffu)), dmin = dm_h2f((f16_t)(r.dmw >> 16));
-  float dd[2], mm[2];
-#pragma unroll
-  for (int k = 0; k < 2; ++k) {
-    const int j = 2 * grp + k;
-    uint32_t s, m;
-    if (j < 4) {
-      s = sc[j] & 63;
-      m = sc[j + 4] & 63;
-    } else {
-      s = (sc[j + 4] & 0xF) | ((sc[j - 4] >> 6) << 4);
-      m = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4);
-    }
-    dd[k] = d * (float)s;
-    mm[k] = dmin * (float)m;
-  }
+  const float dd0 = d * dm_ubyte<0>(sc16), dd1 = d * dm_ubyte<1>(sc16);
+  const float mm0 = -(dmin * dm_ubyte<0>(m16)), mm1 = -(dmin * dm_ubyte<1>(m16));
   uint32_t* out = reinterpret_cast<uint32_t*>(dst);
   const uint32_t w[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const uint32_t b = w[i];
-    const float l0 = dd[0] * (float)(b & 0xF) - mm[0], l1 = dd[0] * (float)((b >> 8) & 0xF) - mm[0];
-    const float l2 = dd[0] * (float)((b >> 16) & 0xF) - mm[0], l3 = dd[0] * (float)((b >> 24) & 0xF) - mm[0];
-    const float h0 = dd[1] * (float)((b >> 4) & 0xF) - mm[1], h1 = dd[1] * (float)((b >> 12) & 0xF) - mm[1];
-    const float h2 = dd[1] * (float)((b >> 20) & 0xF) - mm[1], h3 = dd[1] * (float)(b >> 28) - mm[1];
-    out[2 * i] = pack2(l0, l1);          // low nibbles: weights 4i .. 4i+3
-    out[2 * i + 1] = pack2(l2, l3);
-    out[16 + 2 * i] = pack2(h0, h1);     // high nibbles: the same + 32
-    out[16 + 2 * i + 1] = pack2(h2, h3);
+    const uint32_t lo = w[i] & 0x0f0f0f0fu, hi = (w[i] >> 4) & 0x0f0f0f0fu;
+    out[2 * i] = pack2(dm_fma(dd0, dm_ubyte<0>(lo), mm0), dm_fma(dd0, dm_ubyte<1>(lo), mm0));  // low nibbles: weights 4i .. 4i+3
+    out[2 * i + 1] = pack2(dm_fma(dd0, dm_ubyte<2>(lo), mm0), dm_fma(dd0, dm_ubyte<3>(lo), mm0));
+    out[16 + 2 * i] = pack2(dm_fma(dd1, dm_ubyte<0>(hi), mm1), dm_fma(dd1, dm_ubyte<1>(hi), mm1));  // high nibbles: the same + 32
+    out[16 + 2 * i + 1] = pack2(dm_fma(dd1, dm_ubyte<2>(hi), mm1), dm_fma(dd1, dm_ubyte<3>(hi), mm1));
   }
 }
 
@@ -127,37 +117,29 @@ __device__ __forceinline__ BRegsQ6 load_q6k(const MmArgs& a, int64_t row, int nb
   return r;
 }
 
-// the four weights l, l+32, l+64, l+96 of each position, d*sc*q (q6k.metal:47-77), as bf16
-// into dst[0..128) (dst = start of the half)
+// the four weights l, l+32, l+64, l+96 of each position, d*sc*(q - 32) (q6k.metal:47-77), as
+// bf16 into dst[0..128) (dst = start of the half). The 6-bit codes are put together four at a
+// time in a word; (q - 32) * s is one fma with -32 s.
 __device__ __forceinline__ void dequant_q6k(const BRegsQ6& r, int j, bf16_t* dst) {
   const float d = dm_h2f((f16_t)r.d);
   const uint32_t scw[2] = {r.sc.x, r.sc.y};
   auto scale = [&](int i) { return (float)(int)(int8_t)((scw[i >> 2] >> (8 * (i & 3))) & 0xffu); };
-  const float s1 = d * scale(j), s2 = d * scale(j + 2), s3 = d * scale(j + 4), s4 = d * scale(j + 6);
+  const float sv[4] = {d * scale(j), d * scale(j + 2), d * scale(j + 4), d * scale(j + 6)};
+  const float off[4] = {-32.f * sv[0], -32.f * sv[1], -32.f * sv[2], -32.f * sv[3]};
   const uint32_t la[4] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w}, lb[4] = {r.qb.x, r.qb.y, r.qb.z, r.qb.w},
                  hv[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
   uint32_t* out = reinterpret_cast<uint32_t*>(dst);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    float w1[4], w2[4], w3[4], w4[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const uint32_t a8 = (la[i] >> (8 * b)) & 0xFF, b8 = (lb[i] >> (8 * b)) & 0xFF,
-                     h8 = (hv[i] >> (8 * b)) & 0xFF;
-      w1[b] = s1 * (float)((int)((a8 & 0xF) | ((h8 & 3) << 4)) - 32);
-      w2[b] = s2 * (float)((int)((b8 & 0xF) | (((h8 >> 2) & 3) << 4)) - 32);
-      w3[b] = s3 * (float)((int)((a8 >> 4) | (((h8 >> 4) & 3) << 4)) - 32);
-      w4[b] = s4 * (float)((int)((b8 >> 4) | ((h8 >> 6) << 4)) - 32);
-    }
+    const uint32_t A = la[i], B = lb[i], H = hv[i];
+    const uint32_t c[4] = {(A & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u), (B & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u),
+                           ((A >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u), ((B >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u)};
     const int e = (16 * j + 4 * i) >> 1;
-    out[e] = pack2(w1[0], w1[1]);
-    out[e + 1] = pack2(w1[2], w1[3]);
-    out[16 + e] = pack2(w2[0], w2[1]);
-    out[16 + e + 1] = pack2(w2[2], w2[3]);
-    out[32 + e] = pack2(w3[0], w3[1]);
-    out[32 + e + 1] = pack2(w3[2], w3[3]);
-    out[48 + e] = pack2(w4[0], w4[1]);
-    out[48 + e + 1] = pack2(w4[2], w4[3]);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      out[16 * g + e] = pack2(dm_fma(sv[g], dm_ubyte<0>(c[g]), off[g]), dm_fma(sv[g], dm_ubyte<1>(c[g]), off[g]));
+      out[16 * g + e + 1] = pack2(dm_fma(sv[g], dm_ubyte<2>(c[g]), off[g]), dm_fma(sv[g], dm_ubyte<3>(c[g]), off[g]));
+    }
   }
 }
 
@@ -207,15 +189,17 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
 #pragma unroll
   for (int i = 0; i < NA; ++i) {
     const int idx = tid + 256 * i, r = idx >> 4, c8 = idx & 15;
-    const int64_t src = r < rows_here ? (GATHER ? (int64_t)s_src[r] : (int64_t)(m0 + r)) : -1;
-    asrc[i] = src >= 0 ? a.x + src * a.K + 8 * c8 : nullptr;
+    // rows past the end of the tile read a valid row instead (pair 0's, or the last one): what
+    // they produce lands in output rows the epilogue does not store, and no load needs a branch
+    const int64_t src = GATHER ? (int64_t)s_src[r] : (int64_t)min(m0 + r, a.M - 1);
+    asrc[i] = a.x + src * a.K + 8 * c8;
   }
-  uint4 areg[NA];
+  u32x4_t areg[NA];
   typename BRegsOf<KIND>::type breg;
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < NA; ++i)
-      areg[i] = asrc[i] ? *reinterpret_cast<const uint4*>(asrc[i] + k0) : make_uint4(0, 0, 0, 0);
+      areg[i] = *reinterpret_cast<const u32x4_t*>(asrc[i] + k0);
     if constexpr (KIND == ORNITH_Q4K)
       breg = load_q4k(a, brow, nb, k0 >> 8, ((k0 & 255) >> 6) + bpart);
     else
@@ -235,7 +219,7 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       const int idx = tid + 256 * i;
-      *reinterpret_cast<uint4*>(&As[idx >> 4][8 * (idx & 15)]) = areg[i];
+      *reinterpret_cast<u32x4_t*>(&As[idx >> 4][8 * (idx & 15)]) = areg[i];
     }
     if constexpr (KIND == ORNITH_Q4K)
       dequant_q4k(breg, ((k0 & 255) >> 6) + bpart, &Bs[br][64 * bpart]);
@@ -243,21 +227,27 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
       dequant_q6k(breg, bpart, &Bs[br][0]);
     __syncthreads();
     if (k0 + BK < a.K) fetch(k0 + BK);  // in flight while the matrix cores run
-#pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
+    // fragments of step kk + 1 leave LDS while the matrix cores work on step kk
+    bf16x8_t af[2][TM], bfr[2][TN];
+    auto frags = [&](int kk, bf16x8_t (&fa)[TM], bf16x8_t (&fb)[TN]) {
       const int kc = kk * 16 + 8 * (lane >> 5);
-      bf16x8_t af[TM], bfr[TN];
 #pragma unroll
       for (int i = 0; i < TM; ++i)
-        af[i] = *reinterpret_cast<const bf16x8_t*>(&As[wm * WTM + i * 32 + (lane & 31)][kc]);
+        fa[i] = *reinterpret_cast<const bf16x8_t*>(&As[wm * WTM + i * 32 + (lane & 31)][kc]);
 #pragma unroll
       for (int j = 0; j < TN; ++j)
-        bfr[j] = *reinterpret_cast<const bf16x8_t*>(&Bs[wn * WTN + j * 32 + (lane & 31)][kc]);
+        fb[j] = *reinterpret_cast<const bf16x8_t*>(&Bs[wn * WTN + j * 32 + (lane & 31)][kc]);
+    };
+    frags(0, af[0], bfr[0]);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      if (kk + 1 < BK / 16) frags(kk + 1, af[(kk + 1) & 1], bfr[(kk + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);  // or the reads are sunk to just before their use
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
     }
     __syncthreads();
   }
