@@ -104,6 +104,73 @@ __global__ __launch_bounds__(64) void gdn_front_kernel(FrontArgs p) {
   }
 }
 
+// The same for a run of tokens per workgroup (kernel size 4, prefill widths): the taps are
+// loaded once and each token's inputs are read once and kept as the sliding window, instead of
+// one 64-thread workgroup per token and 128 channels. Per token the arithmetic and its order
+// are those of gdn_front_kernel. grid (D / 128, ceil(T / kFrontRun)), 64 threads.
+constexpr int kFrontRun = 16;
+__global__ __launch_bounds__(64) void gdn_front_run_kernel(FrontArgs p) {
+  constexpr int K = 4, S = K - 1;
+  const int slot = blockIdx.x, t0 = blockIdx.y * kFrontRun, lane = threadIdx.x;
+  const int D = p.D, c0 = slot * 128 + 2 * lane, key_dim = p.Hk * 128;
+  const int t1 = min(t0 + kFrontRun, p.T);
+  float w0[K], w1[K];
+  {
+    const uint2 a = *reinterpret_cast<const uint2*>(p.cw + (size_t)c0 * K);
+    const uint2 b = *reinterpret_cast<const uint2*>(p.cw + (size_t)(c0 + 1) * K);
+    w0[0] = dm_bf2f_lo(a.x); w0[1] = dm_bf2f_hi(a.x); w0[2] = dm_bf2f_lo(a.y); w0[3] = dm_bf2f_hi(a.y);
+    w1[0] = dm_bf2f_lo(b.x); w1[1] = dm_bf2f_hi(b.x); w1[2] = dm_bf2f_lo(b.y); w1[3] = dm_bf2f_hi(b.y);
+  }
+  // window position j holds conv_state[j] for j < S, qkv[j - S] from there on
+  auto input = [&](int j) {
+    const bf16_t* src = (j < S) ? (p.conv_state + (size_t)j * D) : (p.qkv + (size_t)(j - S) * D);
+    return *reinterpret_cast<const uint32_t*>(src + c0);
+  };
+  uint32_t win[K];
+#pragma unroll
+  for (int i = 0; i < S; ++i) win[i] = input(t0 + i);
+  if (t0 == 0) {
+#pragma unroll
+    for (int j = 0; j < S; ++j) *reinterpret_cast<uint32_t*>(p.conv_input + (size_t)j * D + c0) = win[j];
+  }
+  const bool is_qk = slot < 2 * p.Hk, is_q = slot < p.Hk;
+  const float sc = is_q ? p.q_scale : p.k_scale;
+  for (int t = t0; t < t1; ++t) {
+    win[S] = input(t + S);  // = qkv[t]
+    float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+      acc0 = dm_fma(dm_bf2f_lo(win[i]), w0[i], acc0);
+      acc1 = dm_fma(dm_bf2f_hi(win[i]), w1[i], acc1);
+    }
+    *reinterpret_cast<uint32_t*>(p.conv_input + (size_t)(S + t) * D + c0) = win[S];
+#pragma unroll
+    for (int i = 0; i < S; ++i) win[i] = win[i + 1];
+    const float cv0 = dm_rb(acc0), cv1 = dm_rb(acc1);
+    const float y0 = dm_rb(cv0 * dm_sigmoid_bf16(cv0)), y1 = dm_rb(cv1 * dm_sigmoid_bf16(cv1));
+    if (is_qk) {
+      float ss = dm_fma(y0, y0, 0.f);
+      ss = dm_fma(y1, y1, ss);
+      const float inv = dm_rsqrt(dm_wave_sum<64>(ss) / 128.0f + p.eps);
+      bf16_t* dst = (is_q ? p.q : p.k) + (size_t)t * key_dim + (is_q ? c0 : c0 - key_dim);
+      const uint32_t lo = dm_f2bf(sc * dm_rb(y0 * inv)), hi = dm_f2bf(sc * dm_rb(y1 * inv));
+      *reinterpret_cast<uint32_t*>(dst) = lo | (hi << 16);
+    } else {
+      bf16_t* dst = p.v + (size_t)t * (D - 2 * key_dim) + (c0 - 2 * key_dim);
+      *reinterpret_cast<uint32_t*>(dst) = (uint32_t)dm_f2bf(y0) | ((uint32_t)dm_f2bf(y1) << 16);
+    }
+  }
+  if (slot == 0) {
+    for (int i = t0 * p.Hv + lane; i < t1 * p.Hv; i += 64) {
+      const int h = i % p.Hv;
+      const float sp = softplus_bf16(dm_rb(dm_bf2f(p.a_in[i]) + dm_bf2f(p.dt_bias[h])));
+      const float decay = dm_exp(dm_bf2f(p.a_log[h]));
+      p.g[i] = dm_exp(-decay * sp);
+      p.beta[i] = dm_f2bf(dm_sigmoid_bf16(dm_bf2f(p.b_in[i])));
+    }
+  }
+}
+
 struct RecArgs {
   const bf16_t* q;
   const bf16_t* k;
@@ -733,7 +800,11 @@ int ornith_gdn_front(ornith_ctx* ctx, const void* d_conv_state, const void* d_qk
   u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
   memcpy(&p.k_scale, &u, 4);
   p.eps = eps;
-  hipLaunchKernelGGL(gdn_front_kernel, dim3(p.D / 128, T), dim3(64), 0, ctx->stream, p);
+  if (p.K == 4 && T >= 2 * kFrontRun)
+    hipLaunchKernelGGL(gdn_front_run_kernel, dim3(p.D / 128, (T + kFrontRun - 1) / kFrontRun), dim3(64), 0,
+                       ctx->stream, p);
+  else
+    hipLaunchKernelGGL(gdn_front_kernel, dim3(p.D / 128, T), dim3(64), 0, ctx->stream, p);
   ORN_LAUNCH_CHECK("gdn_front_kernel");
   return ORNITH_OK;
 }

@@ -43,34 +43,75 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const bf16_t* gates, in
   }
 }
 
-__global__ void swiglu_kernel(const bf16_t* gate, const bf16_t* up, bf16_t* out, int64_t n) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const float g = dm_bf2f(gate[i]);
-  const float s = dm_rb(g * dm_sigmoid_bf16(g));
-  out[i] = dm_f2bf(s * dm_bf2f(up[i]));
+// V consecutive elements a thread (V = 8: 16-byte loads and stores; V = 1 for odd sizes)
+template <int V>
+struct BfPack;
+template <>
+struct BfPack<8> { typedef unsigned int type __attribute__((ext_vector_type(4))); };
+template <>
+struct BfPack<1> { typedef bf16_t type; };
+template <int V>
+__device__ __forceinline__ float bf_get(const typename BfPack<V>::type& p, int i) {
+  if constexpr (V == 1) return dm_bf2f(p);
+  else return (i & 1) ? dm_bf2f_hi(p[i >> 1]) : dm_bf2f_lo(p[i >> 1]);
+}
+template <int V>
+__device__ __forceinline__ void bf_put(typename BfPack<V>::type& p, int i, float v) {
+  if constexpr (V == 1) p = dm_f2bf(v);
+  else p[i >> 1] = (i & 1) ? (p[i >> 1] & 0xffffu) | ((uint32_t)dm_f2bf(v) << 16) : (uint32_t)dm_f2bf(v);
 }
 
-// one thread per output element; j ascends, every step rounds to bf16
+template <int V>
+__global__ void swiglu_kernel(const bf16_t* gate, const bf16_t* up, bf16_t* out, int64_t n) {
+  typedef typename BfPack<V>::type P;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n / V) return;
+  const P g8 = reinterpret_cast<const P*>(gate)[i], u8 = reinterpret_cast<const P*>(up)[i];
+  P o8;
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const float g = bf_get<V>(g8, e);
+    const float s = dm_rb(g * dm_sigmoid_bf16(g));
+    bf_put<V>(o8, e, s * bf_get<V>(u8, e));
+  }
+  reinterpret_cast<P*>(out)[i] = o8;
+}
+
+// one thread per V output elements of a token; j ascends, every step rounds to bf16
+template <int V>
 __global__ void moe_combine_kernel(const bf16_t* scores, const bf16_t* y, const bf16_t* gate,
                                    const bf16_t* shared, bf16_t* out, int T, int k, int dim,
                                    int normalize) {
+  typedef typename BfPack<V>::type P;
   const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (int64_t)T * dim) return;
-  const int t = (int)(idx / dim), c = (int)(idx - (int64_t)t * dim);
+  const int per_row = dim / V;
+  if (idx >= (int64_t)T * per_row) return;
+  const int t = (int)(idx / per_row), c = (int)(idx - (int64_t)t * per_row) * V;
   const bf16_t* s = scores + (size_t)t * k;
   float denom = 0.f;
   if (normalize)
     for (int j = 0; j < k; ++j) denom = dm_rb(dm_bf2f(s[j]) + denom);
-  float acc = 0.f;
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = 0.f;
   for (int j = 0; j < k; ++j) {
     const float w = normalize ? dm_rb(dm_bf2f(s[j]) / denom) : dm_bf2f(s[j]);
-    const float weighted = dm_rb(dm_bf2f(y[((size_t)t * k + j) * dim + c]) * w);
-    acc = dm_rb(weighted + acc);
+    const P yj = *reinterpret_cast<const P*>(y + ((size_t)t * k + j) * dim + c);
+#pragma unroll
+    for (int e = 0; e < V; ++e) {
+      const float weighted = dm_rb(bf_get<V>(yj, e) * w);
+      acc[e] = dm_rb(weighted + acc[e]);
+    }
   }
   const float g = dm_sigmoid_bf16(dm_bf2f(gate[t]));
-  const float gated = dm_rb(g * dm_bf2f(shared[idx]));
-  out[idx] = dm_f2bf(acc + gated);
+  const P sh = *reinterpret_cast<const P*>(shared + (size_t)t * dim + c);
+  P o;
+#pragma unroll
+  for (int e = 0; e < V; ++e) {
+    const float gated = dm_rb(g * bf_get<V>(sh, e));
+    bf_put<V>(o, e, acc[e] + gated);
+  }
+  *reinterpret_cast<P*>(out + (size_t)t * dim + c) = o;
 }
 
 int launch_router(ornith_ctx* ctx, const bf16_t* gates, int T, int E, int k, uint32_t* inds,
@@ -157,8 +198,13 @@ int ornith_router_topk(ornith_ctx* ctx, const void* d_gates, int T, int E, int k
 int ornith_swiglu(ornith_ctx* ctx, const void* d_gate, const void* d_up, int64_t n, void* d_out) {
   ORN_REQUIRE(ctx && d_gate && d_up && d_out && n >= 0, "swiglu: bad argument");
   if (n == 0) return ORNITH_OK;
-  hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream,
-                     (const bf16_t*)d_gate, (const bf16_t*)d_up, (bf16_t*)d_out, n);
+  // 16-byte pieces when the size and the addresses allow
+  if (n % 8 == 0 && (((uintptr_t)d_gate | (uintptr_t)d_up | (uintptr_t)d_out) & 15) == 0)
+    hipLaunchKernelGGL(swiglu_kernel<8>, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0, ctx->stream,
+                       (const bf16_t*)d_gate, (const bf16_t*)d_up, (bf16_t*)d_out, n);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<1>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, ctx->stream,
+                       (const bf16_t*)d_gate, (const bf16_t*)d_up, (bf16_t*)d_out, n);
   ORN_LAUNCH_CHECK("swiglu_kernel");
   return ORNITH_OK;
 }
@@ -168,10 +214,14 @@ int ornith_moe_combine(ornith_ctx* ctx, const void* d_scores, const void* d_y, c
   ORN_REQUIRE(ctx && d_scores && d_y && d_gate && d_shared && d_out, "moe_combine: null argument");
   ORN_REQUIRE(T >= 1 && k >= 1 && dim >= 1, "moe_combine: T=%d k=%d dim=%d", T, k, dim);
   const int64_t n = (int64_t)T * dim;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-                     ctx->stream, (const bf16_t*)d_scores, (const bf16_t*)d_y,
-                     (const bf16_t*)d_gate, (const bf16_t*)d_shared, (bf16_t*)d_out, T, k, dim,
-                     normalize);
+  if (dim % 8 == 0 && (((uintptr_t)d_y | (uintptr_t)d_shared | (uintptr_t)d_out) & 15) == 0)
+    hipLaunchKernelGGL(moe_combine_kernel<8>, dim3((unsigned)((n / 8 + 255) / 256)), dim3(256), 0,
+                       ctx->stream, (const bf16_t*)d_scores, (const bf16_t*)d_y, (const bf16_t*)d_gate,
+                       (const bf16_t*)d_shared, (bf16_t*)d_out, T, k, dim, normalize);
+  else
+    hipLaunchKernelGGL(moe_combine_kernel<1>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                       ctx->stream, (const bf16_t*)d_scores, (const bf16_t*)d_y, (const bf16_t*)d_gate,
+                       (const bf16_t*)d_shared, (bf16_t*)d_out, T, k, dim, normalize);
   ORN_LAUNCH_CHECK("moe_combine_kernel");
   return ORNITH_OK;
 }

@@ -49,7 +49,9 @@ def _inputs(rng, T, Hk, Hv):
                 dt_bias=util.bf16_normal(rng, (Hv,), 0.5))
 
 
-@pytest.mark.parametrize("T,Hk,Hv", [(1, 16, 32), (2, 16, 32), (4, 16, 32), (3, 2, 4), (7, 1, 1)])
+# from 32 rows a call a workgroup takes a run of 16 tokens (same arithmetic): 32, a ragged 45, 100
+@pytest.mark.parametrize("T,Hk,Hv", [(1, 16, 32), (2, 16, 32), (4, 16, 32), (3, 2, 4), (7, 1, 1), (32, 2, 4), (45, 2, 4),
+                                     (100, 16, 32)])
 def test_gdn_front_bit_exact(orn, ctx, T, Hk, Hv):
     rng = np.random.default_rng(10 + T + Hv)
     i = _inputs(rng, T, Hk, Hv)
