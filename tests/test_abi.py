@@ -67,3 +67,15 @@ def test_host_random_functions_match_known_answers():
     # key = KAT key and the oracle (itself pinned on the three KATs) covers the layout; and here
     # the one KAT that bits() can reach directly: n = 1 hashes (0, 0)
     assert orn.random_bits([0, 0], 1)[0] == 0x6B200159
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """One GPU only: `bench.py --gpus N` with N > 1 exits with a message that says so, before
+    anything touches a device."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stderr + r.stdout)
