@@ -20,6 +20,8 @@
 // Prefill is exempt from the "row r of a batch == row r alone" rule in the reference too
 // (src/ops/invariant.rs:140-168): results agree with the mat-vec path to bf16 rounding of
 // the weights and the order of the fp32 sums, not bit for bit.
+#include <type_traits>
+
 #include "dmath.h"
 #include "rt.h"
 
@@ -269,6 +271,251 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
     }
 }
 
+// ---- the same GEMM with producers and consumers --------------------------------------------
+// Eight wavefronts a workgroup. Four (one a SIMD) run the MFMAs of K slab s out of one LDS
+// buffer; the other four meanwhile write slab s + 1 into the other buffer (activations as they
+// are, weights dequantized, from registers loaded two slabs ahead): the vector work of the
+// dequantization and the matrix cores then run side by side on every SIMD instead of one after
+// the other in one wavefront. K slabs of 64, one barrier a slab.
+constexpr int BK2 = 64, LD2 = BK2 + 8;
+
+struct PipeQ4 {
+  float dd, mm;
+  uint32_t w[8];  // this thread's nibble of each of the 32 code bytes, 4 to a word
+};
+struct PipeQ6 {
+  float sa, sb, oa, ob;
+  uint32_t ca[4], cb[4];  // the 6-bit codes of the positions' two weights, 4 to a word
+};
+
+// what a thread needs of its 32 weights before the quarters: scale, offset, codes
+__device__ __forceinline__ PipeQ4 pipe_prepare(const BRegsQ4& r, int grp, int half) {
+  const int sh16 = (grp & 1) * 16;
+  const uint32_t a = r.s0 >> sh16, b = r.s1 >> sh16, c = r.s2 >> sh16;
+  const bool low = grp < 2;
+  const uint32_t sc16 = low ? (a & 0x3f3fu) : ((c & 0x0f0fu) | ((a & 0xc0c0u) >> 2));
+  const uint32_t m16 = low ? (b & 0x3f3fu) : (((c >> 4) & 0x0f0fu) | ((b & 0xc0c0u) >> 2));
+  const float d = dm_h2f((f16_t)(r.dmw & 0xffffu)), dmin = dm_h2f((f16_t)(r.dmw >> 16));
+  PipeQ4 p;
+  p.dd = d * dm_ubyte<0>(sc16 >> (8 * half));
+  p.mm = -(dmin * dm_ubyte<0>(m16 >> (8 * half)));
+  const uint32_t w[8] = {r.q0.x, r.q0.y, r.q0.z, r.q0.w, r.q1.x, r.q1.y, r.q1.z, r.q1.w};
+#pragma unroll
+  for (int i = 0; i < 8; ++i) p.w[i] = (w[i] >> (4 * half)) & 0x0f0f0f0fu;
+  return p;
+}
+// quarter q: weights 8q .. 8q + 8 of the thread's 32, to dst[8q ..]
+__device__ __forceinline__ void pipe_quarter(const PipeQ4& p, int q, bf16_t* dst) {
+  u32x4_t o;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const uint32_t c = p.w[2 * q + h];
+    o[2 * h] = pack2(dm_fma(p.dd, dm_ubyte<0>(c), p.mm), dm_fma(p.dd, dm_ubyte<1>(c), p.mm));
+    o[2 * h + 1] = pack2(dm_fma(p.dd, dm_ubyte<2>(c), p.mm), dm_fma(p.dd, dm_ubyte<3>(c), p.mm));
+  }
+  *reinterpret_cast<u32x4_t*>(dst + 8 * q) = o;
+}
+
+// Q6_K: the 64-slab `sub` of a 128-half holds weights l and l + 32 (sub 0: low nibbles) or
+// l + 64 and l + 96 (sub 1: high nibbles) of positions l; a thread has positions 16j .. 16j + 16
+__device__ __forceinline__ PipeQ6 pipe_prepare(const BRegsQ6& r, int j, int sub) {
+  const float d = dm_h2f((f16_t)r.d);
+  const uint32_t scw[2] = {r.sc.x, r.sc.y};
+  auto scale = [&](int i) { return (float)(int)(int8_t)((scw[i >> 2] >> (8 * (i & 3))) & 0xffu); };
+  PipeQ6 p;
+  p.sa = d * scale(j + 4 * sub);
+  p.sb = d * scale(j + 2 + 4 * sub);
+  p.oa = -32.f * p.sa;
+  p.ob = -32.f * p.sb;
+  const uint32_t la[4] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w}, lb[4] = {r.qb.x, r.qb.y, r.qb.z, r.qb.w},
+                 hv[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t H = hv[i] >> (4 * sub);  // bits 0-1: the A-side weight's, bits 2-3: the B-side's
+    p.ca[i] = ((la[i] >> (4 * sub)) & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
+    p.cb[i] = ((lb[i] >> (4 * sub)) & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
+  }
+  return p;
+}
+// quarter q: positions 16j + 4q .. + 4: A-side weights to dst[16j + 4q ..], B-side 32 further on
+__device__ __forceinline__ void pipe_quarter(const PipeQ6& p, int q, int j, bf16_t* dst) {
+  uint2 oa, ob;
+  oa.x = pack2(dm_fma(p.sa, dm_ubyte<0>(p.ca[q]), p.oa), dm_fma(p.sa, dm_ubyte<1>(p.ca[q]), p.oa));
+  oa.y = pack2(dm_fma(p.sa, dm_ubyte<2>(p.ca[q]), p.oa), dm_fma(p.sa, dm_ubyte<3>(p.ca[q]), p.oa));
+  ob.x = pack2(dm_fma(p.sb, dm_ubyte<0>(p.cb[q]), p.ob), dm_fma(p.sb, dm_ubyte<1>(p.cb[q]), p.ob));
+  ob.y = pack2(dm_fma(p.sb, dm_ubyte<2>(p.cb[q]), p.ob), dm_fma(p.sb, dm_ubyte<3>(p.cb[q]), p.ob));
+  *reinterpret_cast<uint2*>(dst + 16 * j + 4 * q) = oa;
+  *reinterpret_cast<uint2*>(dst + 32 + 16 * j + 4 * q) = ob;
+}
+
+template <int KIND>
+struct PipeOf { typedef PipeQ4 type; };
+template <>
+struct PipeOf<ORNITH_Q6K> { typedef PipeQ6 type; };
+
+
+template <int KIND, int BM, bool GATHER>
+__global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
+  constexpr int WM = BM >= 128 ? 2 : 1, WN = 4 / WM;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int NA = BM * 8 / 256;  // 16-byte pieces of an activation slab per producer thread
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][BM][LD2];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[2][BN][LD2];
+  __shared__ uint32_t s_src[BM], s_dst[BM];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * BN;
+  const int nb = a.K >> 8;
+  const int nslab = a.K / BK2;  // K is a multiple of 256: a multiple of four slabs
+
+  int rows_here, m0 = 0;
+  int64_t wrow0 = 0;
+  if constexpr (GATHER) {
+    if (blockIdx.y >= *a.n_tiles) return;
+    const uint32_t e = a.tile_expert[blockIdx.y], st = a.tile_start[blockIdx.y];
+    rows_here = (int)a.tile_count[blockIdx.y];
+    wrow0 = (int64_t)e * a.O;
+    for (int r = tid; r < BM; r += 512) {
+      const uint32_t p = r < rows_here ? a.pair[st + r] : 0u;
+      s_src[r] = p / (uint32_t)a.up_div;
+      s_dst[r] = p;
+    }
+    __syncthreads();
+  } else {
+    m0 = blockIdx.y * BM;
+    rows_here = min(BM, a.M - m0);
+  }
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+
+  if (wave >= 4) {
+    // ---- producers ----
+    const int ptid = tid - 256;
+    const int br = ptid >> 1, bpart = ptid & 1;
+    const int64_t brow = wrow0 + min(n0 + br, a.O - 1);
+    const bf16_t* asrc[NA];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      const int idx = ptid + 256 * i, r = idx >> 3, c8 = idx & 7;
+      // rows past the end of the tile read a valid row: what they produce is never stored
+      const int64_t src = GATHER ? (int64_t)s_src[r] : (int64_t)min(m0 + r, a.M - 1);
+      asrc[i] = a.x + src * a.K + 8 * c8;
+    }
+    // Four register sets: slab k travels in set k & 3 and is asked for four slabs before it is
+    // written to LDS buffer k & 1, so a load has about four slab times to arrive. (Sets and
+    // buffers are picked by constants: an index known only at run time would put the arrays
+    // in scratch memory.)
+    u32x4_t areg[4][NA];
+    typename BRegsOf<KIND>::type breg[4];
+    auto fetch = [&](auto set, int k0) {
+      constexpr int SET = decltype(set)::value;
+#pragma unroll
+      for (int i = 0; i < NA; ++i) areg[SET][i] = *reinterpret_cast<const u32x4_t*>(asrc[i] + k0);
+      if constexpr (KIND == ORNITH_Q4K)
+        breg[SET] = load_q4k(a, brow, nb, k0 >> 8, (k0 & 255) >> 6);
+      else
+        breg[SET] = load_q6k(a, brow, nb, k0 >> 8, (k0 & 255) >> 7, bpart);
+    };
+    auto write = [&](auto set, int k0) {
+      constexpr int SET = decltype(set)::value, BUF = SET & 1;
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int idx = ptid + 256 * i;
+        *reinterpret_cast<u32x4_t*>(&As[BUF][idx >> 3][8 * (idx & 7)]) = areg[SET][i];
+      }
+      if constexpr (KIND == ORNITH_Q4K) {
+        const PipeQ4 pp = pipe_prepare(breg[SET], (k0 & 255) >> 6, bpart);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) pipe_quarter(pp, q, &Bs[BUF][br][32 * bpart]);
+      } else {
+        const PipeQ6 pp = pipe_prepare(breg[SET], bpart, (k0 & 127) >> 6);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) pipe_quarter(pp, q, bpart, &Bs[BUF][br][0]);
+      }
+    };
+    using Set2 = std::integral_constant<int, 2>;
+    using Set3 = std::integral_constant<int, 3>;
+    fetch(Set0{}, 0);
+    fetch(Set1{}, BK2);
+    fetch(Set2{}, 2 * BK2);
+    fetch(Set3{}, 3 * BK2);
+    write(Set0{}, 0);
+    if (4 < nslab) fetch(Set0{}, 4 * BK2);
+    __syncthreads();
+    // while the consumers work on slab s + u: slab s + u + 1 into the other buffer, then its
+    // register set asks for the slab four further on
+    auto step = [&](auto set, int k) {
+      if (k < nslab) write(set, k * BK2);
+      if (k + 4 < nslab) fetch(set, (k + 4) * BK2);
+      __syncthreads();
+    };
+    for (int s = 0; s < nslab; s += 4) {
+      step(Set1{}, s + 1);
+      step(Set2{}, s + 2);
+      step(Set3{}, s + 3);
+      step(Set0{}, s + 4);
+    }
+    return;
+  }
+
+  // ---- consumers ----
+  const int wm = wave / WN, wn = wave % WN;
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  auto frags = [&](int buf, int kk, bf16x8_t (&fa)[TM], bf16x8_t (&fb)[TN]) {
+    const int kc = kk * 16 + 8 * (lane >> 5);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      fa[i] = *reinterpret_cast<const bf16x8_t*>(&As[buf][wm * WTM + i * 32 + (lane & 31)][kc]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+      fb[j] = *reinterpret_cast<const bf16x8_t*>(&Bs[buf][wn * WTN + j * 32 + (lane & 31)][kc]);
+  };
+  auto slab = [&](int buf) {
+    bf16x8_t af[2][TM], bfr[2][TN];
+    frags(buf, 0, af[0], bfr[0]);
+#pragma unroll
+    for (int kk = 0; kk < BK2 / 16; ++kk) {
+      if (kk + 1 < BK2 / 16) frags(buf, kk + 1, af[(kk + 1) & 1], bfr[(kk + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);  // or the reads are sunk to just before their use
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
+    }
+  };
+  __syncthreads();  // slab 0 is in buffer 0
+  for (int s = 0; s < nslab; s += 2) {  // (the producers count the same barriers, four a turn)
+    slab(0);
+    __syncthreads();
+    slab(1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: D[row = 8*b + 4*(lane/32) + r][col = lane%32] = acc[4*b + r]
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int o = n0 + wn * WTN + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int r = wm * WTM + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+        if (r < rows_here && o < a.O) {
+          const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
+          a.y[dst * a.O + o] = dm_f2bf(acc[i][j][e]);
+        }
+      }
+    }
+}
+
 // BM == 64 has two 32-row MFMA tiles per wavefront as well (TM = 2), one wavefront column
 static_assert(BN == 128 && BK == 128, "tile constants are baked into the index arithmetic");
 
@@ -351,7 +598,14 @@ int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, 
   const int nx = (w->O + BN - 1) / BN;
   const bool big = M >= 256 && (long)nx * ((M + 255) / 256) >= ctx->compute_units;
   const dim3 grid(nx, big ? (M + 255) / 256 : (M + 127) / 128);
-  if (w->kind == ORNITH_Q4K) {
+  // the 256-row tile runs in its producer / consumer form (the smaller tiles measured no
+  // faster that way: they have too few MFMAs a slab)
+  if (big && ornith_option_gemm_duo()) {
+    if (w->kind == ORNITH_Q4K)
+      hipLaunchKernelGGL((kq_mm_duo_kernel<ORNITH_Q4K, 256, false>), grid, dim3(512), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((kq_mm_duo_kernel<ORNITH_Q6K, 256, false>), grid, dim3(512), 0, ctx->stream, a);
+  } else if (w->kind == ORNITH_Q4K) {
     if (big)
       hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 256, false>), grid, dim3(256), 0, ctx->stream, a);
     else

@@ -43,7 +43,8 @@ Option g_options[] = {{"fuse_moe", "ORNITH_FUSE_MOE", 1, -1},
                       {"kq_iters", "ORNITH_KQ_ITERS", 0, -1},
                       {"gemm_rows", "ORNITH_GEMM_ROWS", 32, -1},
                       {"fuse_gdn", "ORNITH_FUSE_GDN", 1, -1},
-                      {"fuse_norm", "ORNITH_FUSE_NORM", 1, -1}};
+                      {"fuse_norm", "ORNITH_FUSE_NORM", 1, -1},
+                      {"gemm_duo", "ORNITH_GEMM_DUO", 1, -1}};
 int option_value(int i) {
   Option& o = g_options[i];
   if (o.value < 0) {
@@ -60,6 +61,7 @@ int ornith_option_moe_up_iters() { return option_value(2); }
 int ornith_option_kq_iters() { return option_value(3); }
 int ornith_option_fuse_gdn() { return option_value(5); }
 int ornith_option_fuse_norm() { return option_value(6); }
+int ornith_option_gemm_duo() { return option_value(7); }
 int ornith_option_gemm_rows() {
   const int v = option_value(4);
   return v <= 0 ? 1 << 30 : v;
