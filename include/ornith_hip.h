@@ -78,7 +78,10 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *               exact mat-vecs. The one switch that changes results (to bf16 rounding of the
  *               weights): prefill is outside the exact window in the reference as well.
  *   "kq_iters"  (ORNITH_KQ_ITERS, default 0 = chosen by shape; 1..8): output rows each
- *               wavefront of the k-quant mat-vec walks, a tuning knob */
+ *               wavefront of the k-quant mat-vec walks, a tuning knob
+ *   "gemm_duo"  (ORNITH_GEMM_DUO, default 1): the 256-row tile of the prefill GEMM runs with
+ *               producer and consumer wavefronts (0: every wavefront dequantizes, then
+ *               multiplies); same results either way */
 ORNITH_API int ornith_set_option(const char* name, int value);
 ORNITH_API int ornith_timer_begin(ornith_ctx* ctx);
 ORNITH_API int ornith_timer_end(ornith_ctx* ctx, float* ms_out);
