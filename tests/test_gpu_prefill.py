@@ -30,7 +30,10 @@ def _check(got_bits, want64, K, what):
 
 @pytest.mark.parametrize("kind,O,K,M", [(Q4K, 256, 512, 128), (Q4K, 512, 2048, 300), (Q6K, 256, 512, 128),
                                          (Q6K, 384, 2048, 77), (Q4K, 8192, 2048, 256), (Q6K, 2048, 4096, 129),
-                                         (Q4K, 200, 256, 16)])
+                                         (Q4K, 200, 256, 16),
+                                         # enough 256-row tiles to fill the device: the producer / consumer kernel,
+                                         # ragged in rows (1061 = 4 tiles + 37) and a whole number of tiles
+                                         (Q4K, 8192, 512, 1061), (Q6K, 8192, 1024, 1024)])
 def test_kq_matmul_vs_float64(orn, ctx, kind, O, K, M):
     rng = np.random.default_rng(O + K + M + kind)
     t = util.make_kq(kind, rng, 1, O, K)
