@@ -88,19 +88,22 @@ def test_swiglu_and_combine_bit_exact(orn, ctx):
     dg, du, do = ctx.to_device(bits), ctx.to_device(up), ctx.alloc(65536 * 2)
     ctx.swiglu(dg, du, 65536, do)
     assert np.array_equal(do.download(np.uint16, (65536,))[fin], want[fin])
-    T, k, dim = 3, 8, 2048
-    scores = util.f32_to_bf16(rng.random((T, k)).astype(np.float32) * 0.1)
-    y = util.f32_to_bf16(rng.standard_normal((T, k, dim)).astype(np.float32))
-    gate = util.f32_to_bf16(rng.standard_normal(T).astype(np.float32) * 3)
-    shared = util.f32_to_bf16(rng.standard_normal((T, dim)).astype(np.float32))
-    for norm in (1, 0):
-        want = np.empty((T, dim), np.uint16)
-        oracle().orc_moe_combine(p(scores), p(y), p(gate), p(shared), T, k, dim, norm, p(want))
-        bufs = [ctx.to_device(a) for a in (scores, y, gate, shared)]
-        out = ctx.alloc(T * dim * 2)
-        ctx.moe_combine(*bufs, T, k, dim, norm, out)
-        assert np.array_equal(out.download(np.uint16, (T, dim)), want)
-        for b in bufs + [out]: b.free()
+    # a length that is not a multiple of 8 takes the one-element-a-thread form
+    ctx.swiglu(dg, du, 65531, do)
+    assert np.array_equal(do.download(np.uint16, (65536,))[:65531][fin[:65531]], want[:65531][fin[:65531]])
+    for T, k, dim in ((3, 8, 2048), (5, 4, 100)):  # 100: not a multiple of 8 either
+        scores = util.f32_to_bf16(rng.random((T, k)).astype(np.float32) * 0.1)
+        y = util.f32_to_bf16(rng.standard_normal((T, k, dim)).astype(np.float32))
+        gate = util.f32_to_bf16(rng.standard_normal(T).astype(np.float32) * 3)
+        shared = util.f32_to_bf16(rng.standard_normal((T, dim)).astype(np.float32))
+        for norm in (1, 0):
+            want_c = np.empty((T, dim), np.uint16)
+            oracle().orc_moe_combine(p(scores), p(y), p(gate), p(shared), T, k, dim, norm, p(want_c))
+            bufs = [ctx.to_device(a) for a in (scores, y, gate, shared)]
+            out = ctx.alloc(T * dim * 2)
+            ctx.moe_combine(*bufs, T, k, dim, norm, out)
+            assert np.array_equal(out.download(np.uint16, (T, dim)), want_c)
+            for b in bufs + [out]: b.free()
     for b in (dg, du, do): b.free()
 
 
