@@ -42,6 +42,39 @@ def test_moe_fused_equals_unfused_and_oracle(orn, ctx, H, E, I, gk, dk):
         moe.free()
 
 
+# shapes that take the other lane-per-row widths of the two expert kernels: K = 256 (8 Q4_K / 4 Q6_K
+# chunks a row), 1024, 2048 in either format, and the four-rows-a-wavefront form of the up kernel
+@pytest.mark.parametrize("H,E,I,gk,dk,iters", [(2048, 256, 512, Q4K, Q6K, 0), (2048, 256, 512, Q4K, Q6K, 4),
+                                                (256, 64, 256, Q4K, Q6K, 0), (256, 64, 256, Q6K, Q4K, 4),
+                                                (1024, 64, 1024, Q6K, Q4K, 0), (2048, 64, 2048, Q6K, Q4K, 0),
+                                                (512, 64, 256, Q4K, Q4K, 4)])
+def test_moe_experts_entry_equals_block(orn, ctx, H, E, I, gk, dk, iters):
+    """ornith_moe_experts (the expert ids given: the launch bench.py times) gives the bits of
+    ornith_moe_block, which makes the routing itself, and of the oracle."""
+    rng = np.random.default_rng(H + E + I + gk + iters)
+    moe = util.HostMoe(rng, H=H, E=E, I=I, top_k=8, gate_kind=gk, down_kind=dk, router_kind=gk)
+    dw = moe.dev(orn, ctx)
+    k = moe.top_k
+    try:
+        orn.set_option("moe_up_iters", iters)
+        for T in (1, 2, 3, 4):
+            xb = util.bf16_normal(rng, (T, H))
+            want_out, want_inds, want_sc = _block(orn, ctx, moe, dw, xb, T)
+            dx = ctx.to_device(xb)
+            di, ds, de = ctx.to_device(want_inds), ctx.to_device(want_sc), ctx.alloc(T * 2)
+            ctx.linear_matmul(moe._dev[7], dx, T, de)  # the shared expert's scalar gate
+            act, out = ctx.alloc((T * k + T) * I * 2), ctx.alloc(T * H * 2)
+            orn.moe_experts(ctx, dw, dx, T, di, ds, de, act, out, 1)
+            orn.moe_experts(ctx, dw, dx, T, di, ds, de, act, out, 2)
+            assert np.array_equal(out.download(np.uint16, (T, H)), want_out), T
+            if T <= 2:
+                assert np.array_equal(want_out, util.orc_moe_block(moe, xb, T)[0])
+            for b in (dx, di, ds, de, act, out): b.free()
+    finally:
+        orn.set_option("moe_up_iters", 0)
+        moe.free()
+
+
 def test_multi_matrix_launch_equals_separate(orn, ctx):
     rng = np.random.default_rng(5)
     for kind, K in ((Q4K, 2048), (Q6K, 2048), (Q4K, 512), (Q4K, 4096)):
