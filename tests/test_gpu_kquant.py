@@ -138,7 +138,9 @@ def test_config1_q4k_gemv_512x2048(orn, ctx):
     w.free()
 
 
-@pytest.mark.parametrize("kind,K,O", [(Q4K, 2048, 512), (Q6K, 512, 2048), (Q6K, 2048, 64), (Q4K, 512, 128)])
+@pytest.mark.parametrize("kind,K,O", [(Q4K, 2048, 512), (Q6K, 512, 2048), (Q6K, 2048, 64), (Q4K, 512, 128),
+                                       (Q4K, 256, 64), (Q6K, 256, 64), (Q4K, 1024, 96), (Q6K, 1024, 96),
+                                       (Q4K, 4096, 64), (Q6K, 4096, 64)])
 def test_gather_qmv_bit_exact(orn, ctx, kind, K, O):
     rng = np.random.default_rng(300 + kind + K)
     E = 16
@@ -161,7 +163,13 @@ def test_gather_qmv_bit_exact(orn, ctx, kind, K, O):
         dx1 = ctx.to_device(xb[lhs[3]])
         ctx.kq_qmv(we, dx1, orn.BF16, 1, dy1, orn.BF16)
         assert np.array_equal(dy1.download(np.uint16, (O,)), got[3])
-        for b in (dx, dl, dr, dy, dy1, dx1): b.free()
+        # fp32 activations and fp32 outputs through the same gather
+        xf = util.bf16_to_f32(xb)
+        dxf, dyf = ctx.to_device(xf), ctx.alloc(rows * O * 4)
+        ctx.kq_gather_qmv(w, dxf, orn.F32, T, dl, dr, rows, dyf, orn.F32)
+        want32 = util.orc_gather_qmv(kind, *t, E, O, K, xf, lhs, rhs, round_bf16=False)
+        assert np.array_equal(dyf.download(np.float32, (rows, O)).view(np.uint32), want32.view(np.uint32)), T
+        for b in (dx, dl, dr, dy, dy1, dx1, dxf, dyf): b.free()
         we.free()
     w.free()
 
