@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 
 def test_norms_bit_exact(orn, ctx):
     rng = np.random.default_rng(0)
-    for n in (64, 128, 256, 512, 2048, 4096):
+    for n in (64, 128, 256, 512, 1024, 2048, 4096):
         rows = 5
         x = util.bf16_normal(rng, (rows, n), 3.0); b = util.bf16_normal(rng, (rows, n)); w = util.bf16_normal(rng, (n,))
         z = util.bf16_normal(rng, (rows, n), 2.0)

@@ -57,7 +57,7 @@ def test_embedding_and_dense_gather_bit_exact(orn, ctx):
     d.free()
 
 
-@pytest.mark.parametrize("E", [64, 256, 1024])
+@pytest.mark.parametrize("E", [64, 128, 256, 512, 1024])
 def test_router_softmax_topk_bit_exact_with_ties(orn, ctx, E):
     rng = np.random.default_rng(2 + E)
     T, k = 6, 8
