@@ -47,7 +47,7 @@ def test_moe_fused_equals_unfused_and_oracle(orn, ctx, H, E, I, gk, dk):
 @pytest.mark.parametrize("H,E,I,gk,dk,iters", [(2048, 256, 512, Q4K, Q6K, 0), (2048, 256, 512, Q4K, Q6K, 4),
                                                 (256, 64, 256, Q4K, Q6K, 0), (256, 64, 256, Q6K, Q4K, 4),
                                                 (1024, 64, 1024, Q6K, Q4K, 0), (2048, 64, 2048, Q6K, Q4K, 0),
-                                                (512, 64, 256, Q4K, Q4K, 4)])
+                                                (512, 64, 256, Q4K, Q4K, 4), (4096, 64, 256, Q6K, Q4K, 0)])
 def test_moe_experts_entry_equals_block(orn, ctx, H, E, I, gk, dk, iters):
     """ornith_moe_experts (the expert ids given: the launch bench.py times) gives the bits of
     ornith_moe_block, which makes the routing itself, and of the oracle."""
