@@ -90,20 +90,36 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
   {
     KqSeg all[kMaxSeg];
     int nseg = a.nseg;
+    static_assert(kMaxSeg == 4, "the one statement below names every field");
+    // pins the values (not their addresses) in scalar registers in ONE statement, so that all
+    // the argument loads are issued together and waited for once (a statement per segment
+    // made the compiler wait for each segment's loads before issuing the next's)
+    uint64_t q[kMaxSeg], sc[kMaxSeg], d[kMaxSeg], y[kMaxSeg];
+    int so[kMaxSeg], fb[kMaxSeg];
+#pragma unroll
+    for (int i = 0; i < kMaxSeg; ++i) {
+      q[i] = (uint64_t)a.seg[i].qs;
+      sc[i] = (uint64_t)a.seg[i].scales;
+      d[i] = (uint64_t)a.seg[i].dm;
+      y[i] = (uint64_t)a.seg[i].y;
+      so[i] = a.seg[i].O;
+      fb[i] = a.seg[i].first_block;
+    }
+    asm volatile(""
+                 : "+s"(q[0]), "+s"(sc[0]), "+s"(d[0]), "+s"(y[0]), "+s"(so[0]), "+s"(fb[0]), "+s"(q[1]), "+s"(sc[1]),
+                   "+s"(d[1]), "+s"(y[1]), "+s"(so[1]), "+s"(fb[1]), "+s"(q[2]), "+s"(sc[2]), "+s"(d[2]), "+s"(y[2]),
+                   "+s"(so[2]), "+s"(fb[2]), "+s"(q[3]), "+s"(sc[3]), "+s"(d[3]), "+s"(y[3]), "+s"(so[3]), "+s"(fb[3]),
+                   "+s"(nseg), "+s"(a.K), "+s"(a.iters), "+s"(a.y_bf16));
 #pragma unroll
     for (int i = 0; i < kMaxSeg; ++i) {
       all[i] = a.seg[i];
-      // pins the values (not their addresses) in scalar registers here, so that all the
-      // argument loads above are issued together and waited for once
-      uint64_t q = (uint64_t)all[i].qs, sc = (uint64_t)all[i].scales, d = (uint64_t)all[i].dm,
-               y = (uint64_t)all[i].y;
-      asm volatile("" : "+s"(q), "+s"(sc), "+s"(d), "+s"(y), "+s"(all[i].O), "+s"(all[i].first_block));
-      all[i].qs = dm_global_ptr<const uint8_t>(q);
-      all[i].scales = dm_global_ptr<const uint8_t>(sc);
-      all[i].dm = dm_global_ptr<const uint16_t>(d);
-      all[i].y = dm_global_ptr<void>(y);
+      all[i].qs = dm_global_ptr<const uint8_t>(q[i]);
+      all[i].scales = dm_global_ptr<const uint8_t>(sc[i]);
+      all[i].dm = dm_global_ptr<const uint16_t>(d[i]);
+      all[i].y = dm_global_ptr<void>(y[i]);
+      all[i].O = so[i];
+      all[i].first_block = fb[i];
     }
-    asm volatile("" : "+s"(nseg));
     sg = all[0];
 #pragma unroll
     for (int i = 1; i < kMaxSeg; ++i)
