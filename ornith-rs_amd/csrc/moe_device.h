@@ -15,16 +15,17 @@ __device__ __forceinline__ uint32_t dm_xor_lane_u32(uint32_t v) {
   return __builtin_bit_cast(uint32_t, dm_xor_lane<S>(__builtin_bit_cast(float, v)));
 }
 __device__ __forceinline__ uint32_t dm_wave_max_u32(uint32_t v) {
-  uint32_t o;
   float a, b;
   dm_row_swap<32>(__builtin_bit_cast(float, v), a, b);
   v = max(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b));
   dm_row_swap<16>(__builtin_bit_cast(float, v), a, b);
   v = max(__builtin_bit_cast(uint32_t, a), __builtin_bit_cast(uint32_t, b));
-  o = dm_xor_lane_u32<8>(v); v = o > v ? o : v;
-  o = dm_xor_lane_u32<4>(v); v = o > v ? o : v;
-  o = dm_xor_lane_u32<2>(v); v = o > v ? o : v;
-  o = dm_xor_lane_u32<1>(v); v = o > v ? o : v;
+  // max() with a DPP operand is one instruction a step; after the step over 8 the value
+  // repeats every 8 lanes, so a rotate by 4 stands for the exchange with lane l ^ 4
+  v = max(v, dm_xor_lane_u32<8>(v));
+  v = max(v, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x124, 0xF, 0xF, false));
+  v = max(v, dm_xor_lane_u32<2>(v));
+  v = max(v, dm_xor_lane_u32<1>(v));
   return v;
 }
 
