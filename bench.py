@@ -242,6 +242,27 @@ def main():
     total_s = sum(times)
     tok_s = args.tokens * len(times) / total_s
 
+    # Forced acceptance: random-init weights accept no draft, so `value` is the floor of the
+    # loop. With the known output as the drafts every draft is accepted and a cycle yields
+    # depth + 1 tokens: the ceiling. The head still runs for every draft.
+    forced = {}
+    c2 = model.make_cache(cap, 4)
+    head.force_drafts(ar)
+    for d in (1, 2, 3):
+        for it in range(2):   # the first run warms the shapes of this depth
+            c2.reset()
+            (ft, fst), fdt = timed_run(lambda pr: orn.generate_step_mtp(
+                model, head, fr, c2, prompt, d, args.tokens, prefill_step=16,
+                policy=orn.HISTORY_COMMITTED, progress=pr))
+            if ft != ar:
+                sys.exit("bench.py: forced-draft output is NOT identical to plain greedy -- result invalid")
+        forced[f"depth{d}"] = {"tok_s": round(args.tokens / fdt, 1), "cycles": int(fst.cycles),
+                               "accepted": int(fst.accepted), "drafted": int(fst.drafted)}
+        log(f"forced acceptance depth {d}: {args.tokens / fdt:.1f} tok/s, {int(fst.cycles)} cycles, "
+            f"{int(fst.accepted)}/{int(fst.drafted)} accepted")
+    head.force_drafts([])
+    c2.close()
+
     roof = expert_gemv_roofline(orn, ctx, model, util, np, args.layers, T=args.depth + 1)
     log("roofline:", roof)
 
@@ -267,6 +288,7 @@ def main():
                    "tokens_per_step": args.tokens, "byte_identical_to_greedy": True,
                    "plain_greedy_tok_s": round(len(ar) / ar_s, 2),
                    "cycles": int(stats.cycles), "accepted": int(stats.accepted), "drafted": int(stats.drafted),
+                   "forced_acceptance_ceiling": forced,
                    "weights_GB": round(ws.stats()[1] / 1e9, 2), "device": dev_name},
         "roofline": roof,
         "cpu_baseline": cpu,

@@ -505,6 +505,13 @@ ORNITH_API int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspe
                                   void* d_hidden_out, void* d_logits);
 ORNITH_API int ornith_mtp_cache_set_offset(ornith_mtp_head* h, int offset);
 ORNITH_API int ornith_mtp_cache_offset(const ornith_mtp_head* h, int* offset_out);
+/* Measurement aid, no counterpart in the reference: a host list g[0..n) of the tokens a run
+ * is known to produce (g[0] = the first token after the prompt, e.g. the plain greedy output).
+ * While set, ornith_mtp_generate still runs the head for every draft but then replaces the
+ * draft for output position p with g[p], so every draft inside the list is accepted and a
+ * cycle yields depth + 1 tokens: the throughput ceiling of the loop at that depth. n = 0
+ * clears the list. Positions past the list keep the head's own drafts. */
+ORNITH_API int ornith_mtp_force_drafts(ornith_mtp_head* h, const uint32_t* tokens, size_t n);
 
 /* ---- the sampled-token path: TopSampler (src/sample.rs:79-225) -------------------------
  * bf16 throughout except the CDF, as in the reference. Cumulative sums associate in

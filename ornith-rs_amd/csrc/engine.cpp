@@ -209,6 +209,9 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
       } else {
         TRY(ornith_argmax_rows(ctx, d_dlogits, 1, draft_vocab, d_window + i + 1));
       }
+      // a forced draft (measurement aid) takes the place of the head's own
+      const size_t pos = emitted + 1 + (size_t)i;
+      if (pos < head->n_forced) TRY(ornith_copy(ctx, d_window + i + 1, head->d_forced + pos, 4));
       hcur = hid;
     }
     if (want > 0) {

@@ -625,7 +625,29 @@ int ornith_mtp_destroy(ornith_mtp_head* h) {
   ornith_free(h->m->ctx, h->k);
   ornith_free(h->m->ctx, h->v);
   ornith_free(h->m->ctx, h->buf);
+  ornith_free(h->m->ctx, h->d_forced);
   delete h;
+  return ORNITH_OK;
+}
+
+int ornith_mtp_force_drafts(ornith_mtp_head* h, const uint32_t* tokens, size_t n) {
+  ORN_REQUIRE(h && (tokens || n == 0), "mtp_force_drafts: null argument");
+  ornith_ctx* ctx = h->m->ctx;
+  // a generation that still reads the old list has been queued at most; let it finish
+  TRY(ornith_sync(ctx));
+  ornith_free(ctx, h->d_forced);
+  h->d_forced = nullptr;
+  h->n_forced = 0;
+  if (n == 0) return ORNITH_OK;
+  void* d = nullptr;
+  TRY(ornith_alloc(ctx, n * 4, &d));
+  const int rc = ornith_upload(ctx, d, tokens, n * 4);
+  if (rc) {
+    ornith_free(ctx, d);
+    return rc;
+  }
+  h->d_forced = (uint32_t*)d;
+  h->n_forced = n;
   return ORNITH_OK;
 }
 

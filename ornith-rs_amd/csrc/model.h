@@ -151,6 +151,9 @@ struct ornith_mtp_head {
   int capacity = 0, offset = 0;
   void* buf = nullptr;  // step buffers
   int max_rows = 0;
+  // tokens that replace the drafts (ornith_mtp_force_drafts), indexed by output position
+  uint32_t* d_forced = nullptr;
+  size_t n_forced = 0;
 };
 
 // grows the model's RoPE tables to cover `npos` positions

@@ -343,6 +343,14 @@ class MtpHead:
     def set_offset(self, off):
         _check(lib().ornith_mtp_cache_set_offset(self.h, off), "mtp_cache_set_offset")
 
+    def force_drafts(self, tokens):
+        """Measurement aid (not in the reference): the drafts of generate_step_mtp are replaced
+        by tokens[p] for output position p, so every one is accepted when `tokens` is the
+        run's own output. An empty list clears it."""
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        _check(lib().ornith_mtp_force_drafts(self.h, _ptr(t) if len(t) else None, C.c_size_t(len(t))),
+               "mtp_force_drafts")
+
     @property
     def offset(self):
         o = C.c_int()

@@ -179,6 +179,47 @@ def test_generation_loops_small_vocab_exercise_acceptance(orn, ctx, tiny_small_v
     assert acc > 0, "no draft was ever accepted: the acceptance path went untested"
 
 
+def test_forced_drafts_accept_everything(orn, ctx, tiny):
+    """The measurement aid: with the run's own output as the forced drafts every draft is
+    accepted (depth + 1 tokens a cycle), the output stays the greedy one under both history
+    policies, a short list forces only the positions it covers, and clearing it brings the
+    head's own drafts back."""
+    s, ws, model = tiny
+    rng = np.random.default_rng(9)
+    prompt = rng.integers(0, s.cfg["vocab_size"], 9).astype(np.uint32)
+    n = 25
+    cap = 9 + n + 8
+    caches = model.make_cache(cap, 4)
+    ar = orn.generate_step(model, caches, prompt, n, prefill_step=4)
+    head = orn.MtpHead(model, ws, cap)
+    caches.reset()
+    base, base_st = orn.generate_step_mtp(model, head, None, caches, prompt, 2, n, prefill_step=4)
+    assert base == ar
+    head.force_drafts(ar)
+    for depth in (1, 2, 3):
+        for policy in (orn.HISTORY_CYCLE, orn.HISTORY_COMMITTED):
+            caches.reset()
+            toks, st = orn.generate_step_mtp(model, head, None, caches, prompt, depth, n, prefill_step=4,
+                                             policy=policy)
+            assert toks == ar and caches.offset == 9 + n
+            assert st.accepted == st.drafted, (depth, policy, st.accepted, st.drafted)
+            emitted = cycles = drafted = 0
+            while emitted < n:   # every cycle yields its drafts and one more token
+                want = min(depth, n - (emitted + 1))
+                cycles, drafted, emitted = cycles + (want > 0), drafted + want, emitted + want + 1
+            assert (st.cycles, st.drafted) == (cycles, drafted)
+    # a list that ends early: positions past it fall back to the head
+    head.force_drafts(ar[:7])
+    caches.reset()
+    toks, st = orn.generate_step_mtp(model, head, None, caches, prompt, 2, n, prefill_step=4)
+    assert toks == ar and 4 <= st.accepted < st.drafted
+    head.force_drafts([])
+    caches.reset()
+    toks, st = orn.generate_step_mtp(model, head, None, caches, prompt, 2, n, prefill_step=4)
+    assert toks == ar and (st.cycles, st.drafted, st.accepted) == (base_st.cycles, base_st.drafted, base_st.accepted)
+    head.close(); caches.close()
+
+
 def test_stop_callback_and_errors(orn, ctx, tiny):
     s, ws, model = tiny
     prompt = np.arange(5, dtype=np.uint32)
