@@ -248,6 +248,15 @@ def linear_matmul(self, lin, x, M, y):
 
 
 @_ctx_method
+def linear_matmul_multi(self, lins, x, M, ys):
+    """Several Linear over the same activations (one launch when their formats allow)."""
+    n = len(lins)
+    wp = (C.c_void_p * n)(*[C.cast(C.pointer(l.s), C.c_void_p) for l in lins])
+    yp = (C.c_void_p * n)(*[y.ptr for y in ys])
+    _check(lib().ornith_linear_matmul_multi(self.h, wp, n, x.ptr, M, yp), "linear_matmul_multi")
+
+
+@_ctx_method
 def dense_gather_mv(self, w, E, O, K, x, x_rows, lhs, rhs, rows, y):
     _check(lib().ornith_dense_gather_mv(self.h, w.ptr, E, O, K, x.ptr, x_rows, lhs.ptr, rhs.ptr,
                                         rows, y.ptr), "dense_gather_mv")

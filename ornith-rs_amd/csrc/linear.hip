@@ -56,23 +56,34 @@ __global__ __launch_bounds__(64) void affine8_qmv_kernel(const uint8_t* w, const
 // ---- dense bf16 ------------------------------------------------------------
 // grid.x covers rows four at a time (one per wavefront), grid.y is the
 // activation row; GATHER selects expert / activation row through lhs, rhs.
-// rows [0, O) of w -> y; with w2 != null rows [O, O + O2) come from w2 and go to y2
-// (two small projections of the same activations in one launch)
+// Up to four matrices over the same activations in one launch: the rows of the
+// segments follow each other along grid.x, each segment with its own output.
+struct DenseSegs {
+  const bf16_t* w[4];
+  bf16_t* y[4];
+  int O[4];
+  int n;
+};
+
 template <bool GATHER>
-__global__ __launch_bounds__(256) void dense_gemv_kernel(const bf16_t* w, const bf16_t* x,
-                                                         bf16_t* y, int O, int K, int E, int x_rows,
-                                                         const uint32_t* lhs, const uint32_t* rhs,
-                                                         const bf16_t* w2 = nullptr,
-                                                         bf16_t* y2 = nullptr, int O2 = 0) {
+__global__ __launch_bounds__(256) void dense_gemv_kernel(DenseSegs s, const bf16_t* x, int K, int E,
+                                                         int x_rows, const uint32_t* lhs,
+                                                         const uint32_t* rhs) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   int o = blockIdx.x * 4 + wave;
-  if (o >= O + O2) return;
-  if (o >= O) {
-    o -= O;
-    w = w2;
-    y = y2;
-    O = O2;
+  const bf16_t* w = s.w[0];
+  bf16_t* y = s.y[0];
+  int O = s.O[0];
+#pragma unroll
+  for (int i = 1; i < 4; ++i) {
+    if (i < s.n && o >= O) {
+      o -= O;
+      w = s.w[i];
+      y = s.y[i];
+      O = s.O[i];
+    }
   }
+  if (o >= O) return;
   const int r = blockIdx.y;
   const bf16_t* wr;
   const bf16_t* xr;
@@ -102,7 +113,38 @@ __global__ void embedding_kernel(const uint8_t* w, const bf16_t* scales, const b
   out[(size_t)r * K + i] = dm_f2bf(v + b);
 }
 
+template <bool GATHER>
+int launch_dense(ornith_ctx* ctx, const DenseSegs& s, const void* d_x, int K, int E, int x_rows,
+                 const uint32_t* d_lhs, const uint32_t* d_rhs, int rows) {
+  int total = 0;
+  for (int i = 0; i < s.n; ++i) total += s.O[i];
+  hipLaunchKernelGGL(dense_gemv_kernel<GATHER>, dim3((total + 3) / 4, rows), dim3(256), 0, ctx->stream, s,
+                     (const bf16_t*)d_x, K, E, x_rows, d_lhs, d_rhs);
+  ORN_LAUNCH_CHECK(GATHER ? "dense_gemv_kernel<gather>" : "dense_gemv_kernel");
+  return ORNITH_OK;
+}
+
 }  // namespace
+
+// Several stacked expert tensors [E, O, K] gathered over the same (activation row, expert)
+// pairs in one launch (the gate and up projections of dense experts).
+extern "C" int dense_gather_mv_multi(ornith_ctx* ctx, const void* const* d_ws, int n, int E, int O, int K,
+                                     const void* d_x, int x_rows, const uint32_t* d_lhs,
+                                     const uint32_t* d_rhs, int rows, void* const* d_ys) {
+  ORN_REQUIRE(ctx && d_ws && d_ys && d_x && d_lhs && d_rhs && n >= 1 && n <= 4, "dense_gather_mv_multi: bad argument");
+  ORN_REQUIRE(E >= 1 && O >= 1 && K % 8 == 0 && x_rows >= 1 && rows >= 0 && rows <= 65535,
+              "dense_gather_mv: E=%d O=%d K=%d rows=%d", E, O, K, rows);
+  if (rows == 0) return ORNITH_OK;
+  DenseSegs s{};
+  s.n = n;
+  for (int i = 0; i < n; ++i) {
+    ORN_REQUIRE(d_ws[i] && d_ys[i], "dense_gather_mv_multi: null entry %d", i);
+    s.w[i] = (const bf16_t*)d_ws[i];
+    s.y[i] = (bf16_t*)d_ys[i];
+    s.O[i] = O;
+  }
+  return launch_dense<true>(ctx, s, d_x, K, E, x_rows, d_lhs, d_rhs, rows);
+}
 
 extern "C" {
 
@@ -130,11 +172,14 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
       ORN_REQUIRE(w->d_w, "linear_matmul: dense weight missing");
       ORN_REQUIRE(w->K % 8 == 0 && w->O >= 1 && M <= 65535, "linear_matmul: dense O=%d K=%d", w->O,
                   w->K);
-      hipLaunchKernelGGL(dense_gemv_kernel<false>, dim3((w->O + 3) / 4, M), dim3(256), 0,
-                         ctx->stream, (const bf16_t*)w->d_w, (const bf16_t*)d_x, (bf16_t*)d_y, w->O,
-                         w->K, 1, M, nullptr, nullptr);
-      ORN_LAUNCH_CHECK("dense_gemv_kernel");
-      return ORNITH_OK;
+      {
+        DenseSegs s{};
+        s.n = 1;
+        s.w[0] = (const bf16_t*)w->d_w;
+        s.y[0] = (bf16_t*)d_y;
+        s.O[0] = w->O;
+        return launch_dense<false>(ctx, s, d_x, w->K, 1, M, nullptr, nullptr, M);
+      }
     default:
       return ornith_fail(ORNITH_ERR_INVALID, "linear_matmul: unknown mode %d", w->mode);
   }
@@ -154,13 +199,16 @@ int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, 
     for (int i = 0; i < n; ++i) kms[i] = &ws[i]->km;
     return ornith_kq_qmv_multi(ctx, kms, n, d_x, ORNITH_BF16, M, d_ys, ORNITH_BF16);
   }
-  if (fuse && ws[0]->mode == ORNITH_LIN_DENSE && n == 2 && ws[0]->K % 8 == 0 && M <= 65535) {
-    hipLaunchKernelGGL(dense_gemv_kernel<false>, dim3((ws[0]->O + ws[1]->O + 3) / 4, M), dim3(256),
-                       0, ctx->stream, (const bf16_t*)ws[0]->d_w, (const bf16_t*)d_x,
-                       (bf16_t*)d_ys[0], ws[0]->O, ws[0]->K, 1, M, nullptr, nullptr,
-                       (const bf16_t*)ws[1]->d_w, (bf16_t*)d_ys[1], ws[1]->O);
-    ORN_LAUNCH_CHECK("dense_gemv_kernel<pair>");
-    return ORNITH_OK;
+  if (fuse && ws[0]->mode == ORNITH_LIN_DENSE && ws[0]->K % 8 == 0 && M <= 65535) {
+    DenseSegs s{};
+    s.n = n;
+    for (int i = 0; i < n; ++i) {
+      ORN_REQUIRE(ws[i]->d_w && ws[i]->O >= 1, "linear_matmul_multi: dense weight %d missing", i);
+      s.w[i] = (const bf16_t*)ws[i]->d_w;
+      s.y[i] = (bf16_t*)d_ys[i];
+      s.O[i] = ws[i]->O;
+    }
+    return launch_dense<false>(ctx, s, d_x, ws[0]->K, 1, M, nullptr, nullptr, M);
   }
   for (int i = 0; i < n; ++i) {
     int rc = ornith_linear_matmul(ctx, ws[i], d_x, M, d_ys[i]);
@@ -196,11 +244,9 @@ int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K
   ORN_REQUIRE(E >= 1 && O >= 1 && K % 8 == 0 && x_rows >= 1 && rows >= 0 && rows <= 65535,
               "dense_gather_mv: E=%d O=%d K=%d rows=%d", E, O, K, rows);
   if (rows == 0) return ORNITH_OK;
-  hipLaunchKernelGGL(dense_gemv_kernel<true>, dim3((O + 3) / 4, rows), dim3(256), 0, ctx->stream,
-                     (const bf16_t*)d_w, (const bf16_t*)d_x, (bf16_t*)d_y, O, K, E, x_rows, d_lhs,
-                     d_rhs);
-  ORN_LAUNCH_CHECK("dense_gemv_kernel<gather>");
-  return ORNITH_OK;
+  const void* ws[1] = {d_w};
+  void* ys[1] = {d_y};
+  return dense_gather_mv_multi(ctx, ws, 1, E, O, K, d_x, x_rows, d_lhs, d_rhs, rows, ys);
 }
 
 int ornith_embedding(ornith_ctx* ctx, const ornith_linear* table, const uint32_t* d_ids, int n,

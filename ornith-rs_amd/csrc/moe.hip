@@ -13,6 +13,10 @@
 #include "norm_device.h"
 #include "rt.h"
 
+// linear.hip
+extern "C" int dense_gather_mv_multi(ornith_ctx* ctx, const void* const* d_ws, int n, int E, int O, int K,
+                                     const void* d_x, int x_rows, const uint32_t* d_lhs,
+                                     const uint32_t* d_rhs, int rows, void* const* d_ys);
 // moe_fused.hip
 bool moe_fused_supported(const ornith_moe_weights* w);
 bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
@@ -310,17 +314,20 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
                              ctx->stream));
     return ORNITH_OK;
   }
-  TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
-  TRY(ornith_linear_matmul(ctx, &w->sh_gate, d_x, T, sg));
-  TRY(ornith_linear_matmul(ctx, &w->sh_up, d_x, T, su));
-  TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
+  {
+    // the four projections of the block's input: one launch when their formats allow
+    const ornith_linear* in4[4] = {&w->router, &w->sh_gate, &w->sh_up, &w->sh_egate};
+    void* out4[4] = {gates, sg, su, eg};
+    TRY(ornith_linear_matmul_multi(ctx, in4, 4, d_x, T, out4));
+  }
   TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, lhs_tok, lhs_row));
   TRY(ornith_swiglu(ctx, sg, su, (int64_t)T * SI, sact));
   TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
   if (w->ex_dense) {
     ORN_REQUIRE(w->d_ex_gate && w->d_ex_up && w->d_ex_down, "moe_block: dense expert tensor missing");
-    TRY(ornith_dense_gather_mv(ctx, w->d_ex_gate, E, I, H, d_x, T, lhs_tok, inds, T * k, xg));
-    TRY(ornith_dense_gather_mv(ctx, w->d_ex_up, E, I, H, d_x, T, lhs_tok, inds, T * k, xu));
+    const void* gu[2] = {w->d_ex_gate, w->d_ex_up};
+    void* xgu[2] = {xg, xu};
+    TRY(dense_gather_mv_multi(ctx, gu, 2, E, I, H, d_x, T, lhs_tok, inds, T * k, xgu));
     TRY(ornith_swiglu(ctx, xg, xu, (int64_t)T * k * I, act));
     TRY(ornith_dense_gather_mv(ctx, w->d_ex_down, E, H, I, act, T * k, lhs_row, inds, T * k, y));
   } else {

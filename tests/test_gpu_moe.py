@@ -34,6 +34,29 @@ def test_linear_modes_bit_exact(orn, ctx):
         d.free()
 
 
+@pytest.mark.parametrize("sizes", [(33, 5), (33, 5, 1), (7, 64, 1, 130), (1, 1, 1, 1)])
+def test_dense_multi_equals_single_launches(orn, ctx, sizes):
+    """Dense projections of the same activations in one launch: every output row is the
+    oracle's (and so the single launch's), whatever the row counts of the segments."""
+    rng = np.random.default_rng(len(sizes))
+    K, M = 2048, 3
+    lins = [util.HostLinear.dense(rng, O, K) for O in sizes]
+    xb = util.f32_to_bf16(rng.standard_normal((M, K)).astype(np.float32))
+    devs = [l.dev(orn, ctx) for l in lins]
+    dx = ctx.to_device(xb)
+    # canaries after each output: a segment must not write past its own rows
+    ys = [ctx.to_device(np.full(M * l.O + 8, 0xabcd, np.uint16)) for l in lins]
+    ctx.linear_matmul_multi(devs, dx, M, ys)
+    for l, y in zip(lins, ys):
+        want = np.empty((M, l.O), np.uint16)
+        oracle().orc_dense_gemv(p(l.w), l.O, l.K, p(xb), M, p(want))
+        got = y.download(np.uint16, (M * l.O + 8,))
+        assert np.array_equal(got[:M * l.O].reshape(M, l.O), want), sizes
+        assert (got[M * l.O:] == 0xabcd).all()
+    for b in ys + [dx]: b.free()
+    for d in devs: d.free()
+
+
 def test_embedding_and_dense_gather_bit_exact(orn, ctx):
     rng = np.random.default_rng(1)
     tab = util.HostLinear.affine8(rng, 300, 2048)
