@@ -110,23 +110,23 @@ int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, s
   TRY(prefill(m, c, prompt, n_prompt, prefill_step, d_tok, d_hidden, progress, user, &processed));
   // step(): run the n tokens in d_tok and sample from the last position; the one wait of the
   // step is the read-back of the sampled id
-  auto step = [&](size_t n, uint32_t* y) -> int {
-    TRY(ornith_model_forward(m, c, d_tok, (int)n, 0, d_hidden));
+  auto step = [&](const uint32_t* d_in, size_t n, uint32_t* y) -> int {
+    TRY(ornith_model_forward(m, c, d_in, (int)n, 0, d_hidden));
     TRY(ornith_model_logits(m, (char*)d_hidden + (n - 1) * H * 2, 1, d_logits));
     TRY(smp.sample(d_logits, d_out));
     return ornith_download(ctx, y, d_out, 4);
   };
   uint32_t y = 0;
   TRY(ornith_upload(ctx, d_tok, prompt + processed, (n_prompt - processed) * 4));
-  TRY(step(n_prompt - processed, &y));
+  TRY(step(d_tok, n_prompt - processed, &y));
   if (progress) progress(n_prompt, n_prompt, user);
   size_t n = 0;
   for (;;) {
     if (n == max_tokens) return ORNITH_OK;
     uint32_t next = 0;
-    // the token just sampled is fed back from where it lies on the device
-    TRY(ornith_copy(ctx, d_tok, d_out, 4));
-    TRY(step(1, &next));
+    // the token just sampled is fed back from where it lies on the device: the forward
+    // reads it in its first launch, the sampler overwrites it in the step's last
+    TRY(step(d_out, 1, &next));
     if (!on_token(y, user)) return ORNITH_OK;
     y = next;
     ++n;
@@ -156,14 +156,13 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
 
   Bufs b(ctx);
   uint32_t *d_tok, *d_window, *d_targets, *d_local;
-  void *d_hidden, *d_h, *d_vlogits, *d_dlogits, *d_mh, *d_scratch_h;
+  void *d_hidden, *d_vlogits, *d_dlogits, *d_mh, *d_scratch_h;
   const size_t W = (size_t)depth + 1;
   TRY(b.get(R * 4, (void**)&d_tok));
   TRY(b.get(2 * W * 4, (void**)&d_window));  // window, then the targets: one read-back a cycle
   d_targets = d_window + W;
   TRY(b.get(4, (void**)&d_local));
   TRY(b.get(R * H * 2, &d_hidden));
-  TRY(b.get(H * 2, &d_h));
   TRY(b.get(W * V * 2, &d_vlogits));
   TRY(b.get(V * 2, &d_dlogits));
   TRY(b.get(W * H * 2, &d_mh));
@@ -179,7 +178,9 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   TRY(smp.sample(d_vlogits, d_targets));
   uint32_t primary = 0;
   TRY(ornith_download(ctx, &primary, d_targets, 4));
-  TRY(ornith_copy(ctx, d_h, (char*)d_hidden + (rows - 1) * H * 2, H * 2));
+  // the trunk hidden a cycle drafts from is read where the last forward left it: the next
+  // write to d_hidden is the cycle's verify pass, after the drafts
+  const void* d_h = (char*)d_hidden + (rows - 1) * H * 2;
 
   size_t emitted = 0;
   TRY(ornith_mtp_cache_set_offset(head, 0));  // make_mtp_cache()
@@ -267,7 +268,7 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
       TRY(ornith_mtp_cache_set_offset(head, std::min(cycle_mtp_offset + 1, head->capacity)));
       if (k > 0) TRY(ornith_mtp_forward(head, nullptr, d_hidden, d_window + 1, k, d_scratch_h, nullptr));
     }
-    TRY(ornith_copy(ctx, d_h, (char*)d_hidden + (size_t)k * H * 2, H * 2));
+    d_h = (char*)d_hidden + (size_t)k * H * 2;
     // next cycle's primary token: row k's target (the correction or the bonus token)
     TRY(ornith_copy(ctx, d_window, d_targets + k, 4));
 

@@ -250,8 +250,7 @@ static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_to
     TRY(ornith_add_rms_moe_block(ctx, &L.moe, s.x, s.r, L.post_ln, c.rms_norm_eps, T, s.h, s.normed2, s.mo));
   }
   // the last layer's closing add and the model's final norm
-  TRY(ornith_add_rms_norm(ctx, s.h, s.mo, m->final_norm, T, H, c.rms_norm_eps, s.x, s.normed));
-  TRY(ornith_copy(ctx, d_hidden_out, s.normed, (size_t)T * H * 2));
+  TRY(ornith_add_rms_norm(ctx, s.h, s.mo, m->final_norm, T, H, c.rms_norm_eps, s.x, d_hidden_out));
   // every layer advanced together
   cc->conv_cur = 1 - cc->conv_cur;
   cc->conv_off = T;
