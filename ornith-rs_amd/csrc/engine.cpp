@@ -17,13 +17,12 @@
     if (rc__) return rc__; \
   } while (0)
 
-namespace {
+// sample.hip: argmax over a pruned head's rows stored as vocabulary ids (FrSpec::map_id,
+// src/frspec.rs:140-142, inside the argmax's last launch)
+int argmax_rows_mapped(ornith_ctx* ctx, const void* d_logits, int rows, int V, const uint32_t* d_id_map,
+                       uint32_t* d_out);
 
-// FrSpec::map_id (src/frspec.rs:140-142): dst = ids[local], one thread
-__global__ void map_id_kernel(const uint32_t* ids, int n, const uint32_t* local, uint32_t* dst) {
-  const uint32_t l = *local;
-  *dst = ids[l < (uint32_t)n ? l : (uint32_t)(n - 1)];
-}
+namespace {
 
 // device buffers a generation call needs, freed on scope exit
 struct Bufs {
@@ -155,13 +154,12 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   ornith_mtp_stats stats{};
 
   Bufs b(ctx);
-  uint32_t *d_tok, *d_window, *d_targets, *d_local;
+  uint32_t *d_tok, *d_window, *d_targets;
   void *d_hidden, *d_vlogits, *d_dlogits, *d_mh, *d_scratch_h;
   const size_t W = (size_t)depth + 1;
   TRY(b.get(R * 4, (void**)&d_tok));
   TRY(b.get(2 * W * 4, (void**)&d_window));  // window, then the targets: one read-back a cycle
   d_targets = d_window + W;
-  TRY(b.get(4, (void**)&d_local));
   TRY(b.get(R * H * 2, &d_hidden));
   TRY(b.get(W * V * 2, &d_vlogits));
   TRY(b.get(V * 2, &d_dlogits));
@@ -203,10 +201,8 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
       void* hid = (char*)d_mh + (size_t)i * H * 2;
       TRY(ornith_mtp_forward(head, frspec, hcur, d_window + i, 1, hid, d_dlogits));
       if (frspec) {
-        TRY(ornith_argmax_rows(ctx, d_dlogits, 1, draft_vocab, d_local));
-        hipLaunchKernelGGL(map_id_kernel, dim3(1), dim3(1), 0, ctx->stream, frspec->d_ids, frspec->n,
-                           d_local, d_window + i + 1);
-        ORN_LAUNCH_CHECK("map_id_kernel");
+        // FrSpec::map_id rides in the argmax's last launch
+        TRY(argmax_rows_mapped(ctx, d_dlogits, 1, draft_vocab, frspec->d_ids, d_window + i + 1));
       } else {
         TRY(ornith_argmax_rows(ctx, d_dlogits, 1, draft_vocab, d_window + i + 1));
       }

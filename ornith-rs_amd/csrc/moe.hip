@@ -66,10 +66,19 @@ __device__ __forceinline__ void bf_put(typename BfPack<V>::type& p, int i, float
 }
 
 template <int V>
-__global__ void swiglu_kernel(const bf16_t* gate, const bf16_t* up, bf16_t* out, int64_t n) {
+__global__ void swiglu_kernel(const bf16_t* gate, const bf16_t* up, bf16_t* out, int64_t n,
+                              const bf16_t* gate2 = nullptr, const bf16_t* up2 = nullptr,
+                              bf16_t* out2 = nullptr, int64_t n2 = 0) {
   typedef typename BfPack<V>::type P;
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n / V) return;
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // a second, independent range follows the first (two activations in one launch)
+  if (i >= n / V) {
+    i -= n / V;
+    if (i >= n2 / V) return;
+    gate = gate2;
+    up = up2;
+    out = out2;
+  }
   const P g8 = reinterpret_cast<const P*>(gate)[i], u8 = reinterpret_cast<const P*>(up)[i];
   P o8;
 #pragma unroll
@@ -213,6 +222,28 @@ int ornith_swiglu(ornith_ctx* ctx, const void* d_gate, const void* d_up, int64_t
   return ORNITH_OK;
 }
 
+}  // extern "C"
+
+// swiglu over two independent ranges in one launch
+static int swiglu_pair(ornith_ctx* ctx, const void* g1, const void* u1, int64_t n1, void* o1, const void* g2,
+                       const void* u2, int64_t n2, void* o2) {
+  ORN_REQUIRE(g1 && u1 && o1 && g2 && u2 && o2 && n1 >= 0 && n2 >= 0, "swiglu_pair: bad argument");
+  if (n1 + n2 == 0) return ORNITH_OK;
+  const uintptr_t bits = (uintptr_t)g1 | (uintptr_t)u1 | (uintptr_t)o1 | (uintptr_t)g2 | (uintptr_t)u2 | (uintptr_t)o2;
+  if (n1 % 8 == 0 && n2 % 8 == 0 && (bits & 15) == 0)
+    hipLaunchKernelGGL(swiglu_kernel<8>, dim3((unsigned)(((n1 + n2) / 8 + 255) / 256)), dim3(256), 0, ctx->stream,
+                       (const bf16_t*)g1, (const bf16_t*)u1, (bf16_t*)o1, n1, (const bf16_t*)g2,
+                       (const bf16_t*)u2, (bf16_t*)o2, n2);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<1>, dim3((unsigned)((n1 + n2 + 255) / 256)), dim3(256), 0, ctx->stream,
+                       (const bf16_t*)g1, (const bf16_t*)u1, (bf16_t*)o1, n1, (const bf16_t*)g2,
+                       (const bf16_t*)u2, (bf16_t*)o2, n2);
+  ORN_LAUNCH_CHECK("swiglu_kernel<pair>");
+  return ORNITH_OK;
+}
+
+extern "C" {
+
 int ornith_moe_combine(ornith_ctx* ctx, const void* d_scores, const void* d_y, const void* d_gate,
                        const void* d_shared, int T, int k, int dim, int normalize, void* d_out) {
   ORN_REQUIRE(ctx && d_scores && d_y && d_gate && d_shared && d_out, "moe_combine: null argument");
@@ -321,21 +352,22 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
     TRY(ornith_linear_matmul_multi(ctx, in4, 4, d_x, T, out4));
   }
   TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, lhs_tok, lhs_row));
-  TRY(ornith_swiglu(ctx, sg, su, (int64_t)T * SI, sact));
-  TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
   if (w->ex_dense) {
     ORN_REQUIRE(w->d_ex_gate && w->d_ex_up && w->d_ex_down, "moe_block: dense expert tensor missing");
     const void* gu[2] = {w->d_ex_gate, w->d_ex_up};
     void* xgu[2] = {xg, xu};
     TRY(dense_gather_mv_multi(ctx, gu, 2, E, I, H, d_x, T, lhs_tok, inds, T * k, xgu));
-    TRY(ornith_swiglu(ctx, xg, xu, (int64_t)T * k * I, act));
+    // the shared expert's activation and the routed experts' in one launch
+    TRY(swiglu_pair(ctx, sg, su, (int64_t)T * SI, sact, xg, xu, (int64_t)T * k * I, act));
+    TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
     TRY(ornith_dense_gather_mv(ctx, w->d_ex_down, E, H, I, act, T * k, lhs_row, inds, T * k, y));
   } else {
     TRY(ornith_kq_gather_qmv(ctx, &w->ex_gate, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xg,
                              ORNITH_BF16));
     TRY(ornith_kq_gather_qmv(ctx, &w->ex_up, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xu,
                              ORNITH_BF16));
-    TRY(ornith_swiglu(ctx, xg, xu, (int64_t)T * k * I, act));
+    TRY(swiglu_pair(ctx, sg, su, (int64_t)T * SI, sact, xg, xu, (int64_t)T * k * I, act));
+    TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
     TRY(ornith_kq_gather_qmv(ctx, &w->ex_down, act, ORNITH_BF16, T * k, lhs_row, inds, T * k, y,
                              ORNITH_BF16));
   }

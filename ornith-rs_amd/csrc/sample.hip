@@ -125,8 +125,10 @@ __global__ __launch_bounds__(CH) void argmax_chunk_kernel(const bf16_t* logits, 
 }
 
 // pass 3: one wavefront per row over the chunk winners
+// With id_map the winner is stored as id_map[winner]: a pruned head's row number turned into
+// the vocabulary id (FrSpec::map_id, /root/reference/src/frspec.rs:134-142) without a launch.
 __global__ __launch_bounds__(64) void argmax_final_kernel(const float* bv, const int* bi, int nch,
-                                                          int V, uint32_t* out) {
+                                                          int V, uint32_t* out, const uint32_t* id_map) {
   const int r = blockIdx.x, lane = threadIdx.x;
   float v = -DM_INF;
   int idx = 0x7fffffff;
@@ -137,11 +139,14 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* bv, const
     const int oi = __shfl_xor(idx, s, 64);
     best_merge(v, idx, ov, oi);
   }
-  if (lane == 0) out[r] = (idx >= 0 && idx < V) ? (uint32_t)idx : 0u;
+  if (lane == 0) {
+    const uint32_t t = (idx >= 0 && idx < V) ? (uint32_t)idx : 0u;
+    out[r] = id_map ? id_map[t] : t;
+  }
 }
 
 int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens, void* d_lse,
-        bool use_lse, const char* who, ScratchCursor* ws = nullptr) {
+        bool use_lse, const char* who, ScratchCursor* ws = nullptr, const uint32_t* d_id_map = nullptr) {
   ORN_REQUIRE(ctx && d_logits && d_tokens, "%s: null argument", who);
   ORN_REQUIRE(rows >= 1 && rows <= 65535 && V >= 1, "%s: rows=%d V=%d", who, rows, V);
   const int nch = (V + CH - 1) / CH;
@@ -168,7 +173,7 @@ int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_toke
   }
   ORN_LAUNCH_CHECK("argmax_chunk_kernel");
   hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, ctx->stream, bv, bi, nch, V,
-                     d_tokens);
+                     d_tokens, d_id_map);
   ORN_LAUNCH_CHECK("argmax_final_kernel");
   return ORNITH_OK;
 }
@@ -178,6 +183,13 @@ int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_toke
 int ornith_greedy_rows_ws(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens,
                           void* d_lse, ScratchCursor& sc) {
   return run(ctx, d_logits, rows, V, d_tokens, d_lse, true, "greedy_rows", &sc);
+}
+
+// argmax over the V rows of a pruned head, stored as vocabulary ids: d_id_map holds V entries
+int argmax_rows_mapped(ornith_ctx* ctx, const void* d_logits, int rows, int V, const uint32_t* d_id_map,
+                       uint32_t* d_out) {
+  ORN_REQUIRE(d_id_map, "argmax_rows_mapped: null id map");
+  return run(ctx, d_logits, rows, V, d_out, nullptr, false, "argmax_rows", nullptr, d_id_map);
 }
 
 extern "C" {
