@@ -342,6 +342,15 @@ ORNITH_API int ornith_sdpa_prefill_gated(ornith_ctx* ctx, const void* d_q_rot, c
  * index on ties; logits bf16 [rows, V]; d_lse (bf16 [rows]) may be null. */
 ORNITH_API int ornith_greedy_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V,
                                   uint32_t* d_tokens, void* d_lse);
+/* ornith_greedy_rows for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc). No counterpart in the reference. Same
+ * arguments and same results, bit for bit; its per-chunk partials live in a fixed 32 KiB
+ * device array inside the library instead of the context's grow-only scratch block, so the
+ * call reaches no hipMalloc / hipFree. Limits: rows <= 8, V <= 262144 (ORNITH_ERR_INVALID
+ * beyond). Every call on one GPU shares that GPU's array: calls that overlap on one GPU
+ * (two contexts, two streams) race; calls on one context are stream ordered and safe. */
+ORNITH_API int ornith_greedy_rows_noalloc(ornith_ctx* ctx, const void* d_logits, int rows, int V,
+                                          uint32_t* d_tokens, void* d_lse);
 /* greedy_argmax_into (src/ops/sample.rs:174-191): argmax of the raw logits, the draft
  * chain's choice. */
 ORNITH_API int ornith_argmax_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V,

@@ -357,6 +357,13 @@ def greedy_rows(self, logits, rows, V, tokens, lse=None):
 
 
 @_ctx_method
+def greedy_rows_noalloc(self, logits, rows, V, tokens, lse=None):
+    """greedy_rows with its partials in the library's fixed device array: allocates nothing."""
+    _check(lib().ornith_greedy_rows_noalloc(self.h, logits.ptr, rows, V, tokens.ptr, lse.ptr if lse else None),
+           "greedy_rows_noalloc")
+
+
+@_ctx_method
 def argmax_rows(self, logits, rows, V, out):
     _check(lib().ornith_argmax_rows(self.h, logits.ptr, rows, V, out.ptr), "argmax_rows")
 

@@ -57,6 +57,10 @@ int ornith_option_gemm_rows();  // default 32; 0 = never (everything through the
 int ornith_greedy_rows_ws(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens,
                           void* d_lse, ScratchCursor& sc);
 
+// Resolves the device address of the greedy selection's fixed scratch array on `device`
+// (which must be current); ornith_ctx_create calls it once per device.
+int ornith_sample_init_device(int device);
+
 // Records the message for ornith_last_error() and returns `code`.
 int ornith_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 

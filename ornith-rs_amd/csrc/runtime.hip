@@ -114,6 +114,7 @@ int ornith_ctx_create(int device, ornith_ctx** out) {
     return ornith_fail(ORNITH_ERR_UNSUPPORTED,
                        "ornith_ctx_create: device %d is %s; this library is built for gfx950 only",
                        device, prop.gcnArchName);
+  if (int rc = ornith_sample_init_device(device)) return rc;
   ornith_ctx* c = new ornith_ctx();
   c->device = device;
   c->compute_units = prop.multiProcessorCount;

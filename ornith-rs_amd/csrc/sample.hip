@@ -13,9 +13,30 @@
 #include "dmath.h"
 #include "rt.h"
 
+#include <mutex>
+
 namespace {
 
 constexpr int CH = 1024;
+
+// ---- the no-allocation variant's scratch --------------------------------------------
+// ornith_greedy_rows_noalloc keeps its per-chunk partials (maximum, sum of exponentials,
+// best value, best index) in this fixed device array instead of the context's grow-only
+// scratch block, so the call never reaches hipMalloc. Limits: 8 rows of at most 262144
+// logits -> 4 arrays x 8 rows x 256 chunks x 4 bytes = 32 KiB, held by every GPU the
+// library runs on until the process ends.
+constexpr int NA_MAX_ROWS = 8;
+constexpr int NA_MAX_V = 262144;
+constexpr int NA_MAX_NCH = NA_MAX_V / CH;
+constexpr size_t NA_ARRAY_BYTES = (size_t)NA_MAX_ROWS * NA_MAX_NCH * 4;  // a multiple of 256
+constexpr size_t NA_BYTES = 4 * NA_ARRAY_BYTES;
+static __device__ __align__(256) unsigned char scratch[NA_BYTES];
+
+// `scratch` names a host-side stand-in here; the array's device address differs per GPU
+// and is asked for once per device (ornith_sample_init_device) and kept in this table.
+constexpr int NA_MAX_DEVICES = 64;
+void* g_scratch_ptr[NA_MAX_DEVICES] = {};
+std::mutex g_scratch_mu;
 
 __global__ __launch_bounds__(CH) void lse_chunk_kernel(const bf16_t* logits, int V, int nch,
                                                        float* mc, float* lc) {
@@ -180,6 +201,19 @@ int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_toke
 
 }  // namespace
 
+// Called by ornith_ctx_create with `device` current: resolves this GPU's copy of `scratch`.
+int ornith_sample_init_device(int device) {
+  ORN_REQUIRE(device >= 0 && device < NA_MAX_DEVICES, "device %d is beyond the %d this library tracks", device,
+              NA_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[device]) return ORNITH_OK;
+  void* ptr = nullptr;
+  ORN_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  ORN_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null address for the fixed scratch array");
+  g_scratch_ptr[device] = ptr;
+  return ORNITH_OK;
+}
+
 int ornith_greedy_rows_ws(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_tokens,
                           void* d_lse, ScratchCursor& sc) {
   return run(ctx, d_logits, rows, V, d_tokens, d_lse, true, "greedy_rows", &sc);
@@ -201,6 +235,24 @@ int ornith_greedy_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V, u
 
 int ornith_argmax_rows(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_out) {
   return run(ctx, d_logits, rows, V, d_out, nullptr, false, "argmax_rows");
+}
+
+int ornith_greedy_rows_noalloc(ornith_ctx* ctx, const void* d_logits, int rows, int V,
+                               uint32_t* d_tokens, void* d_lse) {
+  ORN_REQUIRE(ctx && d_logits && d_tokens, "greedy_rows_noalloc: null argument");
+  ORN_REQUIRE(rows >= 1 && rows <= NA_MAX_ROWS,
+              "greedy_rows_noalloc: %d rows; the fixed scratch array holds at most %d (use ornith_greedy_rows)",
+              rows, NA_MAX_ROWS);
+  ORN_REQUIRE(V >= 1 && V <= NA_MAX_V,
+              "greedy_rows_noalloc: %d logits a row; the fixed scratch array holds at most %d (use "
+              "ornith_greedy_rows)", V, NA_MAX_V);
+  void* ptr = (ctx->device >= 0 && ctx->device < NA_MAX_DEVICES) ? g_scratch_ptr[ctx->device] : nullptr;
+  ORN_REQUIRE(ptr != nullptr, "greedy_rows_noalloc: the fixed scratch array of device %d was never resolved",
+              ctx->device);
+  // every partial is written by the pass before the one that reads it, for exactly the
+  // rows x chunks of this call, so nothing left by an earlier call is ever read
+  ScratchCursor sc(ptr);
+  return run(ctx, d_logits, rows, V, d_tokens, d_lse, true, "greedy_rows_noalloc", &sc);
 }
 
 }  // extern "C"
