@@ -107,6 +107,17 @@ typedef struct orc_state {
   int moffset;
 } orc_state;
 
+/* Test hook: while a log is set, every MoE block run by orc_forward / orc_mtp_hidden appends
+ * the experts its router picked ([T, top_k] u32 per block, in call order), so a test can
+ * evaluate an independent model on the same experts. NULL turns it off. */
+static struct { uint32_t* buf; int cap, n; } g_picks;
+ORC_API void orc_debug_log_picks(uint32_t* buf, int cap) { g_picks.buf = buf; g_picks.cap = cap; g_picks.n = 0; }
+ORC_API int orc_debug_picks_logged(void) { return g_picks.n; }
+static void log_picks(const uint32_t* inds, int n) {
+  if (!g_picks.buf) return;
+  for (int i = 0; i < n && g_picks.n < g_picks.cap; ++i) g_picks.buf[g_picks.n++] = inds[i];
+}
+
 static int key_dim(const orc_config* c) { return c->linear_num_key_heads * c->linear_key_head_dim; }
 static int value_dim(const orc_config* c) { return c->linear_num_value_heads * c->linear_value_head_dim; }
 static int conv_dim(const orc_config* c) { return 2 * key_dim(c) + value_dim(c); }
@@ -218,7 +229,14 @@ ORC_API void orc_forward(orc_state* s, const uint32_t* tokens, int T, int captur
       attention(c, &Lw->attn, s, normed, T, lc->k, lc->v, s->offset, r);
     }
     orc_add_rms_norm(x, r, Lw->post_ln, T, H, c->rms_norm_eps, h, n2);
-    orc_moe_block(&Lw->moe, n2, T, mo, NULL, NULL, NULL);
+    if (g_picks.buf) {
+      uint32_t* picked = malloc(4 * (size_t)T * Lw->moe.top_k);
+      orc_moe_block(&Lw->moe, n2, T, mo, picked, NULL, NULL);
+      log_picks(picked, T * Lw->moe.top_k);
+      free(picked);
+    } else {
+      orc_moe_block(&Lw->moe, n2, T, mo, NULL, NULL, NULL);
+    }
     orc_add_rms_norm(h, mo, i + 1 < L ? m->layers[i + 1].input_ln : m->final_norm, T, H, c->rms_norm_eps, x,
                      normed);
   }
@@ -258,6 +276,7 @@ static void mtp_moe(const orc_config* c, const orc_mtp_w* w, const bf16_t* x, in
   orc_linear_fwd(&w->moe.router, x, T, gates);
   orc_softmax_bf16(gates, T, E, probs);
   orc_router_topk(probs, T, E, k, inds, scores);
+  log_picks(inds, T * k);
   for (int r = 0; r < T * k; ++r) { lhs[r] = (uint32_t)(r / k); rows[r] = (uint32_t)r; }
   orc_dense_gather_mv(w->ex_gate, I, H, x, lhs, inds, T * k, xg);
   orc_dense_gather_mv(w->ex_up, I, H, x, lhs, inds, T * k, xu);
@@ -362,6 +381,12 @@ ORC_API int orc_generate(orc_state* s, const uint32_t* prompt, int n_prompt, int
   return n;
 }
 
+/* Scripted drafts (test hook, the counterpart of the device library's measurement aid): while
+ * a list is set, the draft for output position p is forced[p] instead of the head's own
+ * (the head still runs). n = 0 clears it. */
+static struct { const uint32_t* toks; int n; } g_forced;
+ORC_API void orc_mtp_force_drafts(const uint32_t* toks, int n) { g_forced.toks = toks; g_forced.n = n; }
+
 typedef struct orc_mtp_stats { int64_t cycles, drafted, accepted, reached[8], accepted_by[8]; } orc_mtp_stats;
 
 /* generate_step_mtp. With the greedy sampler every row's target is taken at once; with a
@@ -417,6 +442,7 @@ ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* f
         orc_linear_fwd(&m->lm_head, hi, 1, dlogits);
         orc_argmax_rows(dlogits, 1, V, &window[i + 1]);
       }
+      if (emitted + 1 + i < g_forced.n) window[i + 1] = g_forced.toks[emitted + 1 + i];
       hcur = hi;
     }
     if (want > 0) { stats->cycles++; stats->drafted += want; }

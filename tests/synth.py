@@ -291,6 +291,12 @@ class OracleRun:
         self.o.orc_set_sampler(kind, C.c_double(float(np.float32(temp))), C.c_double(float(np.float32(top_p))),
                                top_k, C.c_uint64(seed))
 
+    def force_drafts(self, tokens):
+        """Scripted drafts for mtp_generate (position p of the output is drafted as tokens[p]);
+        an empty list clears them. Process-global in the oracle."""
+        self._forced = np.ascontiguousarray(tokens, dtype=np.uint32)
+        self.o.orc_mtp_force_drafts(p(self._forced) if len(self._forced) else None, len(self._forced))
+
     def generate(self, prompt, max_tokens, prefill_step=16):
         prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
         out = np.empty(max_tokens, np.uint32)

@@ -1,0 +1,153 @@
+"""Pins the oracle's model-level composition (CPU only).
+
+oracle/orc_model.c wires the operator restatements into the trunk (orc_forward) and the MTP
+head (orc_mtp_hidden). Every operator has its own pin; this file pins the wiring: the hidden
+rows of a two-layer model (one gated-delta layer, one full-attention layer, a MoE block after
+each) and of the MTP head are compared with tests/f64_model.py, a float64 numpy forward
+written from the reference's Rust (src/model/qwen3_5.rs:231-279,374-390,430-474,478-565;
+src/model/mtp.rs:165-262) that shares no code with the oracle's model file.
+
+Which experts a token is routed to is a discrete choice that a bf16 rounding can flip at a
+near-tie (router logits near 3 are 2^-6 apart in bf16), and one flipped expert moves a row by
+tens of percent. So the oracle logs the experts it picked (orc_debug_log_picks) and the float64
+model is evaluated on those experts with its own softmax weights; that its own top-k is the
+same set wherever the cut is not a near-tie is asserted separately.
+
+Tolerance: every operator of the oracle rounds its output to bf16 (2^-9 relative), some thirty
+roundings deep; measured over seeds 0..11 the two forwards agree to 2.2-4.3 % relative L2 with one outlier at 6.5 % (seed 0, used here: 2.5 %). The bound is
+5 % relative L2 and 8 % of the largest element. A wiring mistake is an O(1) difference: the second test rebuilds the oracle from a
+scratch copy of orc_model.c with one such mistake at a time (residual taken from the wrong
+stream, the concat order swapped, norm weights exchanged, the final norm dropped, a cache
+not carried) and requires this comparison to fail for each.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+import f64_model
+import synth
+import util
+
+CFG = dict(synth.TINY, num_hidden_layers=2, full_attention_interval=2, vocab_size=256, num_experts_per_tok=4)
+SEED = 0
+REL_L2, REL_MAX = 0.05, 0.08
+
+
+def _loud_norms(s, seed):
+    """Norm weights of the test model drawn wide (x0.5 .. x2) so that exchanging two of them,
+    or dropping one, moves the result far beyond the tolerance. In place: the oracle structs
+    and the float64 model both read these arrays."""
+    rng = np.random.default_rng(seed)
+    arrs = [s.final_norm]
+    for lay in s.layers:
+        arrs += [lay["input_ln"], lay["post_ln"]]
+    m = s.mtp
+    arrs += [m["pre_fc_norm_embedding"], m["pre_fc_norm_hidden"], m["input_ln"], m["post_ln"], m["norm"]]
+    for a in arrs:
+        a[...] = util.f32_to_bf16((2.0 ** rng.uniform(-1, 1, a.shape)).astype(np.float32))
+
+
+def _compare():
+    """Worst (rel-L2, rel-max) of oracle vs float64 over the trunk rows and the MTP rows, and
+    the smallest relative gap at a top-k cut the float64 router saw."""
+    s = synth.SynthModel(CFG, seed=SEED)
+    _loud_norms(s, SEED)
+    toks = np.random.default_rng(SEED).integers(0, CFG["vocab_size"], 6).astype(np.uint32)
+    o, f = synth.OracleRun(s, 32), f64_model.F64Model(s)
+    margins, worst, hid = [], [0.0, 0.0], []
+    k = CFG["num_experts_per_tok"]
+    log = np.zeros(4096, np.uint32)
+
+    def run_logged(fn, *a):
+        """fn(*a) on the oracle with the pick log on; hands the picks to the float64 model."""
+        util.oracle().orc_debug_log_picks(util.p(log), log.size)
+        out = fn(*a)
+        n = util.oracle().orc_debug_picks_logged()
+        util.oracle().orc_debug_log_picks(None, 0)
+        assert 0 < n < log.size and n % k == 0
+        f.forced_picks = iter(log[:n].reshape(-1, k).copy())
+        return out
+
+    def note(got_bf16, want):
+        got = util.bf16_to_f32(got_bf16).astype(np.float64)
+        worst[0] = max(worst[0], np.linalg.norm(got - want) / np.linalg.norm(want))
+        worst[1] = max(worst[1], np.max(np.abs(got - want)) / np.max(np.abs(want)))
+
+    # three calls of different widths: the conv window, the recurrent state, the KV rows and the
+    # rotary offset all have to be carried from call to call
+    for chunk in (toks[:3], toks[3:5], toks[5:6]):
+        h = run_logged(o.forward, chunk)
+        hid.append(h)
+        note(h, f.forward(chunk, margins))
+        assert next(f.forced_picks, None) is None        # every logged block was consumed
+    hid = np.concatenate(hid)
+    # the head: rows 0..2 with the tokens that follow them, then two more rows on its own cache
+    for lo, hi in ((0, 3), (3, 5)):
+        got = run_logged(o.mtp_hidden, hid[lo:hi], toks[lo + 1:hi + 1])
+        note(got, f.mtp_hidden(util.bf16_to_f32(hid[lo:hi]), toks[lo + 1:hi + 1], margins))
+    o.close()
+    # the float64 router's own top-k is the oracle's wherever the cut is clear (a 10 % gap)
+    clear = [(own, forced) for gap, own, forced in margins if gap > 0.10]
+    agree = sum(own == forced for own, forced in clear)
+    return worst[0], worst[1], (agree, len(clear), len(margins))
+
+
+def test_oracle_forward_and_mtp_head_match_float64_model():
+    l2, mx, (agree, clear, total) = _compare()
+    assert clear >= total // 3 and agree == clear, (agree, clear, total)
+    assert l2 <= REL_L2 and mx <= REL_MAX, (l2, mx)
+
+
+MUTATIONS = {
+    "closing residual taken from x instead of h":
+        ("orc_add_rms_norm(h, mo, i + 1 < L ?", "orc_add_rms_norm(x, mo, i + 1 < L ?"),
+    "post-attention norm weight exchanged with the input norm's":
+        ("orc_add_rms_norm(x, r, Lw->post_ln,", "orc_add_rms_norm(x, r, Lw->input_ln,"),
+    "final norm dropped":
+        ("memcpy(hidden_out, normed, hb);", "memcpy(hidden_out, x, hb);"),
+    "mixer fed the residual stream instead of its norm":
+        ("orc_linear_fwd(&g->in_proj_qkv, normed, T, qkv);", "orc_linear_fwd(&g->in_proj_qkv, x, T, qkv);"),
+    "recurrent state not carried between calls":
+        ("memcpy(lc->state, snaps + se * (size_t)(T - 1), 4 * se);", ""),
+    "conv window not carried between calls":
+        ("memcpy(lc->conv, ci + (size_t)T * D, 2 * (size_t)S * D);", ""),
+    "attention position stuck at zero":
+        ("attention(c, &Lw->attn, s, normed, T, lc->k, lc->v, s->offset, r);",
+         "attention(c, &Lw->attn, s, normed, T, lc->k, lc->v, 0, r);"),
+    "MTP concat order swapped":
+        ("memcpy(joined + (size_t)t * 2 * H, e + (size_t)t * H, 2 * (size_t)H);\n"
+         "    memcpy(joined + (size_t)t * 2 * H + H, hh + (size_t)t * H, 2 * (size_t)H);",
+         "memcpy(joined + (size_t)t * 2 * H, hh + (size_t)t * H, 2 * (size_t)H);\n"
+         "    memcpy(joined + (size_t)t * 2 * H + H, e + (size_t)t * H, 2 * (size_t)H);"),
+    "MTP pre-fc norms exchanged":
+        ("orc_rms_norm(emb, w->pre_fc_norm_embedding,", "orc_rms_norm(emb, w->pre_fc_norm_hidden,"),
+    "MTP closing residual taken from x instead of h":
+        ("orc_add_rms_norm(h2, mo, w->norm,", "orc_add_rms_norm(x, mo, w->norm,"),
+    "MTP head's own norm replaced by the layer's":
+        ("orc_add_rms_norm(h2, mo, w->norm,", "orc_add_rms_norm(h2, mo, w->post_ln,"),
+}
+
+
+def test_wiring_mistakes_in_a_scratch_copy_of_the_oracle_fail_the_comparison(tmp_path, monkeypatch):
+    src_dir = util.ORACLE_DIR
+    model_c = open(os.path.join(src_dir, "orc_model.c")).read()
+    others = sorted(os.path.join(src_dir, f) for f in os.listdir(src_dir)
+                    if f.startswith("orc_") and f.endswith(".c") and f != "orc_model.c")
+    flags = ["-O1", "-std=c11", "-fPIC", "-ffp-contract=off", "-fno-fast-math", "-mfma", "-msse4.1", "-fopenmp",
+             "-fvisibility=hidden", "-w", "-shared", "-I", src_dir]
+    for i, (what, (old, new)) in enumerate(MUTATIONS.items()):
+        assert model_c.count(old) == 1, f"mutation '{what}' no longer matches orc_model.c exactly once"
+        c_path, so_path = str(tmp_path / f"orc_model_mut{i}.c"), str(tmp_path / f"liborc_mut{i}.so")
+        with open(c_path, "w") as fh:
+            fh.write(model_c.replace(old, new))
+        subprocess.check_call(["gcc", *flags, "-o", so_path, c_path, *others, "-lm"])
+        lib = C.CDLL(so_path)
+        lib.orc_tree64_export.restype = C.c_float
+        monkeypatch.setattr(util, "_orc", lib)
+        l2, mx, _ = _compare()
+        assert l2 > 2 * REL_L2, (what, l2, mx)
+    monkeypatch.undo()
+    l2, mx, _ = _compare()      # and the real oracle passes again afterwards
+    assert l2 <= REL_L2 and mx <= REL_MAX
