@@ -81,7 +81,15 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *               wavefront of the k-quant mat-vec walks, a tuning knob
  *   "gemm_duo"  (ORNITH_GEMM_DUO, default 1): the 256-row tile of the prefill GEMM runs with
  *               producer and consumer wavefronts (0: every wavefront dequantizes, then
- *               multiplies); same results either way */
+ *               multiplies); same results either way
+ *   "fuse_moe_one" (ORNITH_FUSE_MOE_ONE, default 0): the MoE block's phases as ranges of
+ *               workgroups of ONE launch that hand their intermediates over through memory
+ *               (1: router + up + down, 2: up + down after a router launch). Bit-identical,
+ *               measured slower than the separate launches on this part, kept for that
+ *               measurement (hidden size 2048, expert width 512, T <= 4 only)
+ *   "ho_spins"  (ORNITH_HO_SPINS, default 2^20): polling rounds a wait between workgroups of
+ *               such a launch may take before it gives up; the failure is reported by the next
+ *               ornith_sync / ornith_download (ORNITH_ERR_HIP) */
 ORNITH_API int ornith_set_option(const char* name, int value);
 ORNITH_API int ornith_timer_begin(ornith_ctx* ctx);
 ORNITH_API int ornith_timer_end(ornith_ctx* ctx, float* ms_out);

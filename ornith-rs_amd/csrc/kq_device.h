@@ -16,10 +16,23 @@
 #include "../../include/ornith_hip.h"
 #include "dmath.h"
 
-// 16 consecutive activations -> fp32 registers
-template <bool XF32>
+// 16 consecutive activations -> fp32 registers. COH: the row was written by another
+// workgroup of this launch (handoff.h), so it is read with agent-scope loads (bf16 only).
+template <bool XF32, bool COH = false>
 __device__ __forceinline__ void load_x16(const void* xrow, int off, float (&v)[16]) {
-  if constexpr (XF32) {
+  if constexpr (COH) {
+    static_assert(!XF32, "hand-off rows are bf16");
+    const uint64_t* p = reinterpret_cast<const uint64_t*>(static_cast<const bf16_t*>(xrow) + off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint64_t w = __hip_atomic_load(p + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t lo = (uint32_t)w, hi = (uint32_t)(w >> 32);
+      v[4 * i + 0] = dm_bf2f_lo(lo);
+      v[4 * i + 1] = dm_bf2f_hi(lo);
+      v[4 * i + 2] = dm_bf2f_lo(hi);
+      v[4 * i + 3] = dm_bf2f_hi(hi);
+    }
+  } else if constexpr (XF32) {
     const float4* p = reinterpret_cast<const float4*>(static_cast<const float*>(xrow) + off);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -64,14 +77,14 @@ struct Q4Lane {
     h = chunk & 1;
   }
 
-  template <bool XF32>
+  template <bool XF32, bool COH = false>
   __device__ __forceinline__ void load_x(const void* const (&xrow)[M], int chunk) {
     set_chunk(chunk);
     const int off = 256 * b + 64 * g + 16 * h;
 #pragma unroll
     for (int t = 0; t < M; ++t) {
-      load_x16<XF32>(xrow[t], off, xl[t]);
-      load_x16<XF32>(xrow[t], off + 32, xh[t]);
+      load_x16<XF32, COH>(xrow[t], off, xl[t]);
+      load_x16<XF32, COH>(xrow[t], off + 32, xh[t]);
       float a = 0.f, c = 0.f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
@@ -165,14 +178,14 @@ struct Q6Lane {
     u = chunk & 1;
   }
 
-  template <bool XF32>
+  template <bool XF32, bool COH = false>
   __device__ __forceinline__ void load_x(const void* const (&xrow)[M], int chunk) {
     set_chunk(chunk);
     const int off = 256 * b + 128 * n + 16 * u;
 #pragma unroll
     for (int t = 0; t < M; ++t)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) load_x16<XF32>(xrow[t], off + 32 * g, x[t][g]);
+      for (int g = 0; g < 4; ++g) load_x16<XF32, COH>(xrow[t], off + 32 * g, x[t][g]);
   }
 };
 

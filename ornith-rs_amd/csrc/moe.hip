@@ -21,6 +21,9 @@ extern "C" int dense_gather_mv_multi(ornith_ctx* ctx, const void* const* d_ws, i
 bool moe_fused_supported(const ornith_moe_weights* w);
 bool moe_fused_router(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       void* d_gates, void* d_egate, int* rc, const PreNorm* pre);
+bool moe_one_launch(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, void* d_gates,
+                    void* d_egate, uint32_t* d_inds, void* d_scores, void* d_act, void* d_out,
+                    const PreNorm* pre, int* rc);
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
                       void* d_out, int phases, const void* d_gates);
@@ -323,8 +326,17 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
     if (rc) return rc;  \
   } while (0)
   if (ornith_option_fuse_moe() && moe_fused_supported(w)) {
-    // gates + shared-expert gate, softmax + top-k, then the two expert kernels
     int rrc = ORNITH_OK;
+    // router, up and down as one launch where the shapes are in its family
+    if (moe_one_launch(ctx, w, d_x, T, gates, eg, inds, scores, act, d_out, pre, &rrc)) {
+      if (rrc) return rrc;
+      if (d_inds_out)
+        ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice, ctx->stream));
+      if (d_scores_out)
+        ORN_HIP(hipMemcpyAsync(d_scores_out, scores, 2 * (size_t)T * k, hipMemcpyDeviceToDevice, ctx->stream));
+      return ORNITH_OK;
+    }
+    // gates + shared-expert gate, softmax + top-k, then the two expert kernels
     if (moe_fused_router(ctx, w, d_x, T, gates, eg, &rrc, pre)) {
       if (rrc) return rrc;
     } else {

@@ -33,17 +33,39 @@ __device__ __forceinline__ uint32_t dm_wave_max_u32(uint32_t v) {
 // E = 64 * PER <= 1024 so an index fits 10 bits: a candidate is the single integer
 // (bf16 probability bits << 16 | index) + 1, whose order is exactly (value, index) for
 // the non-negative probabilities a softmax produces; 0 marks a taken entry.
-template <int PER>
+// COH: the gates were written by other workgroups of this launch (handoff.h) and are read
+// with agent-scope loads.
+template <int PER, bool COH = false>
 __device__ __forceinline__ void router_topk_wave(const bf16_t* gates_row, int k, uint32_t* inds_row,
                                                  bf16_t* scores_row, bf16_t* probs_row, int lane) {
   const bf16_t* g = gates_row + lane * PER;
   float v[PER];
   float m = -DM_INF;
+  if constexpr (COH) {
+    if constexpr (PER == 1) {
+      v[0] = dm_bf2f(__hip_atomic_load(g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    } else if constexpr (PER == 2) {
+      const uint32_t w = __hip_atomic_load(reinterpret_cast<const uint32_t*>(g), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+      v[0] = dm_bf2f_lo(w);
+      v[1] = dm_bf2f_hi(w);
+    } else {
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    v[i] = dm_bf2f(g[i]);
-    m = v[i] > m ? v[i] : m;
+      for (int q = 0; q < PER / 4; ++q) {
+        const uint64_t w = __hip_atomic_load(reinterpret_cast<const uint64_t*>(g) + q, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+        v[4 * q + 0] = dm_bf2f_lo((uint32_t)w);
+        v[4 * q + 1] = dm_bf2f_hi((uint32_t)w);
+        v[4 * q + 2] = dm_bf2f_lo((uint32_t)(w >> 32));
+        v[4 * q + 3] = dm_bf2f_hi((uint32_t)(w >> 32));
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) v[i] = dm_bf2f(g[i]);
   }
+#pragma unroll
+  for (int i = 0; i < PER; ++i) m = v[i] > m ? v[i] : m;
   m = dm_wave_max<64>(m);
   float s = 0.f;
 #pragma unroll

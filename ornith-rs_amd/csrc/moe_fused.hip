@@ -23,6 +23,7 @@
 // verify width 2 a launch moves ~19 MB / ~15 MB, less than the chip can hold in
 // flight, so every wavefront issues ALL of its weight loads first (they depend on
 // nothing but the index list), then the activation loads, and only then computes.
+#include "handoff.h"
 #include "kq_device.h"
 #include "moe_device.h"
 #include "norm_device.h"
@@ -352,6 +353,311 @@ void launch_router_fused(ornith_ctx* ctx, const RouterArgs& a, int M) {
   }
 }
 
+// ---- the whole block in ONE launch ---------------------------------------------------
+// Router, expert up and expert down as three ranges of workgroups of one grid, handing
+// their small intermediates (gates, the normed input rows, the routing, the expert
+// activations) over through memory as handoff.h describes. Same arithmetic as the three
+// kernels above, operation for operation; what changes is that two launch boundaries are
+// gone, that the down workgroups have their weight rows in flight while the up workgroups
+// still compute, and that nothing but flag words is waited for.
+//
+//   [0, n_router)            router rows (+ the shared expert's scalar gate in the last one);
+//                            workgroup 0 also stores h and the normed rows
+//   [n_router, +n_up)        (row r, column block bx): waits for the router, makes the top-k,
+//                            gate + up + swiglu -> act; one workgroup per token stores the routing
+//   [.., +n_down)            (token t, column block bx): waits for the routing, requests its
+//                            down rows, waits for its act rows, down + combine -> out
+struct OneArgs {
+  RouterArgs r;
+  UpArgs u;
+  DownArgs d;
+  uint32_t* rflag;  // [n_router]
+  uint32_t* iflag;  // [T]
+  uint32_t* aflag;  // [(T*k + T) * up_x]
+  uint32_t* err;
+  uint32_t epoch;
+  int n_router, up_x, n_up, down_x, max_spins;
+};
+
+template <int KIND, int LPR, int M>
+__device__ __forceinline__ void one_router(const OneArgs& o, int wg, char* lds) {
+  if (threadIdx.x >= 256) return;
+  const RouterArgs& a = o.r;
+  using KL = KqLane<KIND, 1>;
+  constexpr int RPW = 64 / LPR;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  PreNormLds<M>& pn = *reinterpret_cast<PreNormLds<M>*>(lds);
+  const bool pre = a.pre.res != nullptr;
+  if (wg == o.n_router - 1) {
+    if (pre) prenorm_rows<M, true>(a.pre, false, pn);
+    if (wave < M) {
+      const float e = egate_row_dot(a, pre ? &pn.xn[wave][0] : a.x + (size_t)wave * a.K, lane);
+      if (lane == 0) ho_store_u16(&a.egate[wave], dm_f2bf(e));
+    }
+    ho_publish(&o.rflag[wg], o.epoch);
+    return;
+  }
+  const int slot = lane / LPR, c = lane % LPR;
+  const int nb = a.K >> 8;
+  typename KL::Lane L;
+  L.set_chunk(c);
+  const int row_o = (wg * 4 + wave) * RPW + slot;
+  const typename KL::Row row = KL::load(a.w.qs, a.w.scales, a.w.dm, row_o < a.E ? row_o : a.E - 1, nb, L);
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  if (pre) prenorm_rows<M, true>(a.pre, wg == 0, pn);
+  // one token at a time over the same weight registers (a row's sum does not depend on how
+  // many rows share the pass)
+#pragma unroll
+  for (int t = 0; t < M; ++t) {
+    const void* xrow[1] = {pre ? (const void*)&pn.xn[t][0] : (const void*)(a.x + (size_t)t * a.K)};
+    L.template load_x<false>(xrow, c);
+    float acc[1] = {0.f};
+    KL::accumulate(row, L, acc);
+    const float v = dm_wave_sum<LPR>(acc[0]);
+    if (c == 0 && row_o < a.E) ho_store_u16(&a.gates[(size_t)t * a.E + row_o], dm_f2bf(v));
+  }
+  ho_publish(&o.rflag[wg], o.epoch);
+}
+
+// RIN: the router runs inside this launch (gates and input rows are hand-offs); otherwise they
+// were written by earlier launches and are read the ordinary way.
+template <int KIND, int LPR, bool RIN>
+__device__ __forceinline__ void one_up(const OneArgs& o, int u, char* lds) {
+  if (threadIdx.x >= 256) return;
+  const UpArgs& a = o.u;
+  using KL = KqLane<KIND, 1>;
+  constexpr int RPW = 64 / LPR, ITERS = 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int slot = lane / LPR, c = lane % LPR;
+  const int nb = a.K >> 8;
+  const int bx = u % o.up_x, r = u / o.up_x;
+  const int routed = a.T * a.k;
+  uint32_t* s_inds = reinterpret_cast<uint32_t*>(lds);
+  bf16_t* s_scores = reinterpret_cast<bf16_t*>(lds + 64);
+  KqPtr pin[4] = {a.gate, a.up, a.sgate, a.sup};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    uint64_t q = (uint64_t)pin[i].qs, sc = (uint64_t)pin[i].scales, d = (uint64_t)pin[i].dm;
+    asm volatile("" : "+s"(q), "+s"(sc), "+s"(d));
+    pin[i].qs = dm_global_ptr<const uint8_t>(q);
+    pin[i].scales = dm_global_ptr<const uint8_t>(sc);
+    pin[i].dm = dm_global_ptr<const uint16_t>(d);
+  }
+  int token;
+  int64_t row0;
+  KqPtr wg_, wu_;
+  const bool is_routed = r < routed;
+  if (is_routed) {
+    token = r / a.k;
+    if (wave == 0) {
+      if constexpr (RIN) ho_wait(o.rflag, o.n_router, o.epoch, o.max_spins, o.err, lane);
+      const bf16_t* g = a.gates + (size_t)token * a.E;
+      switch (a.E / 64) {
+        case 1: router_topk_wave<1, RIN>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+        case 2: router_topk_wave<2, RIN>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+        case 4: router_topk_wave<4, RIN>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+        case 8: router_topk_wave<8, RIN>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+        default: router_topk_wave<16, RIN>(g, a.k, s_inds, s_scores, nullptr, lane); break;
+      }
+    }
+    __syncthreads();
+    const uint32_t e = s_inds[r - token * a.k];
+    row0 = (int64_t)min(e, (uint32_t)(a.E - 1)) * a.I;
+    wg_ = pin[0];
+    wu_ = pin[1];
+  } else {
+    token = r - routed;
+    row0 = 0;
+    wg_ = pin[2];
+    wu_ = pin[3];
+  }
+  typename KL::Lane L;
+  L.set_chunk(c);
+  const int base = (bx * 4 + wave) * (RPW * ITERS);
+  typename KL::Row rg[ITERS], ru[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int oo = base + it * RPW + slot;
+    const int64_t row = row0 + (oo < a.I ? oo : a.I - 1);
+    rg[it] = KL::load(wg_.qs, wg_.scales, wg_.dm, row, nb, L);
+    ru[it] = KL::load(wu_.qs, wu_.scales, wu_.dm, row, nb, L);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of everything below
+  if (is_routed) {
+    // one workgroup per token stores the routing: for the down workgroups when the router runs
+    // in this launch (a hand-off), for the caller otherwise
+    if (bx == 0 && r == token * a.k && wave == 0) {
+      if (lane < a.k) {
+        ho_store_u32(&a.inds_out[r + lane], s_inds[lane]);
+        ho_store_u16(&a.scores_out[r + lane], s_scores[lane]);
+      }
+      if constexpr (RIN) {
+        ho_wait_stores();
+        if (lane == 0) ho_store_u32(&o.iflag[token], o.epoch);
+      }
+    }
+  } else if constexpr (RIN) {
+    // the shared expert's rows need no routing, only the normed input rows
+    ho_wait(o.rflag, o.n_router, o.epoch, o.max_spins, o.err, lane);
+  }
+  const void* xrow[1] = {a.x + (size_t)token * a.K};
+  L.template load_x<false, RIN>(xrow, c);
+  if constexpr (LPR == 64) {
+#pragma unroll
+    for (int it = 0; it < ITERS; it += 2) {
+      float g0[1] = {0.f}, u0[1] = {0.f}, g1[1] = {0.f}, u1[1] = {0.f};
+      KL::accumulate(rg[it], L, g0);
+      KL::accumulate(ru[it], L, u0);
+      KL::accumulate(rg[it + 1], L, g1);
+      KL::accumulate(ru[it + 1], L, u1);
+      const float red = dm_wave_sum4(g0[0], u0[0], g1[0], u1[0], lane);
+      float gsum, usum;
+      dm_row_swap<32>(red, gsum, usum);
+      const int oo = base + it + ((lane >> 4) & 1);
+      if ((lane & 47) == 0 && oo < a.I) ho_store_u16(&a.act[(size_t)r * a.I + oo], swiglu_bf16(gsum, usum));
+    }
+  } else {
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int oo = base + it * RPW + slot;
+      float ag[1] = {0.f}, au[1] = {0.f};
+      KL::accumulate(rg[it], L, ag);
+      KL::accumulate(ru[it], L, au);
+      const float g = dm_wave_sum<LPR>(ag[0]);
+      const float uu = dm_wave_sum<LPR>(au[0]);
+      if (c == 0 && oo < a.I) ho_store_u16(&a.act[(size_t)r * a.I + oo], swiglu_bf16(g, uu));
+    }
+  }
+  ho_publish(&o.aflag[(size_t)r * o.up_x + bx], o.epoch);
+}
+
+// Down role: wavefront w of the workgroup takes expert slots 2w and 2w+1 (slot k is the shared
+// expert), so (k + 1 + 1) / 2 wavefronts cover the k + 1 rows that meet in LDS.
+template <int KIND, int LPR, bool RIN>
+__device__ __forceinline__ void one_down(const OneArgs& o, int dd, char* lds) {
+  const DownArgs& a = o.d;
+  using KL = KqLane<KIND, 1>;
+  constexpr int RPW = 64 / LPR, COLS = RPW;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int slot = lane / LPR, c = lane % LPR;
+  const int nb = a.I >> 8;
+  const int t = dd / o.down_x, k = a.k;
+  const int c0 = (dd % o.down_x) * COLS;
+  float(*yl)[COLS] = reinterpret_cast<float(*)[COLS]>(lds);
+  float* wj = reinterpret_cast<float*>(lds + sizeof(float) * (kMaxK + 1) * COLS);
+  float* gsig = wj + kMaxK;
+  const int j0 = 2 * wave;
+  const bool two = j0 + 1 <= k;
+
+  typename KL::Lane L;
+  L.set_chunk(c);
+  const int oo = c0 + slot;
+  const int64_t orow = oo < a.H ? oo : a.H - 1;
+  typename KL::Row rr[2];
+  int arow[2];
+  uint32_t* s_inds = reinterpret_cast<uint32_t*>(gsig + 1);
+  bf16_t* s_scores = reinterpret_cast<bf16_t*>(s_inds + 16);
+  if constexpr (RIN) {
+    if (j0 < k) ho_wait(&o.iflag[t], 1, o.epoch, o.max_spins, o.err, lane);
+  } else {
+    // the gates are an earlier launch's: every workgroup makes its token's routing itself,
+    // so nothing but its own act rows is ever waited for
+    if (wave == 0) {
+      const bf16_t* g = o.u.gates + (size_t)t * a.E;
+      switch (a.E / 64) {
+        case 1: router_topk_wave<1>(g, k, s_inds, s_scores, nullptr, lane); break;
+        case 2: router_topk_wave<2>(g, k, s_inds, s_scores, nullptr, lane); break;
+        case 4: router_topk_wave<4>(g, k, s_inds, s_scores, nullptr, lane); break;
+        case 8: router_topk_wave<8>(g, k, s_inds, s_scores, nullptr, lane); break;
+        default: router_topk_wave<16>(g, k, s_inds, s_scores, nullptr, lane); break;
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const int j = j0 + q;
+    const bool shared = j >= k;  // also the unused second slot of the last wavefront (harmless reload)
+    arow[q] = shared ? a.T * k + t : t * k + j;
+    const KqPtr w = shared ? a.sdown : a.down;
+    int64_t row0 = 0;
+    if (!shared) {
+      const uint32_t e = RIN ? ho_load_u32(&a.inds[t * k + j]) : s_inds[j];
+      row0 = (int64_t)min(e, (uint32_t)(a.E - 1)) * a.H;
+    }
+    rr[q] = KL::load(w.qs, w.scales, w.dm, row0 + orow, nb, L);
+  }
+  __builtin_amdgcn_sched_barrier(0);  // the weight rows are in flight while the act rows are awaited
+  if (wave == 0) {
+    // with the router in this launch the scores arrived with the routing (iflag), and the shared
+    // expert's scalar gate was published before any routing could be made
+    const bf16_t* s = a.scores + (size_t)t * k;
+    float denom = 0.f;
+    if (a.normalize)
+      for (int i = 0; i < k; ++i) denom = dm_rb(dm_bf2f(RIN ? ho_load_u16(&s[i]) : s_scores[i]) + denom);
+    if (lane < k) {
+      const float sv = dm_bf2f(RIN ? ho_load_u16(&s[lane]) : s_scores[lane]);
+      wj[lane] = a.normalize ? dm_rb(sv / denom) : sv;
+    }
+    if (lane == 0) *gsig = dm_sigmoid_bf16(dm_bf2f(RIN ? ho_load_u16(&a.egate[t]) : a.egate[t]));
+  }
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    if (j0 + q > k) break;  // a slot past the shared expert
+    ho_wait(&o.aflag[(size_t)arow[q] * o.up_x], o.up_x, o.epoch, o.max_spins, o.err, lane);
+    const void* xrow[1] = {a.act + (size_t)arow[q] * a.I};
+    L.template load_x<false, true>(xrow, c);
+    float acc[1] = {0.f};
+    KL::accumulate(rr[q], L, acc);
+    const float v = dm_wave_sum<LPR>(acc[0]);
+    if (c == 0) yl[j0 + q][slot] = dm_rb(v);
+  }
+  __syncthreads();
+  const int col = threadIdx.x;
+  if (col < COLS && c0 + col < a.H) {
+    float acc = 0.f;
+    for (int i = 0; i < k; ++i) {
+      const float weighted = dm_rb(yl[i][col] * wj[i]);
+      acc = dm_rb(weighted + acc);
+    }
+    const float gated = dm_rb(*gsig * yl[k][col]);
+    a.out[(size_t)t * a.H + c0 + col] = dm_f2bf(acc + gated);
+  }
+}
+
+template <int M>
+constexpr size_t one_lds_bytes() {
+  constexpr size_t down = sizeof(float) * ((kMaxK + 1) * 16 + kMaxK + 1) + 16 * 4 + 16 * 2;
+  return sizeof(PreNormLds<M>) > down ? sizeof(PreNormLds<M>) : down;
+}
+
+constexpr int kOneThreads = 64 * ((kMaxK + 2) / 2);  // 320: five wavefronts, of which up / router use four
+
+template <int RK, int RLPR, int M, int UK, int ULPR, int DK, int DLPR>
+__global__ __launch_bounds__(kOneThreads) void moe_one_kernel(OneArgs a) {
+  __shared__ __attribute__((aligned(16))) char lds[one_lds_bytes<M>()];
+  const int wg = blockIdx.x;
+  if (wg < a.n_router) {
+    one_router<RK, RLPR, M>(a, wg, lds);
+  } else if (wg < a.n_router + a.n_up) {
+    one_up<UK, ULPR, true>(a, wg - a.n_router, lds);
+  } else {
+    one_down<DK, DLPR, true>(a, wg - a.n_router - a.n_up, lds);
+  }
+}
+
+// up + down only: the router (and the norm in its head) stays a launch of its own
+template <int UK, int ULPR, int DK, int DLPR>
+__global__ __launch_bounds__(kOneThreads) void moe_updown_kernel(OneArgs a) {
+  __shared__ __attribute__((aligned(16))) char lds[one_lds_bytes<1>() > 1024 ? 1024 : one_lds_bytes<1>()];
+  const int wg = blockIdx.x;
+  if (wg < a.n_up) {
+    one_up<UK, ULPR, false>(a, wg, lds);
+  } else {
+    one_down<DK, DLPR, false>(a, wg - a.n_up, lds);
+  }
+}
+
 KqPtr ptr_of(const ornith_kmatrix& m) {
   return KqPtr{(const uint8_t*)m.d_qs, (const uint8_t*)m.d_scales, (const uint16_t*)m.d_dm};
 }
@@ -526,6 +832,131 @@ int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
     ORN_LAUNCH_CHECK("moe_down_kernel");
   }
   return ORNITH_OK;
+}
+
+// The block in one launch (moe_one_kernel). Returns false with nothing launched when the
+// shapes / formats are outside the instantiated family: hidden size 2048 and expert width
+// 512 in one of the format mixes (router, gate/up, down) = (Q6_K, Q4_K, Q6_K), all Q4_K or
+// all Q6_K, T <= 4, a power-of-two expert count the top-k wavefront covers.
+// d_x: the block's input rows, or with `pre` where the normed rows are to be stored.
+bool moe_one_launch(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, void* d_gates,
+                    void* d_egate, uint32_t* d_inds, void* d_scores, void* d_act, void* d_out,
+                    const PreNorm* pre, int* rc) {
+  *rc = ORNITH_OK;
+  const ornith_linear& r = w->router;
+  const ornith_linear& g = w->sh_egate;
+  const int E = r.O, H = r.K, I = w->ex_gate.O, k = w->top_k;
+  const int how = ornith_option_fuse_moe_one();  // 1: router + up + down, 2: up + down (router launched first)
+  if (!how || !moe_fused_supported(w) || T < 1 || T > 4) return false;
+  if (r.mode != ORNITH_LIN_KQUANT || (g.mode != ORNITH_LIN_AFFINE8 && g.mode != ORNITH_LIN_DENSE)) return false;
+  if (H != kPreN || I != 512 || w->sh_gate.O != I || g.K != H) return false;
+  if (E % 64 != 0 || E > 1024 || ((E / 64) & (E / 64 - 1)) != 0 || k > kMaxK || k > E) return false;
+  const int rk = r.km.kind, uk = w->ex_gate.kind, dk = w->ex_down.kind;
+  const int mix = rk == ORNITH_Q6K && uk == ORNITH_Q4K && dk == ORNITH_Q6K   ? 0
+                  : rk == ORNITH_Q4K && uk == ORNITH_Q4K && dk == ORNITH_Q4K ? 1
+                  : rk == ORNITH_Q6K && uk == ORNITH_Q6K && dk == ORNITH_Q6K ? 2
+                                                                              : -1;
+  if (mix < 0) return false;
+  // flag words: router | routing | act, all inside the context's block
+  const int rlpr = rk == ORNITH_Q4K ? 64 : 32, ulpr = uk == ORNITH_Q4K ? 64 : 32, dlpr = dk == ORNITH_Q4K ? 16 : 8;
+  OneArgs a{};
+  a.n_router = how == 1 ? (E + (64 / rlpr) * 4 - 1) / ((64 / rlpr) * 4) + 1 : 0;
+  if (how != 1) {
+    // the router (with the norm in its head) as its own launch first
+    if (!moe_fused_router(ctx, w, d_x, T, d_gates, d_egate, rc, pre)) return false;
+    if (*rc) return true;
+    pre = nullptr;
+  }
+  a.up_x = (I + (64 / ulpr) * 4 * 2 - 1) / ((64 / ulpr) * 4 * 2);
+  const int rows_y = T * k + T;
+  a.n_up = a.up_x * rows_y;
+  a.down_x = (H + (64 / dlpr) - 1) / (64 / dlpr);
+  const int n_down = a.down_x * T;
+  if ((size_t)a.n_router + 4 + (size_t)rows_y * a.up_x > ornith_ctx::kHoFlagWords) return false;
+  if (ctx->ho_epoch == 0xffffffffu) {
+    // the epoch numbers are used up: start over from clean flag words
+    if (hipStreamSynchronize(ctx->stream) != hipSuccess ||
+        hipMemset(ctx->ho_flags, 0, sizeof(uint32_t) * ornith_ctx::kHoFlagWords) != hipSuccess) {
+      *rc = ornith_fail(ORNITH_ERR_HIP, "moe_block: resetting the hand-off flags failed");
+      return true;
+    }
+    ctx->ho_epoch = 0;
+  }
+  a.epoch = ++ctx->ho_epoch;
+  a.rflag = ctx->ho_flags;
+  a.iflag = a.rflag + a.n_router;
+  a.aflag = a.iflag + 4;
+  a.err = ctx->ho_err_dev;
+  a.max_spins = ornith_option_ho_spins();
+
+  a.r.w = ptr_of(r.km);
+  a.r.x = (const bf16_t*)d_x;
+  a.r.gates = (bf16_t*)d_gates;
+  a.r.egate = (bf16_t*)d_egate;
+  a.r.eg_w = g.d_w;
+  a.r.eg_s = (const bf16_t*)g.d_scales;
+  a.r.eg_b = (const bf16_t*)g.d_biases;
+  a.r.eg_affine = g.mode == ORNITH_LIN_AFFINE8;
+  a.r.E = E;
+  a.r.K = H;
+  if (pre) a.r.pre = *pre;
+
+  a.u.gate = ptr_of(w->ex_gate);
+  a.u.up = ptr_of(w->ex_up);
+  a.u.sgate = ptr_of(w->sh_gate.km);
+  a.u.sup = ptr_of(w->sh_up.km);
+  a.u.x = (const bf16_t*)d_x;
+  a.u.inds = d_inds;
+  a.u.act = (bf16_t*)d_act;
+  a.u.T = T;
+  a.u.k = k;
+  a.u.E = E;
+  a.u.I = I;
+  a.u.K = H;
+  a.u.gates = (const bf16_t*)d_gates;
+  a.u.inds_out = d_inds;
+  a.u.scores_out = (bf16_t*)d_scores;
+
+  a.d.down = ptr_of(w->ex_down);
+  a.d.sdown = ptr_of(w->sh_down.km);
+  a.d.act = (const bf16_t*)d_act;
+  a.d.inds = d_inds;
+  a.d.scores = (const bf16_t*)d_scores;
+  a.d.egate = (const bf16_t*)d_egate;
+  a.d.out = (bf16_t*)d_out;
+  a.d.T = T;
+  a.d.k = k;
+  a.d.E = E;
+  a.d.H = H;
+  a.d.I = I;
+  a.d.normalize = w->norm_topk_prob;
+
+  const dim3 grid(a.n_router + a.n_up + n_down), block(kOneThreads);
+#define ONE_M(RK, RL, UK, UL, DK, DL)                                                                         \
+  switch (T) {                                                                                                \
+    case 1: hipLaunchKernelGGL((moe_one_kernel<RK, RL, 1, UK, UL, DK, DL>), grid, block, 0, ctx->stream, a); break; \
+    case 2: hipLaunchKernelGGL((moe_one_kernel<RK, RL, 2, UK, UL, DK, DL>), grid, block, 0, ctx->stream, a); break; \
+    case 3: hipLaunchKernelGGL((moe_one_kernel<RK, RL, 3, UK, UL, DK, DL>), grid, block, 0, ctx->stream, a); break; \
+    default: hipLaunchKernelGGL((moe_one_kernel<RK, RL, 4, UK, UL, DK, DL>), grid, block, 0, ctx->stream, a); break; \
+  }
+  if (how != 1) {
+    if (mix == 0)
+      hipLaunchKernelGGL((moe_updown_kernel<ORNITH_Q4K, 64, ORNITH_Q6K, 8>), grid, block, 0, ctx->stream, a);
+    else if (mix == 1)
+      hipLaunchKernelGGL((moe_updown_kernel<ORNITH_Q4K, 64, ORNITH_Q4K, 16>), grid, block, 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((moe_updown_kernel<ORNITH_Q6K, 32, ORNITH_Q6K, 8>), grid, block, 0, ctx->stream, a);
+  } else if (mix == 0) {
+    ONE_M(ORNITH_Q6K, 32, ORNITH_Q4K, 64, ORNITH_Q6K, 8)
+  } else if (mix == 1) {
+    ONE_M(ORNITH_Q4K, 64, ORNITH_Q4K, 64, ORNITH_Q4K, 16)
+  } else {
+    ONE_M(ORNITH_Q6K, 32, ORNITH_Q6K, 32, ORNITH_Q6K, 8)
+  }
+#undef ONE_M
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) *rc = ornith_fail(ORNITH_ERR_HIP, "launch of moe_one_kernel failed: %s", hipGetErrorString(e));
+  return true;
 }
 
 extern "C" {

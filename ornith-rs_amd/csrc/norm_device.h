@@ -8,6 +8,7 @@
 #pragma once
 
 #include "dmath.h"
+#include "handoff.h"
 
 // PER consecutive bf16 values <-> fp32 registers, widest aligned access
 template <int PER>
@@ -123,7 +124,9 @@ struct PreNormLds {
   float inv[4];
 };
 
-template <int T>
+// COH: the normed rows stored by the `write_global` workgroup are read by other workgroups of
+// the same launch (handoff.h), so they go out as agent-scope stores.
+template <int T, bool COH = false>
 __device__ __forceinline__ void prenorm_rows(const PreNorm& p, bool write_global, PreNormLds<T>& s) {
   static_assert(T >= 1 && T <= 4, "one wavefront per row");
   constexpr int PER = kPreN / 64;
@@ -160,7 +163,15 @@ __device__ __forceinline__ void prenorm_rows(const PreNorm& p, bool write_global
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[t][i] = dm_rb(wv[i] * dm_rb(x[t][i] * inv));
     store_bf16<8>(&s.xn[t][e0], x[t]);
-    if (write_global) store_bf16<8>(p.normed_out + (size_t)t * kPreN + e0, x[t]);
+    if (write_global) {
+      if constexpr (COH) {
+        uint64_t* dst = reinterpret_cast<uint64_t*>(p.normed_out + (size_t)t * kPreN + e0);
+        ho_store_u64(dst, (uint64_t)pack_bf16x2(x[t][0], x[t][1]) | ((uint64_t)pack_bf16x2(x[t][2], x[t][3]) << 32));
+        ho_store_u64(dst + 1, (uint64_t)pack_bf16x2(x[t][4], x[t][5]) | ((uint64_t)pack_bf16x2(x[t][6], x[t][7]) << 32));
+      } else {
+        store_bf16<8>(p.normed_out + (size_t)t * kPreN + e0, x[t]);
+      }
+    }
   }
   __syncthreads();
 }

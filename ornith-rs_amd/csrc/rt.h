@@ -23,7 +23,18 @@ struct ornith_ctx {
   // a copy into pinned memory completes without the runtime's pageable detour
   void* pinned = nullptr;
   static constexpr size_t kPinnedBytes = 4096;
+  // hand-offs inside a launch (handoff.h): the flag words, the epoch handed to the next such
+  // launch, and the word a wait that ran out of its bound reports through (pinned host
+  // memory the kernels write directly; checked after every synchronisation)
+  uint32_t* ho_flags = nullptr;
+  static constexpr size_t kHoFlagWords = 16384;
+  uint32_t ho_epoch = 0;
+  volatile uint32_t* ho_err = nullptr;
+  uint32_t* ho_err_dev = nullptr;
 };
+
+// After the stream has been synchronised: fails if a hand-off wait inside a launch gave up.
+int ornith_check_handoffs(ornith_ctx* ctx);
 
 // Returns at least `bytes` of device scratch (256-byte aligned). Growing it
 // synchronises the stream; callers that must not allocate size it once up front.
@@ -96,5 +107,7 @@ int ornith_option_fuse_norm();
 int ornith_option_gemm_duo();  // 1: prefill GEMM with producer and consumer wavefronts; 0: every wavefront does both in turn
 int ornith_option_kq_iters();      // output rows per wavefront pass of the mat-vec kernels; 0 = by shape
 int ornith_option_moe_up_iters();  // rows per wavefront of the fused gate+up kernel; 0 = by shape
+int ornith_option_fuse_moe_one();  // 1: the MoE block's router, up and down phases in one launch
+int ornith_option_ho_spins();      // polling rounds a hand-off wait inside a launch may take
 
 static inline size_t ornith_dtype_size(int dt) { return dt == ORNITH_F32 ? 4 : 2; }

@@ -44,7 +44,9 @@ Option g_options[] = {{"fuse_moe", "ORNITH_FUSE_MOE", 1, -1},
                       {"gemm_rows", "ORNITH_GEMM_ROWS", 32, -1},
                       {"fuse_gdn", "ORNITH_FUSE_GDN", 1, -1},
                       {"fuse_norm", "ORNITH_FUSE_NORM", 1, -1},
-                      {"gemm_duo", "ORNITH_GEMM_DUO", 1, -1}};
+                      {"gemm_duo", "ORNITH_GEMM_DUO", 1, -1},
+                      {"fuse_moe_one", "ORNITH_FUSE_MOE_ONE", 0, -1},
+                      {"ho_spins", "ORNITH_HO_SPINS", 1 << 20, -1}};
 int option_value(int i) {
   Option& o = g_options[i];
   if (o.value < 0) {
@@ -62,6 +64,18 @@ int ornith_option_kq_iters() { return option_value(3); }
 int ornith_option_fuse_gdn() { return option_value(5); }
 int ornith_option_fuse_norm() { return option_value(6); }
 int ornith_option_gemm_duo() { return option_value(7); }
+int ornith_option_fuse_moe_one() { return option_value(8); }
+int ornith_option_ho_spins() { return option_value(9) < 1 ? 1 : option_value(9); }
+
+int ornith_check_handoffs(ornith_ctx* ctx) {
+  if (ctx->ho_err && *ctx->ho_err) {
+    *ctx->ho_err = 0;
+    return ornith_fail(ORNITH_ERR_HIP,
+                       "a wait between workgroups inside a launch ran out of its bound (ho_spins = %d): "
+                       "the results of that launch are invalid", ornith_option_ho_spins());
+  }
+  return ORNITH_OK;
+}
 int ornith_option_gemm_rows() {
   const int v = option_value(4);
   return v <= 0 ? 1 << 30 : v;
@@ -122,6 +136,13 @@ int ornith_ctx_create(int device, ornith_ctx** out) {
   ORN_HIP(hipEventCreate(&c->ev0));
   ORN_HIP(hipEventCreate(&c->ev1));
   ORN_HIP(hipHostMalloc(&c->pinned, ornith_ctx::kPinnedBytes, hipHostMallocDefault));
+  ORN_HIP(hipMalloc((void**)&c->ho_flags, sizeof(uint32_t) * ornith_ctx::kHoFlagWords));
+  ORN_HIP(hipMemset(c->ho_flags, 0, sizeof(uint32_t) * ornith_ctx::kHoFlagWords));
+  void* err_host = nullptr;
+  ORN_HIP(hipHostMalloc(&err_host, 256, hipHostMallocDefault));
+  memset(err_host, 0, 256);
+  c->ho_err = static_cast<volatile uint32_t*>(err_host);
+  ORN_HIP(hipHostGetDevicePointer((void**)&c->ho_err_dev, err_host, 0));
   *out = c;
   return ORNITH_OK;
 }
@@ -131,6 +152,8 @@ int ornith_ctx_destroy(ornith_ctx* ctx) {
   (void)hipStreamSynchronize(ctx->stream);
   if (ctx->scratch) (void)hipFree(ctx->scratch);
   if (ctx->pinned) (void)hipHostFree(ctx->pinned);
+  if (ctx->ho_flags) (void)hipFree(ctx->ho_flags);
+  if (ctx->ho_err) (void)hipHostFree(const_cast<uint32_t*>(ctx->ho_err));
   (void)hipEventDestroy(ctx->ev0);
   (void)hipEventDestroy(ctx->ev1);
   (void)hipStreamDestroy(ctx->stream);
@@ -141,7 +164,7 @@ int ornith_ctx_destroy(ornith_ctx* ctx) {
 int ornith_sync(ornith_ctx* ctx) {
   ORN_REQUIRE(ctx, "ornith_sync: null ctx");
   ORN_HIP(hipStreamSynchronize(ctx->stream));
-  return ORNITH_OK;
+  return ornith_check_handoffs(ctx);
 }
 
 int ornith_alloc(ornith_ctx* ctx, size_t bytes, void** d_out) {
@@ -177,11 +200,11 @@ int ornith_download(ornith_ctx* ctx, void* host, const void* d_src, size_t bytes
     ORN_HIP(hipMemcpyAsync(ctx->pinned, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
     ORN_HIP(hipStreamSynchronize(ctx->stream));
     memcpy(host, ctx->pinned, bytes);
-    return ORNITH_OK;
+    return ornith_check_handoffs(ctx);
   }
   ORN_HIP(hipMemcpyAsync(host, d_src, bytes, hipMemcpyDeviceToHost, ctx->stream));
   ORN_HIP(hipStreamSynchronize(ctx->stream));
-  return ORNITH_OK;
+  return ornith_check_handoffs(ctx);
 }
 
 int ornith_memset(ornith_ctx* ctx, void* d_dst, int byte, size_t bytes) {

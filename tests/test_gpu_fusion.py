@@ -42,6 +42,61 @@ def test_moe_fused_equals_unfused_and_oracle(orn, ctx, H, E, I, gk, dk):
         moe.free()
 
 
+@pytest.mark.parametrize("gk,dk,rk", [(Q4K, Q6K, Q6K), (Q4K, Q4K, Q4K), (Q6K, Q6K, Q6K)])
+def test_moe_block_in_one_launch_equals_separate_launches(orn, ctx, gk, dk, rk):
+    """The block's phases as workgroup ranges of one launch, handing gates / routing / expert
+    activations over through memory inside the launch (option fuse_moe_one = 1: router + up +
+    down, 2: up + down): same bits as the separate launches and as the oracle, T = 1..4, on the
+    three format mixes the launch is instantiated for; repeated so that every call meets the
+    flag words its predecessors left."""
+    rng = np.random.default_rng(77 + gk + 2 * dk)
+    moe = util.HostMoe(rng, H=2048, E=256, I=512, top_k=8, gate_kind=gk, down_kind=dk, router_kind=rk)
+    dw = moe.dev(orn, ctx)
+    try:
+        for T in (1, 2, 3, 4, 2):
+            xb = util.bf16_normal(rng, (T, 2048))
+            orn.set_option("fuse_moe_one", 0)
+            want = _block(orn, ctx, moe, dw, xb, T)
+            for how in (1, 2, 1):
+                orn.set_option("fuse_moe_one", how)
+                got = _block(orn, ctx, moe, dw, xb, T)
+                for a, b in zip(got, want):
+                    assert np.array_equal(a, b), (T, how)
+            if T == 2:
+                want_out, want_inds, _, _ = util.orc_moe_block(moe, xb, T)
+                assert np.array_equal(want[1], want_inds) and np.array_equal(want[0], want_out)
+    finally:
+        orn.set_option("fuse_moe_one", 0)
+        moe.free()
+
+
+def test_wait_inside_a_launch_gives_up_and_reports(orn, ctx):
+    """A wait between workgroups is bounded: with the bound forced to one polling round from the
+    host the consumers give up at once, every wavefront still exits, and the next
+    synchronisation reports the failure; the following call (bound restored) is right again."""
+    rng = np.random.default_rng(5)
+    moe = util.HostMoe(rng, H=2048, E=256, I=512, top_k=8)
+    dw = moe.dev(orn, ctx)
+    T = 2
+    xb = util.bf16_normal(rng, (T, 2048))
+    try:
+        orn.set_option("fuse_moe_one", 0)
+        want = _block(orn, ctx, moe, dw, xb, T)
+        orn.set_option("fuse_moe_one", 1)
+        orn.set_option("ho_spins", 1)
+        with pytest.raises(orn.OrnithError, match="ran out of its bound"):
+            for _ in range(4):       # a single polling round can succeed by luck; four launches do not
+                _block(orn, ctx, moe, dw, xb, T)
+        orn.set_option("ho_spins", 1 << 20)
+        got = _block(orn, ctx, moe, dw, xb, T)
+        for a, b in zip(got, want):
+            assert np.array_equal(a, b)
+    finally:
+        orn.set_option("ho_spins", 1 << 20)
+        orn.set_option("fuse_moe_one", 0)
+        moe.free()
+
+
 # shapes that take the other lane-per-row widths of the two expert kernels: K = 256 (8 Q4_K / 4 Q6_K
 # chunks a row), 1024, 2048 in either format, and the four-rows-a-wavefront form of the up kernel
 @pytest.mark.parametrize("H,E,I,gk,dk,iters", [(2048, 256, 512, Q4K, Q6K, 0), (2048, 256, 512, Q4K, Q6K, 4),
