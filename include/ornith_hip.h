@@ -563,16 +563,59 @@ ORNITH_API int ornith_top_sampler_destroy(ornith_top_sampler* s);
 ORNITH_API int ornith_top_sampler_sample(ornith_top_sampler* s, const void* d_logits_row,
                                          uint32_t* d_token_out);
 
+/* Which generator a TopSampler draws its random words from (default ORNITH_RNG_THREEFRY), and
+ * the next raw word of its stream (one key split, or one Philox counter value, per word). */
+ORNITH_API int ornith_top_sampler_set_rng(ornith_top_sampler* s, int rng);
+ORNITH_API int ornith_top_sampler_next_bits(ornith_top_sampler* s, uint32_t* bits_out);
+/* Philox4x32-10 (Salmon et al., SC'11; Random123's philox4x32 at 10 rounds): host function. */
+ORNITH_API void ornith_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]);
+
+/* ---- speculative sampling: no counterpart in the reference, which accepts drafts by token
+ * equality only and says so (src/mtp_generate.rs:27-35). A distribution is carried as
+ * unnormalised fp32 weights w[0..V) with their total in w[V] (V + 1 floats on the device);
+ * the probabilities are w[i] / w[V]. ---------------------------------------------------- */
+/* The distribution TopSampler draws from for one row of logits (log-softmax, top-p, top-k,
+ * temperature: src/sample.rs:79-190) as such weights. Consumes no random word. */
+ORNITH_API int ornith_sampler_weights(ornith_top_sampler* s, const void* d_logits_row, int V, float* d_w);
+/* inverse-CDF draw from such weights with the raw random word given (the draw of
+ * categorical_sampling, src/sample.rs:138-190, on weights already made) */
+ORNITH_API int ornith_draw_weights(ornith_ctx* ctx, const float* d_w, int V, uint32_t raw_bits,
+                                   uint32_t* d_token_out);
+/* weights over a pruned draft vocabulary (n entries, d_ids their vocabulary ids) placed in
+ * vocabulary space: zero off the list */
+ORNITH_API int ornith_spec_scatter(ornith_ctx* ctx, const float* d_w_local, const uint32_t* d_ids, int n,
+                                   int V, float* d_w_full);
+/* the draft token *d_x was drawn from q: *d_accept_out = (u * q(x) < p(x)), u uniform in [0, 1)
+ * from raw_bits, i.e. acceptance with probability min(1, p(x) / q(x)) */
+ORNITH_API int ornith_spec_accept(ornith_ctx* ctx, const float* d_wp, const float* d_wq, int V,
+                                  const uint32_t* d_x, uint32_t raw_bits, uint32_t* d_accept_out);
+/* the token for a rejected position: a draw from norm(max(0, p - q)); from p if that is empty */
+ORNITH_API int ornith_spec_resample(ornith_ctx* ctx, const float* d_wp, const float* d_wq, int V,
+                                    uint32_t raw_bits, uint32_t* d_token_out);
+
 /* ---- generation loops ---------------------------------------------------------------- */
 /* Sampler (src/generate.rs:36-64, src/sample.rs:205-225). rows_are_independent is
  * true for GREEDY. */
 #define ORNITH_SAMPLER_GREEDY 0
 #define ORNITH_SAMPLER_TOP_P 1
+/* how generate_step_mtp decides on a draft under a sampling sampler */
+#define ORNITH_ACCEPT_EQUALITY 0 /* the reference's rule: the target's own sample must equal the draft
+                                    (src/mtp_generate.rs:27-35, 255-279); drafts are the head's argmax */
+#define ORNITH_ACCEPT_RATIO 1    /* speculative sampling, which the reference names as not carried
+                                    (src/mtp_generate.rs:27-30): drafts are drawn from the head's
+                                    distribution q, accepted with probability min(1, p/q), and a
+                                    rejected position is redrawn from norm(max(0, p - q)) */
+/* where the sampler's random words come from */
+#define ORNITH_RNG_THREEFRY 0 /* the reference's key sequence (src/ops/random.rs:16-67) */
+#define ORNITH_RNG_PHILOX 1   /* Philox4x32-10: draw n of a seed is word 0 of
+                                 philox(counter = (n, 0, 0, 0) as 64 + 64 bits, key = seed) */
 typedef struct ornith_sampler {
   int kind;
-  float temperature, top_p;
+  double temperature, top_p; /* as TopSampler::new(f64, f64, ..) takes them (src/sample.rs:205-225) */
   int top_k;
   uint64_t seed;
+  int accept; /* ORNITH_ACCEPT_*; ignored by GREEDY and by generate_step */
+  int rng;    /* ORNITH_RNG_* */
 } ornith_sampler;
 /* on_token: return 0 to stop (FnMut(u32) -> bool); progress: (done, total) prompt tokens */
 typedef int (*ornith_token_cb)(uint32_t token, void* user);

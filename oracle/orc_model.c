@@ -328,26 +328,52 @@ static struct {
   double temp, top_p;
   int top_k;
   uint64_t seed;
+  int accept; /* 0: token equality (the reference), 1: probability ratio (speculative sampling) */
+  int rng;    /* 0: threefry key sequence (the reference), 1: Philox4x32-10 counter stream */
   uint32_t key[2];
+  uint64_t philox_n;
 } g_sampler;
 extern void orc_key_from_seed(uint64_t seed, uint32_t key[2]);
-extern uint32_t orc_top_sample(const bf16_t* logits, int V, double temp, double top_p, int top_k,
-                               uint32_t key_state[2]);
-ORC_API void orc_set_sampler(int kind, double temp, double top_p, int top_k, uint64_t seed) {
+extern void orc_key_next(uint32_t state[2], uint32_t sub[2]);
+extern void orc_random_bits(const uint32_t key[2], int n, uint32_t* out);
+extern uint32_t orc_philox_draw(uint64_t seed, uint64_t n);
+extern uint32_t orc_top_sample_bits(const bf16_t* logits, int V, double temp, double top_p, int top_k, uint32_t raw);
+extern float orc_sampler_weights(const bf16_t* logits, int V, double temp, double top_p, int top_k, float* w);
+extern uint32_t orc_draw_weights(const float* w, int V, uint32_t bits);
+extern int orc_spec_accept(const float* wp, float sp, const float* wq, float sq, uint32_t x, uint32_t bits);
+extern uint32_t orc_spec_resample(const float* wp, float sp, const float* wq, float sq, int V, uint32_t bits);
+ORC_API void orc_set_sampler2(int kind, double temp, double top_p, int top_k, uint64_t seed, int accept, int rng) {
   g_sampler.kind = kind;
   g_sampler.temp = temp;
   g_sampler.top_p = top_p;
   g_sampler.top_k = top_k;
   g_sampler.seed = seed;
+  g_sampler.accept = accept;
+  g_sampler.rng = rng;
 }
-static void sampler_begin(void) { orc_key_from_seed(g_sampler.seed, g_sampler.key); }
+ORC_API void orc_set_sampler(int kind, double temp, double top_p, int top_k, uint64_t seed) {
+  orc_set_sampler2(kind, temp, top_p, top_k, seed, 0, 0);
+}
+static void sampler_begin(void) {
+  orc_key_from_seed(g_sampler.seed, g_sampler.key);
+  g_sampler.philox_n = 0;
+}
+/* the next raw random word of the sampler's stream: one key split (threefry) or one counter
+ * value (Philox) per draw */
+static uint32_t next_bits(void) {
+  if (g_sampler.rng == 1) return orc_philox_draw(g_sampler.seed, g_sampler.philox_n++);
+  uint32_t sub[2], raw;
+  orc_key_next(g_sampler.key, sub);
+  orc_random_bits(sub, 1, &raw);
+  return raw;
+}
 static uint32_t sample_row(const bf16_t* logits, int V) {
   if (g_sampler.kind == 0) {
     uint32_t t;
     orc_greedy_rows(logits, 1, V, &t, NULL);
     return t;
   }
-  return orc_top_sample(logits, V, g_sampler.temp, g_sampler.top_p, g_sampler.top_k, g_sampler.key);
+  return orc_top_sample_bits(logits, V, g_sampler.temp, g_sampler.top_p, g_sampler.top_k, next_bits());
 }
 
 /* generate_step; returns the number of tokens written */
@@ -407,6 +433,16 @@ ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* f
   bf16_t *vlogits = malloc(2 * (size_t)W * V), *dlogits = malloc(2 * (size_t)V), *tmp = malloc(2 * (size_t)W * H);
   uint32_t* window = malloc(4 * (size_t)W);
   uint32_t* targets = malloc(4 * (size_t)W);
+  /* probability-ratio acceptance: the drafts are DRAWN from the head's distribution q (under the
+   * sampler's own temperature / top-p / top-k) and kept, in vocabulary space, for the verify */
+  const int ratio = g_sampler.kind != 0 && g_sampler.accept == 1;
+  float *wq = NULL, *wp = NULL, *wloc = NULL, *sq = NULL;
+  if (ratio) {
+    wq = calloc((size_t)depth * V, 4);
+    wp = malloc(4 * (size_t)V);
+    wloc = malloc(4 * (size_t)V);
+    sq = malloc(4 * (size_t)depth);
+  }
   int processed = 0;
   while (n_prompt - processed > 1) {
     int n = prefill_step < n_prompt - processed - 1 ? prefill_step : n_prompt - processed - 1;
@@ -433,7 +469,16 @@ ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* f
     for (int i = 0; i < want; ++i) {
       bf16_t* hi = mh + (size_t)i * H;
       orc_mtp_hidden(s, w, hcur, window + i, 1, hi);
-      if (fr_head) {
+      if (ratio) {
+        const int Vd = fr_head ? fr_n : V;
+        orc_linear_fwd(fr_head ? fr_head : &m->lm_head, hi, 1, dlogits);
+        sq[i] = orc_sampler_weights(dlogits, Vd, g_sampler.temp, g_sampler.top_p, g_sampler.top_k, wloc);
+        const uint32_t local = orc_draw_weights(wloc, Vd, next_bits());
+        window[i + 1] = fr_head ? fr_ids[local] : local;
+        float* q = wq + (size_t)i * V;
+        memset(q, 0, 4 * (size_t)V);
+        for (int l = 0; l < Vd; ++l) q[fr_head ? fr_ids[l] : (uint32_t)l] = wloc[l];
+      } else if (fr_head) {
         uint32_t local;
         orc_linear_fwd(fr_head, hi, 1, dlogits);
         orc_argmax_rows(dlogits, 1, fr_n, &local);
@@ -454,9 +499,21 @@ ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* f
     int k = 0, have = 0;
     uint32_t next_primary = 0;
     while (k < want) {
-      const uint32_t target = independent ? targets[k] : sample_row(vlogits + (size_t)k * V, V);
-      stats->reached[k]++;
-      if (target != window[1 + k]) { next_primary = target; have = 1; break; }
+      if (ratio) {
+        const float sp = orc_sampler_weights(vlogits + (size_t)k * V, V, g_sampler.temp, g_sampler.top_p,
+                                             g_sampler.top_k, wp);
+        const float* q = wq + (size_t)k * V;
+        stats->reached[k]++;
+        if (!orc_spec_accept(wp, sp, q, sq[k], window[1 + k], next_bits())) {
+          next_primary = orc_spec_resample(wp, sp, q, sq[k], V, next_bits());
+          have = 1;
+          break;
+        }
+      } else {
+        const uint32_t target = independent ? targets[k] : sample_row(vlogits + (size_t)k * V, V);
+        stats->reached[k]++;
+        if (target != window[1 + k]) { next_primary = target; have = 1; break; }
+      }
       stats->accepted_by[k]++;
       stats->accepted++;
       k++;
@@ -476,5 +533,6 @@ ORC_API int orc_mtp_generate(orc_state* s, const orc_mtp_w* w, const uint32_t* f
   }
 done:
   free(hid); free(h); free(mh); free(vlogits); free(dlogits); free(tmp); free(window); free(targets);
+  free(wq); free(wp); free(wloc); free(sq);
   return emitted;
 }

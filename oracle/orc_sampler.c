@@ -194,18 +194,27 @@ ORC_API void orc_apply_top_k(const bf16_t* lp, int V, int top_k, bf16_t* out) {
   free(order);
 }
 
-/* mx.random.categorical(logits * (1/temp)) with the given raw random word */
-ORC_API uint32_t orc_categorical(const bf16_t* lp, int V, double temp, uint32_t bits) {
+/* weights of mx.random.categorical(lp * (1/temp)): x = float(bf16(lp * bf16(1/temp))), m = max x,
+ * w = isinf(m) ? (x == m) : exp(x - m); returns their sum in the scan's order */
+ORC_API float orc_categorical_weights(const bf16_t* lp, int V, double temp, float* w) {
   const float scale = orc_bf16_to_f32(orc_f32_to_bf16((float)(1.0 / temp)));
-  float* x = (float*)malloc(sizeof(float) * (size_t)V * 3);
-  float *w = x + V, *cdf = w + V;
   float m = -INFINITY;
   for (int i = 0; i < V; ++i) {
-    x[i] = orc_rb(orc_bf16_to_f32(lp[i]) * scale);
-    m = x[i] > m ? x[i] : m;
+    w[i] = orc_rb(orc_bf16_to_f32(lp[i]) * scale);
+    m = w[i] > m ? w[i] : m;
   }
   const int inf = (m == INFINITY) || (m == -INFINITY);
-  for (int i = 0; i < V; ++i) w[i] = inf ? (x[i] == m ? 1.f : 0.f) : orc_expf(x[i] - m);
+  for (int i = 0; i < V; ++i) w[i] = inf ? (w[i] == m ? 1.f : 0.f) : orc_expf(w[i] - m);
+  float* cdf = (float*)malloc(sizeof(float) * (size_t)V);
+  const float total = orc_cumsum_f32(w, V, cdf);
+  free(cdf);
+  return total;
+}
+
+/* inverse-CDF draw from unnormalised weights with the given raw random word: the first index
+ * whose inclusive cumulative sum exceeds u * total, else the last index of positive weight */
+ORC_API uint32_t orc_draw_weights(const float* w, int V, uint32_t bits) {
+  float* cdf = (float*)malloc(sizeof(float) * (size_t)V);
   const float total = orc_cumsum_f32(w, V, cdf);
   const float u = orc_uniform_scaled(bits, total);
   uint32_t tok = 0xffffffffu, last = 0;
@@ -213,15 +222,22 @@ ORC_API uint32_t orc_categorical(const bf16_t* lp, int V, double temp, uint32_t 
     if (w[i] > 0.f) last = (uint32_t)i;
     if (tok == 0xffffffffu && cdf[i] > u) tok = (uint32_t)i;
   }
-  free(x);
+  free(cdf);
   return tok == 0xffffffffu ? last : tok;
 }
 
-/* TopSampler::sample (sample.rs:205-225): one token from one row of logits; advances the key */
-ORC_API uint32_t orc_top_sample(const bf16_t* logits, int V, double temp, double top_p, int top_k,
-                                uint32_t key_state[2]) {
-  bf16_t* a = (bf16_t*)malloc(sizeof(bf16_t) * (size_t)V * 2);
-  bf16_t* b = a + V;
+/* mx.random.categorical(logits * (1/temp)) with the given raw random word */
+ORC_API uint32_t orc_categorical(const bf16_t* lp, int V, double temp, uint32_t bits) {
+  float* w = (float*)malloc(sizeof(float) * (size_t)V);
+  orc_categorical_weights(lp, V, temp, w);
+  const uint32_t tok = orc_draw_weights(w, V, bits);
+  free(w);
+  return tok;
+}
+
+/* log-softmax, then top-p / top-k as configured: the filtered log-probabilities the draw sees */
+static void filtered_logprobs(const bf16_t* logits, int V, double top_p, int top_k, bf16_t* a) {
+  bf16_t* b = (bf16_t*)malloc(sizeof(bf16_t) * (size_t)V);
   orc_logprobs_row(logits, V, a);
   if (top_p > 0.0 && top_p < 1.0) {
     orc_apply_top_p(a, V, top_p, b);
@@ -231,10 +247,91 @@ ORC_API uint32_t orc_top_sample(const bf16_t* logits, int V, double temp, double
     orc_apply_top_k(a, V, top_k, b);
     memcpy(a, b, sizeof(bf16_t) * (size_t)V);
   }
+  free(b);
+}
+
+/* The sampler's distribution over one row of logits as unnormalised weights (the probabilities
+ * TopSampler draws with are w / total); returns the total. */
+ORC_API float orc_sampler_weights(const bf16_t* logits, int V, double temp, double top_p, int top_k, float* w) {
+  bf16_t* a = (bf16_t*)malloc(sizeof(bf16_t) * (size_t)V);
+  filtered_logprobs(logits, V, top_p, top_k, a);
+  const float total = orc_categorical_weights(a, V, temp, w);
+  free(a);
+  return total;
+}
+
+/* TopSampler::sample with the raw random word given (sample.rs:205-225) */
+ORC_API uint32_t orc_top_sample_bits(const bf16_t* logits, int V, double temp, double top_p, int top_k,
+                                     uint32_t raw) {
+  bf16_t* a = (bf16_t*)malloc(sizeof(bf16_t) * (size_t)V);
+  filtered_logprobs(logits, V, top_p, top_k, a);
+  const uint32_t tok = orc_categorical(a, V, temp, raw);
+  free(a);
+  return tok;
+}
+
+/* TopSampler::sample (sample.rs:205-225): one token from one row of logits; advances the key */
+ORC_API uint32_t orc_top_sample(const bf16_t* logits, int V, double temp, double top_p, int top_k,
+                                uint32_t key_state[2]) {
   uint32_t sub[2], raw;
   orc_key_next(key_state, sub);
   orc_random_bits(sub, 1, &raw);
-  const uint32_t tok = orc_categorical(a, V, temp, raw);
-  free(a);
+  return orc_top_sample_bits(logits, V, temp, top_p, top_k, raw);
+}
+
+/* ---- Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3",
+ * SC'11; the Random123 library's philox4x32 with 10 rounds). Not in the reference, whose
+ * sampler draws from threefry keys; the counter-based generator the sampled speculative
+ * configuration asks for. ctr: 128-bit counter, key: 64-bit key. ------------------------- */
+ORC_API void orc_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* the sampler's stream under Philox: draw number n of seed s is word 0 of
+ * philox(counter = (n_lo, n_hi, 0, 0), key = (s_lo, s_hi)) */
+ORC_API uint32_t orc_philox_draw(uint64_t seed, uint64_t n) {
+  const uint32_t ctr[4] = {(uint32_t)n, (uint32_t)(n >> 32), 0u, 0u};
+  const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  uint32_t out[4];
+  orc_philox4x32_10(ctr, key, out);
+  return out[0];
+}
+
+/* ---- speculative sampling (Leviathan, Kalman, Matias 2023; Chen et al. 2023). Not carried by
+ * the reference, which accepts a draft by token equality only and says so
+ * (src/mtp_generate.rs:27-35). The draft token x was drawn from q; it is accepted with
+ * probability min(1, p(x) / q(x)); on rejection the token is drawn from norm(max(0, p - q)).
+ * The committed token is then distributed exactly as p whatever q is.
+ *   wp / wq: unnormalised weights over the vocabulary, sp / sq their totals (q lives in
+ *   vocabulary space: zero outside a pruned draft vocabulary).
+ * orc_spec_accept: u = uniform(bits); accept iff u * q(x) < p(x), p(x) = wp[x] / sp,
+ *   q(x) = wq[x] / sq (so p(x) >= q(x) always accepts, since u < 1).
+ * orc_spec_resample: r_y = max(0, wp[y] / sp - wq[y] / sq), inverse-CDF draw over r with
+ *   fresh bits; if every r_y is zero (p == q to the last bit) the draw is over wp instead. */
+ORC_API int orc_spec_accept(const float* wp, float sp, const float* wq, float sq, uint32_t x, uint32_t bits) {
+  const float px = wp[x] / sp, qx = wq[x] / sq;
+  const float u = orc_uniform_scaled(bits, 1.0f);
+  return u * qx < px;
+}
+
+ORC_API uint32_t orc_spec_resample(const float* wp, float sp, const float* wq, float sq, int V, uint32_t bits) {
+  float* r = (float*)malloc(sizeof(float) * (size_t)V * 2);
+  float* cdf = r + V;
+  for (int y = 0; y < V; ++y) {
+    const float d = wp[y] / sp - wq[y] / sq;
+    r[y] = d > 0.f ? d : 0.f;
+  }
+  const float total = orc_cumsum_f32(r, V, cdf);
+  const uint32_t tok = total > 0.f ? orc_draw_weights(r, V, bits) : orc_draw_weights(wp, V, bits);
+  free(r);
   return tok;
 }

@@ -46,6 +46,7 @@ struct LoopSampler {
   ornith_ctx* ctx = nullptr;
   ornith_top_sampler* top = nullptr;
   int V = 0;
+  bool ratio = false;  // drafts drawn from the head's distribution and accepted by probability ratio
   ~LoopSampler() {
     if (top) ornith_top_sampler_destroy(top);
   }
@@ -55,8 +56,14 @@ struct LoopSampler {
     V = vocab;
     if (s->kind == ORNITH_SAMPLER_GREEDY) return ORNITH_OK;
     ORN_REQUIRE(s->kind == ORNITH_SAMPLER_TOP_P, "unknown sampler kind %d", s->kind);
-    return ornith_top_sampler_create(c, s->temperature, s->top_p, s->top_k, s->seed, vocab, &top);
+    ORN_REQUIRE(s->accept == ORNITH_ACCEPT_EQUALITY || s->accept == ORNITH_ACCEPT_RATIO,
+                "unknown acceptance rule %d", s->accept);
+    ORN_REQUIRE(s->rng == ORNITH_RNG_THREEFRY || s->rng == ORNITH_RNG_PHILOX, "unknown generator %d", s->rng);
+    TRY(ornith_top_sampler_create(c, s->temperature, s->top_p, s->top_k, s->seed, vocab, &top));
+    ratio = s->accept == ORNITH_ACCEPT_RATIO;
+    return ornith_top_sampler_set_rng(top, s->rng);
   }
+  int next_bits(uint32_t* bits) { return ornith_top_sampler_next_bits(top, bits); }
   bool rows_are_independent() const { return top == nullptr; }
   // one row of logits -> token on the device
   int sample(const void* d_logits_row, uint32_t* d_token) {
@@ -93,6 +100,11 @@ int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, s
                     ornith_progress_cb progress, ornith_token_cb on_token, void* user) {
   ORN_REQUIRE(m && c && prompt && on_token, "generate: null argument");
   ORN_REQUIRE(n_prompt >= 1, "generate_step needs a prompt");
+  // the caches are of fixed capacity (the reference's grow in steps of 256): refuse a run that
+  // cannot finish before any token has been handed out
+  ORN_REQUIRE((size_t)c->offset + n_prompt + max_tokens <= (size_t)c->capacity,
+              "generate: %d cached + %zu prompt + %zu new tokens exceed cache capacity %d", c->offset, n_prompt,
+              max_tokens, c->capacity);
   ornith_ctx* ctx = m->ctx;
   const size_t H = m->cfg.hidden_size, V = m->cfg.vocab_size, R = m->max_rows;
   LoopSampler smp;
@@ -147,11 +159,29 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   ORN_REQUIRE(policy == ORNITH_HISTORY_CYCLE || policy == ORNITH_HISTORY_COMMITTED,
               "mtp_generate: unknown history policy %d", policy);
   ORN_REQUIRE(head->m == m && (!frspec || frspec->m == m), "mtp_generate: head / frspec of another model");
+  if (stats_out) *stats_out = ornith_mtp_stats{};  // defined on every return, error returns included
+  // fixed-capacity caches: a verify window holds up to `depth` rows beyond the committed ones;
+  // the head's own cache holds one row per committed token under Committed, a cycle's rows under
+  // Cycle. Refuse up front rather than fail between two tokens already handed out.
+  ORN_REQUIRE((size_t)c->offset + n_prompt + max_tokens + (size_t)depth <= (size_t)c->capacity,
+              "mtp_generate: %d cached + %zu prompt + %zu new tokens + a %d-row window exceed cache capacity %d",
+              c->offset, n_prompt, max_tokens, depth, c->capacity);
+  ORN_REQUIRE((size_t)head->capacity >= (policy == ORNITH_HISTORY_COMMITTED ? max_tokens + (size_t)depth : (size_t)depth),
+              "mtp_generate: the head's cache of %d rows is too small for %zu tokens at depth %d under this "
+              "history policy", head->capacity, max_tokens, depth);
   ornith_ctx* ctx = m->ctx;
   const size_t H = m->cfg.hidden_size, V = m->cfg.vocab_size, R = m->max_rows;
   LoopSampler smp;
   TRY(smp.init(ctx, sampler, (int)V));
   ornith_mtp_stats stats{};
+  // an error return below still reports the cycles counted so far
+  struct StatsOut {
+    ornith_mtp_stats* out;
+    const ornith_mtp_stats* cur;
+    ~StatsOut() {
+      if (out) *out = *cur;
+    }
+  } stats_guard{stats_out, &stats};
 
   Bufs b(ctx);
   uint32_t *d_tok, *d_window, *d_targets;
@@ -165,6 +195,16 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   TRY(b.get(V * 2, &d_dlogits));
   TRY(b.get(W * H * 2, &d_mh));
   TRY(b.get(W * H * 2, &d_scratch_h));
+  // probability-ratio acceptance keeps every draft level's distribution q (vocabulary space)
+  // for the verify pass, the target's p of the row in hand, and a flag word
+  float *d_wq = nullptr, *d_wp = nullptr, *d_wloc = nullptr;
+  uint32_t* d_flag = nullptr;
+  if (smp.ratio) {
+    TRY(b.get((size_t)depth * (V + 1) * 4, (void**)&d_wq));
+    TRY(b.get((V + 1) * 4, (void**)&d_wp));
+    TRY(b.get((V + 1) * 4, (void**)&d_wloc));
+    TRY(b.get(4, (void**)&d_flag));
+  }
 
   size_t processed = 0;
   TRY(prefill(m, c, prompt, n_prompt, prefill_step, d_tok, d_hidden, progress, user, &processed));
@@ -200,7 +240,21 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
     for (int i = 0; i < want; ++i) {
       void* hid = (char*)d_mh + (size_t)i * H * 2;
       TRY(ornith_mtp_forward(head, frspec, hcur, d_window + i, 1, hid, d_dlogits));
-      if (frspec) {
+      if (smp.ratio) {
+        // the draft is DRAWN from the head's distribution under the sampler's own settings
+        float* q = d_wq + (size_t)i * (V + 1);
+        uint32_t bits = 0;
+        TRY(smp.next_bits(&bits));
+        if (frspec) {
+          TRY(ornith_sampler_weights(smp.top, d_dlogits, draft_vocab, d_wloc));
+          TRY(ornith_draw_weights(ctx, d_wloc, draft_vocab, bits, d_flag));
+          TRY(ornith_gather_rows(ctx, frspec->d_ids, 4, d_flag, 1, d_window + i + 1));  // map_id
+          TRY(ornith_spec_scatter(ctx, d_wloc, frspec->d_ids, draft_vocab, (int)V, q));
+        } else {
+          TRY(ornith_sampler_weights(smp.top, d_dlogits, (int)V, q));
+          TRY(ornith_draw_weights(ctx, q, (int)V, bits, d_window + i + 1));
+        }
+      } else if (frspec) {
         // FrSpec::map_id rides in the argmax's last launch
         TRY(argmax_rows_mapped(ctx, d_dlogits, 1, draft_vocab, frspec->d_ids, d_window + i + 1));
       } else {
@@ -242,13 +296,32 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
     bool have_next = false;
     uint32_t next_primary = 0;
     while (k < want) {
-      uint32_t target = 0;
-      TRY(take(k, &target));
-      stats.reached_by_depth[k] += 1;
-      if (target != win[1 + k]) {
-        next_primary = target;
-        have_next = true;
-        break;
+      if (smp.ratio) {
+        // accept with probability min(1, p(x) / q(x)); a rejected position is redrawn from
+        // norm(max(0, p - q)) and ends the cycle
+        const float* q = d_wq + (size_t)k * (V + 1);
+        uint32_t bits = 0, ok = 0;
+        TRY(ornith_sampler_weights(smp.top, (const char*)d_vlogits + (size_t)k * V * 2, (int)V, d_wp));
+        TRY(smp.next_bits(&bits));
+        TRY(ornith_spec_accept(ctx, d_wp, q, (int)V, d_window + 1 + k, bits, d_flag));
+        TRY(ornith_download(ctx, &ok, d_flag, 4));
+        stats.reached_by_depth[k] += 1;
+        if (!ok) {
+          TRY(smp.next_bits(&bits));
+          TRY(ornith_spec_resample(ctx, d_wp, q, (int)V, bits, d_targets + k));
+          TRY(ornith_download(ctx, &next_primary, d_targets + k, 4));
+          have_next = true;
+          break;
+        }
+      } else {
+        uint32_t target = 0;
+        TRY(take(k, &target));
+        stats.reached_by_depth[k] += 1;
+        if (target != win[1 + k]) {
+          next_primary = target;
+          have_next = true;
+          break;
+        }
       }
       stats.accepted_by_depth[k] += 1;
       stats.accepted += 1;

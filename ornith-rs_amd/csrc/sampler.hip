@@ -54,6 +54,21 @@ void threefry2x32(const uint32_t key[2], uint32_t c0, uint32_t c1, uint32_t out[
   out[1] = y;
 }
 
+// ---- Philox4x32-10 (host): Salmon, Moraes, Dror, Shaw, "Parallel random numbers: as easy as
+// 1, 2, 3" (SC'11); Random123's philox4x32 at 10 rounds ---------------------------------
+void philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3], k0 = key[0], k1 = key[1];
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n1 = (uint32_t)p1;
+    const uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1, n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
 // ---- radix sort ----------------------------------------------------------------------
 __device__ __forceinline__ uint32_t sort_key(uint32_t b) {
   return (b & 0x8000u) ? (0xFFFFu - b) : (b | 0x8000u);
@@ -348,11 +363,14 @@ __global__ __launch_bounds__(RB) void cat_weights_kernel(float* x, int n, const 
 }
 
 // u = min(float(bits) / 2^32, nextafter(1, 0)) * total; first index with cdf > u, last with w > 0
+// (first_last[2], when asked for, receives the bits of the row total)
 __global__ __launch_bounds__(RB) void cat_search_kernel(const float* vloc, const float* segoff,
                                                         const float* chunk_tot, const float* w, int n,
-                                                        int nch, uint32_t bits, uint32_t* first_last) {
+                                                        int nch, uint32_t bits, uint32_t* first_last,
+                                                        bool store_total) {
   float base, total;
   chunk_base<false>(chunk_tot, nch, base, total);
+  if (store_total && blockIdx.x == 0 && threadIdx.x == 0) first_last[2] = __float_as_uint(total);
   const int i = blockIdx.x * RB + threadIdx.x;
   float u = (float)bits / 4294967296.0f;
   const float upper = __uint_as_float(0x3f7fffffu);
@@ -468,10 +486,90 @@ int categorical_impl(ornith_ctx* ctx, const bf16_t* lp, int V, double temp, uint
                      b.segoff, b.chunk_tot);
   hipLaunchKernelGGL(cat_init_kernel, dim3(1), dim3(1), 0, ctx->stream, fl);
   hipLaunchKernelGGL(cat_search_kernel, dim3(nch), dim3(RB), 0, ctx->stream, b.vloc, b.segoff,
-                     b.chunk_tot, x, V, nch, bits, fl);
+                     b.chunk_tot, x, V, nch, bits, fl, false);
   hipLaunchKernelGGL(cat_pick_kernel, dim3(1), dim3(1), 0, ctx->stream, fl, token);
   ORN_LAUNCH_CHECK("categorical kernels");
   return ORNITH_OK;
+}
+
+// ---- distributions as weights, speculative sampling ----------------------------------------
+// w[n] = the row total of w[0..n) in the scan's order
+__global__ __launch_bounds__(RB) void weights_total_kernel(const float* chunk_tot, int nch, float* w, int n) {
+  float base, total;
+  chunk_base<false>(chunk_tot, nch, base, total);
+  if (threadIdx.x == 0) w[n] = total;
+}
+
+// the categorical weights of filtered log-probabilities: w[0..V) and their total in w[V]
+int weights_impl(ornith_ctx* ctx, const bf16_t* lp, int V, double temp, float* w, ScratchCursor& sc) {
+  const int nch = nchunks(V);
+  float* pmax = sc.take<float>(nch);
+  ScanBufs b = scan_bufs(sc, V);
+  const float s32 = (float)(1.0 / temp);
+  uint32_t u;
+  memcpy(&u, &s32, 4);
+  u = (u + 0x7fffu + ((u >> 16) & 1u)) & 0xffff0000u;
+  float scale;
+  memcpy(&scale, &u, 4);
+  hipLaunchKernelGGL(cat_scale_kernel, dim3(nch), dim3(RB), 0, ctx->stream, lp, V, scale, w, pmax);
+  hipLaunchKernelGGL(cat_weights_kernel, dim3(nch), dim3(RB), 0, ctx->stream, w, V, pmax, nch);
+  hipLaunchKernelGGL(scan_local_kernel<false>, dim3(nch), dim3(RB), 0, ctx->stream, w, V, b.vloc, b.segoff,
+                     b.chunk_tot);
+  hipLaunchKernelGGL(weights_total_kernel, dim3(1), dim3(RB), 0, ctx->stream, b.chunk_tot, nch, w, V);
+  ORN_LAUNCH_CHECK("sampler weights kernels");
+  return ORNITH_OK;
+}
+
+// scan + search of one weight vector; leaves (first, last[, total bits]) in fl
+int search_weights(ornith_ctx* ctx, const float* w, int V, uint32_t bits, uint32_t* fl, bool store_total,
+                   ScratchCursor& sc) {
+  const int nch = nchunks(V);
+  ScanBufs b = scan_bufs(sc, V);
+  hipLaunchKernelGGL(scan_local_kernel<false>, dim3(nch), dim3(RB), 0, ctx->stream, w, V, b.vloc, b.segoff,
+                     b.chunk_tot);
+  hipLaunchKernelGGL(cat_init_kernel, dim3(1), dim3(1), 0, ctx->stream, fl);
+  hipLaunchKernelGGL(cat_search_kernel, dim3(nch), dim3(RB), 0, ctx->stream, b.vloc, b.segoff, b.chunk_tot, w, V,
+                     nch, bits, fl, store_total);
+  return ORNITH_OK;
+}
+
+__global__ void spec_zero_kernel(float* w, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) w[i] = 0.f;
+}
+// full[ids[l]] = local[l]; full[V] = local[n]
+__global__ void spec_scatter_kernel(const float* local, const uint32_t* ids, int n, int V, float* full) {
+  const int l = blockIdx.x * blockDim.x + threadIdx.x;
+  if (l < n) {
+    const uint32_t id = ids[l];
+    if (id < (uint32_t)V) full[id] = local[l];
+  }
+  if (l == 0) full[V] = local[n];
+}
+// accept iff u * q(x) < p(x)
+__global__ void spec_accept_kernel(const float* wp, const float* wq, int V, const uint32_t* x_ptr, uint32_t bits,
+                                   uint32_t* accept) {
+  const uint32_t x = min(x_ptr[0], (uint32_t)(V - 1));
+  const float px = wp[x] / wp[V], qx = wq[x] / wq[V];
+  float u = (float)bits / 4294967296.0f;
+  const float upper = __uint_as_float(0x3f7fffffu);
+  u = u < upper ? u : upper;
+  u = 1.0f * u + 0.0f;
+  u = u * 1.0f;
+  accept[0] = u * qx < px ? 1u : 0u;
+}
+// r = max(0, p - q)
+__global__ void spec_residual_kernel(const float* wp, const float* wq, int V, float* r) {
+  const int y = blockIdx.x * blockDim.x + threadIdx.x;
+  if (y < V) {
+    const float d = wp[y] / wp[V] - wq[y] / wq[V];
+    r[y] = d > 0.f ? d : 0.f;
+  }
+}
+// the residual's draw if it has any mass, the target's otherwise
+__global__ void spec_pick_kernel(const uint32_t* fl_r, const uint32_t* fl_p, uint32_t* token) {
+  const uint32_t* fl = __uint_as_float(fl_r[2]) > 0.f ? fl_r : fl_p;
+  token[0] = fl[0] != 0xffffffffu ? fl[0] : fl[1];
 }
 
 size_t sampler_workspace(int V) {
@@ -487,7 +585,44 @@ struct ornith_top_sampler {
   double temp, top_p;
   int top_k, vocab;
   uint32_t key[2];
+  int rng = ORNITH_RNG_THREEFRY;
+  uint64_t seed = 0, philox_n = 0;
 };
+
+namespace {
+// the filtered log-probabilities of one row (log-softmax, top-p, top-k): returns the buffer
+// holding them (one of two taken from sc); sc.off is left past both rows
+int filtered_logprobs(ornith_top_sampler* s, const void* d_logits_row, int V, ScratchCursor& sc,
+                      const bf16_t** out) {
+  ornith_ctx* ctx = s->ctx;
+  bf16_t* a = sc.take<bf16_t>(V);
+  bf16_t* b = sc.take<bf16_t>(V);
+  bf16_t* lse = sc.take<bf16_t>(1);
+  uint32_t* tok_tmp = sc.take<uint32_t>(1);
+  const size_t mark = sc.off;
+  // lse through the greedy selector's kernels (its token output is not used)
+  int rc = ornith_greedy_rows_ws(ctx, d_logits_row, 1, V, tok_tmp, lse, sc);
+  if (rc) return rc;
+  hipLaunchKernelGGL(logprob_kernel, dim3(nchunks(V)), dim3(RB), 0, ctx->stream,
+                     (const bf16_t*)d_logits_row, lse, V, a);
+  bf16_t *cur = a, *nxt = b;
+  if (s->top_p > 0.0 && s->top_p < 1.0) {
+    sc.off = mark;
+    rc = top_p_impl(ctx, cur, V, s->top_p, nxt, sc);
+    if (rc) return rc;
+    std::swap(cur, nxt);
+  }
+  if (s->top_k > 0 && s->top_k < V) {
+    sc.off = mark;
+    rc = top_k_impl(ctx, cur, V, s->top_k, nxt, sc);
+    if (rc) return rc;
+    std::swap(cur, nxt);
+  }
+  sc.off = mark;
+  *out = cur;
+  return ORNITH_OK;
+}
+}  // namespace
 
 extern "C" {
 
@@ -598,6 +733,7 @@ int ornith_top_sampler_create(ornith_ctx* ctx, double temp, double top_p, int to
   if (rc) return rc;
   auto* s = new ornith_top_sampler{ctx, temp, top_p, top_k, vocab, {0, 0}};
   ornith_random_key(seed, s->key);
+  s->seed = seed;
   *out = s;
   return ORNITH_OK;
 }
@@ -605,6 +741,33 @@ int ornith_top_sampler_create(ornith_ctx* ctx, double temp, double top_p, int to
 int ornith_top_sampler_destroy(ornith_top_sampler* s) {
   delete s;
   return ORNITH_OK;
+}
+
+int ornith_top_sampler_set_rng(ornith_top_sampler* s, int rng) {
+  ORN_REQUIRE(s, "top_sampler_set_rng: null sampler");
+  ORN_REQUIRE(rng == ORNITH_RNG_THREEFRY || rng == ORNITH_RNG_PHILOX, "top_sampler_set_rng: unknown generator %d", rng);
+  s->rng = rng;
+  return ORNITH_OK;
+}
+
+int ornith_top_sampler_next_bits(ornith_top_sampler* s, uint32_t* bits_out) {
+  ORN_REQUIRE(s && bits_out, "top_sampler_next_bits: null argument");
+  if (s->rng == ORNITH_RNG_PHILOX) {
+    const uint64_t n = s->philox_n++;
+    const uint32_t ctr[4] = {(uint32_t)n, (uint32_t)(n >> 32), 0u, 0u};
+    const uint32_t key[2] = {(uint32_t)s->seed, (uint32_t)(s->seed >> 32)};
+    uint32_t out[4];
+    philox4x32_10(ctr, key, out);
+    *bits_out = out[0];
+    return ORNITH_OK;
+  }
+  uint32_t sub[2];
+  ornith_random_split(s->key, sub);
+  return ornith_random_bits(sub, 1, bits_out);
+}
+
+void ornith_philox4x32_10(const uint32_t counter[4], const uint32_t key[2], uint32_t out[4]) {
+  philox4x32_10(counter, key, out);
 }
 
 int ornith_top_sampler_sample(ornith_top_sampler* s, const void* d_logits_row, uint32_t* d_token_out) {
@@ -615,34 +778,80 @@ int ornith_top_sampler_sample(ornith_top_sampler* s, const void* d_logits_row, u
   int rc = ornith_scratch(ctx, sampler_workspace(V), &base);
   if (rc) return rc;
   ScratchCursor sc(base);
-  bf16_t* a = sc.take<bf16_t>(V);
-  bf16_t* b = sc.take<bf16_t>(V);
-  bf16_t* lse = sc.take<bf16_t>(1);
-  uint32_t* tok_tmp = sc.take<uint32_t>(1);
-  const size_t mark = sc.off;
-  // lse through the greedy selector's kernels (its token output is not used)
-  rc = ornith_greedy_rows_ws(ctx, d_logits_row, 1, V, tok_tmp, lse, sc);
+  const bf16_t* cur = nullptr;
+  rc = filtered_logprobs(s, d_logits_row, V, sc, &cur);
   if (rc) return rc;
-  hipLaunchKernelGGL(logprob_kernel, dim3(nchunks(V)), dim3(RB), 0, ctx->stream,
-                     (const bf16_t*)d_logits_row, lse, V, a);
-  bf16_t *cur = a, *nxt = b;
-  if (s->top_p > 0.0 && s->top_p < 1.0) {
-    sc.off = mark;
-    rc = top_p_impl(ctx, cur, V, s->top_p, nxt, sc);
-    if (rc) return rc;
-    std::swap(cur, nxt);
-  }
-  if (s->top_k > 0) {
-    sc.off = mark;
-    rc = top_k_impl(ctx, cur, V, s->top_k, nxt, sc);
-    if (rc) return rc;
-    std::swap(cur, nxt);
-  }
-  uint32_t sub[2], raw;
-  ornith_random_split(s->key, sub);
-  ornith_random_bits(sub, 1, &raw);
-  sc.off = mark;
+  uint32_t raw;
+  rc = ornith_top_sampler_next_bits(s, &raw);
+  if (rc) return rc;
   return categorical_impl(ctx, cur, V, s->temp, raw, d_token_out, sc);
+}
+
+int ornith_sampler_weights(ornith_top_sampler* s, const void* d_logits_row, int V, float* d_w) {
+  ORN_REQUIRE(s && d_logits_row && d_w, "sampler_weights: null argument");
+  ORN_REQUIRE(V >= 2 && V <= s->vocab, "sampler_weights: V=%d outside the sampler's vocabulary of %d", V, s->vocab);
+  ornith_ctx* ctx = s->ctx;
+  void* base = nullptr;
+  int rc = ornith_scratch(ctx, sampler_workspace(s->vocab), &base);
+  if (rc) return rc;
+  ScratchCursor sc(base);
+  const bf16_t* cur = nullptr;
+  rc = filtered_logprobs(s, d_logits_row, V, sc, &cur);
+  if (rc) return rc;
+  return weights_impl(ctx, cur, V, s->temp, d_w, sc);
+}
+
+int ornith_draw_weights(ornith_ctx* ctx, const float* d_w, int V, uint32_t raw_bits, uint32_t* d_token_out) {
+  ORN_REQUIRE(ctx && d_w && d_token_out && V >= 1, "draw_weights: bad argument");
+  void* base = nullptr;
+  int rc = ornith_scratch(ctx, scan_workspace(V) + 1024, &base);
+  if (rc) return rc;
+  ScratchCursor sc(base);
+  uint32_t* fl = sc.take<uint32_t>(4);
+  rc = search_weights(ctx, d_w, V, raw_bits, fl, false, sc);
+  if (rc) return rc;
+  hipLaunchKernelGGL(cat_pick_kernel, dim3(1), dim3(1), 0, ctx->stream, fl, d_token_out);
+  ORN_LAUNCH_CHECK("draw_weights kernels");
+  return ORNITH_OK;
+}
+
+int ornith_spec_scatter(ornith_ctx* ctx, const float* d_w_local, const uint32_t* d_ids, int n, int V,
+                        float* d_w_full) {
+  ORN_REQUIRE(ctx && d_w_local && d_ids && d_w_full && n >= 1 && n <= V, "spec_scatter: bad argument");
+  hipLaunchKernelGGL(spec_zero_kernel, dim3((V + 255) / 256), dim3(256), 0, ctx->stream, d_w_full, V);
+  hipLaunchKernelGGL(spec_scatter_kernel, dim3((n + 255) / 256), dim3(256), 0, ctx->stream, d_w_local, d_ids, n, V,
+                     d_w_full);
+  ORN_LAUNCH_CHECK("spec_scatter kernels");
+  return ORNITH_OK;
+}
+
+int ornith_spec_accept(ornith_ctx* ctx, const float* d_wp, const float* d_wq, int V, const uint32_t* d_x,
+                       uint32_t raw_bits, uint32_t* d_accept_out) {
+  ORN_REQUIRE(ctx && d_wp && d_wq && d_x && d_accept_out && V >= 1, "spec_accept: bad argument");
+  hipLaunchKernelGGL(spec_accept_kernel, dim3(1), dim3(1), 0, ctx->stream, d_wp, d_wq, V, d_x, raw_bits,
+                     d_accept_out);
+  ORN_LAUNCH_CHECK("spec_accept_kernel");
+  return ORNITH_OK;
+}
+
+int ornith_spec_resample(ornith_ctx* ctx, const float* d_wp, const float* d_wq, int V, uint32_t raw_bits,
+                         uint32_t* d_token_out) {
+  ORN_REQUIRE(ctx && d_wp && d_wq && d_token_out && V >= 1, "spec_resample: bad argument");
+  void* base = nullptr;
+  int rc = ornith_scratch(ctx, (size_t)V * 4 + 2 * scan_workspace(V) + 2048, &base);
+  if (rc) return rc;
+  ScratchCursor sc(base);
+  float* r = sc.take<float>(V);
+  uint32_t* fl_r = sc.take<uint32_t>(4);
+  uint32_t* fl_p = sc.take<uint32_t>(4);
+  hipLaunchKernelGGL(spec_residual_kernel, dim3((V + 255) / 256), dim3(256), 0, ctx->stream, d_wp, d_wq, V, r);
+  rc = search_weights(ctx, r, V, raw_bits, fl_r, true, sc);
+  if (rc) return rc;
+  rc = search_weights(ctx, d_wp, V, raw_bits, fl_p, false, sc);
+  if (rc) return rc;
+  hipLaunchKernelGGL(spec_pick_kernel, dim3(1), dim3(1), 0, ctx->stream, fl_r, fl_p, d_token_out);
+  ORN_LAUNCH_CHECK("spec_resample kernels");
+  return ORNITH_OK;
 }
 
 }  // extern "C"

@@ -80,13 +80,18 @@ class TextConfig(C.Structure):
         return (i + 1) % self.full_attention_interval != 0
 
 
+ACCEPT_EQUALITY, ACCEPT_RATIO = 0, 1
+RNG_THREEFRY, RNG_PHILOX = 0, 1
+
+
 class Sampler(C.Structure):
-    _fields_ = [("kind", C.c_int), ("temperature", C.c_float), ("top_p", C.c_float),
-                ("top_k", C.c_int), ("seed", C.c_uint64)]
+    """ornith_sampler: (kind, temperature, top_p, top_k, seed, accept, rng)."""
+    _fields_ = [("kind", C.c_int), ("temperature", C.c_double), ("top_p", C.c_double),
+                ("top_k", C.c_int), ("seed", C.c_uint64), ("accept", C.c_int), ("rng", C.c_int)]
 
     @staticmethod
     def greedy():
-        return Sampler(0, 0.0, 1.0, 0, 0)
+        return Sampler(0, 0.0, 1.0, 0, 0, 0, 0)
 
 
 class MtpStats(C.Structure):
@@ -461,11 +466,46 @@ class TopSampler:
         _check(lib().ornith_top_sampler_sample(self.h, logits_row.ptr, self._tok.ptr), "top_sampler_sample")
         return int(self._tok.download(np.uint32, (1,))[0])
 
+    def set_rng(self, rng):
+        _check(lib().ornith_top_sampler_set_rng(self.h, rng), "top_sampler_set_rng")
+
+    def next_bits(self):
+        b = C.c_uint32()
+        _check(lib().ornith_top_sampler_next_bits(self.h, C.byref(b)), "top_sampler_next_bits")
+        return b.value
+
+    def weights(self, logits_row, V, w):
+        """The sampler's distribution over bf16 logits [V] as fp32 weights [V] + their total: w is
+        a DeviceBuffer of V + 1 floats."""
+        _check(lib().ornith_sampler_weights(self.h, logits_row.ptr, V, w.ptr), "sampler_weights")
+
     def close(self):
         if self.h:
             lib().ornith_top_sampler_destroy(self.h)
             self.h = None
             self._tok.free()
+
+
+def philox4x32_10(counter, key):
+    c, k, out = (C.c_uint32 * 4)(*counter), (C.c_uint32 * 2)(*key), (C.c_uint32 * 4)()
+    lib().ornith_philox4x32_10(c, k, out)
+    return list(out)
+
+
+def draw_weights(ctx, w, V, bits, tok):
+    _check(lib().ornith_draw_weights(ctx.h, w.ptr, V, C.c_uint32(bits), tok.ptr), "draw_weights")
+
+
+def spec_scatter(ctx, w_local, ids, n, V, w_full):
+    _check(lib().ornith_spec_scatter(ctx.h, w_local.ptr, ids.ptr, n, V, w_full.ptr), "spec_scatter")
+
+
+def spec_accept(ctx, wp, wq, V, x, bits, flag):
+    _check(lib().ornith_spec_accept(ctx.h, wp.ptr, wq.ptr, V, x.ptr, C.c_uint32(bits), flag.ptr), "spec_accept")
+
+
+def spec_resample(ctx, wp, wq, V, bits, tok):
+    _check(lib().ornith_spec_resample(ctx.h, wp.ptr, wq.ptr, V, C.c_uint32(bits), tok.ptr), "spec_resample")
 
 
 # ---- prefill-width k-quant GEMM (src/ops/kquant.rs:783-1027) --------------------------------

@@ -285,11 +285,12 @@ class OracleRun:
         self.o.orc_mtp_hidden(self.st, C.byref(self.mtp), p(trunk_hidden), p(next_ids), len(next_ids), p(out))
         return out
 
-    def set_sampler(self, kind=0, temp=1.0, top_p=1.0, top_k=0, seed=0):
-        """kind 0 greedy, 1 top-p/top-k/temperature; temp and top_p as the float32 values the
-        C struct carries. Process-global in the oracle: reset to greedy when done."""
-        self.o.orc_set_sampler(kind, C.c_double(float(np.float32(temp))), C.c_double(float(np.float32(top_p))),
-                               top_k, C.c_uint64(seed))
+    def set_sampler(self, kind=0, temp=1.0, top_p=1.0, top_k=0, seed=0, accept=0, rng=0):
+        """kind 0 greedy, 1 top-p/top-k/temperature; accept 0 token equality, 1 probability
+        ratio; rng 0 threefry keys, 1 Philox4x32-10. Process-global in the oracle: reset to
+        greedy when done."""
+        self.o.orc_set_sampler2(kind, C.c_double(float(temp)), C.c_double(float(top_p)), top_k, C.c_uint64(seed),
+                                accept, rng)
 
     def force_drafts(self, tokens):
         """Scripted drafts for mtp_generate (position p of the output is drafted as tokens[p]);

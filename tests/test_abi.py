@@ -69,6 +69,14 @@ def test_host_random_functions_match_known_answers():
     assert orn.random_bits([0, 0], 1)[0] == 0x6B200159
 
 
+def test_host_philox_matches_known_answers(orn):
+    """Philox4x32-10 is host code inside the library: the published Random123 vectors."""
+    assert orn.philox4x32_10([0, 0, 0, 0], [0, 0]) == [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert orn.philox4x32_10([0xFFFFFFFF] * 4, [0xFFFFFFFF] * 2) == [0x408F276D, 0x41C83B0E, 0xA20BC7C6, 0x6D5451FD]
+    assert orn.philox4x32_10([0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344], [0xA4093822, 0x299F31D0]) == \
+        [0xD16CFE09, 0x94FDCCEB, 0x5001E420, 0x24126EA1]
+
+
 def test_bench_refuses_more_than_one_gpu():
     """One GPU only: `bench.py --gpus N` with N > 1 exits with a message that says so, before
     anything touches a device."""

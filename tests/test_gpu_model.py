@@ -233,6 +233,20 @@ def test_stop_callback_and_errors(orn, ctx, tiny):
         orn.generate_step_mtp(model, head, None, caches, prompt, 3, 5)
     with pytest.raises(orn.OrnithError, match="exceed cache capacity"):
         model.forward(caches, np.zeros(16, np.uint32)); model.forward(caches, np.zeros(16, np.uint32)); model.forward(caches, np.zeros(1, np.uint32))
+    # a run that cannot fit is refused before any token is handed out, and leaves defined stats
+    seen.clear()
+    with pytest.raises(orn.OrnithError, match="exceed cache capacity"):
+        orn.generate_step(model, caches, prompt, 2, on_token=lambda t: (seen.append(t), True)[1])
+    caches.reset()
+    with pytest.raises(orn.OrnithError, match="exceed cache capacity"):
+        orn.generate_step_mtp(model, head, None, caches, prompt, 1, 27, on_token=lambda t: (seen.append(t), True)[1])
+    small_head = orn.MtpHead(model, ws, 4)
+    with pytest.raises(orn.OrnithError, match="head's cache"):
+        orn.generate_step_mtp(model, small_head, None, caches, prompt, 1, 10, on_token=lambda t: (seen.append(t), True)[1])
+    toks, _ = orn.generate_step_mtp(model, small_head, None, caches, prompt, 1, 10, policy=orn.HISTORY_CYCLE)
+    assert len(toks) == 10 and not seen
+    small_head.close()
+    caches.reset()
     with pytest.raises(orn.OrnithError, match="sampler kind"):
         orn.generate_step(model, caches, prompt, 2, sampler=orn.Sampler(7, 0.8, 0.95, 0, 1))
     with pytest.raises(orn.OrnithError, match="temp"):

@@ -49,13 +49,27 @@ def _loud_norms(s, seed):
         a[...] = util.f32_to_bf16((2.0 ** rng.uniform(-1, 1, a.shape)).astype(np.float32))
 
 
+_cache = {}
+
+
+def _model():
+    """The seeded test model and its float64 twin (weights dequantized once)."""
+    if SEED not in _cache:
+        s = synth.SynthModel(CFG, seed=SEED)
+        _loud_norms(s, SEED)
+        _cache[SEED] = (s, f64_model.F64Model(s))
+    s, f = _cache[SEED]
+    f.reset()
+    f.mtp_kv = ([], [])
+    return s, f
+
+
 def _compare():
     """Worst (rel-L2, rel-max) of oracle vs float64 over the trunk rows and the MTP rows, and
-    the smallest relative gap at a top-k cut the float64 router saw."""
-    s = synth.SynthModel(CFG, seed=SEED)
-    _loud_norms(s, SEED)
+    how often the float64 router's own top-k agreed with the oracle's where the cut was clear."""
+    s, f = _model()
     toks = np.random.default_rng(SEED).integers(0, CFG["vocab_size"], 6).astype(np.uint32)
-    o, f = synth.OracleRun(s, 32), f64_model.F64Model(s)
+    o = synth.OracleRun(s, 32)
     margins, worst, hid = [], [0.0, 0.0], []
     k = CFG["num_experts_per_tok"]
     log = np.zeros(4096, np.uint32)
