@@ -22,7 +22,9 @@ def _mk(rng, T, Hq, Hkv, hd, cap, offset):
     (1, 16, 2, 256, 4096, 4000), (2, 16, 2, 256, 4096, 255), (4, 16, 2, 256, 4096, 1021),
     (3, 4, 1, 256, 512, 0), (2, 4, 2, 128, 768, 300), (1, 2, 2, 256, 256, 7),
     # many live key blocks: the launch switches to its 256-thread form (same sums)
-    (4, 16, 2, 256, 4096, 4000), (4, 16, 2, 128, 4096, 3000)])
+    (4, 16, 2, 256, 4096, 4000), (4, 16, 2, 128, 4096, 3000),
+    # the long-context configuration: a depth-3 verify window at the end of a 16384-row cache
+    (4, 16, 2, 256, 16384, 16380), (1, 16, 2, 256, 16384, 6621)])
 def test_attention_bit_exact(orn, ctx, T, Hq, Hkv, hd, cap, offset):
     rng = np.random.default_rng(T * 1000 + offset)
     qg, kx, vx, qw, kw, kc, vc = _mk(rng, T, Hq, Hkv, hd, cap, offset)

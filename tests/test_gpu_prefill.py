@@ -33,7 +33,10 @@ def _check(got_bits, want64, K, what):
                                          (Q4K, 200, 256, 16),
                                          # enough 256-row tiles to fill the device: the producer / consumer kernel,
                                          # ragged in rows (1061 = 4 tiles + 37) and a whole number of tiles
-                                         (Q4K, 8192, 512, 1061), (Q6K, 8192, 1024, 1024)])
+                                         (Q4K, 8192, 512, 1061), (Q6K, 8192, 1024, 1024),
+                                         # a 4096-row prompt chunk through the widest projection of a gated-delta
+                                         # layer and through q_proj: the sampled configuration's prefill call
+                                         (Q4K, 8192, 2048, 4096), (Q6K, 8192, 2048, 4096)])
 def test_kq_matmul_vs_float64(orn, ctx, kind, O, K, M):
     rng = np.random.default_rng(O + K + M + kind)
     t = util.make_kq(kind, rng, 1, O, K)
@@ -200,6 +203,45 @@ def test_prefill_attention_close_to_exact_kernel(orn, ctx, T, Hq, Hkv, cap, offs
     rel = np.linalg.norm(g - w, axis=1) / np.linalg.norm(w, axis=1)
     assert rel.max() < 0.01, float(rel.max())
     for b in (dq, dk, dv, dg, dout): b.free()
+
+
+def test_prefill_attention_at_the_long_context_sizes(orn, ctx):
+    """The sampled configuration's sizes: a 4096-row prompt chunk behind 4096 cached rows in a
+    16384-row cache, 16 query heads over 2 KV heads of 256. Checked on 96 sampled (row, head)
+    pairs (first and last rows included) against a float64 softmax attention of the same bf16
+    operands, and for chunk invariance: the same rows in eight 512-row calls agree with the one
+    call to rounding."""
+    T, Hq, Hkv, hd, cap, offset = 4096, 16, 2, 256, 16384, 4096
+    rng = np.random.default_rng(55)
+    q = util.bf16_normal(rng, (T, Hq, hd)); qg = util.bf16_normal(rng, (T, Hq, 2 * hd))
+    kc = np.full((Hkv, cap, hd), 0x7FC0, np.uint16); vc = np.full((Hkv, cap, hd), 0x7FC0, np.uint16)
+    kc[:, :offset + T] = util.bf16_normal(rng, (Hkv, offset + T, hd)); vc[:, :offset + T] = util.bf16_normal(rng, (Hkv, offset + T, hd))
+    dq, dk, dv, dg = ctx.to_device(q), ctx.to_device(kc), ctx.to_device(vc), ctx.to_device(qg)
+    dout = ctx.alloc(T * Hq * hd * 2)
+    ctx.sdpa_decode_gated(dq, dk, dv, dg, T, Hq, Hkv, hd, offset, cap, hd ** -0.5, dout)
+    got = util.bf16_to_f32(dout.download(np.uint16, (T, Hq, hd))).astype(np.float64)
+    assert np.isfinite(got).all()
+    K64 = util.bf16_to_f32(kc[:, :offset + T]).astype(np.float64); V64 = util.bf16_to_f32(vc[:, :offset + T]).astype(np.float64)
+    rows = [0, 1, T - 1, T - 2] + list(rng.integers(2, T - 2, 20))
+    worst = 0.0
+    for t in rows:
+        for h in rng.choice(Hq, 4, replace=False):
+            n = offset + t + 1
+            sc = (K64[h // (Hq // Hkv), :n] @ util.bf16_to_f32(q[t, h]).astype(np.float64)) * hd ** -0.5
+            pr = np.exp(sc - sc.max()); pr /= pr.sum()
+            gate = util.bf16_to_f32(qg[t, h, hd:]).astype(np.float64)
+            want = (pr @ V64[h // (Hq // Hkv), :n]) / (1 + np.exp(-gate))
+            worst = max(worst, np.linalg.norm(got[t, h] - want) / np.linalg.norm(want))
+    assert worst < 0.01, worst
+    # the same rows in 512-row calls
+    dq2, dg2, dout2 = ctx.alloc(512 * Hq * hd * 2), ctx.alloc(512 * Hq * 2 * hd * 2), ctx.alloc(512 * Hq * hd * 2)
+    for c0 in (0, 2048, 3584):
+        dq2.upload(q[c0:c0 + 512]); dg2.upload(qg[c0:c0 + 512])
+        ctx.sdpa_decode_gated(dq2, dk, dv, dg2, 512, Hq, Hkv, hd, offset + c0, cap, hd ** -0.5, dout2)
+        part = util.bf16_to_f32(dout2.download(np.uint16, (512, Hq, hd))).astype(np.float64)
+        rel = np.linalg.norm((part - got[c0:c0 + 512]).reshape(-1, hd), axis=1) / np.linalg.norm(got[c0:c0 + 512].reshape(-1, hd), axis=1)
+        assert rel.max() < 0.01, (c0, float(rel.max()))
+    for b in (dq, dk, dv, dg, dout, dq2, dg2, dout2): b.free()
 
 
 def test_model_forward_at_the_reference_chunk_width(orn, ctx):
