@@ -8,15 +8,27 @@ random-init Qwen3.5-35B-A3B-shaped model (40 layers = 30 gated-delta + 10 full a
 MTP head, FR-Spec draft vocabulary of 32768 ids), 51-token seeded prompt, greedy depth-1
 MTP decode of 200 tokens, whose output must be byte-identical to plain greedy decode.
 A "step" is one such 200-token generation; the timed region starts when the prompt has
-been consumed (weights, caches and prompt state are resident in HBM) and `value` is
-generated tokens per second.
+been consumed and its last position sampled from (weights, caches and prompt state are
+resident in HBM) and `value` is generated tokens per second.
+
+`value` is a FLOOR: random-init weights accept no draft, so every cycle pays a two-row verify
+plus a draft for one token. The same line carries plain greedy decode and the forced-acceptance
+ceilings (every draft accepted) beside it.
 
 Also measured in the same run and printed on the same JSON line:
-  roofline      the expert gate+up gather-GEMV kernel (the largest share of the step):
-                algorithmic bytes per launch (distinct routed experts + the shared one,
-                two Q4_K matrices each, + activations) over the average launch duration
-                from HIP events on the library's stream, against 8 TB/s
-  cpu_baseline  the CPU oracle running the same loop on the host cores (bounded sample)
+  roofline      the expert gather-GEMV as the model runs it: the up launch (routing made in its
+                head, gate + up + swiglu) and the down launch (down + combine) of the MoE block,
+                back to back over all 40 layers' resident weights with the router's own picks, at
+                verify width 2: algorithmic bytes (distinct routed experts + the shared one, three
+                matrices each, + activations) over the pair's average duration from HIP events on
+                the library's stream, against 8 TB/s. `by_width` repeats it at T = 1, 2, 4 with the
+                number of distinct experts; `standalone_up` is the up kernel alone with the expert
+                ids given (no routing head).
+  per_config    BASELINE configs 1-3: the 512x2048 Q4_K mat-vec, one MoE block at T = 1, 2, 4, one
+                gated-delta layer at T = 2 with per-token snapshots, each with the oracle's time on
+                the host cores
+  cpu_baseline  the CPU oracle running the same loop on the host cores (bounded sample); the only
+                part of this script that loads anything under oracle/
 """
 import argparse
 import ctypes as C
@@ -31,69 +43,255 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
+EXPERT_BYTES = 2 * 589_824 + 860_160       # gate + up (Q4_K 512x2048) + down (Q6_K 2048x512)
 
-# HBM bytes per launch of the expert gate+up kernel at verify width 2 (17 distinct experts),
-# from two `rocprofv3 --pmc` runs of `bench.py --roofline-only` (FETCH_SIZE, then WRITE_SIZE,
-# KiB per dispatch), each scaled by what the same counter reads for the 256 MiB device copies
-# that run issues: FETCH_SIZE 9866.6 x 2.0 (the copy reads 131,086 for 262,144 KiB),
-# WRITE_SIZE 36.0 x 1.0. Counters cannot be read from inside this script; other widths: null.
-PMC_TRAFFIC_BYTES = {2: int(round((9866.6 * 2.0 + 36.0 * 1.0) * 1024))}
+# HBM bytes per launch of the up kernel at verify width 2 with 17 experts, from two
+# `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch) recorded in
+# profiles/moe_up_T2_pmc.md, each scaled by what the same counter reads for a 256 MiB device
+# copy (fetch x 2.0, write x 1.0). Counters cannot be read from inside this script: the figure
+# is carried from that profile and labelled so.
+PROFILE_TRAFFIC = {"bytes": int(round((9866.6 * 2.0 + 36.0 * 1.0) * 1024)), "algorithmic_bytes": 20_080_704,
+                   "kernel": "moe_up_kernel (T = 2, 17 experts)", "source": "profiles/moe_up_T2_pmc.md"}
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def expert_gemv_roofline(orn, ctx, model, util, np, n_layers, T, launches=800):
-    """Times the expert gate+up gather-GEMV kernel (Q4_K: top-8 of 256 routed experts plus the
-    shared expert, gate and up projections and swiglu in one launch) at verify width T on the
-    model's resident weights, cycling through every layer so no launch finds its experts in
-    cache. Algorithmic bytes per launch: (distinct routed experts + 1) x 2 matrices x 512 x
-    2048 weights x 144/256 bytes, plus the activations read and written."""
+class _Lin:
+    """A Linear held by the model, seen through the struct the library hands out."""
+
+    def __init__(self, s):
+        self.s = s
+
+
+def _time_loop(ctx, fn, n, warm):
+    for i in range(warm):
+        fn(i)
+    ctx.sync()
+    ctx.timer_begin()
+    for i in range(n):
+        fn(i)
+    return ctx.timer_end() * 1000.0 / n       # microseconds per call
+
+
+def expert_roofline(orn, ctx, model, np, n_layers, T, pairs=400):
+    """The expert gather-GEMV as the model runs it, at verify width T: per layer the router's
+    gates are made once from seeded activations, then the up launch (softmax + top-8 in its head,
+    gate + up + swiglu) and the down launch (down + combine) are timed back to back, cycling
+    through every layer's resident weights so that no launch finds its experts in cache.
+    Algorithmic bytes per pair: (distinct routed experts + 1) x 2,039,808 + the activation rows
+    read and written (x, act twice, out)."""
     rng = np.random.default_rng(123)
     H, I, E, k = 2048, 512, 256, 8
     moes = [model.moe_weights(i) for i in range(n_layers)]
-    xb = util.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32))
-    inds = np.concatenate([rng.permutation(E)[:k] for _ in range(T)]).astype(np.uint32)
-    U = len(np.unique(inds))
-    scores = util.f32_to_bf16(rng.random((T, k)).astype(np.float32))
-    eg = util.f32_to_bf16(rng.standard_normal(T).astype(np.float32))
-    dx, di, ds, de = ctx.to_device(xb), ctx.to_device(inds), ctx.to_device(scores), ctx.to_device(eg)
+    x = ctx.to_device(orn.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32)))
+    gates = [ctx.alloc(T * E * 2) for _ in moes]
+    egate = ctx.alloc(T * 2)
+    inds, scores = ctx.alloc(T * k * 4), ctx.alloc(T * k * 2)
     act, out = ctx.alloc((T * k + T) * I * 2), ctx.alloc(T * H * 2)
-    for w in moes:
-        orn.moe_experts(ctx, w, dx, T, di, ds, de, act, out, 1)
-    ctx.sync()
-    ctx.timer_begin()
-    for i in range(launches):
-        orn.moe_experts(ctx, moes[i % len(moes)], dx, T, di, ds, de, act, out, 1)
-    us = ctx.timer_end() * 1000.0 / launches
-    bytes_per_launch = (U + 1) * 2 * I * (H // 256) * 144 + T * H * 2 + (T * k + T) * I * 2 + T * k * 4
-    for b in (dx, di, ds, de, act, out):
+    U = []
+    for w, g in zip(moes, gates):
+        ctx.linear_matmul(_Lin(w.router), x, T, g)
+        ctx.linear_matmul(_Lin(w.sh_egate), x, T, egate)
+        orn.moe_experts_from_gates(ctx, w, x, T, g, egate, inds, scores, act, out)
+        U.append(len(np.unique(inds.download(np.uint32, (T * k,)))))
+    us = _time_loop(ctx, lambda i: orn.moe_experts_from_gates(ctx, moes[i % n_layers], x, T, gates[i % n_layers], egate,
+                                                              inds, scores, act, out), pairs, n_layers)
+    u_mean = float(np.mean(U))
+    acts = T * H * 2 + 2 * (T * k + T) * I * 2 + T * H * 2
+    nbytes = (u_mean + 1) * EXPERT_BYTES + acts
+    # the up kernel alone with the ids given (no routing head): the figure earlier reports carried
+    ids = np.concatenate([rng.permutation(E)[:k] for _ in range(T)]).astype(np.uint32)
+    d_ids = ctx.to_device(ids)
+    us_up = _time_loop(ctx, lambda i: orn.moe_experts(ctx, moes[i % n_layers], x, T, d_ids, scores, egate, act, out, 1),
+                       pairs, n_layers)
+    up_bytes = (len(np.unique(ids)) + 1) * 2 * 589_824 + T * H * 2 + (T * k + T) * I * 2 + T * k * 4
+    for b in [x, egate, inds, scores, act, out, d_ids] + gates:
         b.free()
-    achieved = bytes_per_launch / (us * 1e-6) / 1e9
-    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": PMC_TRAFFIC_BYTES.get(T) if U == 16 else None,
-            "kernel": "moe_up_kernel<0, 64, 2, false> (Q4_K expert gate+up gather-GEMV + swiglu, expert ids given)",
-            "us_per_launch": round(us, 3), "bytes_per_launch": int(bytes_per_launch),
-            "distinct_experts": int(U), "verify_width": int(T)}
+    ach = nbytes / (us * 1e-6) / 1e9
+    return {"verify_width": T, "distinct_experts_mean": round(u_mean, 2), "us_per_pair": round(us, 3),
+            "bytes_per_pair": int(nbytes), "achieved": round(ach, 1), "frac": round(ach / HBM_PEAK_GBS, 4),
+            "standalone_up": {"us_per_launch": round(us_up, 3), "bytes_per_launch": int(up_bytes),
+                              "achieved": round(up_bytes / (us_up * 1e-6) / 1e9, 1),
+                              "frac": round(up_bytes / (us_up * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}}
 
 
-def cpu_baseline(synth, synth_model, np, depth, tokens):
-    """The oracle's generate_step_mtp on the host cores, whole call timed."""
+def per_config(orn, ctx, np, with_cpu):
+    """BASELINE configs 1-3 on their own seeded tensors: GPU time from HIP events over chained
+    launches; CPU time of the oracle's restatement of the same operator (best of 5)."""
+    import util
+    res = {}
+
+    def cpu_us(fn, reps=5):
+        best = 1e30
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            best = min(best, time.perf_counter() - t0)
+        return round(best * 1e6, 1)
+
+    # ---- config 1: Q4_K mat-vec 512 x 2048, fp32 activations in and out
+    rng = np.random.default_rng(1)
+    O, K = 512, 2048
+    t = util.make_q4k(rng, 1, O, K)
+    w = orn.KMatrix(ctx, orn.Q4K, *t, 1, O, K)
+    xf = rng.standard_normal((1, K)).astype(np.float32)
+    dx, dy = ctx.to_device(xf), ctx.alloc(O * 4)
+    us = _time_loop(ctx, lambda i: ctx.kq_qmv(w, dx, orn.F32, 1, dy, orn.F32), 2000, 100)
+    nbytes = 589_824 + 8_192 + 2_048
+    c1 = {"workload": "Q4_K dequant mat-vec 512x2048, fp32 x [1,2048] -> fp32 y [1,512], 2000 chained launches",
+          "us_per_launch": round(us, 3), "algorithmic_bytes": nbytes, "GB_s": round(nbytes / (us * 1e-6) / 1e9, 1)}
+    if with_cpu:
+        got = dy.download(np.float32, (1, O))
+        want64 = util.orc_matvec_f64(util.Q4K, *t, O, K, xf)
+        c1["max_abs_err_vs_f64"] = float(np.max(np.abs(got - want64)))
+        c1["global_rel_err_vs_f64"] = util.global_rel(got, want64)
+        c1["bit_exact_vs_oracle"] = bool(np.array_equal(got.view(np.uint32), util.orc_qmv(util.Q4K, *t, O, K, xf).view(np.uint32)))
+        c1["cpu_us"] = cpu_us(lambda: util.orc_qmv(util.Q4K, *t, O, K, xf))
+    for b in (dx, dy):
+        b.free()
+    w.free()
+    res["config1"] = c1
+
+    # ---- config 2: one MoE block at T = 1, 2, 4 (four sets of weights cycled: 2.1 GB)
+    rng = np.random.default_rng(2)
+    moes = [util.HostMoe(rng) for _ in range(4)]
+    devs = [m.dev(orn, ctx) for m in moes]
+    c2 = {"workload": "one MoE block: hidden 2048, 256 experts top-8 (gate/up Q4_K, down Q6_K) + shared expert, "
+                      "router Q6_K, bf16 activations; router + up + down launches", "by_width": []}
+    for T in (1, 2, 4):
+        xb = orn.f32_to_bf16(rng.standard_normal((T, 2048)).astype(np.float32))
+        dxb, dout = ctx.to_device(xb), ctx.alloc(T * 2048 * 2)
+        di, ds = ctx.alloc(T * 8 * 4), ctx.alloc(T * 8 * 2)
+        ctx.moe_block(devs[0], dxb, T, dout, di, ds)
+        inds = di.download(np.uint32, (T, 8))
+        U = len(np.unique(inds))
+        us = _time_loop(ctx, lambda i: ctx.moe_block(devs[i % 4], dxb, T, dout), 400, 8)
+        nbytes = (U + 1) * EXPERT_BYTES + 430_080 + 2_208 + T * 2048 * 2 * 2 + 2 * 9 * T * 1024
+        e = {"T": T, "distinct_experts": U, "us_per_block": round(us, 3), "algorithmic_bytes": int(nbytes),
+             "GB_s": round(nbytes / (us * 1e-6) / 1e9, 1), "frac_of_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}
+        if with_cpu:
+            _, oinds, _, _ = util.orc_moe_block(moes[0], xb, T)
+            e["expert_indices_bit_exact"] = bool(np.array_equal(oinds, inds))
+            e["cpu_us"] = cpu_us(lambda: util.orc_moe_block(moes[0], xb, T), reps=3)
+        c2["by_width"].append(e)
+        for b in (dxb, dout, di, ds):
+            b.free()
+    for m in moes:
+        m.free()
+    res["config2"] = c2
+
+    # ---- config 3: one gated-delta layer at T = 2 with per-token snapshots (rollback is a cursor move)
+    rng = np.random.default_rng(3)
+    H, Hk, Hv, D = 2048, 16, 32, 8192
+    T = 2
+    lin = {n: util.HostLinear.kq(rng, util.Q4K, o, k) for n, (o, k) in
+           (("qkv", (D, H)), ("z", (4096, H)), ("out", (H, 4096)))}
+    dl = {n: l.dev(orn, ctx) for n, l in lin.items()}
+    wa, wb = util.HostLinear.dense(rng, Hv, H), util.HostLinear.dense(rng, Hv, H)
+    bf = lambda shape, std=1.0: orn.f32_to_bf16((rng.standard_normal(shape) * std).astype(np.float32))
+    host = dict(xn=bf((T, H)), conv=bf((3, D)), cw=bf((D, 4), 0.5), a_log=bf((Hv,), 0.5), dt=bf((Hv,), 0.5),
+                nw=bf((128,)), S0=(rng.standard_normal((Hv, 128, 128)) * 0.1).astype(np.float32))
+    d = {n: ctx.to_device(a) for n, a in host.items()}
+    d["wa"], d["wb"] = ctx.to_device(wa.w), ctx.to_device(wb.w)
+    qkv, z = ctx.alloc(T * D * 2), ctx.alloc(T * 4096 * 2)
+    snaps, ci, gated, r = ctx.alloc(T * Hv * 128 * 128 * 4), ctx.alloc((3 + T) * D * 2), ctx.alloc(T * 4096 * 2), ctx.alloc(T * H * 2)
+
+    def layer(i):
+        ctx.linear_matmul_multi([dl["qkv"], dl["z"]], d["xn"], T, [qkv, z])
+        orn.gdn_step(ctx, d["conv"], qkv, d["cw"], d["wa"], d["wb"], d["xn"], H, d["a_log"], d["dt"], T, 4, Hk, 128, Hv,
+                     128, d["S0"], snaps, True, d["nw"], z, ci, gated)
+        ctx.linear_matmul(dl["out"], gated, T, r)
+
+    us = _time_loop(ctx, layer, 400, 8)
+    wbytes = 9_437_184 + 4_718_592 + 4_718_592 + 2 * 131_072 + 65_536
+    state = 2_097_152 * (1 + T)
+    c3 = {"workload": "one gated-delta layer, T = 2 verify rows with a state snapshot per row: in_proj qkv+z, "
+                      "mixer core (a/b projections, conv, recurrence, gated norm), out_proj; 3 launches, the same "
+                      "weights every call; rollback of the rejected row is a cursor move (no launch)",
+          "us_per_layer": round(us, 3), "weight_bytes": wbytes, "state_bytes_moved": state,
+          "GB_s": round((wbytes + state) / (us * 1e-6) / 1e9, 1)}
+    if with_cpu:
+        def cpu_layer():
+            x32 = util.bf16_to_f32(host["xn"])
+            qkv_h = util.f32_to_bf16(util.orc_qmv(util.Q4K, lin["qkv"].km.qs, lin["qkv"].km.scales, lin["qkv"].km.dm, D, H, x32, True))
+            z_h = util.f32_to_bf16(util.orc_qmv(util.Q4K, lin["z"].km.qs, lin["z"].km.scales, lin["z"].km.dm, 4096, H, x32, True))
+            a_h, b_h = np.empty((T, Hv), np.uint16), np.empty((T, Hv), np.uint16)
+            util.oracle().orc_dense_gemv(util.p(wa.w), Hv, H, util.p(host["xn"]), T, util.p(a_h))
+            util.oracle().orc_dense_gemv(util.p(wb.w), Hv, H, util.p(host["xn"]), T, util.p(b_h))
+            q, k, v, beta, g, _ = util.orc_gdn_front(host["conv"], qkv_h, host["cw"], a_h, b_h, host["a_log"], host["dt"], Hk, Hv)
+            y, _ = util.orc_gdn_recurrence(q, k, v, g, beta, host["S0"])
+            gated_h = util.orc_rms_norm_gated(y.reshape(T * Hv, 128), host["nw"], z_h.reshape(T * Hv, 128))
+            return util.f32_to_bf16(util.orc_qmv(util.Q4K, lin["out"].km.qs, lin["out"].km.scales, lin["out"].km.dm, H, 4096,
+                                                 util.bf16_to_f32(gated_h.reshape(T, 4096)), True))
+
+        want = cpu_layer()
+        c3["bit_exact_vs_oracle"] = bool(np.array_equal(r.download(np.uint16, (T, H)), want))
+        c3["cpu_us"] = cpu_us(cpu_layer, reps=3)
+    for b in list(d.values()) + [qkv, z, snaps, ci, gated, r]:
+        b.free()
+    for l in dl.values():
+        l.free()
+    res["config3"] = c3
+    return res
+
+
+def cpu_baseline(synth, synth_model, np, depth, tokens, prompt):
+    """The oracle's generate_step_mtp on the host cores with the benchmark's own prompt; the
+    prefill (timed separately on a second state) is taken off the whole call."""
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    rng = np.random.default_rng(99)
-    prompt = rng.integers(0, synth_model.cfg["vocab_size"], 2).astype(np.uint32)
     fr_ids = synth.zipf_frspec_ids(synth_model.cfg["vocab_size"], 32768, seed=1)
     fr_host = synth.prune_head(synth_model.lm_head, fr_ids)
-    run = synth.OracleRun(synth_model, 64)
+    pre = synth.OracleRun(synth_model, 128)
+    t0 = time.time()
+    for i in range(0, len(prompt) - 1, 16):
+        pre.forward(prompt[i:min(i + 16, len(prompt) - 1)])
+    t_pre = time.time() - t0
+    pre.close()
+    run = synth.OracleRun(synth_model, 128)
     t0 = time.time()
     toks, st = run.mtp_generate(prompt, depth, tokens, fr_ids, fr_host, policy=1, prefill_step=16)
     dt = time.time() - t0
     run.close()
-    return {"value": round(len(toks) / dt, 4), "unit": "tok/s", "cores": threads, "kind": "port",
-            "sample": f"oracle generate_step_mtp depth {depth} + FR-Spec, 2-token prompt, {len(toks)} tokens, "
-                      f"whole call {dt:.1f} s ({int(st.cycles)} cycles, {int(st.accepted)} accepted)"}, toks, prompt
+    dec = max(dt - t_pre, 1e-9)
+    return {"value": round(len(toks) / dec, 4), "unit": "tok/s", "cores": threads, "kind": "port",
+            "sample": f"oracle generate_step_mtp depth {depth} + FR-Spec on the {len(prompt)}-token prompt, first "
+                      f"{len(toks)} tokens: whole call {dt:.1f} s, of which prefill {t_pre:.1f} s "
+                      f"({int(st.cycles)} cycles, {int(st.accepted)} accepted)"}, toks
+
+
+def moe_ab(orn, ctx, model, np, n_layers):
+    """The MoE block (norm + router + up + down) as separate launches (fuse_moe_one = 0), as one
+    launch with in-launch hand-offs (1), and as router + one up/down launch (2), on the resident
+    weights of every layer in turn. Prints a JSON table."""
+    lib = orn.lib()
+    H = 2048
+    rng = np.random.default_rng(5)
+    moes = [model.moe_weights(i) for i in range(n_layers)]
+    wn = ctx.to_device(orn.f32_to_bf16((1 + 0.1 * rng.standard_normal(H)).astype(np.float32)))
+    rows = []
+    for T in (1, 2, 4):
+        res, y = (ctx.to_device(orn.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32))) for _ in range(2))
+        h, nx, out = ctx.alloc(T * H * 2), ctx.alloc(T * H * 2), ctx.alloc(T * H * 2)
+        ref = None
+        for how in (0, 1, 2):
+            orn.set_option("fuse_moe_one", how)
+
+            def run(i):
+                rc = lib.ornith_add_rms_moe_block(ctx.h, C.byref(moes[i % n_layers]), res.ptr, y.ptr, wn.ptr,
+                                                  C.c_float(1e-6), T, h.ptr, nx.ptr, out.ptr)
+                assert rc == 0, lib.ornith_last_error()
+
+            us = _time_loop(ctx, run, 400, n_layers)
+            run(0)
+            o = out.download(np.uint16, (T, H))
+            ref = o if ref is None else ref
+            rows.append({"T": T, "fuse_moe_one": how, "us_per_block": round(us, 2), "identical": bool(np.array_equal(o, ref))})
+        for b in (res, y, h, nx, out):
+            b.free()
+    orn.set_option("fuse_moe_one", 0)
+    print(json.dumps({"moe_block_launch_structure": rows}), flush=True)
 
 
 def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
@@ -106,7 +304,9 @@ def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
     fr = orn.FrSpec(model, ids=fr_ids)
     rng = np.random.default_rng(6621)
     prompt = rng.integers(0, cfg["vocab_size"], n_prompt).astype(np.uint32)
-    smp = orn.Sampler(1, 0.8, 0.95, 0, 2025)
+    accept = orn.ACCEPT_RATIO if args.accept == "ratio" else orn.ACCEPT_EQUALITY
+    gen = orn.RNG_PHILOX if args.rng == "philox" else orn.RNG_THREEFRY
+    smp = orn.Sampler(1, 0.8, 0.95, 0, 2025, accept, gen)
     res = []
     for it in range(2):
         caches.reset()
@@ -138,12 +338,14 @@ def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
     flops_tok = 2.0 * (30 * per_layer_gdn + 10 * per_layer_att + 40 * per_layer_moe)
     line = {"workload": f"config5: {n_prompt}-token prefill (chunks of {args.prefill_chunk}) into a {cap}-token context, "
                         f"then sampled MTP depth-{depth} + FR-Spec decode of {n_gen} tokens (temperature 0.8, top-p 0.95, "
-                        "seeded threefry keys)",
+                        f"{'probability-ratio (rejection-sampling)' if args.accept == 'ratio' else 'token-equality'} "
+                        f"acceptance, seeded {'Philox4x32-10' if args.rng == 'philox' else 'threefry'} stream)",
             "prefill_s": round(t_pre, 4), "prefill_tok_s": round(n_prompt / t_pre, 1),
             "prefill_gemm_tflops": round(flops_tok * n_prompt / t_pre / 1e12, 2),
             "prefill_frac_of_bf16_mfma_peak": round(flops_tok * n_prompt / t_pre / 2.5e15, 4),
             "decode_tok_s": round(n_gen / t_dec, 2), "cycles": int(st.cycles), "drafted": int(st.drafted),
-            "accepted": int(st.accepted), "tokens_per_verify_step": round(n_gen / max(1, int(st.cycles)), 3),
+            "accepted": int(st.accepted), "accepted_tokens_per_verify_step": round(int(st.accepted) / max(1, int(st.cycles)), 4),
+            "tokens_per_verify_step": round(n_gen / max(1, int(st.cycles)), 3),
             "repeatable": True, "device": dev_name, "data": "synthetic"}
     print(json.dumps(line), flush=True)
 
@@ -156,20 +358,26 @@ def main():
     ap.add_argument("--tokens", type=int, default=200)
     ap.add_argument("--depth", type=int, default=1)
     ap.add_argument("--layers", type=int, default=40, help="trunk layers (40 = the named config)")
-    ap.add_argument("--cpu-tokens", type=int, default=48)
-    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-tokens", type=int, default=40)
+    ap.add_argument("--no-cpu", action="store_true", help="skip every leg that runs the CPU oracle")
     ap.add_argument("--config5", action="store_true",
                     help="instead of the metric's workload: BASELINE config 5 (6621-token prefill into a "
                          "16384-token context through the matrix-core path, then sampled depth-3 MTP "
                          "decode of 256 tokens, temperature 0.8, top-p 0.95); prints its own JSON line")
+    ap.add_argument("--accept", choices=("ratio", "equality"), default="ratio",
+                    help="with --config5: probability-ratio (rejection-sampling) acceptance, or the reference's token equality")
+    ap.add_argument("--rng", choices=("philox", "threefry"), default="philox",
+                    help="with --config5: the sampler's random stream")
     ap.add_argument("--prefill-chunk", type=int, default=4096,
                     help="rows per prefill call with --config5 (the reference's prefill_step_size is 2048; up to 4096 here)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="with --config5: stop after the first generated token (a short run for "
                          "profiling the matrix-core prefill kernels)")
     ap.add_argument("--roofline-only", action="store_true",
-                    help="only the expert-kernel timing loop plus three 256 MiB device copies "
+                    help="only the expert-kernel timing loops plus three 256 MiB device copies "
                          "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--moe-ab", action="store_true",
+                    help="only the A/B of the MoE block's launch structure (option fuse_moe_one = 0, 1, 2)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (one process, one stream); "
@@ -177,7 +385,6 @@ def main():
 
     import numpy as np
     import synth
-    import util
     orn = importlib.import_module("ornith-rs_amd")
     ctx = orn.Ctx(0)
     dev_name, cus, mem = ctx.device_info()
@@ -192,13 +399,15 @@ def main():
     log(f"uploaded in {time.time() - t0:.1f} s")
     model = orn.TextModel(ctx, ws, sm.text_config(orn))
     if args.roofline_only:
-        roof = expert_gemv_roofline(orn, ctx, model, util, np, args.layers, T=args.depth + 1, launches=200)
+        roof = expert_roofline(orn, ctx, model, np, args.layers, T=args.depth + 1, pairs=200)
         a, b = ctx.alloc(256 << 20), ctx.alloc(256 << 20)
         for _ in range(3):
             ctx.copy(a, b, 256 << 20)
         ctx.sync()
         print(json.dumps({"roofline": roof}), flush=True)
         return
+    if args.moe_ab:
+        return moe_ab(orn, ctx, model, np, args.layers)
     if args.config5:
         return config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name)
     rng = np.random.default_rng(51)
@@ -210,7 +419,8 @@ def main():
     fr = orn.FrSpec(model, ids=fr_ids)
 
     def timed_run(fn):
-        """fn(progress) -> tokens; returns (tokens, decode seconds, extra)."""
+        """fn(progress) -> tokens; returns (tokens, decode seconds). Both loops report the
+        prompt consumed at the same point: after its last position has been sampled from."""
         mark = {}
 
         def progress(done, total):
@@ -223,6 +433,8 @@ def main():
         return out, time.perf_counter() - mark["t0"]
 
     # plain greedy, for the byte-identity check and as the non-speculative figure
+    caches.reset()
+    orn.generate_step(model, caches, prompt, 8, prefill_step=16)      # warm the shapes
     caches.reset()
     ar, ar_s = timed_run(lambda pr: orn.generate_step(model, caches, prompt, args.tokens, prefill_step=16, progress=pr))
     log(f"plain greedy: {len(ar)} tokens in {ar_s * 1e3:.1f} ms = {len(ar) / ar_s:.1f} tok/s")
@@ -263,34 +475,45 @@ def main():
     head.force_drafts([])
     c2.close()
 
-    roof = expert_gemv_roofline(orn, ctx, model, util, np, args.layers, T=args.depth + 1)
+    by_width = [expert_roofline(orn, ctx, model, np, args.layers, T) for T in (1, 2, 4)]
+    main_w = next(w for w in by_width if w["verify_width"] == 2)
+    roof = {"bound": "hbm", "achieved": main_w["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": main_w["frac"],
+            "traffic": None, "traffic_from_profile": PROFILE_TRAFFIC,
+            "kernel": "moe_up_kernel<Q4_K, 64, 2, routing made in the launch> + moe_down_kernel<Q6_K, 8, 1>: the expert "
+                      "gather-GEMV of one MoE block as the model launches it (gate + up + swiglu, down + combine), "
+                      "verify width 2, the router's own picks",
+            "us_per_launch": main_w["us_per_pair"], "launches_per_unit": 2, "bytes_per_launch": main_w["bytes_per_pair"],
+            "distinct_experts": main_w["distinct_experts_mean"], "verify_width": 2, "by_width": by_width}
     log("roofline:", roof)
+
+    configs = per_config(orn, ctx, np, with_cpu=not args.no_cpu)
+    log("per_config:", configs)
 
     cpu = None
     if not args.no_cpu:
-        cpu, cpu_toks, cpu_prompt = cpu_baseline(synth, sm, np, args.depth, args.cpu_tokens)
-        # the same short run on the GPU must give the same tokens
-        caches.reset()
-        g, _ = orn.generate_step_mtp(model, head, fr, caches, cpu_prompt, args.depth, args.cpu_tokens,
-                                     prefill_step=16, policy=orn.HISTORY_COMMITTED)
-        cpu["gpu_tokens_match"] = bool(g == cpu_toks)
+        cpu, cpu_toks = cpu_baseline(synth, sm, np, args.depth, args.cpu_tokens, prompt)
+        # the same tokens must have come out of the GPU
+        cpu["gpu_tokens_match"] = bool(ar[:len(cpu_toks)] == cpu_toks)
         log("cpu_baseline:", cpu)
 
     line = {
         "metric": "decode tok/s @MTP depth 1 (1 GPU, byte-exact); expert GEMV HBM GB/s vs peak",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(total_s / len(times) * 1e3, 3), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32",
+        "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
+        "value_is": "the zero-acceptance floor of the depth-1 loop (random-init weights accept no draft: one token per "
+                    "two-row verify + draft); see plain_greedy_tok_s and forced_acceptance_ceiling beside it",
+        "plain_greedy_tok_s": round(len(ar) / ar_s, 2),
+        "forced_acceptance_ceiling": forced,
         "config": {"workload": f"config4: greedy MTP depth-{args.depth} + FR-Spec(32768) decode of {args.tokens} tokens, "
                                f"51-token prompt, Qwen3.5-35B-A3B shape, {args.layers} layers, KV capacity {cap}",
-                   "arithmetic": "fp32 accumulate over bf16 activations and Q4_K/Q6_K/int8/bf16 weights",
+                   "arithmetic": "bf16 activations, fp32 accumulation, Q4_K/Q6_K/int8/bf16 weights",
                    "tokens_per_step": args.tokens, "byte_identical_to_greedy": True,
-                   "plain_greedy_tok_s": round(len(ar) / ar_s, 2),
                    "cycles": int(stats.cycles), "accepted": int(stats.accepted), "drafted": int(stats.drafted),
-                   "forced_acceptance_ceiling": forced,
                    "weights_GB": round(ws.stats()[1] / 1e9, 2), "device": dev_name},
         "roofline": roof,
+        "per_config": configs,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line), flush=True)

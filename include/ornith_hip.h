@@ -264,6 +264,15 @@ ORNITH_API int ornith_moe_experts(ornith_ctx* ctx, const ornith_moe_weights* w, 
                                   const uint32_t* d_inds, const void* d_scores, const void* d_egate,
                                   void* d_act, void* d_out, int phases);
 
+/* The same two launches as ornith_moe_block issues them after its router launch: the routing
+ * (softmax + top-k, src/ops/moe.rs:688-697) is made from the router's gates (d_gates bf16
+ * [T,E]) in the head of the up launch and stored to d_inds_out / d_scores_out, then the down
+ * launch. What a caller times to see the expert gather-GEMV as the model runs it. */
+ORNITH_API int ornith_moe_experts_from_gates(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x,
+                                             int T, const void* d_gates, const void* d_egate,
+                                             uint32_t* d_inds_out, void* d_scores_out, void* d_act,
+                                             void* d_out);
+
 /* ---- norms: src/ops/norm.rs:19-220 (vendored rms_norm.metal:12-81,
  * kernels/ornith_norm.metal:28-183). Rows of n bf16 values, n = 64 * 2^j <= 4096. */
 /* norm::rms_norm: out = w * (x * rsqrt(mean(x^2) + eps)); d_w may be null (weight 1). */

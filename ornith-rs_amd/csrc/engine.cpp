@@ -211,11 +211,12 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
   const size_t rows = n_prompt - processed;
   TRY(ornith_upload(ctx, d_tok, prompt + processed, rows * 4));
   TRY(ornith_model_forward(m, c, d_tok, (int)rows, 0, d_hidden));
-  if (progress) progress(n_prompt, n_prompt, user);
   TRY(ornith_model_logits(m, (char*)d_hidden + (rows - 1) * H * 2, 1, d_vlogits));
   TRY(smp.sample(d_vlogits, d_targets));
   uint32_t primary = 0;
   TRY(ornith_download(ctx, &primary, d_targets, 4));
+  // the prompt is consumed once its last position has been sampled from, as in generate_step
+  if (progress) progress(n_prompt, n_prompt, user);
   // the trunk hidden a cycle drafts from is read where the last forward left it: the next
   // write to d_hidden is the cycle's verify pass, after the drafts
   const void* d_h = (char*)d_hidden + (rows - 1) * H * 2;

@@ -974,4 +974,18 @@ int ornith_moe_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void*
   return moe_fused_experts(ctx, w, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, phases, nullptr);
 }
 
+int ornith_moe_experts_from_gates(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
+                                  const void* d_gates, const void* d_egate, uint32_t* d_inds_out,
+                                  void* d_scores_out, void* d_act, void* d_out) {
+  ORN_REQUIRE(ctx && w && d_x && d_gates && d_egate && d_inds_out && d_scores_out && d_act && d_out,
+              "moe_experts_from_gates: null argument");
+  ORN_REQUIRE(T >= 1 && T <= 64, "moe_experts_from_gates: T=%d", T);
+  const int E = w->router.O, k = w->top_k;
+  if (!moe_fused_supported(w) || E % 64 != 0 || E > 1024 || ((E / 64) & (E / 64 - 1)) != 0 || k > 16)
+    return ornith_fail(ORNITH_ERR_UNSUPPORTED,
+                       "moe_experts_from_gates: needs k-quant routed and shared experts of matching formats, "
+                       "top_k <= %d and a power-of-two multiple of 64 experts up to 1024", kMaxK);
+  return moe_fused_experts(ctx, w, d_x, T, d_inds_out, d_scores_out, d_egate, d_act, d_out, 3, d_gates);
+}
+
 }  // extern "C"

@@ -508,6 +508,22 @@ def spec_resample(ctx, wp, wq, V, bits, tok):
     _check(lib().ornith_spec_resample(ctx.h, wp.ptr, wq.ptr, V, C.c_uint32(bits), tok.ptr), "spec_resample")
 
 
+def moe_experts_from_gates(ctx, w, x, T, gates, egate, inds, scores, act, out):
+    """The up + down launches of the MoE block with the routing made from the gates in the head
+    of the up launch (what the model runs after its router launch)."""
+    _check(lib().ornith_moe_experts_from_gates(ctx.h, C.byref(w), x.ptr, T, gates.ptr, egate.ptr, inds.ptr,
+                                               scores.ptr, act.ptr, out.ptr), "moe_experts_from_gates")
+
+
+def gdn_step(ctx, conv_state, qkv, cw, wa, wb, xn, H, a_log, dt_bias, T, K, Hk, Dk, Hv, Dv, state_in, snapshots,
+             snap_all, norm_w, z, conv_input, gated_out, eps=1e-6, norm_eps=1e-6):
+    """ornith_gdn_step with the a / b projections made from dense weights inside the launch."""
+    _check(lib().ornith_gdn_step(ctx.h, conv_state.ptr, qkv.ptr, cw.ptr, None, None, wa.ptr, wb.ptr, xn.ptr, H,
+                                 a_log.ptr, dt_bias.ptr, T, K, Hk, Dk, Hv, Dv, C.c_float(eps), state_in.ptr,
+                                 snapshots.ptr, int(snap_all), norm_w.ptr, z.ptr, C.c_float(norm_eps),
+                                 conv_input.ptr, gated_out.ptr), "gdn_step")
+
+
 # ---- prefill-width k-quant GEMM (src/ops/kquant.rs:783-1027) --------------------------------
 def kq_matmul(ctx, w, x, M, y):
     _check(lib().ornith_kq_matmul(ctx.h, C.byref(w.s), x.ptr, M, y.ptr), "kq_matmul")

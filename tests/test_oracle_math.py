@@ -47,11 +47,16 @@ def test_bf16_rne_and_f16_conversions():
     # bf16: exhaustive over the upper 16 bits is the identity; ties go to even
     bits = np.arange(65536, dtype=np.uint32)
     f = (bits << 16).view(np.float32)
-    got = util.f32_to_bf16(f)
+    got = util.orc_f32_to_bf16(f)
     nan = np.isnan(f)
     assert np.array_equal(got[~nan], bits[~nan].astype(np.uint16))
     tie = np.array([0x3F808000, 0x3F818000, 0x3F808001, 0x3F807FFF], np.uint32).view(np.float32)
-    assert list(util.f32_to_bf16(tie)) == [0x3F80, 0x3F82, 0x3F81, 0x3F80]
+    assert list(util.orc_f32_to_bf16(tie)) == [0x3F80, 0x3F82, 0x3F81, 0x3F80]
+    # the numpy conversion the tests build their inputs with is the same function, bit for bit,
+    # NaN and infinities included
+    rnd = np.random.default_rng(0).integers(0, 2 ** 32, 2_000_000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    for v in (f, tie, rnd):
+        assert np.array_equal(util.f32_to_bf16(v), util.orc_f32_to_bf16(v))
     # f16 -> f32 exhaustive vs numpy; f32 -> f16 on random values vs numpy (RNE)
     h = np.arange(65536, dtype=np.uint16)
     out = np.empty(65536, np.float32)

@@ -33,6 +33,17 @@ def p(a):
 
 # ---- bf16 / f16 on the host ------------------------------------------------
 def f32_to_bf16(a):
+    """Round to nearest even, NaN -> quiet NaN (src/array.rs:229-237), in numpy: building
+    inputs must not need the oracle's library (tests/test_oracle_math.py holds this against
+    the oracle's own conversion)."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
+
+
+def orc_f32_to_bf16(a):
     a = np.ascontiguousarray(a, dtype=np.float32)
     out = np.empty(a.shape, dtype=np.uint16)
     oracle().orc_f32_to_bf16_n(p(a), p(out), C.c_int64(a.size))
