@@ -227,11 +227,24 @@ static inline size_t kq_qs_row(int kind, int K) { return (size_t)(K / 256) * (ki
 static inline size_t kq_sc_row(int kind, int K) { return (size_t)(K / 256) * (kind == ORC_Q4K ? 12 : 16); }
 static inline size_t kq_dm_row(int kind, int K) { return (size_t)(K / 256) * (kind == ORC_Q4K ? 2 : 1); }
 
+/* orc_ref_order.c: the same dot product in the reference's 32-lane schedule, selected for
+ * every k-quant mat-vec of the oracle by orc_set_row_order (a measurement aid) */
+extern int orc_row_order;
+float orc_q4k_row_dot_ref32(const uint8_t* qs, const uint8_t* scales, const f16_t* dm, int K, const float* x,
+                            int fma, int tree);
+float orc_q6k_row_dot_ref32(const uint8_t* w, const uint8_t* scales, const f16_t* dm, int K, const float* x,
+                            int fma, int tree);
+
 float orc_kq_row_dot(int kind, const uint8_t* qs, const uint8_t* scales, const f16_t* dm,
                      int K, int64_t row, const float* x) {
   const uint8_t* q = qs + row * kq_qs_row(kind, K);
   const uint8_t* s = scales + row * kq_sc_row(kind, K);
   const f16_t* d = dm + row * kq_dm_row(kind, K);
+  if (orc_row_order > 0) {
+    const int v = orc_row_order - 1, tree = v % 3, fma = v / 3;
+    return kind == ORC_Q4K ? orc_q4k_row_dot_ref32(q, s, d, K, x, fma, tree)
+                           : orc_q6k_row_dot_ref32(q, s, d, K, x, fma, tree);
+  }
   return kind == ORC_Q4K ? orc_q4k_row_dot(q, s, d, K, x) : orc_q6k_row_dot(q, s, d, K, x);
 }
 
