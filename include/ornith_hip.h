@@ -512,6 +512,32 @@ typedef struct ornith_frspec ornith_frspec;
 /* FrSpec::load: file = u32 n, then n x u32 LE; rejects n == 0, n >= vocab, ids out of
  * range, duplicates. FrSpec::prune: row-gathers lm_head's tensors into an n-row head. */
 ORNITH_API int ornith_frspec_load(ornith_model* m, const char* path, ornith_frspec** out);
+/* frspec::default_path (src/frspec.rs:153-158): $ORNITH_FRSPEC, else
+ * <$ORNITH_REFS or "refs">/frspec/ids_64k.bin. ornith_frspec_load(m, NULL, ..) reads from there. */
+ORNITH_API int ornith_frspec_default_path(char* buf, size_t len);
+/* The list file on the host (src/frspec.rs:101-117; tools/merge_frspec.py:74-92). read: ids in
+ * file order, *n_out their number (ids_out == NULL only asks for it); write: sorted and
+ * de-duplicated, refusing an empty list, one that is not a strict pruning of `vocab`, or an id
+ * outside it. */
+ORNITH_API int ornith_frspec_read_ids(const char* path, uint32_t* ids_out, size_t cap, size_t* n_out);
+ORNITH_API int ornith_frspec_write_ids(const char* path, const uint32_t* ids, size_t n, uint32_t vocab,
+                                       size_t* n_written);
+/* The superset merge of tools/merge_frspec.py:176-204 on token ids: merged = base + every id the
+ * corpus (a token-id stream) used at least min_count times and base lacks + `extra` (e.g. every
+ * id of one script), sorted and de-duplicated. It only adds, so coverage of what the base list
+ * covered is unchanged by construction. out == NULL only computes the statistics. */
+typedef struct ornith_frspec_merge_stats {
+  size_t n_merged;         /* ids in the merged list */
+  size_t corpus_tokens;    /* tokens in the corpus */
+  size_t covered_before;   /* of them inside the base list */
+  size_t covered_after;    /* inside the merged list, corpus additions only (the script's count apart) */
+  size_t missing_distinct; /* distinct corpus ids the base lacks */
+  size_t missing_kept;     /* of them seen >= min_count times */
+  size_t extra_new;        /* distinct extra ids the base lacks */
+} ornith_frspec_merge_stats;
+ORNITH_API int ornith_frspec_merge(const uint32_t* base, size_t n_base, const uint32_t* corpus, size_t n_corpus,
+                                   uint32_t min_count, const uint32_t* extra, size_t n_extra, uint32_t vocab,
+                                   uint32_t* out, size_t out_cap, ornith_frspec_merge_stats* stats);
 ORNITH_API int ornith_frspec_from_ids(ornith_model* m, const uint32_t* ids, int n, ornith_frspec** out);
 ORNITH_API int ornith_frspec_destroy(ornith_frspec* f);
 /* the pruned head as a Linear (for tests: pruned row == original row) and its size */

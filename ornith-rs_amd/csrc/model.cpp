@@ -24,6 +24,9 @@
 
 static const int kMaxRows = 16;  // activation rows a single forward may carry
 
+// frspec_list.cpp: reads and validates an FR-Spec id file
+int frspec_read_file(const char* path, std::vector<uint32_t>& ids);
+
 #define TRY(e)         \
   do {                 \
     int rc__ = (e);    \
@@ -288,12 +291,12 @@ int ornith_model_load(ornith_ctx* ctx, const ornith_weights* ws, const ornith_te
     if (rc) return fail(rc);       \
   } while (0)
   LTRY(ws_linear(ws, std::string(P) + "embed_tokens", &m->embed_tokens));
-  ORN_REQUIRE(m->embed_tokens.mode == ORNITH_LIN_AFFINE8 && m->embed_tokens.O == c.vocab_size &&
-                  m->embed_tokens.K == c.hidden_size,
-              "model_load: embed_tokens must be the 8-bit affine [vocab, hidden] table");
+  if (!(m->embed_tokens.mode == ORNITH_LIN_AFFINE8 && m->embed_tokens.O == c.vocab_size &&
+        m->embed_tokens.K == c.hidden_size))
+    return fail(ornith_fail(ORNITH_ERR_INVALID, "model_load: embed_tokens must be the 8-bit affine [vocab, hidden] table"));
   LTRY(ws_linear(ws, "language_model.lm_head", &m->lm_head));
-  ORN_REQUIRE(m->lm_head.O == c.vocab_size && m->lm_head.K == c.hidden_size,
-              "model_load: lm_head is [%d,%d]", m->lm_head.O, m->lm_head.K);
+  if (!(m->lm_head.O == c.vocab_size && m->lm_head.K == c.hidden_size))
+    return fail(ornith_fail(ORNITH_ERR_INVALID, "model_load: lm_head is [%d,%d]", m->lm_head.O, m->lm_head.K));
   LTRY(ws_tensor(ws, std::string(P) + "norm.weight", ORNITH_DT_BF16, c.hidden_size, &m->final_norm));
   const int Hv = c.linear_num_value_heads, H = c.hidden_size;
   m->layers.resize(c.num_hidden_layers);
@@ -538,27 +541,16 @@ int ornith_frspec_from_ids(ornith_model* m, const uint32_t* ids, int n, ornith_f
 }
 
 int ornith_frspec_load(ornith_model* m, const char* path, ornith_frspec** out) {
-  ORN_REQUIRE(m && path && out, "frspec_load: null argument");
-  FILE* fp = fopen(path, "rb");
-  if (!fp) return ornith_fail(ORNITH_ERR_IO, "%s: cannot open", path);
-  uint32_t n = 0;
-  if (fread(&n, 4, 1, fp) != 1) {
-    fclose(fp);
-    return ornith_fail(ORNITH_ERR_IO, "%s: %d bytes is too short to hold a count", path, 0);
+  ORN_REQUIRE(m && out, "frspec_load: null argument");
+  char dflt[4096];
+  if (!path) {
+    TRY(ornith_frspec_default_path(dflt, sizeof dflt));
+    path = dflt;
   }
-  fseek(fp, 0, SEEK_END);
-  const long size = ftell(fp);
-  if (size != 4 + 4 * (long)n) {
-    fclose(fp);
-    return ornith_fail(ORNITH_ERR_IO, "%s: header says %u ids, file holds %ld bytes", path, n, size);
-  }
-  fseek(fp, 4, SEEK_SET);
-  std::vector<uint32_t> ids(n);
-  const size_t got = n ? fread(ids.data(), 4, n, fp) : 0;
-  fclose(fp);
-  if (got != n) return ornith_fail(ORNITH_ERR_IO, "%s: short read", path);
-  ORN_REQUIRE(n > 0, "%s: FR-Spec list is empty", path);
-  return ornith_frspec_from_ids(m, ids.data(), (int)n, out);
+  std::vector<uint32_t> ids;
+  TRY(frspec_read_file(path, ids));
+  ORN_REQUIRE(!ids.empty(), "%s: FR-Spec list is empty", path);
+  return ornith_frspec_from_ids(m, ids.data(), (int)ids.size(), out);
 }
 
 int ornith_frspec_destroy(ornith_frspec* f) {

@@ -53,6 +53,10 @@ struct ornith_weights {
   // (WeightStore::tensor, /root/reference/src/weights.rs:101-108), hence mutable
   mutable std::map<std::string, Tensor> t;
   mutable size_t total_bytes = 0;
+  // set when copying a tensor in on first use failed (allocation / upload): find() then
+  // returns null for a tensor that does exist, and the caller reports this code instead of
+  // "no such tensor" (the message of the failing call is already recorded)
+  mutable int fault_rc = 0;
   ornith_weights_files* files = nullptr;
   QuantTable quant;
   const Tensor* find(const std::string& name) const {
@@ -61,6 +65,19 @@ struct ornith_weights {
     return files ? ws_fault_in(this, name) : nullptr;
   }
 };
+
+// A lookup came back null: the reason is a failed copy-in if there was one, else a missing tensor.
+#define ORN_REQUIRE_TENSOR(ws, t, ...)                               \
+  do {                                                               \
+    if (!(t)) {                                                      \
+      if ((ws)->fault_rc) {                                          \
+        const int rc__ = (ws)->fault_rc;                             \
+        (ws)->fault_rc = 0;                                          \
+        return rc__;                                                 \
+      }                                                              \
+      return ornith_fail(ORNITH_ERR_INVALID, __VA_ARGS__);           \
+    }                                                                \
+  } while (0)
 
 // Resolves module `path` into a Linear by the tensors present (k-quant / affine8 / dense).
 int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* out);

@@ -547,7 +547,6 @@ __device__ __forceinline__ void one_down(const OneArgs& o, int dd, char* lds) {
   float* wj = reinterpret_cast<float*>(lds + sizeof(float) * (kMaxK + 1) * COLS);
   float* gsig = wj + kMaxK;
   const int j0 = 2 * wave;
-  const bool two = j0 + 1 <= k;
 
   typename KL::Lane L;
   L.set_chunk(c);

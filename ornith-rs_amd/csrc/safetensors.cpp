@@ -615,16 +615,20 @@ const Tensor* ws_fault_in(const ornith_weights* ws, const std::string& name) {
   const StTensor* info = st->get(name);
   if (!info) return nullptr;
   if (info->nbytes == 0) {
-    ornith_fail(ORNITH_ERR_INVALID, "%s: empty tensor", name.c_str());
+    ws->fault_rc = ornith_fail(ORNITH_ERR_INVALID, "%s: empty tensor", name.c_str());
     return nullptr;
   }
   Tensor t;
   t.dtype = info->dtype;
   t.shape = info->shape;
   t.bytes = info->nbytes;
-  if (ornith_alloc(ws->ctx, t.bytes, &t.d)) return nullptr;
-  if (ornith_upload(ws->ctx, t.d, st->bytes(*info), t.bytes)) {
+  if (int rc = ornith_alloc(ws->ctx, t.bytes, &t.d)) {
+    ws->fault_rc = rc;
+    return nullptr;
+  }
+  if (int rc = ornith_upload(ws->ctx, t.d, st->bytes(*info), t.bytes)) {
     ornith_free(ws->ctx, t.d);
+    ws->fault_rc = rc;
     return nullptr;
   }
   ws->total_bytes += t.bytes;
@@ -802,7 +806,7 @@ int ornith_weights_fetch(const ornith_weights* ws, const char* name, int* dtype,
                          int* ndim, void* host_out, size_t host_bytes) {
   ORN_REQUIRE(ws && name, "weights_fetch: null argument");
   const Tensor* t = ws->find(name);
-  ORN_REQUIRE(t, "no tensor named %s", name);
+  ORN_REQUIRE_TENSOR(ws, t, "no tensor named %s", name);
   if (dtype) *dtype = t->dtype;
   if (ndim) *ndim = (int)t->shape.size();
   if (shape)

@@ -38,7 +38,7 @@ static int kq_from(const ornith_weights* ws, const std::string& path, bool route
   const Tensor* w = ws->find(path + ".weight");
   const Tensor* s = ws->find(path + ".scales");
   const Tensor* d = ws->find(path + ".dm");
-  ORN_REQUIRE(w && s && d, "%s: k-quant module needs .weight, .scales and .dm", path.c_str());
+  ORN_REQUIRE_TENSOR(ws, w && s && d, "%s: k-quant module needs .weight, .scales and .dm", path.c_str());
   ORN_REQUIRE(w->dtype == ORNITH_DT_U32 || w->dtype == ORNITH_DT_U8, "%s.weight must be uint32",
               path.c_str());
   ORN_REQUIRE(s->dtype == ORNITH_DT_U8, "%s.scales must be uint8", path.c_str());
@@ -69,7 +69,7 @@ int ws_kmatrix(const ornith_weights* ws, const std::string& path, ornith_kmatrix
 int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* out) {
   memset(out, 0, sizeof *out);
   const Tensor* w = ws->find(path + ".weight");
-  ORN_REQUIRE(w, "%s.weight: no such tensor", path.c_str());
+  ORN_REQUIRE_TENSOR(ws, w, "%s.weight: no such tensor", path.c_str());
   if (ornith_weights_has(ws, (path + ".dm").c_str())) {
     out->mode = ORNITH_LIN_KQUANT;
     int rc = kq_from(ws, path, false, &out->km);
@@ -118,7 +118,7 @@ int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* 
 int ws_tensor(const ornith_weights* ws, const std::string& name, int dtype, int64_t numel,
               const void** out) {
   const Tensor* t = ws->find(name);
-  ORN_REQUIRE(t, "%s: no such tensor", name.c_str());
+  ORN_REQUIRE_TENSOR(ws, t, "%s: no such tensor", name.c_str());
   ORN_REQUIRE(t->dtype == dtype, "%s: dtype %d, expected %d", name.c_str(), t->dtype, dtype);
   ORN_REQUIRE(t->numel() == numel, "%s: %lld elements, expected %lld", name.c_str(),
               (long long)t->numel(), (long long)numel);

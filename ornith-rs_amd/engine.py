@@ -300,10 +300,13 @@ class FrSpec:
     """FrSpec::load / from a list of ids; holds the pruned head."""
 
     def __init__(self, model, ids=None, path=None):
+        """ids: the list itself; path: a list file; neither: the default location
+        (frspec::default_path: $ORNITH_FRSPEC, else <refs>/frspec/ids_64k.bin)."""
         self.model = model
         h = C.c_void_p()
-        if path is not None:
-            _check(lib().ornith_frspec_load(model.h, str(path).encode(), C.byref(h)), "frspec_load")
+        if path is not None or ids is None:
+            _check(lib().ornith_frspec_load(model.h, str(path).encode() if path is not None else None, C.byref(h)),
+                   "frspec_load")
         else:
             ids = np.ascontiguousarray(ids, dtype=np.uint32)
             _check(lib().ornith_frspec_from_ids(model.h, _ptr(ids), len(ids), C.byref(h)), "frspec_from_ids")
@@ -522,6 +525,48 @@ def gdn_step(ctx, conv_state, qkv, cw, wa, wb, xn, H, a_log, dt_bias, T, K, Hk, 
                                  a_log.ptr, dt_bias.ptr, T, K, Hk, Dk, Hv, Dv, C.c_float(eps), state_in.ptr,
                                  snapshots.ptr, int(snap_all), norm_w.ptr, z.ptr, C.c_float(norm_eps),
                                  conv_input.ptr, gated_out.ptr), "gdn_step")
+
+
+# ---- FR-Spec id lists on the host (src/frspec.rs:101-158, tools/merge_frspec.py) ------------------
+class FrSpecMergeStats(C.Structure):
+    _fields_ = [(n, C.c_size_t) for n in ("n_merged", "corpus_tokens", "covered_before", "covered_after",
+                                           "missing_distinct", "missing_kept", "extra_new")]
+
+
+def frspec_default_path():
+    buf = C.create_string_buffer(4096)
+    _check(lib().ornith_frspec_default_path(buf, C.c_size_t(4096)), "frspec_default_path")
+    return buf.value.decode()
+
+
+def frspec_read_ids(path):
+    n = C.c_size_t()
+    _check(lib().ornith_frspec_read_ids(str(path).encode(), None, C.c_size_t(0), C.byref(n)), "frspec_read_ids")
+    out = np.empty(n.value, np.uint32)
+    _check(lib().ornith_frspec_read_ids(str(path).encode(), _ptr(out), C.c_size_t(out.size), C.byref(n)), "frspec_read_ids")
+    return out
+
+
+def frspec_write_ids(path, ids, vocab):
+    ids = np.ascontiguousarray(ids, dtype=np.uint32)
+    n = C.c_size_t()
+    _check(lib().ornith_frspec_write_ids(str(path).encode(), _ptr(ids), C.c_size_t(ids.size), C.c_uint32(vocab),
+                                         C.byref(n)), "frspec_write_ids")
+    return n.value
+
+
+def frspec_merge(base, corpus, min_count, extra, vocab):
+    """The superset merge on token ids: returns (merged ids, FrSpecMergeStats)."""
+    base = np.ascontiguousarray(base, dtype=np.uint32)
+    corpus = np.ascontiguousarray(corpus if corpus is not None else [], dtype=np.uint32)
+    extra = np.ascontiguousarray(extra if extra is not None else [], dtype=np.uint32)
+    st = FrSpecMergeStats()
+    args = (_ptr(base), C.c_size_t(base.size), _ptr(corpus) if corpus.size else None, C.c_size_t(corpus.size),
+            C.c_uint32(min_count), _ptr(extra) if extra.size else None, C.c_size_t(extra.size), C.c_uint32(vocab))
+    _check(lib().ornith_frspec_merge(*args, None, C.c_size_t(0), C.byref(st)), "frspec_merge")
+    out = np.empty(st.n_merged, np.uint32)
+    _check(lib().ornith_frspec_merge(*args, _ptr(out), C.c_size_t(out.size), C.byref(st)), "frspec_merge")
+    return out, st
 
 
 # ---- prefill-width k-quant GEMM (src/ops/kquant.rs:783-1027) --------------------------------

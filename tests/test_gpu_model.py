@@ -113,6 +113,14 @@ def test_frspec_prune_map_and_file_format(orn, ctx, tiny, tmp_path):
     fr = orn.FrSpec(model, path=path)
     assert fr.head()[1] == 256
     fr.close()
+    # no path at all: the default location (frspec::default_path, src/frspec.rs:153-158)
+    os.environ["ORNITH_FRSPEC"] = str(path)
+    try:
+        fr = orn.FrSpec(model)
+        assert fr.head()[1] == 256
+        fr.close()
+    finally:
+        del os.environ["ORNITH_FRSPEC"]
     bad = {
         "empty": struct.pack("<I", 0),
         "too many": struct.pack("<I", V) + np.arange(V, dtype="<u4").tobytes(),
@@ -121,7 +129,7 @@ def test_frspec_prune_map_and_file_format(orn, ctx, tiny, tmp_path):
         "holds": struct.pack("<I", 5) + np.array([1, 2], "<u4").tobytes(),
     }
     msgs = {"empty": "empty", "too many": "nothing to prune", "out of range": "outside the vocabulary",
-            "listed twice": "listed twice", "holds": "header says"}
+            "listed twice": "listed twice", "holds": "says 5 ids"}
     for k, blob in bad.items():
         path.write_bytes(blob)
         with pytest.raises(orn.OrnithError, match=msgs[k]):
