@@ -161,13 +161,16 @@ ORNITH_API int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w,
 #define ORNITH_LIN_KQUANT 0  /* Linear::K(KMatrix) */
 #define ORNITH_LIN_AFFINE8 1 /* Linear::Mlx, mlx affine 8-bit group 64 (quantized.rs:311-333) */
 #define ORNITH_LIN_DENSE 2   /* bf16 [O,K], ops::matmul::gemv (matmul.rs:334-438) */
+#define ORNITH_LIN_AFFINE4 3 /* Linear::Mlx, mlx affine 4-bit group 32, the published artifact's format
+                                (quantized.rs:311-333; vendored quantized.h:235-244) */
 typedef struct ornith_linear {
   int mode;
   int O, K;
   ornith_kmatrix km;    /* KQUANT */
-  const void* d_w;      /* AFFINE8: u8[O,K] (the reference's u32[O,K/4] bytes); DENSE: bf16[O,K] */
-  const void* d_scales; /* AFFINE8: bf16[O,K/64] */
-  const void* d_biases; /* AFFINE8: bf16[O,K/64] */
+  const void* d_w;      /* AFFINE8: u8[O,K] (the reference's u32[O,K/4] bytes); DENSE: bf16[O,K];
+                           AFFINE4: u8[O,K/2] (the reference's u32[O,K/8] bytes, lowest nibble first) */
+  const void* d_scales; /* AFFINE8: bf16[O,K/64]; AFFINE4: bf16[O,K/32] */
+  const void* d_biases; /* as d_scales */
 } ornith_linear;
 
 /* Linear::matmul (src/ops/linear.rs:60-110): y[M,O] = x[M,K] . W^T, bf16 in/out. */
@@ -199,8 +202,16 @@ ORNITH_API int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, i
                                       const void* d_x, int x_rows, const uint32_t* d_lhs,
                                       const uint32_t* d_rhs, int rows, void* d_y);
 
-/* ops::embedding::embedding (src/ops/embedding.rs:18-46): 8-bit affine g64 table
- * rows -> bf16; ids are device u32, clamped to the table. */
+/* quantized::gather_qmv for the 4-bit affine format (src/ops/quantized.rs:531-589): stacked
+ * experts w u8[E,O,K/2], scales / biases bf16[E,O,K/32]; out[r] = x[lhs[r]] . W[rhs[r]]^T, bf16 in
+ * and out. Ids past the end are clamped to the last row / expert. */
+ORNITH_API int ornith_affine4_gather_qmv(ornith_ctx* ctx, const void* d_w, const void* d_scales,
+                                         const void* d_biases, int E, int O, int K, const void* d_x,
+                                         int x_rows, const uint32_t* d_lhs, const uint32_t* d_rhs, int rows,
+                                         void* d_y);
+
+/* ops::embedding::embedding (src/ops/embedding.rs:18-46): affine table rows (8-bit group 64 or
+ * 4-bit group 32) -> bf16; ids are device u32, clamped to the table. */
 ORNITH_API int ornith_embedding(ornith_ctx* ctx, const ornith_linear* table, const uint32_t* d_ids,
                                 int n, void* d_out);
 

@@ -29,6 +29,13 @@ void orc_dense_gather_mv(const bf16_t* w, int O, int K, const bf16_t* x, const u
                          const uint32_t* rhs, int rows, bf16_t* y);
 void orc_embedding(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K,
                    const uint32_t* ids, int n, bf16_t* out);
+void orc_embedding4(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K,
+                    const uint32_t* ids, int n, bf16_t* out);
+/* the token embedding through whichever affine format the table is in */
+static void embed_rows(const orc_linear* t, int K, const uint32_t* ids, int n, bf16_t* out) {
+  if (t->mode == 3) orc_embedding4(t->aw, t->as, t->ab, K, ids, n, out);
+  else orc_embedding(t->aw, t->as, t->ab, K, ids, n, out);
+}
 void orc_rms_norm(const bf16_t* x, const bf16_t* w, int rows, int n, float eps, bf16_t* out);
 void orc_add_rms_norm(const bf16_t* a, const bf16_t* b, const bf16_t* w, int rows, int n, float eps,
                       bf16_t* h_out, bf16_t* out);
@@ -193,7 +200,7 @@ ORC_API void orc_forward(orc_state* s, const uint32_t* tokens, int T, int captur
             Dv = c->linear_value_head_dim, K = c->linear_conv_kernel_dim, S = K - 1, D = conv_dim(c);
   const size_t hb = 2 * (size_t)T * H, se = state_elems(c);
   bf16_t *x = malloc(hb), *normed = malloc(hb), *r = malloc(hb), *h = malloc(hb), *n2 = malloc(hb), *mo = malloc(hb);
-  orc_embedding(m->embed.aw, m->embed.as, m->embed.ab, H, tokens, T, x);
+  embed_rows(&m->embed, H, tokens, T, x);
   orc_rms_norm(x, m->layers[0].input_ln, T, H, c->rms_norm_eps, normed);
   for (int i = 0; i < L; ++i) {
     const orc_layer_w* Lw = &m->layers[i];
@@ -301,7 +308,7 @@ ORC_API void orc_mtp_hidden(orc_state* s, const orc_mtp_w* w, const bf16_t* trun
   const size_t hb = 2 * (size_t)T * H;
   bf16_t *emb = malloc(hb), *e = malloc(hb), *hh = malloc(hb), *joined = malloc(2 * hb), *x = malloc(hb);
   bf16_t *normed = malloc(hb), *r = malloc(hb), *h2 = malloc(hb), *n2 = malloc(hb), *mo = malloc(hb), *sum = malloc(hb);
-  orc_embedding(m->embed.aw, m->embed.as, m->embed.ab, H, next_ids, T, emb);
+  embed_rows(&m->embed, H, next_ids, T, emb);
   orc_rms_norm(emb, w->pre_fc_norm_embedding, T, H, c->rms_norm_eps, e);
   orc_rms_norm(trunk_hidden, w->pre_fc_norm_hidden, T, H, c->rms_norm_eps, hh);
   for (int t = 0; t < T; ++t) {

@@ -138,6 +138,68 @@ ORC_API void orc_affine8_qmv(const uint8_t* w, const bf16_t* scales, const bf16_
   free(xf);
 }
 
+/* ---- 4-bit affine, group 32 (the published artifact's format: mlx affine, bits 4, group 32;
+ * /root/reference/src/ops/quantized.rs:311-333, vendored quantized.h:235-244 qdot at bits = 4):
+ * w holds K/2 bytes a row, element i in the low (even i) or high (odd i) nibble of byte i/2
+ * (mlx packs eight nibbles into a u32, lowest first); scales/biases bf16[O,K/32].
+ * y = sum_g (s_g * sum x q + b_g * sum x). Lane l owns 16-element chunks j = l + 64c (two a
+ * group); per chunk one fma chain over x*q and one plain sum of x, p = fma(sum_x, bias,
+ * scale * accum); tree64. */
+float orc_affine4_row_dot(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K,
+                          const float* x) {
+  float lanes[64];
+  for (int l = 0; l < 64; ++l) lanes[l] = 0.f;
+  for (int j = 0; j < K / 16; ++j) {
+    const float s = orc_bf16_to_f32(scales[j / 2]), b = orc_bf16_to_f32(biases[j / 2]);
+    float acc = 0.f, sum = 0.f;
+    for (int i = 0; i < 16; ++i) {
+      const uint8_t byte = w[8 * j + i / 2];
+      const float q = (float)((i & 1) ? (byte >> 4) : (byte & 0xF));
+      acc = fmaf(x[16 * j + i], q, acc);
+      sum = sum + x[16 * j + i];
+    }
+    float pp = s * acc;
+    pp = fmaf(sum, b, pp);
+    lanes[j % 64] = lanes[j % 64] + pp;
+  }
+  return orc_tree64(lanes);
+}
+
+/* E == 1, lhs == rhs == NULL: plain mat-vec over M = rows rows of x. Otherwise the gathered
+ * form (quantized.rs:531-589): y[r] = x[lhs[r]] . W[rhs[r]]^T over stacked experts [E,O,K]. */
+ORC_API void orc_affine4_gather_qmv(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int E, int O,
+                                    int K, const bf16_t* x, const uint32_t* lhs, const uint32_t* rhs, int rows,
+                                    bf16_t* y) {
+  (void)E;
+#pragma omp parallel for schedule(dynamic)
+  for (int r = 0; r < rows; ++r) {
+    float* xf = (float*)malloc(sizeof(float) * (size_t)K);
+    const size_t xr = lhs ? lhs[r] : (size_t)r, e = rhs ? rhs[r] : 0;
+    for (int i = 0; i < K; ++i) xf[i] = orc_bf16_to_f32(x[xr * K + i]);
+    for (int o = 0; o < O; ++o) {
+      const size_t row = e * O + o;
+      y[(size_t)r * O + o] = orc_f32_to_bf16(orc_affine4_row_dot(w + row * (K / 2), scales + row * (K / 32),
+                                                                 biases + row * (K / 32), K, xf));
+    }
+    free(xf);
+  }
+}
+
+/* 4-bit embedding rows: out = bf16(bf16(q * scale) + bias), as the 8-bit lookup below */
+ORC_API void orc_embedding4(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K,
+                            const uint32_t* ids, int n, bf16_t* out) {
+  for (int r = 0; r < n; ++r) {
+    const size_t row = ids[r];
+    for (int i = 0; i < K; ++i) {
+      const uint8_t byte = w[row * (K / 2) + i / 2];
+      const float q = (float)((i & 1) ? (byte >> 4) : (byte & 0xF));
+      const float s = orc_bf16_to_f32(scales[row * (K / 32) + i / 32]);
+      const float b = orc_bf16_to_f32(biases[row * (K / 32) + i / 32]);
+      out[(size_t)r * K + i] = orc_f32_to_bf16(orc_rb(q * s) + b);
+    }
+  }
+}
+
 /* embedding row lookup: out = bf16(bf16(q * scale) + bias)
  * (vendored quantized.h affine_dequantize at T = bf16; src/ops/embedding.rs:18-46) */
 ORC_API void orc_embedding(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K,
@@ -172,6 +234,9 @@ void orc_linear_fwd(const orc_linear* L, const bf16_t* x, int M, bf16_t* y) {
       else if (L->mode == 1)
         v = orc_affine8_row_dot(L->aw + (size_t)o * K, L->as + (size_t)o * (K / 64),
                                 L->ab + (size_t)o * (K / 64), K, xf);
+      else if (L->mode == 3)
+        v = orc_affine4_row_dot(L->aw + (size_t)o * (K / 2), L->as + (size_t)o * (K / 32),
+                                L->ab + (size_t)o * (K / 32), K, xf);
       else
         v = orc_dense_row_dot((const bf16_t*)L->aw + (size_t)o * K, K, xf);
       y[(size_t)m * O + o] = orc_f32_to_bf16(v);

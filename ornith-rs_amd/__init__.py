@@ -187,7 +187,7 @@ FN_XOR_LANE = 9  # + i: value of lane l ^ 2**i, i = 0..5
 
 
 # ---- Linear / MoE ---------------------------------------------------------------
-LIN_KQUANT, LIN_AFFINE8, LIN_DENSE = 0, 1, 2
+LIN_KQUANT, LIN_AFFINE8, LIN_DENSE, LIN_AFFINE4 = 0, 1, 2, 3
 
 
 class LinearStruct(C.Structure):
@@ -227,6 +227,14 @@ class Linear:
                                    bufs[2].ptr), bufs)
 
     @staticmethod
+    def affine4(ctx, w, scales, biases):
+        """w: u8 [O, K/2] (two 4-bit codes a byte, low nibble first); scales / biases bf16 [O, K/32]."""
+        O, K = scales.shape[0], scales.shape[1] * 32
+        bufs = [ctx.to_device(t) for t in (w, scales, biases)]
+        return Linear(LinearStruct(LIN_AFFINE4, O, K, KMatrixStruct(), bufs[0].ptr, bufs[1].ptr,
+                                   bufs[2].ptr), bufs)
+
+    @staticmethod
     def dense(ctx, w):
         O, K = w.shape
         buf = ctx.to_device(w)
@@ -260,6 +268,12 @@ def linear_matmul_multi(self, lins, x, M, ys):
 def dense_gather_mv(self, w, E, O, K, x, x_rows, lhs, rhs, rows, y):
     _check(lib().ornith_dense_gather_mv(self.h, w.ptr, E, O, K, x.ptr, x_rows, lhs.ptr, rhs.ptr,
                                         rows, y.ptr), "dense_gather_mv")
+
+
+@_ctx_method
+def affine4_gather_qmv(self, w, scales, biases, E, O, K, x, x_rows, lhs, rhs, rows, y):
+    _check(lib().ornith_affine4_gather_qmv(self.h, w.ptr, scales.ptr, biases.ptr, E, O, K, x.ptr, x_rows, lhs.ptr,
+                                           rhs.ptr, rows, y.ptr), "affine4_gather_qmv")
 
 
 @_ctx_method

@@ -53,6 +53,53 @@ __global__ __launch_bounds__(64) void affine8_qmv_kernel(const uint8_t* w, const
   if (lane == 0) y[(size_t)m * O + o] = dm_f2bf(v);
 }
 
+// ---- 4-bit affine, group 32 ------------------------------------------------
+// One wavefront per output row (four rows a workgroup); lane l owns the 16-element chunks
+// j = l + 64c: 8 code bytes and 16 activations, both one aligned load. GATHER selects the
+// expert and the activation row through lhs / rhs.
+template <bool GATHER>
+__global__ __launch_bounds__(256) void affine4_qmv_kernel(const uint8_t* w, const bf16_t* scales,
+                                                          const bf16_t* biases, const bf16_t* x, bf16_t* y,
+                                                          int E, int O, int K, int x_rows, const uint32_t* lhs,
+                                                          const uint32_t* rhs) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int o = blockIdx.x * 4 + wave, r = blockIdx.y;
+  if (o >= O) return;
+  size_t row = o, xi = r;
+  if constexpr (GATHER) {
+    xi = min(lhs[r], (uint32_t)(x_rows - 1));
+    row = (size_t)min(rhs[r], (uint32_t)(E - 1)) * O + o;
+  }
+  const uint8_t* wr = w + row * (K / 2);
+  const bf16_t* sr = scales + row * (K / 32);
+  const bf16_t* br = biases + row * (K / 32);
+  const bf16_t* xr = x + xi * K;
+  float acc_lane = 0.f;
+  for (int j = lane; j < K / 16; j += 64) {
+    const uint2 q = *reinterpret_cast<const uint2*>(wr + 8 * j);
+    const uint4 xa = *reinterpret_cast<const uint4*>(xr + 16 * j);
+    const uint4 xb = *reinterpret_cast<const uint4*>(xr + 16 * j + 8);
+    const float xs[16] = {dm_bf2f_lo(xa.x), dm_bf2f_hi(xa.x), dm_bf2f_lo(xa.y), dm_bf2f_hi(xa.y),
+                          dm_bf2f_lo(xa.z), dm_bf2f_hi(xa.z), dm_bf2f_lo(xa.w), dm_bf2f_hi(xa.w),
+                          dm_bf2f_lo(xb.x), dm_bf2f_hi(xb.x), dm_bf2f_lo(xb.y), dm_bf2f_hi(xb.y),
+                          dm_bf2f_lo(xb.z), dm_bf2f_hi(xb.z), dm_bf2f_lo(xb.w), dm_bf2f_hi(xb.w)};
+    const uint32_t qw[2] = {q.x, q.y};
+    float acc = 0.f, sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float qf = (float)((qw[i >> 3] >> (4 * (i & 7))) & 0xfu);
+      acc = dm_fma(xs[i], qf, acc);
+      sum = sum + xs[i];
+    }
+    const float s = dm_bf2f(sr[j >> 1]), b = dm_bf2f(br[j >> 1]);
+    float p = s * acc;
+    p = dm_fma(sum, b, p);
+    acc_lane = acc_lane + p;
+  }
+  const float v = dm_wave_sum<64>(acc_lane);
+  if (lane == 0) y[(size_t)r * O + o] = dm_f2bf(v);
+}
+
 // ---- dense bf16 ------------------------------------------------------------
 // grid.x covers rows four at a time (one per wavefront), grid.y is the
 // activation row; GATHER selects expert / activation row through lhs, rhs.
@@ -113,6 +160,20 @@ __global__ void embedding_kernel(const uint8_t* w, const bf16_t* scales, const b
   out[(size_t)r * K + i] = dm_f2bf(v + b);
 }
 
+// 4-bit table rows: out = bf16(bf16(q * scale) + bias)
+__global__ void embedding4_kernel(const uint8_t* w, const bf16_t* scales, const bf16_t* biases,
+                                  const uint32_t* ids, bf16_t* out, int V, int K) {
+  const int r = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= K) return;
+  const size_t row = min(ids[r], (uint32_t)(V - 1));
+  const uint8_t byte = w[row * (K / 2) + i / 2];
+  const float q = (float)((i & 1) ? (byte >> 4) : (byte & 0xF));
+  const float s = dm_bf2f(scales[row * (K / 32) + i / 32]);
+  const float b = dm_bf2f(biases[row * (K / 32) + i / 32]);
+  out[(size_t)r * K + i] = dm_f2bf(dm_rb(q * s) + b);
+}
+
 template <bool GATHER>
 int launch_dense(ornith_ctx* ctx, const DenseSegs& s, const void* d_x, int K, int E, int x_rows,
                  const uint32_t* d_lhs, const uint32_t* d_rhs, int rows) {
@@ -167,6 +228,15 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
                          (const uint8_t*)w->d_w, (const bf16_t*)w->d_scales,
                          (const bf16_t*)w->d_biases, (const bf16_t*)d_x, (bf16_t*)d_y, w->O, w->K);
       ORN_LAUNCH_CHECK("affine8_qmv_kernel");
+      return ORNITH_OK;
+    case ORNITH_LIN_AFFINE4:
+      ORN_REQUIRE(w->d_w && w->d_scales && w->d_biases, "linear_matmul: affine tensor missing");
+      ORN_REQUIRE(w->K % 32 == 0 && w->O >= 1 && M <= 65535, "linear_matmul: 4-bit affine O=%d K=%d", w->O, w->K);
+      hipLaunchKernelGGL(affine4_qmv_kernel<false>, dim3((w->O + 3) / 4, M), dim3(256), 0, ctx->stream,
+                         (const uint8_t*)w->d_w, (const bf16_t*)w->d_scales, (const bf16_t*)w->d_biases,
+                         (const bf16_t*)d_x, (bf16_t*)d_y, 1, w->O, w->K, M, (const uint32_t*)nullptr,
+                         (const uint32_t*)nullptr);
+      ORN_LAUNCH_CHECK("affine4_qmv_kernel");
       return ORNITH_OK;
     case ORNITH_LIN_DENSE:
       ORN_REQUIRE(w->d_w, "linear_matmul: dense weight missing");
@@ -249,14 +319,35 @@ int ornith_dense_gather_mv(ornith_ctx* ctx, const void* d_w, int E, int O, int K
   return dense_gather_mv_multi(ctx, ws, 1, E, O, K, d_x, x_rows, d_lhs, d_rhs, rows, ys);
 }
 
+int ornith_affine4_gather_qmv(ornith_ctx* ctx, const void* d_w, const void* d_scales, const void* d_biases,
+                              int E, int O, int K, const void* d_x, int x_rows, const uint32_t* d_lhs,
+                              const uint32_t* d_rhs, int rows, void* d_y) {
+  ORN_REQUIRE(ctx && d_w && d_scales && d_biases && d_x && d_lhs && d_rhs && d_y, "affine4_gather_qmv: null argument");
+  ORN_REQUIRE(E >= 1 && O >= 1 && K % 32 == 0 && x_rows >= 1 && rows >= 0 && rows <= 65535,
+              "affine4_gather_qmv: E=%d O=%d K=%d rows=%d", E, O, K, rows);
+  if (rows == 0) return ORNITH_OK;
+  hipLaunchKernelGGL(affine4_qmv_kernel<true>, dim3((O + 3) / 4, rows), dim3(256), 0, ctx->stream,
+                     (const uint8_t*)d_w, (const bf16_t*)d_scales, (const bf16_t*)d_biases, (const bf16_t*)d_x,
+                     (bf16_t*)d_y, E, O, K, x_rows, d_lhs, d_rhs);
+  ORN_LAUNCH_CHECK("affine4_qmv_kernel<gather>");
+  return ORNITH_OK;
+}
+
 int ornith_embedding(ornith_ctx* ctx, const ornith_linear* table, const uint32_t* d_ids, int n,
                      void* d_out) {
   ORN_REQUIRE(ctx && table && d_ids && d_out, "embedding: null argument");
-  ORN_REQUIRE(table->mode == ORNITH_LIN_AFFINE8,
-              "embedding: table mode %d; the lookup is defined for the 8-bit affine table only",
+  ORN_REQUIRE(table->mode == ORNITH_LIN_AFFINE8 || table->mode == ORNITH_LIN_AFFINE4,
+              "embedding: table mode %d; the lookup is defined for the affine tables only",
               table->mode);
   ORN_REQUIRE(table->K % 64 == 0 && n >= 0 && n <= 65535, "embedding: K=%d n=%d", table->K, n);
   if (n == 0) return ORNITH_OK;
+  if (table->mode == ORNITH_LIN_AFFINE4) {
+    hipLaunchKernelGGL(embedding4_kernel, dim3((table->K + 255) / 256, n), dim3(256), 0, ctx->stream,
+                       (const uint8_t*)table->d_w, (const bf16_t*)table->d_scales,
+                       (const bf16_t*)table->d_biases, d_ids, (bf16_t*)d_out, table->O, table->K);
+    ORN_LAUNCH_CHECK("embedding4_kernel");
+    return ORNITH_OK;
+  }
   hipLaunchKernelGGL(embedding_kernel, dim3((table->K + 255) / 256, n), dim3(256), 0, ctx->stream,
                      (const uint8_t*)table->d_w, (const bf16_t*)table->d_scales,
                      (const bf16_t*)table->d_biases, d_ids, (bf16_t*)d_out, table->O, table->K);

@@ -291,9 +291,9 @@ int ornith_model_load(ornith_ctx* ctx, const ornith_weights* ws, const ornith_te
     if (rc) return fail(rc);       \
   } while (0)
   LTRY(ws_linear(ws, std::string(P) + "embed_tokens", &m->embed_tokens));
-  if (!(m->embed_tokens.mode == ORNITH_LIN_AFFINE8 && m->embed_tokens.O == c.vocab_size &&
-        m->embed_tokens.K == c.hidden_size))
-    return fail(ornith_fail(ORNITH_ERR_INVALID, "model_load: embed_tokens must be the 8-bit affine [vocab, hidden] table"));
+  if (!((m->embed_tokens.mode == ORNITH_LIN_AFFINE8 || m->embed_tokens.mode == ORNITH_LIN_AFFINE4) &&
+        m->embed_tokens.O == c.vocab_size && m->embed_tokens.K == c.hidden_size))
+    return fail(ornith_fail(ORNITH_ERR_INVALID, "model_load: embed_tokens must be an affine [vocab, hidden] table"));
   LTRY(ws_linear(ws, "language_model.lm_head", &m->lm_head));
   if (!(m->lm_head.O == c.vocab_size && m->lm_head.K == c.hidden_size))
     return fail(ornith_fail(ORNITH_ERR_INVALID, "model_load: lm_head is [%d,%d]", m->lm_head.O, m->lm_head.K));

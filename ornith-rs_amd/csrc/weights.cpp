@@ -82,25 +82,32 @@ int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* 
   if (rc) return rc;
   if (const Tensor* b = ws->find(path + ".biases")) {
     const Tensor* s = ws->find(path + ".scales");
-    if (ws->quant.loaded) {
-      const QuantSpec q = ws->quant.lookup(path);
-      ORN_REQUIRE(q.bits == 8 && q.group_size == 64,
-                  "%s: affine %d-bit group %d is not carried (8-bit group 64 only)", path.c_str(),
-                  q.bits, q.group_size);
-    }
     ORN_REQUIRE(s, "%s: affine module needs .scales", path.c_str());
     ORN_REQUIRE(s->dtype == ORNITH_DT_BF16 && b->dtype == ORNITH_DT_BF16,
                 "%s: affine scales/biases must be bfloat16", path.c_str());
     ORN_REQUIRE(w->dtype == ORNITH_DT_U32 || w->dtype == ORNITH_DT_U8, "%s.weight must be uint32",
                 path.c_str());
-    ORN_REQUIRE(s->shape.size() == 2 && b->shape == s->shape, "%s: scales/biases must be [O, K/64]",
+    ORN_REQUIRE(s->shape.size() == 2 && b->shape == s->shape, "%s: scales/biases must be [O, K/group]",
                 path.c_str());
-    out->mode = ORNITH_LIN_AFFINE8;
+    // two affine layouts are carried: 8-bit group 64 and 4-bit group 32 (the published
+    // artifact's). The quantization block says which; without one the byte count does
+    // (64 weight bytes per group against 16).
+    const size_t groups = (size_t)s->shape[0] * (size_t)s->shape[1];
+    ORN_REQUIRE(groups > 0, "%s: empty scales", path.c_str());
+    int bits = w->bytes == groups * 64 ? 8 : w->bytes == groups * 16 ? 4 : 0, group = bits == 8 ? 64 : 32;
+    if (ws->quant.loaded) {
+      const QuantSpec q = ws->quant.lookup(path);
+      ORN_REQUIRE((q.bits == 8 && q.group_size == 64) || (q.bits == 4 && q.group_size == 32),
+                  "%s: affine %d-bit group %d is not carried (8-bit group 64 and 4-bit group 32 only)",
+                  path.c_str(), q.bits, q.group_size);
+      ORN_REQUIRE(bits == q.bits, "%s.weight: %zu bytes is not %d-bit group-%d for its %zu groups", path.c_str(),
+                  w->bytes, q.bits, q.group_size, groups);
+    }
+    ORN_REQUIRE(bits != 0, "%s.weight: %zu bytes is neither 8-bit group-64 nor 4-bit group-32 for [%lld, %lld] groups",
+                path.c_str(), w->bytes, (long long)s->shape[0], (long long)s->shape[1]);
+    out->mode = bits == 8 ? ORNITH_LIN_AFFINE8 : ORNITH_LIN_AFFINE4;
     out->O = (int)s->shape[0];
-    out->K = (int)s->shape[1] * 64;
-    ORN_REQUIRE(w->bytes == (size_t)out->O * out->K,
-                "%s.weight: %zu bytes is not 8-bit group-64 for [%d, %d]", path.c_str(), w->bytes,
-                out->O, out->K);
+    out->K = (int)s->shape[1] * group;
     out->d_w = w->d;
     out->d_scales = s->d;
     out->d_biases = b->d;

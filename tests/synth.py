@@ -84,7 +84,11 @@ def _norm_w(rng, n):
 class SynthModel:
     """All tensors of a trunk (+ optional MTP head) for a config dict."""
 
-    def __init__(self, cfg, seed=0, with_mtp=True, with_oracle=True):
+    def __init__(self, cfg, seed=0, with_mtp=True, with_oracle=True, affine="affine8"):
+        """affine: the format of the two affine modules (embed_tokens, shared_expert_gate):
+        'affine8' (8-bit group 64, as in the k-quant artifact) or 'affine4' (4-bit group 32, the
+        published artifact's format)."""
+        self.affine = affine
         self.cfg = dict(cfg)
         self.rng = np.random.default_rng(seed)
         self.tensors = {}     # name -> (array, dtype code)
@@ -97,7 +101,7 @@ class SynthModel:
         D, Hv = 2 * kd + vd, c["linear_num_value_heads"]
         hd, Hq, Hkv = c["head_dim"], c["num_attention_heads"], c["num_key_value_heads"]
         P = "language_model.model."
-        self.embed = self._linear(P + "embed_tokens", "affine8", c["vocab_size"], H)
+        self.embed = self._linear(P + "embed_tokens", affine, c["vocab_size"], H)
         self.lm_head = self._linear("language_model.lm_head", Q4K, c["vocab_size"], H)
         self.final_norm = self._plain(P + "norm.weight", _norm_w(self.rng, H))
         self.layers = []
@@ -148,8 +152,8 @@ class SynthModel:
         self.tensors[path + ".dm"] = (km.dm.reshape(lead + (nb, db)), DT_F16)
 
     def _linear(self, path, mode, O, K):
-        if mode == "affine8":
-            lin = HostLinear.affine8(self.rng, O, K)
+        if mode in ("affine8", "affine4"):
+            lin = HostLinear.affine8(self.rng, O, K) if mode == "affine8" else HostLinear.affine4(self.rng, O, K)
             self.tensors[path + ".weight"] = (lin.w.view(np.uint32), DT_U32)
             self.tensors[path + ".scales"] = (lin.scales, DT_BF16)
             self.tensors[path + ".biases"] = (lin.biases, DT_BF16)
@@ -192,7 +196,7 @@ class SynthModel:
             m["sh_gate"] = self._linear(p_ + "shared_expert.gate_proj", Q4K, SI, H)
             m["sh_up"] = self._linear(p_ + "shared_expert.up_proj", Q4K, SI, H)
             m["sh_down"] = self._linear(p_ + "shared_expert.down_proj", Q6K, H, SI)
-            m["sh_egate"] = self._linear(p_ + "shared_expert_gate", "affine8", 1, H)
+            m["sh_egate"] = self._linear(p_ + "shared_expert_gate", self.affine, 1, H)
         return m
 
     # ---- device side ----------------------------------------------------------------------

@@ -109,4 +109,4 @@ def test_config_and_tensors_must_agree(orn, ctx, artifact, tmp_path):
     assert "laid out as q4k" in load_with(lambda q: q[lm].update(mode="q6k"))
     emb = "language_model.model.embed_tokens"
     assert "no " + emb + ".dm" in load_with(lambda q: q.update({emb: {"group_size": 256, "bits": 4, "mode": "q4k"}}))
-    assert "8-bit group 64 only" in load_with(lambda q: q.update({emb: {"bits": 4}}))
+    assert "is not carried" in load_with(lambda q: q.update({emb: {"bits": 4}}))   # 4-bit needs group 32

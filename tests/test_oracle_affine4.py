@@ -1,0 +1,62 @@
+"""Pins for the oracle's 4-bit affine (group 32) mat-vec and lookup, the published artifact's
+format (src/ops/quantized.rs:311-333, vendored quantized.h:235-244): the nibble order against
+mlx's packing stated as `(word >> 4*(i % 8)) & 15` on the u32 words, the product against
+float64, and the gathered form against the plain one. CPU only."""
+import ctypes as C
+
+import numpy as np
+
+import util
+from util import oracle, p
+
+
+def _dequant(lin):
+    words = lin.w.view(np.uint32)                                    # [O, K/8], as the artifact stores it
+    i = np.arange(lin.K)
+    q = (words[:, i // 8] >> (4 * (i % 8)).astype(np.uint32)) & 15   # mlx: eight codes a word, lowest first
+    s = np.repeat(util.bf16_to_f32(lin.scales).astype(np.float64), 32, 1)
+    b = np.repeat(util.bf16_to_f32(lin.biases).astype(np.float64), 32, 1)
+    return q.astype(np.float64) * s + b
+
+
+def _qmv(lin, xb, lhs=None, rhs=None, E=1):
+    rows = len(rhs) if rhs is not None else xb.shape[0]
+    O = lin.O // E
+    y = np.empty((rows, O), np.uint16)
+    oracle().orc_affine4_gather_qmv(p(lin.w), p(lin.scales), p(lin.biases), E, O, lin.K, p(xb),
+                                    p(lhs) if lhs is not None else None, p(rhs) if rhs is not None else None, rows, p(y))
+    return y
+
+
+def test_affine4_matvec_vs_float64_and_nibble_order():
+    rng = np.random.default_rng(0)
+    for O, K in ((6, 2048), (3, 32), (5, 4096), (2, 96)):
+        lin = util.HostLinear.affine4(rng, O, K)
+        W = _dequant(lin)
+        xb = util.bf16_normal(rng, (3, K))
+        want = util.bf16_to_f32(xb).astype(np.float64) @ W.T
+        got = util.bf16_to_f32(_qmv(lin, xb)).astype(np.float64)
+        assert np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-5 * np.abs(want).max()), (O, K)
+        # one-hot activations pick out single weights: every nibble position, both ends of a group
+        for col in sorted(set(list(rng.integers(0, K, 24)) + [0, 1, 7, 8, 15, 16, 31, K - 1])):
+            e = np.zeros((1, K), np.float32); e[0, col] = 1.0
+            y = util.bf16_to_f32(_qmv(lin, util.f32_to_bf16(e)))[0].astype(np.float64)
+            assert np.all(np.abs(y - W[:, col]) <= 2.0 ** -8 * np.abs(W[:, col]) + 1e-12), (K, col)
+
+
+def test_affine4_gather_equals_plain_rows_and_embedding_vs_double():
+    rng = np.random.default_rng(1)
+    E, O, K = 5, 12, 256
+    lin = util.HostLinear.affine4(rng, E * O, K)
+    xb = util.bf16_normal(rng, (4, K))
+    lhs = np.array([0, 3, 3, 1, 2, 0], np.uint32); rhs = np.array([4, 0, 2, 2, 1, 3], np.uint32)
+    got = _qmv(lin, xb, lhs, rhs, E)
+    full = _qmv(lin, xb)                                             # every expert's rows for every x row
+    for r in range(len(rhs)):
+        assert np.array_equal(got[r], full[lhs[r], rhs[r] * O:(rhs[r] + 1) * O])
+    ids = np.array([7, 0, 59], np.uint32)
+    out = np.empty((3, K), np.uint16)
+    oracle().orc_embedding4(p(lin.w), p(lin.scales), p(lin.biases), K, p(ids), 3, p(out))
+    W = _dequant(lin)
+    bias = np.repeat(util.bf16_to_f32(lin.biases).astype(np.float64), 32, 1)
+    assert np.all(np.abs(util.bf16_to_f32(out) - W[ids]) <= 2.0 ** -7 * np.abs(W[ids]) + 2.0 ** -8 * np.abs(bias[ids]))

@@ -221,6 +221,16 @@ class HostLinear:
         return HostLinear("affine8", O, K, w=w, scales=scales, biases=biases)
 
     @staticmethod
+    def affine4(rng, O, K, out_std=1.0):
+        """mlx affine 4-bit group 32: codes two a byte (low nibble first), weight = s*q + b,
+        centred (b = -7.5 s; std(q) = 4.61)."""
+        w = rng.integers(0, 256, size=(O, K // 2), dtype=np.uint8)
+        s = (out_std / (4.61 * np.sqrt(K))) * (0.5 + rng.random((O, K // 32)))
+        scales = f32_to_bf16(s.astype(np.float32))
+        biases = f32_to_bf16((-7.5 * bf16_to_f32(scales)).astype(np.float32))
+        return HostLinear("affine4", O, K, w=w, scales=scales, biases=biases)
+
+    @staticmethod
     def dense(rng, O, K, out_std=1.0):
         w = f32_to_bf16((rng.standard_normal((O, K)) * (out_std / np.sqrt(K))).astype(np.float32))
         return HostLinear("dense", O, K, w=w)
@@ -231,6 +241,8 @@ class HostLinear:
         km = OrcKmat(0, 1, self.O, self.K, None, None, None)
         if self.mode == "affine8":
             return OrcLinear(1, km, p(self.w), p(self.scales), p(self.biases))
+        if self.mode == "affine4":
+            return OrcLinear(3, km, p(self.w), p(self.scales), p(self.biases))
         return OrcLinear(2, km, p(self.w), None, None)
 
     def dev(self, orn, ctx):
@@ -238,6 +250,8 @@ class HostLinear:
             return orn.Linear.kquant(ctx, self.km.kind, self.km.qs, self.km.scales, self.km.dm, self.O, self.K)
         if self.mode == "affine8":
             return orn.Linear.affine8(ctx, self.w, self.scales, self.biases)
+        if self.mode == "affine4":
+            return orn.Linear.affine4(ctx, self.w, self.scales, self.biases)
         return orn.Linear.dense(ctx, self.w)
 
     def nbytes(self):
