@@ -689,7 +689,16 @@ void launch_down(ornith_ctx* ctx, const DownArgs& a) {
   constexpr int RPW = 64 / LPR;
   dim3 block(64 * (a.k + 1));
   const long groups1 = (long)(a.H + RPW - 1) / RPW * a.T;
-  if (groups1 >= (long)ctx->compute_units * 4) {
+  const int forced = ornith_option_moe_down_iters();
+  // About one workgroup (k + 1 wavefronts) per compute unit is the fastest shape at every verify
+  // width: measured (us, 1 / 2 / 4 column groups a workgroup) T = 1: 5.4 / 6.1 / 8.7, T = 2:
+  // 9.0 / 6.8 / 9.2, T = 3: 12.6 / 11.4 / 10.0, T = 4: 16.2 / 12.1 / 10.9
+  const long cu = ctx->compute_units;
+  const int iters = forced ? forced : groups1 >= 3 * cu ? 4 : groups1 >= 2 * cu ? 2 : 1;
+  if (iters >= 4) {
+    dim3 grid((a.H + RPW * 4 - 1) / (RPW * 4), a.T);
+    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 4>), grid, block, 0, ctx->stream, a);
+  } else if (iters == 2) {
     dim3 grid((a.H + RPW * 2 - 1) / (RPW * 2), a.T);
     hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 2>), grid, block, 0, ctx->stream, a);
   } else {
