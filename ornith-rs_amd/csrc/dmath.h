@@ -40,6 +40,13 @@ __device__ __forceinline__ bf16_t dm_f2bf(float f) {
   const __bf16 b = (__bf16)f;
   return __builtin_bit_cast(bf16_t, b);
 }
+// two values in one instruction, element 0 in the low half; each half equals dm_f2bf of its value
+__device__ __forceinline__ uint32_t dm_f2bf2(float lo, float hi) {
+  typedef float f2v __attribute__((ext_vector_type(2)));
+  typedef __bf16 b2v __attribute__((ext_vector_type(2)));
+  const f2v v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, b2v));
+}
 // round to bf16 precision, keep as float
 __device__ __forceinline__ float dm_rb(float f) { return dm_bf2f(dm_f2bf(f)); }
 

@@ -105,6 +105,14 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
       so[i] = a.seg[i].O;
       fb[i] = a.seg[i].first_block;
     }
+    if constexpr (PRE) {
+      // the norm's three input pointers ride along with the same batch of argument loads
+      uint64_t pr = (uint64_t)a.pre.res, py = (uint64_t)a.pre.y, pw = (uint64_t)a.pre.w;
+      asm volatile("" : "+s"(pr), "+s"(py), "+s"(pw));
+      a.pre.res = dm_global_ptr<const bf16_t>(pr);
+      a.pre.y = dm_global_ptr<const bf16_t>(py);
+      a.pre.w = dm_global_ptr<const bf16_t>(pw);
+    }
     asm volatile(""
                  : "+s"(q[0]), "+s"(sc[0]), "+s"(d[0]), "+s"(y[0]), "+s"(so[0]), "+s"(fb[0]), "+s"(q[1]), "+s"(sc[1]),
                    "+s"(d[1]), "+s"(y[1]), "+s"(so[1]), "+s"(fb[1]), "+s"(q[2]), "+s"(sc[2]), "+s"(d[2]), "+s"(y[2]),
@@ -159,14 +167,22 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
     const int o = base + it * RPW + slot;
     return row0 + (o < O ? o : O - 1);
   };
+  // The rows the norm is made from are a few KB that sit in cache; their loads go out first
+  // because loads return in issue order: behind the cold weight rows they would hold the
+  // norm back until the weights had arrived.
+  PreNormRegs<PRE ? M : 1> pg;
+  if constexpr (PRE) {
+    prenorm_issue<M>(a.pre, pg);
+    __builtin_amdgcn_sched_barrier(0);
+  }
   typename KL::Row pf[PF];
 #pragma unroll
   for (int i = 0; i < PF; ++i) pf[i] = KL::load(sg.qs, sg.scales, sg.dm, row_of(i), nb, L);
-  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of everything that follows
   ORN_MARK(1);
   if constexpr (PRE) {
     __shared__ PreNormLds<M> pn;
-    prenorm_rows<M>(a.pre, blockIdx.x == 0, pn);
+    prenorm_finish<M>(a.pre, pg, blockIdx.x == 0, pn);
 #pragma unroll
     for (int t = 0; t < M; ++t) xrow[t] = &pn.xn[t][0];
   }

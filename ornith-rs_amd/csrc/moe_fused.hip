@@ -323,9 +323,14 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
   typename KL::Lane L;
   L.set_chunk(c);
   const int o = (blockIdx.x * 4 + wave) * RPW + slot;
+  // the norm's inputs first (cached, back early), the weight row right behind them: loads
+  // return in issue order
+  PreNormRegs<M> pg;
+  if (pre) prenorm_issue<M>(a.pre, pg);
+  __builtin_amdgcn_sched_barrier(0);
   const typename KL::Row row = KL::load(a.w.qs, a.w.scales, a.w.dm, o < a.E ? o : a.E - 1, nb, L);
-  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
-  if (pre) prenorm_rows<M>(a.pre, blockIdx.x == 0, pn);
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of everything that follows
+  if (pre) prenorm_finish<M>(a.pre, pg, blockIdx.x == 0, pn);
   const void* xrow[M];
 #pragma unroll
   for (int t = 0; t < M; ++t) xrow[t] = pre ? (const void*)&pn.xn[t][0] : (const void*)(a.x + (size_t)t * a.K);

@@ -41,9 +41,7 @@ __device__ __forceinline__ void load_bf16(const bf16_t* p, float (&v)[PER]) {
   }
 }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  return (uint32_t)dm_f2bf(a) | ((uint32_t)dm_f2bf(b) << 16);
-}
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) { return dm_f2bf2(a, b); }
 
 // rounds each value to bf16 and stores
 template <int PER>
@@ -104,8 +102,9 @@ __device__ __forceinline__ void rms_row(const bf16_t* a, const bf16_t* b, const 
 // kernels that consume the normed rows themselves: h = bf16(res + y),
 // normed = bf16(w * bf16(h * inv)). The rows land in LDS (xn); the workgroup for which
 // `write_global` holds also stores h and normed for later consumers. Same arithmetic and
-// order as rms_wide_kernel<32, NORM_ADD> (wavefront t sums row t), so a consumer that
-// recomputes the norm per workgroup sees the bits the stand-alone kernel would have written.
+// order as rms_wide_kernel<32, NORM_ADD> (64 lane chains of 32 squares, then the 64-lane
+// butterfly), so a consumer that recomputes the norm per workgroup sees the bits the
+// stand-alone kernel would have written.
 struct PreNorm {
   const bf16_t* res;     // [T, 2048]
   const bf16_t* y;       // [T, 2048]
@@ -119,59 +118,113 @@ constexpr int kPreN = 2048;
 
 template <int T>
 struct PreNormLds {
-  float xs[T * kPreN];
   __attribute__((aligned(16))) bf16_t xn[T][kPreN];
-  float inv[4];
+  float part[T][64];  // the 64 canonical lanes' sums of squares
 };
+
+// The global loads of the prologue, kept apart from the arithmetic: loads return in issue
+// order, so a kernel that also has cold weight rows to fetch issues these first (they hit in
+// cache and come back early) and the weight loads right after, and the norm is worked out
+// while the weights are still on their way.
+template <int T>
+struct PreNormRegs {
+  uint4 w, r[T], y[T];
+};
+
+__device__ __forceinline__ void unpack_bf16x8(const uint4& w, float (&v)[8]) {
+  v[0] = dm_bf2f_lo(w.x);
+  v[1] = dm_bf2f_hi(w.x);
+  v[2] = dm_bf2f_lo(w.y);
+  v[3] = dm_bf2f_hi(w.y);
+  v[4] = dm_bf2f_lo(w.z);
+  v[5] = dm_bf2f_hi(w.z);
+  v[6] = dm_bf2f_lo(w.w);
+  v[7] = dm_bf2f_hi(w.w);
+}
+
+template <int T>
+__device__ __forceinline__ void prenorm_issue(const PreNorm& p, PreNormRegs<T>& g) {
+  const int e0 = threadIdx.x * 8;
+  g.w = *reinterpret_cast<const uint4*>(p.w + e0);
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    g.r[t] = *reinterpret_cast<const uint4*>(p.res + (size_t)t * kPreN + e0);
+    g.y[t] = *reinterpret_cast<const uint4*>(p.y + (size_t)t * kPreN + e0);
+  }
+}
 
 // COH: the normed rows stored by the `write_global` workgroup are read by other workgroups of
 // the same launch (handoff.h), so they go out as agent-scope stores.
 template <int T, bool COH = false>
-__device__ __forceinline__ void prenorm_rows(const PreNorm& p, bool write_global, PreNormLds<T>& s) {
-  static_assert(T >= 1 && T <= 4, "one wavefront per row");
-  constexpr int PER = kPreN / 64;
-  const int tid = threadIdx.x, e0 = tid * 8, lane = tid & 63, wave = tid >> 6;
-  const int lane_of = e0 / PER, pos0 = e0 % PER;
+__device__ __forceinline__ void prenorm_finish(const PreNorm& p, const PreNormRegs<T>& g, bool write_global,
+                                               PreNormLds<T>& s) {
+  static_assert(T >= 1 && T <= 4, "rows of the exact window");
+  // Thread tid holds values [8 tid, 8 tid + 8): canonical lane l = tid / 4 (32 values, one
+  // fma chain in ascending order) is the four threads of a quad. The chain runs down the quad:
+  // every thread continues from what its left neighbour handed over, so after four steps the
+  // quad's last thread holds the lane's sum with the canonical association.
+  const int tid = threadIdx.x, e0 = tid * 8, lane = tid & 63;
   float x[T][8], wv[8];
-  load_bf16<8>(p.w + e0, wv);
+  unpack_bf16x8(g.w, wv);
 #pragma unroll
   for (int t = 0; t < T; ++t) {
-    float yv[8];
-    load_bf16<8>(p.res + (size_t)t * kPreN + e0, x[t]);
-    load_bf16<8>(p.y + (size_t)t * kPreN + e0, yv);
+    float rv[8], yv[8];
+    unpack_bf16x8(g.r[t], rv);
+    unpack_bf16x8(g.y[t], yv);
+    // h = bf16(res + y), two values a conversion; the packed words are what gets stored
+    uint32_t hp[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) x[t][i] = dm_rb(x[t][i] + yv[i]);
-    if (write_global) store_bf16<8>(p.h_out + (size_t)t * kPreN + e0, x[t]);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) s.xs[t * kPreN + (pos0 + i) * 64 + lane_of] = x[t][i];
-  }
-  __syncthreads();
-  if (wave < T) {
+    for (int j = 0; j < 4; ++j) {
+      hp[j] = dm_f2bf2(rv[2 * j] + yv[2 * j], rv[2 * j + 1] + yv[2 * j + 1]);
+      x[t][2 * j] = dm_bf2f_lo(hp[j]);
+      x[t][2 * j + 1] = dm_bf2f_hi(hp[j]);
+    }
+    if (write_global)
+      *reinterpret_cast<uint4*>(p.h_out + (size_t)t * kPreN + e0) = make_uint4(hp[0], hp[1], hp[2], hp[3]);
     float acc = 0.f;
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const float v = s.xs[wave * kPreN + i * 64 + lane];
-      acc = dm_fma(v, v, acc);
+    for (int step = 0; step < 4; ++step) {
+      // quad_perm [0,0,1,2]: each thread reads its left neighbour in the quad
+      float in = 0.f;
+      if (step > 0)
+        in = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x90, 0xF, 0xF, false));
+      acc = in;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc = dm_fma(x[t][i], x[t][i], acc);
     }
-    const float inv = dm_rsqrt(dm_wave_sum<64>(acc) / (float)kPreN + p.eps);
-    if (lane == 0) s.inv[wave] = inv;
+    if ((tid & 3) == 3) s.part[t][tid >> 2] = acc;
   }
   __syncthreads();
+  float invs[T];
+#pragma unroll
+  for (int t = 0; t < T; ++t)
+    invs[t] = dm_rsqrt(dm_wave_sum<64>(s.part[t][lane]) / (float)kPreN + p.eps);
 #pragma unroll
   for (int t = 0; t < T; ++t) {
-    const float inv = s.inv[t];
+    const float inv = invs[t];
+    uint32_t np[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) x[t][i] = dm_rb(wv[i] * dm_rb(x[t][i] * inv));
-    store_bf16<8>(&s.xn[t][e0], x[t]);
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t a = dm_f2bf2(x[t][2 * j] * inv, x[t][2 * j + 1] * inv);
+      np[j] = dm_f2bf2(wv[2 * j] * dm_bf2f_lo(a), wv[2 * j + 1] * dm_bf2f_hi(a));
+    }
+    *reinterpret_cast<uint4*>(&s.xn[t][e0]) = make_uint4(np[0], np[1], np[2], np[3]);
     if (write_global) {
       if constexpr (COH) {
         uint64_t* dst = reinterpret_cast<uint64_t*>(p.normed_out + (size_t)t * kPreN + e0);
-        ho_store_u64(dst, (uint64_t)pack_bf16x2(x[t][0], x[t][1]) | ((uint64_t)pack_bf16x2(x[t][2], x[t][3]) << 32));
-        ho_store_u64(dst + 1, (uint64_t)pack_bf16x2(x[t][4], x[t][5]) | ((uint64_t)pack_bf16x2(x[t][6], x[t][7]) << 32));
+        ho_store_u64(dst, (uint64_t)np[0] | ((uint64_t)np[1] << 32));
+        ho_store_u64(dst + 1, (uint64_t)np[2] | ((uint64_t)np[3] << 32));
       } else {
-        store_bf16<8>(p.normed_out + (size_t)t * kPreN + e0, x[t]);
+        *reinterpret_cast<uint4*>(p.normed_out + (size_t)t * kPreN + e0) = make_uint4(np[0], np[1], np[2], np[3]);
       }
     }
   }
   __syncthreads();
+}
+
+template <int T, bool COH = false>
+__device__ __forceinline__ void prenorm_rows(const PreNorm& p, bool write_global, PreNormLds<T>& s) {
+  PreNormRegs<T> g;
+  prenorm_issue<T>(p, g);
+  prenorm_finish<T, COH>(p, g, write_global, s);
 }
