@@ -270,7 +270,9 @@ ORNITH_API int ornith_add_rms_moe_block(ornith_ctx* ctx, const ornith_moe_weight
  * d_inds u32 [T,k], d_scores bf16 [T,k] (router_topk outputs), d_egate bf16 [T]
  * (shared_expert_gate's output). Needs k-quant routed and shared experts of matching
  * formats and top_k <= 8 (ORNITH_ERR_UNSUPPORTED otherwise; ornith_moe_block falls back
- * to one launch per operator by itself). */
+ * to one launch per operator by itself). The ids live on the device and are not validated:
+ * an id >= num_experts is read as the last expert (clamped for memory safety), so a corrupt
+ * routing buffer gives plausible output, not an error. */
 ORNITH_API int ornith_moe_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                                   const uint32_t* d_inds, const void* d_scores, const void* d_egate,
                                   void* d_act, void* d_out, int phases);
