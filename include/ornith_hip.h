@@ -692,6 +692,78 @@ ORNITH_API int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const
                                    size_t prefill_step, int policy, ornith_progress_cb progress,
                                    ornith_token_cb on_token, void* user, ornith_mtp_stats* stats_out);
 
+/* ---- text in, text out: tokenizer, streaming detokenizer, chat template (host only) ----
+ * The callers' side of the loops (src/main.rs:651-741): a prompt is rendered by the chat
+ * template, encoded, generated from, and the tokens handed to on_token go through the
+ * detokenizer. Nothing here touches the GPU. Strings are UTF-8 with explicit lengths (no
+ * terminator needed or written). Every function that returns text or a list takes a buffer,
+ * its capacity and a count pointer: with a NULL buffer it only reports the size needed. */
+typedef struct ornith_tokenizer ornith_tokenizer;
+typedef struct ornith_detokenizer ornith_detokenizer;
+/* split::Dialect (src/tokenizer/split.rs:55-78): which of the two split patterns runs */
+#define ORNITH_DIALECT_TOKENIZER_JSON 0 /* the pattern tokenizer.json carries, \p{M} beside \p{L} */
+#define ORNITH_DIALECT_TRANSFORMERS 1   /* transformers' PRETOKENIZE_REGEX, without \p{M} */
+/* Tokenizer::load / load_as (src/tokenizer/mod.rs:78-259): reads tokenizer.json,
+ * tokenizer_config.json (added tokens only the config knows, eos_token) and, when present,
+ * generation_config.json (eos_token_id). A file that asks for a pipeline other than
+ * NFC -> Split(the pattern, Isolated) + ByteLevel -> BPE without dropout / unk / fallback is
+ * refused (ORNITH_ERR_UNSUPPORTED) where the reference asserts. */
+ORNITH_API int ornith_tokenizer_load(const char* model_dir, int dialect, ornith_tokenizer** out);
+ORNITH_API int ornith_tokenizer_destroy(ornith_tokenizer* tk);
+/* Tokenizer::vocab_size (mod.rs:261-263): ids the tokenizer has a string for, added ones included */
+ORNITH_API int ornith_tokenizer_vocab_size(const ornith_tokenizer* tk, size_t* n_out);
+/* Tokenizer::encode (mod.rs:279-308): tokenizer.encode(text, add_special_tokens=False).
+ * The text must be valid UTF-8 (ORNITH_ERR_INVALID otherwise; the reference takes &str). */
+ORNITH_API int ornith_tokenizer_encode(const ornith_tokenizer* tk, const char* text, size_t text_len,
+                                       uint32_t* ids_out, size_t cap, size_t* n_out);
+/* Tokenizer::decode (mod.rs:330-346): ByteLevel decoding, ill-formed bytes as U+FFFD */
+ORNITH_API int ornith_tokenizer_decode(const ornith_tokenizer* tk, const uint32_t* ids, size_t n, char* out,
+                                       size_t cap, size_t* n_out);
+/* Tokenizer::token (mod.rs:349-355): the token string of an id; "!" for an id past the entries */
+ORNITH_API int ornith_tokenizer_token(const ornith_tokenizer* tk, uint32_t id, char* out, size_t cap,
+                                      size_t* n_out);
+/* Tokenizer::id (mod.rs:265-271): token is NUL-terminated; ORNITH_ERR_INVALID when absent */
+ORNITH_API int ornith_tokenizer_id(const ornith_tokenizer* tk, const char* token, uint32_t* id_out);
+/* Tokenizer::is_special (mod.rs:273-275): 1 / 0 */
+ORNITH_API int ornith_tokenizer_is_special(const ornith_tokenizer* tk, uint32_t id);
+/* Tokenizer::eos_ids (mod.rs:230-247) */
+ORNITH_API int ornith_tokenizer_eos_ids(const ornith_tokenizer* tk, uint32_t* ids_out, size_t cap,
+                                        size_t* n_out);
+/* The pattern string a dialect spells (Dialect::TOKENIZER_JSON_PATTERN / TRANSFORMERS_PATTERN) */
+ORNITH_API const char* ornith_tokenizer_split_pattern(int dialect);
+/* Detokenizer (mod.rs:352-417, mlx-lm's BPEStreamingDetokenizer with its two quirks: the single
+ * leading space of a generation is dropped; the character standing for byte 0 is emitted as
+ * itself while streaming). add_token holds back an unfinished UTF-8 sequence and a lone space;
+ * last_segment returns (and, with a buffer, consumes) the text made since its last call. */
+ORNITH_API int ornith_detokenizer_create(const ornith_tokenizer* tk, ornith_detokenizer** out);
+ORNITH_API int ornith_detokenizer_destroy(ornith_detokenizer* d);
+ORNITH_API int ornith_detokenizer_add_token(ornith_detokenizer* d, uint32_t token);
+ORNITH_API int ornith_detokenizer_finalize(ornith_detokenizer* d);
+ORNITH_API int ornith_detokenizer_last_segment(ornith_detokenizer* d, char* out, size_t cap, size_t* n_out);
+ORNITH_API int ornith_detokenizer_text(const ornith_detokenizer* d, char* out, size_t cap, size_t* n_out);
+/* The tokenizer's layers one by one, as the reference's tests reach them (tests/tokenizer.rs):
+ * nfc::nfc (src/tokenizer/nfc.rs:121-170); split::pre_split (split.rs:134-153: the byte offset
+ * at which each piece ends); the class the split pattern puts a code point in (1 letter or
+ * mark, 2 number, 3 white space, 0 other; split.rs:100-118). */
+ORNITH_API int ornith_text_nfc(const char* text, size_t n, char* out, size_t cap, size_t* n_out);
+ORNITH_API int ornith_text_pre_split(const char* text, size_t n, int dialect, size_t* ends_out, size_t cap,
+                                     size_t* n_out);
+ORNITH_API int ornith_text_char_class(uint32_t code_point);
+/* chat::apply_chat_template (src/chat.rs:196-352): the artifact's chat template written out as
+ * code. messages_json: the list tokenizer.apply_chat_template takes, [{"role": "system" |
+ * "user" | "assistant" | "tool", "content": string | [{"type": "text" | "image" | "video", ...}]
+ * | null, "reasoning_content"?, "tool_calls"?: [{"function"?: {"name", "arguments": {...}}}]}];
+ * tools_json: a list of tool schemas, or NULL / empty for none. The template's own errors
+ * ("No messages provided.", "No user query found in messages.", "System message must be at
+ * the beginning.", "System message cannot contain images." / "videos.") come back as
+ * ORNITH_ERR_INVALID with that text. */
+ORNITH_API int ornith_chat_apply_template(const char* messages_json, size_t messages_len, const char* tools_json,
+                                          size_t tools_len, int add_generation_prompt, int enable_thinking,
+                                          char* out, size_t cap, size_t* n_out);
+/* json::Value::to_json (src/json.rs): json.dumps(value, ensure_ascii=False) of a JSON text,
+ * keys in their written order - what the template's tojson filter produces. */
+ORNITH_API int ornith_json_dumps(const char* json, size_t len, char* out, size_t cap, size_t* n_out);
+
 /* ---- self test ------------------------------------------------------------------
  * Evaluates one of the library's scalar device functions element-wise (fp32 in,
  * fp32 out) so their bits can be compared with a CPU evaluation. No reference

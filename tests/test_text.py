@@ -1,0 +1,357 @@
+"""The tokenizer, the streaming detokenizer and the chat template (host code: CPU only).
+
+Layers, narrowest first, as /root/reference/tests/tokenizer.rs has them: the character classes
+the split pattern asks about, NFC, the pre-tokenizer's pieces, then whole-pipeline encode and
+decode; then the detokenizer and /root/reference/tests/chat.rs's two layers (the JSON writer,
+the rendered template).
+
+What pins them: tests/golden/tokenizer/ holds what the `tokenizers` library - the
+implementation the reference checks itself against - makes of a trained byte-level BPE of the
+model's pipeline shape (tests/golden/make_tokenizer_fixture.py wrote it; nothing of the
+reference was run): oniguruma's classes for every code point, NFC outputs, pieces, ids under
+both split patterns, decoded text. Independent of that fixture: Python's unicodedata for NFC,
+bytes.decode("utf-8", "replace") for the lossy decoder, json.dumps for the JSON writer,
+str.strip for the template's trim, and the expectations the reference's own unit tests spell
+out in source (src/tokenizer/split.rs:240-290, nfc.rs:172-199, chat.rs:354-370).
+Parity unpinned: the rendered chat template beyond those in-source cases (the artifact's
+chat_template.jinja and the reference's refs/ fixtures are not available), and the streaming
+detokenizer against mlx-lm itself (not installed) - both follow the reference's source.
+"""
+import importlib
+import json
+import os
+import random
+import shutil
+import unicodedata as ud
+
+import pytest
+
+orn = importlib.import_module("ornith-rs_amd")
+text = importlib.import_module("ornith-rs_amd.text")
+
+FIX = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tokenizer")
+CASES = json.load(open(os.path.join(FIX, "cases.json")))
+
+
+@pytest.fixture(scope="module")
+def tk():
+    t = text.Tokenizer(FIX)
+    yield t
+    t.close()
+
+
+@pytest.fixture(scope="module")
+def tk_tr():
+    t = text.Tokenizer(FIX, text.TRANSFORMERS)
+    yield t
+    t.close()
+
+
+# ---- character classes ---------------------------------------------------------------
+def test_character_classes_match_oniguruma():
+    """Every code point Python's Unicode 13 tables know lands in the class oniguruma puts it in
+    (oniguruma's tables are newer: code points assigned since are skipped, not compared)."""
+    onig = json.load(open(os.path.join(FIX, "classes.json")))
+    want = bytearray(0x110000)
+    for name, cls in (("s", 3), ("N", 2), ("M", 1), ("L", 1)):
+        for a, b in onig[name]:
+            for c in range(a, b + 1):
+                want[c] = cls
+    bad, skipped = [], 0
+    for c in range(0x110000):
+        if 0xD800 <= c <= 0xDFFF:
+            continue
+        if ud.category(chr(c)) == "Cn":
+            skipped += want[c] != 0
+            continue
+        if text.char_class(c) != want[c]:
+            bad.append((hex(c), text.char_class(c), want[c]))
+    assert not bad, bad[:20]
+    assert skipped < 12000          # letters / marks / numbers assigned after Unicode 13
+    # \s is the White_Space property, not Ruby's ASCII \s and not Python's isspace
+    assert text.char_class(0xA0) == 3 and text.char_class(0x3000) == 3 and text.char_class(0x85) == 3
+    assert text.char_class(0x200B) == 0 and text.char_class(0x1C) == 0
+
+
+# ---- NFC -------------------------------------------------------------------------------
+def test_nfc_matches_the_tokenizers_normalizer_and_unicodedata():
+    for s, want in zip(CASES["text"], CASES["nfc"]):
+        assert text.nfc(s) == want, [hex(ord(c)) for c in s]
+    # the cases the reference spells out (nfc.rs:176-198)
+    for s, want in [("abc", "abc"), ("é", "é"), ("é", "é"), ("Ḑ̇", "Ḑ̇"),
+                    ("Å", "Å"), ("각", "각"), ("क़", "क़"),
+                    ("क़", "क़"), ("ཷ", "ཷ"), ("̈́", "̈́")]:
+        assert text.nfc(s) == want
+    # random strings over the characters that take part in normalization, against unicodedata
+    rng = random.Random(5)
+    pool = [c for c in range(0x110000) if not 0xD800 <= c <= 0xDFFF and ud.category(chr(c)) != "Cn"
+            and (ud.combining(chr(c)) or ud.decomposition(chr(c)) or 0x1100 <= c <= 0x11FF or 0xAC00 <= c <= 0xD7A3)]
+    base = [ord(c) for c in "aeiouAEDdnN कאاあ"]
+    for _ in range(3000):
+        s = "".join(chr(rng.choice(pool if rng.random() < 0.6 else base)) for _ in range(rng.randint(1, 8)))
+        assert text.nfc(s) == ud.normalize("NFC", s), [hex(ord(c)) for c in s]
+    # every single code point
+    for c in pool:
+        assert text.nfc(chr(c)) == ud.normalize("NFC", chr(c)), hex(c)
+
+
+# ---- the split pattern -----------------------------------------------------------------
+def test_both_split_patterns_are_the_ones_in_play():
+    assert text.split_pattern(text.TOKENIZER_JSON) == CASES["pattern_json"]
+    assert text.split_pattern(text.TRANSFORMERS) == CASES["pattern_transformers"]
+    tj = json.load(open(os.path.join(FIX, "tokenizer.json")))
+    assert tj["pre_tokenizer"]["pretokenizers"][0]["pattern"]["Regex"] == CASES["pattern_json"]
+
+
+def test_pre_split_matches_the_live_pre_tokenizer():
+    for s, pj, pt in zip(CASES["nfc"], CASES["pieces_json"], CASES["pieces_transformers"]):
+        assert text.pre_split(s, text.TOKENIZER_JSON) == pj, repr(s)
+        assert text.pre_split(s, text.TRANSFORMERS) == pt, repr(s)
+    # the shapes the reference documents (split.rs:247-262, 266-285)
+    for s, want in [("don't", ["don", "'t"]), ("it'ss", ["it", "'s", "s"]), ("it'ſs", ["it", "'ſ", "s"]),
+                    ("123abc", ["1", "2", "3", "abc"]), ("--x", ["--", "x"]), ("  \n\n  x", ["  \n\n", " ", " x"]),
+                    ("a   ", ["a", "   "]), ("a  b", ["a", " ", " b"]), ("a  x", ["a", " ", " x"]),
+                    ("a   b", ["a", "  ", " b"])]:
+        assert text.pre_split(s) == want
+    hindi = "हिन"
+    assert text.pre_split(hindi, text.TOKENIZER_JSON) == [hindi]
+    assert text.pre_split(hindi, text.TRANSFORMERS) == ["ह", "िन"]
+
+
+def test_pre_split_random_strings_against_a_live_pre_tokenizer():
+    tokenizers = pytest.importorskip("tokenizers")
+    rng = random.Random(11)
+    alphabet = list("ab Z9'\n\r\t.,!-_sStTrReEvVmMlLdD") + [" ", " ", "́", "ि", "ह", "　", "ſ",
+                                                            "é", "中", "٣", "½", "\U0001F600", "️", "​"]
+    for dialect, pat in ((text.TOKENIZER_JSON, CASES["pattern_json"]), (text.TRANSFORMERS, CASES["pattern_transformers"])):
+        live = tokenizers.pre_tokenizers.Split(tokenizers.Regex(pat), behavior="isolated")
+        for _ in range(1500):
+            s = "".join(rng.choice(alphabet) for _ in range(rng.randint(1, 14)))
+            assert text.pre_split(s, dialect) == [p for p, _ in live.pre_tokenize_str(s)], repr(s)
+
+
+# ---- encode / decode ---------------------------------------------------------------------
+def test_encode_and_decode_match_tokenizers(tk, tk_tr):
+    assert tk.vocab_size == len(CASES["tokenmap"])
+    for i, want in enumerate(CASES["tokenmap"]):
+        assert tk.token(i) == want, i
+    assert tk.token(len(CASES["tokenmap"]) + 5) == "!"      # ids past the entries
+    for s, ij, it, dec in zip(CASES["text"], CASES["ids_json"], CASES["ids_transformers"], CASES["decoded"]):
+        assert tk.encode(s) == ij, repr(s)
+        assert tk_tr.encode(s) == it, repr(s)
+        assert tk.decode(ij) == dec, repr(s)
+    assert any(a != b for a, b in zip(CASES["ids_json"], CASES["ids_transformers"]))   # the dialects differ on marks
+    # prefixes that cut a character in two decode with U+FFFD, as tokenizers' decoder does
+    for ids, outs in zip(CASES["ids_json"], CASES["prefix_decoded"]):
+        for k, want in enumerate(outs):
+            assert tk.decode(ids[:k]) == want
+    with pytest.raises(orn.OrnithError, match="not valid UTF-8"):
+        tk.encode(b"ab\xff")
+
+
+def test_encode_random_strings_against_a_live_tokenizer(tk):
+    tokenizers = pytest.importorskip("tokenizers")
+    live = tokenizers.Tokenizer.from_file(os.path.join(FIX, "tokenizer.json"))
+    cfg = json.load(open(os.path.join(FIX, "tokenizer_config.json")))
+    have = {t.content for t in live.get_added_tokens_decoder().values()}
+    live.add_special_tokens([tokenizers.AddedToken(v["content"], special=True, normalized=False)
+                             for _, v in sorted(cfg["added_tokens_decoder"].items(), key=lambda kv: int(kv[0]))
+                             if v["content"] not in have])
+    rng = random.Random(3)
+    words = CASES["text"][:24] + ["<|im_start|>", "<|im_end|>", "<think>", "</think>", "<|audio_start|>", "<|im_start|>x", " ", "\n", "é"]
+    for _ in range(400):
+        s = "".join(rng.choice(words)[rng.randint(0, 3):][:rng.randint(1, 30)] for _ in range(rng.randint(1, 5)))
+        assert tk.encode(s) == live.encode(s, add_special_tokens=False).ids, repr(s)
+        ids = tk.encode(s)
+        assert tk.decode(ids) == live.decode(ids, skip_special_tokens=False)
+
+
+def test_added_tokens_and_end_of_sequence_ids(tk):
+    cfg_only = tk.id("<|audio_start|>")
+    assert cfg_only is not None and tk.is_special(cfg_only)          # known to tokenizer_config.json alone
+    assert tk.id("<think>") is not None and not tk.is_special(tk.id("<think>"))
+    assert tk.id("no such token") is None
+    assert tk.eos_ids == json.load(open(os.path.join(FIX, "generation_config.json")))["eos_token_id"]
+    # leftmost-longest: "<|im_start|>x" is an added token of its own and wins over "<|im_start|>"
+    assert tk.encode("<|im_start|>x") == [tk.id("<|im_start|>x")]
+    assert tk.encode("<|im_start|>y")[0] == tk.id("<|im_start|>")
+
+
+def test_lossy_utf8_matches_python():
+    """decode() reads its bytes like String::from_utf8_lossy; Python's "replace" handler follows the
+    same maximal-subpart rule. Driven through token strings of single bytes."""
+    rng = random.Random(9)
+    t = text.Tokenizer(FIX)
+    byte_tok = {}
+    alphabet = {}
+    n = 0
+    for b in range(256):
+        printable = 0x21 <= b <= 0x7E or 0xA1 <= b <= 0xAC or b >= 0xAE
+        alphabet[b] = chr(b) if printable else chr(256 + n)
+        n += 0 if printable else 1
+        byte_tok[b] = t.id(alphabet[b])
+    interesting = [0x41, 0x80, 0xBF, 0xC0, 0xC2, 0xE0, 0xA0, 0x9F, 0xED, 0xEF, 0xF0, 0x90, 0x8F, 0xF4, 0xF5, 0xFF, 0xE2, 0x82, 0xAC]
+    for _ in range(3000):
+        bs = bytes(rng.choice(interesting) for _ in range(rng.randint(1, 7)))
+        assert t.decode([byte_tok[b] for b in bs]) == bs.decode("utf-8", "replace"), bs
+    t.close()
+
+
+def test_refuses_a_pipeline_it_does_not_implement(tmp_path):
+    for edit, msg in [(lambda j: j["normalizer"].update(type="NFKC"), "normalizer"),
+                      (lambda j: j["model"].update(byte_fallback=True), "byte_fallback"),
+                      (lambda j: j["pre_tokenizer"]["pretokenizers"][0]["pattern"].update(Regex=r"\s+"), "split pattern"),
+                      (lambda j: j["pre_tokenizer"]["pretokenizers"][1].update(add_prefix_space=True), "ByteLevel"),
+                      (lambda j: j["added_tokens"][0].update(lstrip=True), "lstrip")]:
+        d = tmp_path / msg.replace(" ", "_")
+        shutil.copytree(FIX, d)
+        j = json.load(open(d / "tokenizer.json"))
+        edit(j)
+        json.dump(j, open(d / "tokenizer.json", "w"))
+        with pytest.raises(orn.OrnithError, match=msg):
+            text.Tokenizer(d)
+    with pytest.raises(orn.OrnithError, match="tokenizer.json"):
+        text.Tokenizer(tmp_path / "nowhere")
+
+
+# ---- streaming detokenizer ---------------------------------------------------------------
+def test_streaming_detokenizer(tk):
+    for s, ids in zip(CASES["text"], CASES["ids_json"]):
+        d = tk.detokenizer()
+        segs = []
+        for t in ids:
+            d.add_token(t)
+            seg = d.last_segment()
+            assert "�" not in seg or "�" in tk.decode(ids)      # no half characters leak out
+            segs.append(seg)
+        d.finalize()
+        segs.append(d.last_segment())
+        whole = tk.decode(ids)
+        want = whole[1:] if whole.startswith(" ") else whole              # the one leading space is dropped
+        if "\x00" not in whole:
+            assert "".join(segs) == want == d.text, repr(s)
+        d.close()
+    # a character split over two tokens comes out when it completes; a lone space waits
+    euro = [tk.id(c) for c in ("â", "Ĥ", "¬")]              # the byte-level spelling of E2 82 AC
+    if all(e is not None for e in euro):
+        d = tk.detokenizer()
+        out = []
+        for t in euro:
+            d.add_token(t)
+            out.append(d.last_segment())
+        assert out == ["", "", "€"]
+        d.close()
+    sp, a = tk.id("Ġ"), tk.id("a")
+    d = tk.detokenizer()
+    d.add_token(sp)
+    assert d.last_segment() == ""          # held back
+    d.add_token(a)
+    assert d.last_segment() == "a"         # ... and dropped: it was the generation's leading space
+    d.add_token(sp)
+    d.add_token(a)
+    assert d.last_segment() == " a"
+    d.finalize()
+    assert d.text == "a a"
+    d.close()
+
+
+# ---- chat template -------------------------------------------------------------------------
+def test_tojson_matches_python():
+    values = [{"type": "function", "function": {"name": "get_weather", "description": "Wetter für Zürich \"heute\"\n",
+                                                 "parameters": {"type": "object", "properties": {"city": {"type": "string"}, "days": {"type": "integer", "default": 3}},
+                                                                "required": ["city"]}}},
+              [1, -2, 0, 2.5, -0.0, 1e16, 1e15, 123456789012345680.0, 1.5e-7, 0.0001, 0.00001, 1e-5, 3.14159, 1 / 3, 2 ** 70, True, False, None],
+              {"nested": {"empty_list": [], "empty_obj": {}, "s": "tab\tcr\rbs\\ \u0001 \u007f é 日本 \U0001F600"}}, "plain", 7, [], {}]
+    for v in values:
+        src = json.dumps(v)                       # ASCII-escaped on the way in
+        assert text.json_dumps(src) == json.dumps(json.loads(src), ensure_ascii=False), src
+        src2 = json.dumps(v, ensure_ascii=False, separators=(",", ":"))
+        assert text.json_dumps(src2) == json.dumps(v, ensure_ascii=False)
+    assert text.json_dumps('{"b": 1, "a": 2}') == '{"b": 1, "a": 2}'          # written order kept
+
+
+def _expected_render(messages, tools, add_generation_prompt, enable_thinking):
+    """The template's documented behaviour (src/chat.rs:13-27), composed from Python's own
+    str.strip and json.dumps; the cases below keep to shapes where that description is complete."""
+    out = ""
+    if tools:
+        out += "<|im_start|>system\n# Tools\n\nYou have access to the following functions:\n\n<tools>"
+        out += "".join("\n" + json.dumps(t, ensure_ascii=False) for t in tools) + "\n</tools>" + TOOL_TEXT
+        if messages[0]["role"] == "system" and messages[0]["content"].strip():
+            out += "\n\n" + messages[0]["content"].strip()
+        out += "<|im_end|>\n"
+    elif messages[0]["role"] == "system":
+        out += "<|im_start|>system\n" + messages[0]["content"].strip() + "<|im_end|>\n"
+    for i, m in enumerate(messages):
+        c = (m.get("content") or "").strip()
+        if m["role"] == "user":
+            out += "<|im_start|>user\n" + c + "<|im_end|>\n"
+        elif m["role"] == "assistant":
+            out += "<|im_start|>assistant\n<think>\n" + m.get("reasoning_content", "").strip() + "\n</think>\n\n" + c + "<|im_end|>\n"
+        elif m["role"] == "tool":
+            if messages[i - 1]["role"] != "tool":
+                out += "<|im_start|>user"
+            out += "\n<tool_response>\n" + c + "\n</tool_response>"
+            if i + 1 == len(messages) or messages[i + 1]["role"] != "tool":
+                out += "<|im_end|>\n"
+    if add_generation_prompt:
+        out += "<|im_start|>assistant\n" + ("<think>\n" if enable_thinking else "<think>\n\n</think>\n\n")
+    return out
+
+
+TOOL_TEXT = ("\n\nIf you choose to call a function ONLY reply in the following format with NO suffix:\n\n<tool_call>\n"
+             "<function=example_function_name>\n<parameter=example_parameter_1>\nvalue_1\n</parameter>\n"
+             "<parameter=example_parameter_2>\nThis is the value for the second parameter\nthat can span\nmultiple lines\n"
+             "</parameter>\n</function>\n</tool_call>\n\n<IMPORTANT>\nReminder:\n- Function calls MUST follow the specified format: "
+             "an inner <function=...></function> block must be nested within <tool_call></tool_call> XML tags\n"
+             "- Required parameters MUST be specified\n- You may provide optional reasoning for your function call in natural "
+             "language BEFORE the function call, but NOT after\n- If there is no function call available, answer the question like "
+             "normal with your current knowledge and do not tell the user about function calls\n</IMPORTANT>")
+
+
+def test_chat_template_renders():
+    # the reference's in-source cases (chat.rs:357-369)
+    hi = [{"role": "user", "content": "hi"}]
+    assert text.apply_chat_template(hi, None, True, False) == "<|im_start|>user\nhi<|im_end|>\n<|im_start|>assistant\n<think>\n\n</think>\n\n"
+    assert text.apply_chat_template(hi, None, True, True) == "<|im_start|>user\nhi<|im_end|>\n<|im_start|>assistant\n<think>\n"
+    with pytest.raises(orn.OrnithError, match="No user query found"):
+        text.apply_chat_template([{"role": "system", "content": "be nice"}])
+    tools = [{"type": "function", "function": {"name": "f", "parameters": {"type": "object", "properties": {"x": {"type": "number"}}}}}]
+    convs = [
+        [{"role": "system", "content": "  be brief\n"}, {"role": "user", "content": "\thi there \x1f"}],
+        [{"role": "user", "content": "a"}, {"role": "assistant", "content": "b", "reasoning_content": " because \n"}, {"role": "user", "content": "c"}],
+        [{"role": "user", "content": "look it up"}, {"role": "assistant", "content": ""}, {"role": "tool", "content": "42"},
+         {"role": "tool", "content": " 43 "}, {"role": "user", "content": "thanks"}],
+        [{"role": "system", "content": ""}, {"role": "user", "content": "q"}],
+    ]
+    for conv in convs:
+        for tl in (None, tools):
+            for gen in (True, False):
+                for think in (True, False):
+                    assert text.apply_chat_template(conv, tl, gen, think) == _expected_render(conv, tl, gen, think)
+    # parts, think blocks inside content, tool calls in both shapes (chat.rs:150-190, 266-330)
+    got = text.apply_chat_template([{"role": "user", "content": [{"type": "image"}, {"type": "text", "text": " what is this? "}, {"video": "v.mp4"}]}], None, False)
+    assert got == "<|im_start|>user\n<|vision_start|><|image_pad|><|vision_end|> what is this? <|vision_start|><|video_pad|><|vision_end|><|im_end|>\n"
+    got = text.apply_chat_template([{"role": "user", "content": "q"}, {"role": "assistant", "content": "<think>\nold\n</think>\n\n<think>\nwhy\n</think>\n\nanswer"}], None, False)
+    assert got == "<|im_start|>user\nq<|im_end|>\n<|im_start|>assistant\n<think>\nold\n</think>\n\nanswer<|im_end|>\n"
+    calls = [{"function": {"name": "f", "arguments": {"x": 1.5, "s": "raw text", "o": {"k": [1, 2]}}}}, {"name": "g"}]
+    got = text.apply_chat_template([{"role": "user", "content": "q"}, {"role": "assistant", "content": "calling", "tool_calls": calls}], None, False)
+    assert got == ("<|im_start|>user\nq<|im_end|>\n<|im_start|>assistant\n<think>\n\n</think>\n\ncalling\n\n<tool_call>\n<function=f>\n"
+                   "<parameter=x>\n1.5\n</parameter>\n<parameter=s>\nraw text\n</parameter>\n<parameter=o>\n{\"k\": [1, 2]}\n</parameter>\n"
+                   "</function>\n</tool_call>\n<tool_call>\n<function=g>\n</function>\n</tool_call><|im_end|>\n")
+    got = text.apply_chat_template([{"role": "user", "content": "q"}, {"role": "assistant", "content": None, "tool_calls": calls[1:]}], None, False)
+    assert got.endswith("<think>\n\n</think>\n\n<tool_call>\n<function=g>\n</function>\n</tool_call><|im_end|>\n")
+    # the template's own errors
+    for conv, msg in [([], "No messages provided"), ([{"role": "user", "content": "a"}, {"role": "system", "content": "late"}], "System message must be at the beginning"),
+                      ([{"role": "system", "content": [{"type": "image"}]}, {"role": "user", "content": "a"}], "cannot contain images"),
+                      ([{"role": "user", "content": "<tool_response>\nx\n</tool_response>"}], "No user query found")]:
+        with pytest.raises(orn.OrnithError, match=msg):
+            text.apply_chat_template(conv)
+
+
+def test_rendered_prompt_round_trips_through_the_tokenizer(tk):
+    prompt = text.apply_chat_template([{"role": "system", "content": "Be brief."}, {"role": "user", "content": "It's 9 o'clock"}], None, True, False)
+    ids = tk.encode(prompt)
+    assert ids[0] == tk.id("<|im_start|>") and ids.count(tk.id("<|im_end|>")) == 2
+    assert tk.id("<think>") in ids and tk.id("</think>") in ids
+    assert tk.decode(ids) == prompt
