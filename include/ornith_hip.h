@@ -37,6 +37,9 @@ extern "C" {
 /* k-quant kinds (src/ops/kquant.rs KQuant) */
 #define ORNITH_Q4K 0
 #define ORNITH_Q6K 1
+/* a third kind a stacked-expert descriptor may carry (the MoE block only; the k-quant
+ * operators refuse it): mlx 4-bit affine, group 32 - the published artifact's switch_mlp */
+#define ORNITH_AFFINE4_G32 2
 
 typedef struct ornith_ctx ornith_ctx;
 
@@ -98,9 +101,11 @@ ORNITH_API int ornith_timer_end(ornith_ctx* ctx, float* ms_out);
  * Three device tensors in the reference's layout:
  *   Q4_K qs u32[E,O,K/8]     scales u8[E,O,K/256,12]  dm f16[E,O,K/256,2]
  *   Q6_K qs u32[E,O,3K/16]   scales u8[E,O,K/256,16]  dm f16[E,O,K/256,1]
- * E == 1 for a plain matrix. */
+ * E == 1 for a plain matrix. For routed experts in the 4-bit affine format
+ * (src/ops/quantized.rs:531-589) the same three slots carry kind ORNITH_AFFINE4_G32:
+ *   qs u32[E,O,K/8] (eight codes a word)   scales bf16[E,O,K/32]   dm = biases bf16[E,O,K/32] */
 typedef struct ornith_kmatrix {
-  int kind; /* ORNITH_Q4K / ORNITH_Q6K */
+  int kind; /* ORNITH_Q4K / ORNITH_Q6K (/ ORNITH_AFFINE4_G32: expert stacks of a MoE block) */
   int E, O, K;
   const void* d_qs;
   const void* d_scales;

@@ -38,7 +38,10 @@ typedef uint16_t bf16_t; /* raw bits */
 typedef uint16_t f16_t;  /* raw bits */
 
 enum { ORC_F32 = 0, ORC_BF16 = 1 };
-enum { ORC_Q4K = 0, ORC_Q6K = 1 };
+enum { ORC_Q4K = 0, ORC_Q6K = 1,
+       /* stacked experts in the 4-bit affine group-32 format riding in an orc_kmat: qs = packed
+        * codes u8[E,O,K/2], scales = bf16 scales [E,O,K/32], dm = bf16 biases [E,O,K/32] */
+       ORC_AFFINE4_G32 = 2 };
 
 static inline uint32_t orc_f2u(float f) {
   uint32_t u;

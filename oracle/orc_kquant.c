@@ -235,8 +235,13 @@ float orc_q4k_row_dot_ref32(const uint8_t* qs, const uint8_t* scales, const f16_
 float orc_q6k_row_dot_ref32(const uint8_t* w, const uint8_t* scales, const f16_t* dm, int K, const float* x,
                             int fma, int tree);
 
+float orc_affine4_row_dot(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K, const float* x);  /* orc_moe.c */
+
 float orc_kq_row_dot(int kind, const uint8_t* qs, const uint8_t* scales, const f16_t* dm,
                      int K, int64_t row, const float* x) {
+  if (kind == ORC_AFFINE4_G32)  /* quantized::gather_qmv, 4-bit affine (src/ops/quantized.rs:531-589) */
+    return orc_affine4_row_dot(qs + row * (K / 2), (const bf16_t*)scales + row * (K / 32),
+                               (const bf16_t*)dm + row * (K / 32), K, x);
   const uint8_t* q = qs + row * kq_qs_row(kind, K);
   const uint8_t* s = scales + row * kq_sc_row(kind, K);
   const f16_t* d = dm + row * kq_dm_row(kind, K);

@@ -392,6 +392,16 @@ extern "C" {
 
 int ornith_kmatrix_check(const ornith_kmatrix* w, size_t qs_bytes, size_t scales_bytes,
                          size_t dm_bytes) {
+  if (w && w->kind == ORNITH_AFFINE4_G32) {
+    ORN_REQUIRE(w->E >= 1 && w->O >= 1 && w->K >= 32 && w->K % 32 == 0, "KMatrix: bad dims E=%d O=%d K=%d", w->E,
+                w->O, w->K);
+    ORN_REQUIRE(w->d_qs && w->d_scales && w->d_dm, "KMatrix: null tensor");
+    const size_t groups = (size_t)w->E * w->O * (w->K / 32);
+    ORN_REQUIRE(qs_bytes == groups * 16 && scales_bytes == groups * 2 && dm_bytes == groups * 2,
+                "affine4 sizes: %zu / %zu / %zu bytes, %zu groups want %zu / %zu / %zu", qs_bytes, scales_bytes,
+                dm_bytes, groups, groups * 16, groups * 2, groups * 2);
+    return ORNITH_OK;
+  }
   int rc = check_matrix(w, "KMatrix");
   if (rc) return rc;
   const size_t blocks = (size_t)w->E * w->O * (w->K / 256);

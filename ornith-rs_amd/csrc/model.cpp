@@ -527,6 +527,13 @@ int ornith_frspec_from_ids(ornith_model* m, const uint32_t* ids, int n, ornith_f
       f->head.d_w = f->owned[0];
       f->head.d_scales = f->owned[1];
       f->head.d_biases = f->owned[2];
+    } else if (lm.mode == ORNITH_LIN_AFFINE4) {
+      rc = gather_rows_dev(m->ctx, lm.d_w, (size_t)lm.K / 2, f->ids, &f->owned[0]);
+      if (!rc) rc = gather_rows_dev(m->ctx, lm.d_scales, (size_t)lm.K / 32 * 2, f->ids, &f->owned[1]);
+      if (!rc) rc = gather_rows_dev(m->ctx, lm.d_biases, (size_t)lm.K / 32 * 2, f->ids, &f->owned[2]);
+      f->head.d_w = f->owned[0];
+      f->head.d_scales = f->owned[1];
+      f->head.d_biases = f->owned[2];
     } else {
       rc = gather_rows_dev(m->ctx, lm.d_w, (size_t)lm.K * 2, f->ids, &f->owned[0]);
       f->head.d_w = f->owned[0];

@@ -292,11 +292,15 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
     if (rcn) return rcn;
     pre = nullptr;
   }
-  if (T >= kPrefillRows && !w->ex_dense) {
+  const bool ex_affine4 = !w->ex_dense && w->ex_gate.kind == ORNITH_AFFINE4_G32;
+  if (ex_affine4)
+    ORN_REQUIRE(w->ex_up.kind == ORNITH_AFFINE4_G32 && w->ex_down.kind == ORNITH_AFFINE4_G32,
+                "moe_block: the three expert stacks must share the 4-bit affine format");
+  if (T >= kPrefillRows && !w->ex_dense && !ex_affine4) {
     ORN_REQUIRE(!d_inds_out && !d_scores_out, "moe_block: index outputs are a decode-width feature");
     return moe_block_prefill(ctx, w, d_x, T, d_out);
   }
-  ORN_REQUIRE(T <= 64, "moe_block: T=%d with dense experts (decode/verify widths only)", T);
+  ORN_REQUIRE(T <= 64, "moe_block: T=%d with dense or 4-bit affine experts (decode/verify widths only)", T);
 
   const size_t need = 2 * ((size_t)T * E * 2 + (size_t)T * SI * 3 + (size_t)T * H + T +
                            (size_t)(T * k + T) * (2 * I + I + SI + H + 1)) +
@@ -373,6 +377,16 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
     TRY(swiglu_pair(ctx, sg, su, (int64_t)T * SI, sact, xg, xu, (int64_t)T * k * I, act));
     TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
     TRY(ornith_dense_gather_mv(ctx, w->d_ex_down, E, H, I, act, T * k, lhs_row, inds, T * k, y));
+  } else if (ex_affine4) {
+    // quantized::gather_qmv over the stacked 4-bit affine experts (src/ops/quantized.rs:531-589)
+    TRY(ornith_affine4_gather_qmv(ctx, w->ex_gate.d_qs, w->ex_gate.d_scales, w->ex_gate.d_dm, E, I, H, d_x, T,
+                                  lhs_tok, inds, T * k, xg));
+    TRY(ornith_affine4_gather_qmv(ctx, w->ex_up.d_qs, w->ex_up.d_scales, w->ex_up.d_dm, E, I, H, d_x, T, lhs_tok,
+                                  inds, T * k, xu));
+    TRY(swiglu_pair(ctx, sg, su, (int64_t)T * SI, sact, xg, xu, (int64_t)T * k * I, act));
+    TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
+    TRY(ornith_affine4_gather_qmv(ctx, w->ex_down.d_qs, w->ex_down.d_scales, w->ex_down.d_dm, E, H, I, act, T * k,
+                                  lhs_row, inds, T * k, y));
   } else {
     TRY(ornith_kq_gather_qmv(ctx, &w->ex_gate, d_x, ORNITH_BF16, T, lhs_tok, inds, T * k, xg,
                              ORNITH_BF16));

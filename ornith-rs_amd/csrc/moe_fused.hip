@@ -723,6 +723,7 @@ extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_up(long
 // Whether the two fused kernels cover this block's shapes and formats.
 bool moe_fused_supported(const ornith_moe_weights* w) {
   if (w->ex_dense) return false;
+  if (w->ex_gate.kind > ORNITH_Q6K || w->ex_down.kind > ORNITH_Q6K) return false;  // 4-bit affine stacks
   const ornith_linear* sh[3] = {&w->sh_gate, &w->sh_up, &w->sh_down};
   for (auto* l : sh)
     if (l->mode != ORNITH_LIN_KQUANT) return false;

@@ -38,6 +38,31 @@ static int kq_from(const ornith_weights* ws, const std::string& path, bool route
   const Tensor* w = ws->find(path + ".weight");
   const Tensor* s = ws->find(path + ".scales");
   const Tensor* d = ws->find(path + ".dm");
+  if (routed && w && s && !d && ornith_weights_has(ws, (path + ".biases").c_str())) {
+    // stacked experts in the 4-bit affine group-32 format (the published artifact's switch_mlp)
+    const Tensor* b = ws->find(path + ".biases");
+    ORN_REQUIRE_TENSOR(ws, b, "%s.biases: no such tensor", path.c_str());
+    int rc = check_mode(ws, path, false, 0);
+    if (rc) return rc;
+    ORN_REQUIRE(w->dtype == ORNITH_DT_U32 || w->dtype == ORNITH_DT_U8, "%s.weight must be uint32", path.c_str());
+    ORN_REQUIRE(s->dtype == ORNITH_DT_BF16 && b->dtype == ORNITH_DT_BF16, "%s: affine scales/biases must be bfloat16",
+                path.c_str());
+    ORN_REQUIRE(s->shape.size() == 3 && b->shape == s->shape, "%s: scales/biases must be [E, O, K/32]", path.c_str());
+    if (ws->quant.loaded) {
+      const QuantSpec q = ws->quant.lookup(path);
+      ORN_REQUIRE(q.bits == 4 && q.group_size == 32,
+                  "%s: affine %d-bit group %d experts are not carried (4-bit group 32 only)", path.c_str(), q.bits,
+                  q.group_size);
+    }
+    out->kind = ORNITH_AFFINE4_G32;
+    out->E = (int)s->shape[0];
+    out->O = (int)s->shape[1];
+    out->K = (int)s->shape[2] * 32;
+    out->d_qs = w->d;
+    out->d_scales = s->d;
+    out->d_dm = b->d;
+    return ornith_kmatrix_check(out, w->bytes, s->bytes, b->bytes);
+  }
   ORN_REQUIRE_TENSOR(ws, w && s && d, "%s: k-quant module needs .weight, .scales and .dm", path.c_str());
   ORN_REQUIRE(w->dtype == ORNITH_DT_U32 || w->dtype == ORNITH_DT_U8, "%s.weight must be uint32",
               path.c_str());

@@ -84,11 +84,16 @@ def _norm_w(rng, n):
 class SynthModel:
     """All tensors of a trunk (+ optional MTP head) for a config dict."""
 
-    def __init__(self, cfg, seed=0, with_mtp=True, with_oracle=True, affine="affine8"):
+    def __init__(self, cfg, seed=0, with_mtp=True, with_oracle=True, affine="affine8", trunk="kq"):
         """affine: the format of the two affine modules (embed_tokens, shared_expert_gate):
         'affine8' (8-bit group 64, as in the k-quant artifact) or 'affine4' (4-bit group 32, the
-        published artifact's format)."""
+        published artifact's format). trunk: 'kq' (the k-quant artifact: Q4_K / Q6_K
+        projections and experts) or 'affine4' (the published artifact: every projection, the
+        routed and shared experts and lm_head 4-bit affine group 32, the router 8-bit)."""
         self.affine = affine
+        self.trunk = trunk
+        t4 = (lambda kind: "affine4") if trunk == "affine4" else (lambda kind: kind)
+        self._fmt = t4
         self.cfg = dict(cfg)
         self.rng = np.random.default_rng(seed)
         self.tensors = {}     # name -> (array, dtype code)
@@ -102,7 +107,7 @@ class SynthModel:
         hd, Hq, Hkv = c["head_dim"], c["num_attention_heads"], c["num_key_value_heads"]
         P = "language_model.model."
         self.embed = self._linear(P + "embed_tokens", affine, c["vocab_size"], H)
-        self.lm_head = self._linear("language_model.lm_head", Q4K, c["vocab_size"], H)
+        self.lm_head = self._linear("language_model.lm_head", t4(Q4K), c["vocab_size"], H)
         self.final_norm = self._plain(P + "norm.weight", _norm_w(self.rng, H))
         self.layers = []
         for i in range(L):
@@ -113,9 +118,9 @@ class SynthModel:
             if lay["linear"]:
                 g = lp + "linear_attn."
                 lay["gdn"] = dict(
-                    in_proj_qkv=self._linear(g + "in_proj_qkv", Q4K, D, H),
-                    in_proj_z=self._linear(g + "in_proj_z", Q4K, vd, H),
-                    out_proj=self._linear(g + "out_proj", Q4K, H, vd),
+                    in_proj_qkv=self._linear(g + "in_proj_qkv", t4(Q4K), D, H),
+                    in_proj_z=self._linear(g + "in_proj_z", t4(Q4K), vd, H),
+                    out_proj=self._linear(g + "out_proj", t4(Q4K), H, vd),
                     in_proj_a=self._linear(g + "in_proj_a", "dense", Hv, H),
                     in_proj_b=self._linear(g + "in_proj_b", "dense", Hv, H),
                     conv1d=self._plain(g + "conv1d.weight", util.bf16_normal(self.rng, (D, 4, 1), 0.5)),
@@ -123,7 +128,7 @@ class SynthModel:
                     a_log=self._plain(g + "A_log", util.bf16_normal(self.rng, (Hv,), 0.5)),
                     norm=self._plain(g + "norm.weight", _norm_w(self.rng, c["linear_value_head_dim"])))
             else:
-                lay["attn"] = self._attn(lp + "self_attn.", Q6K)
+                lay["attn"] = self._attn(lp + "self_attn.", t4(Q6K))
             lay["moe"] = self._moe(lp + "mlp.", dense=False)
             self.layers.append(lay)
         self.mtp = None
@@ -144,6 +149,11 @@ class SynthModel:
         return self.tensors[name][0]
 
     def _reg_kmat(self, path, km, routed):
+        if km.kind == util.AFFINE4:
+            self.tensors[path + ".weight"] = (km.qs.view(np.uint32), DT_U32)
+            self.tensors[path + ".scales"] = (km.scales, DT_BF16)
+            self.tensors[path + ".biases"] = (km.dm, DT_BF16)
+            return
         nb = km.K // 256
         cb, sb, db = (128, 12, 2) if km.kind == Q4K else (192, 16, 1)
         lead = (km.E, km.O) if routed else (km.O,)
@@ -188,14 +198,15 @@ class SynthModel:
             m["sh_down"] = self._linear(p_ + "shared_expert.down_proj", "dense", H, SI)
             m["sh_egate"] = self._linear(p_ + "shared_expert_gate", "dense", 1, H)
         else:
-            m["router"] = self._linear(p_ + "gate", Q6K, E, H)
+            a4 = self.trunk == "affine4"
+            m["router"] = self._linear(p_ + "gate", "affine8" if a4 else Q6K, E, H)
             for n, kind, (o, k) in (("gate", Q4K, (I, H)), ("up", Q4K, (I, H)), ("down", Q6K, (H, I))):
-                km = HostKMat.random(self.rng, kind, E, o, k)
+                km = HostKMat.random(self.rng, util.AFFINE4 if a4 else kind, E, o, k)
                 self._reg_kmat(f"{p_}switch_mlp.{n}_proj", km, routed=True)
                 m["ex_" + n] = km
-            m["sh_gate"] = self._linear(p_ + "shared_expert.gate_proj", Q4K, SI, H)
-            m["sh_up"] = self._linear(p_ + "shared_expert.up_proj", Q4K, SI, H)
-            m["sh_down"] = self._linear(p_ + "shared_expert.down_proj", Q6K, H, SI)
+            m["sh_gate"] = self._linear(p_ + "shared_expert.gate_proj", self._fmt(Q4K), SI, H)
+            m["sh_up"] = self._linear(p_ + "shared_expert.up_proj", self._fmt(Q4K), SI, H)
+            m["sh_down"] = self._linear(p_ + "shared_expert.down_proj", self._fmt(Q6K), H, SI)
             m["sh_egate"] = self._linear(p_ + "shared_expert_gate", self.affine, 1, H)
         return m
 
@@ -327,6 +338,9 @@ class OracleRun:
 def prune_head(lin, ids):
     """FrSpec::prune on the host (for the oracle): row-gather of a k-quant head."""
     ids = np.asarray(ids, dtype=np.int64)
+    if lin.mode in ("affine4", "affine8"):
+        return HostLinear(lin.mode, len(ids), lin.K, w=np.ascontiguousarray(lin.w[ids]),
+                          scales=np.ascontiguousarray(lin.scales[ids]), biases=np.ascontiguousarray(lin.biases[ids]))
     km = lin.km
     return HostLinear("kq", len(ids), lin.K, km=HostKMat(km.kind, 1, len(ids), km.K, (km.qs[ids], km.scales[ids], km.dm[ids])))
 
@@ -385,8 +399,15 @@ def write_artifact(synth, model_dir, shards=3, nested=True):
     with open(os.path.join(model_dir, "model.safetensors.index.json"), "w") as f:
         json.dump({"metadata": {"total_size": synth.total_bytes()}, "weight_map": weight_map}, f)
 
-    quant = {"group_size": 64, "bits": 8, "mode": "affine"}
+    a4 = getattr(synth, "trunk", "kq") == "affine4"
+    quant = {"group_size": 32, "bits": 4, "mode": "affine"} if a4 else {"group_size": 64, "bits": 8, "mode": "affine"}
     for n, (arr, dt) in synth.tensors.items():
+        if n.endswith(".biases"):
+            # a module that departs from the artifact's default gets its own entry (mlx's per-layer overrides)
+            groups, wbytes = synth.tensors[n[:-7] + ".scales"][0].size, synth.tensors[n[:-7] + ".weight"][0].nbytes
+            bits = 8 if wbytes == groups * 64 else 4
+            if bits != quant["bits"]:
+                quant[n[:-7]] = {"group_size": 64 if bits == 8 else 32, "bits": bits, "mode": "affine"}
         if n.endswith(".dm"):
             q4 = synth.tensors[n[:-3] + ".scales"][0].shape[-1] == 12
             quant[n[:-3]] = {"group_size": 256, "bits": 4 if q4 else 6, "mode": "q4k" if q4 else "q6k"}

@@ -69,3 +69,55 @@ def test_model_with_4bit_affine_modules_matches_oracle(orn, ctx):
         assert ar == want and spec == ar
     finally:
         head.close(); caches.close(); model.close(); ws.close()
+
+
+@pytest.mark.parametrize("T", [1, 2, 4, 9])
+def test_moe_block_with_4bit_affine_experts_bit_exact(orn, ctx, T):
+    """The published artifact's block: routed and shared experts 4-bit affine group 32, router and
+    shared gate 8-bit. Expert ids, scores and output by bits against the oracle."""
+    rng = np.random.default_rng(40 + T)
+    moe = util.HostMoe(rng, H=1024, E=64, I=256, top_k=8, gate_kind=util.AFFINE4)
+    xb = util.bf16_normal(rng, (T, 1024))
+    want, winds, wscores, _ = util.orc_moe_block(moe, xb, T)
+    w = moe.dev(orn, ctx)
+    dx = ctx.to_device(xb)
+    out, inds, scores = ctx.alloc(T * 1024 * 2), ctx.alloc(T * 8 * 4), ctx.alloc(T * 8 * 2)
+    try:
+        ctx.moe_block(w, dx, T, out, inds, scores)
+        assert np.array_equal(inds.download(np.uint32, (T, 8)), winds)
+        assert np.array_equal(scores.download(np.uint16, (T, 8)), wscores)
+        assert np.array_equal(out.download(np.uint16, (T, 1024)), want)
+    finally:
+        for b in (dx, out, inds, scores): b.free()
+        moe.free()
+
+
+def test_model_in_the_published_artifacts_format_matches_oracle(orn, ctx):
+    """Every projection, the routed and shared experts, embed_tokens and lm_head 4-bit affine
+    group 32 (routers 8-bit), as the published mlx artifact stores them: both loops, with and
+    without a pruned draft head, token for token against the oracle."""
+    s = synth.SynthModel(dict(synth.TINY, vocab_size=256), seed=33, affine="affine4", trunk="affine4")
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    prompt = np.random.default_rng(2).integers(0, 256, 9).astype(np.uint32)
+    caches = model.make_cache(48, 3)
+    head = orn.MtpHead(model, ws, 48)
+    fr_ids = synth.zipf_frspec_ids(256, 96, seed=3)
+    fr = orn.FrSpec(model, ids=fr_ids)
+    try:
+        ar = orn.generate_step(model, caches, prompt, 14, prefill_step=4)
+        o = synth.OracleRun(s, 48)
+        want = o.generate(prompt, 14, prefill_step=4)
+        o.close()
+        assert ar == want
+        for frs, frh in ((None, None), (fr, synth.prune_head(s.lm_head, fr_ids))):
+            caches.reset()
+            head.set_offset(0)
+            spec, st = orn.generate_step_mtp(model, head, frs, caches, prompt, 2, 14, prefill_step=4)
+            o = synth.OracleRun(s, 48)
+            wspec, wst = o.mtp_generate(prompt, 2, 14, fr_ids if frs else None, frh, prefill_step=4)
+            o.close()
+            assert spec == ar == wspec
+            assert (st.cycles, st.drafted, st.accepted) == (wst.cycles, wst.drafted, wst.accepted)
+    finally:
+        fr.close(); head.close(); caches.close(); model.close(); ws.close()

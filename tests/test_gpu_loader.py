@@ -110,3 +110,48 @@ def test_config_and_tensors_must_agree(orn, ctx, artifact, tmp_path):
     emb = "language_model.model.embed_tokens"
     assert "no " + emb + ".dm" in load_with(lambda q: q.update({emb: {"group_size": 256, "bits": 4, "mode": "q4k"}}))
     assert "is not carried" in load_with(lambda q: q.update({emb: {"bits": 4}}))   # 4-bit needs group 32
+
+
+def test_published_artifact_format_from_files(orn, ctx, tmp_path):
+    """The published mlx artifact's layout: 4-bit affine group 32 by default (projections, stacked
+    experts, embed_tokens, lm_head), 8-bit group 64 for the routers, said by config.json's
+    quantization block with per-module overrides. Read from files it generates the tokens of the
+    same model put by name and of the oracle."""
+    s = synth.SynthModel(dict(synth.TINY, vocab_size=256), seed=23, affine="affine4", trunk="affine4")
+    d = str(tmp_path / "model")
+    side = synth.write_artifact(s, d, shards=2)
+    q = json.load(open(os.path.join(d, "config.json")))["quantization"]
+    assert (q["bits"], q["group_size"]) == (4, 32)
+    assert q["language_model.model.layers.0.mlp.gate"] == {"group_size": 64, "bits": 8, "mode": "affine"}
+    cfg, _ = orn.TextConfig.load(d)
+    prompt = np.random.default_rng(4).integers(0, 256, 7).astype(np.uint32)
+
+    def run(ws, config):
+        model = orn.TextModel(ctx, ws, config)
+        head = orn.MtpHead(model, ws, 48)
+        caches = model.make_cache(48, 4)
+        greedy = orn.generate_step(model, caches, prompt, 10, prefill_step=4)
+        caches.reset()
+        spec, _ = orn.generate_step_mtp(model, head, None, caches, prompt, 2, 10, prefill_step=4)
+        for o in (head, caches, model):
+            o.close()
+        return greedy, spec
+
+    ws = orn.WeightStore.open(ctx, d, extra=[side])
+    assert ws.quant_config("language_model.model.layers.1.mlp.switch_mlp.down_proj") == (32, 4, orn.QM_AFFINE)
+    got = run(ws, cfg)
+    ws.close()
+    ws_put = s.upload(orn, ctx)
+    want = run(ws_put, s.text_config(orn))
+    ws_put.close()
+    orc = synth.OracleRun(s, 48)
+    assert got == want and got[0] == got[1] == orc.generate(prompt, 10, prefill_step=4)
+    orc.close()
+    # 8-bit stacked experts are not carried: the loader says so
+    cj = json.load(open(os.path.join(d, "config.json")))
+    cj["quantization"]["language_model.model.layers.0.mlp.switch_mlp.gate_proj"] = {"group_size": 64, "bits": 8, "mode": "affine"}
+    json.dump(cj, open(os.path.join(d, "config.json"), "w"))
+    ws = orn.WeightStore.open(ctx, d, extra=[side])
+    with pytest.raises(orn.OrnithError, match="4-bit group 32 only"):
+        orn.TextModel(ctx, ws, cfg)
+    ws.close()

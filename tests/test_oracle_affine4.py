@@ -60,3 +60,48 @@ def test_affine4_gather_equals_plain_rows_and_embedding_vs_double():
     W = _dequant(lin)
     bias = np.repeat(util.bf16_to_f32(lin.biases).astype(np.float64), 32, 1)
     assert np.all(np.abs(util.bf16_to_f32(out) - W[ids]) <= 2.0 ** -7 * np.abs(W[ids]) + 2.0 ** -8 * np.abs(bias[ids]))
+
+
+def test_moe_block_with_4bit_affine_experts_matches_float64_composition():
+    """The published artifact's MoE block (4-bit affine group-32 routed and shared experts, 8-bit
+    router and shared gate; src/ops/moe.rs:662-741 over quantized::gather_qmv) against a float64
+    restatement built from dequantized weights: same experts chosen where the cut is clear,
+    output within bf16 tolerance."""
+    rng = np.random.default_rng(6)
+    H, E, I, k, T = 512, 64, 256, 8, 3
+    moe = util.HostMoe(rng, H=H, E=E, I=I, top_k=k, gate_kind=util.AFFINE4)
+    xb = util.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32))
+    out, inds, scores, probs = util.orc_moe_block(moe, xb, T)
+    x = util.bf16_to_f32(xb).astype(np.float64)
+
+    def deq4(w, s, b, K):
+        w = np.ascontiguousarray(w)
+        words = w.view(np.uint32).reshape(-1, K // 8)
+        i = np.arange(K)
+        q = (words[:, i // 8] >> (4 * (i % 8)).astype(np.uint32)) & 15
+        sc = np.repeat(util.bf16_to_f32(s).astype(np.float64).reshape(-1, K // 32), 32, 1)
+        bi = np.repeat(util.bf16_to_f32(b).astype(np.float64).reshape(-1, K // 32), 32, 1)
+        return q.astype(np.float64) * sc + bi
+
+    def deq8(lin):
+        return lin.w.astype(np.float64) * np.repeat(util.bf16_to_f32(lin.scales), 64, 1) + np.repeat(util.bf16_to_f32(lin.biases), 64, 1)
+
+    Wg = deq4(moe.ex_gate.qs, moe.ex_gate.scales, moe.ex_gate.dm, H).reshape(E, I, H)
+    Wu = deq4(moe.ex_up.qs, moe.ex_up.scales, moe.ex_up.dm, H).reshape(E, I, H)
+    Wd = deq4(moe.ex_down.qs, moe.ex_down.scales, moe.ex_down.dm, I).reshape(E, H, I)
+    Sg, Su, Sd = (deq4(l.w, l.scales, l.biases, l.K) for l in (moe.sh_gate, moe.sh_up, moe.sh_down))
+    g = x @ deq8(moe.router).T
+    pr = np.exp(g - g.max(1, keepdims=True)); pr /= pr.sum(1, keepdims=True)
+    we = deq8(moe.sh_egate)[0]
+    silu = lambda v: v / (1 + np.exp(-v))
+    for t in range(T):
+        srt = np.sort(pr[t])
+        if srt[-k] - srt[-k - 1] > 2.0 ** -7 * srt[-k]:
+            assert set(np.argsort(pr[t], kind="stable")[-k:]) == set(int(i) for i in inds[t])
+        w = pr[t][inds[t].astype(int)]; w = w / w.sum()
+        acc = np.zeros(H)
+        for j, e in enumerate(inds[t].astype(int)):
+            acc += w[j] * (Wd[e] @ (silu(Wg[e] @ x[t]) * (Wu[e] @ x[t])))
+        want = acc + (Sd @ (silu(Sg @ x[t]) * (Su @ x[t]))) / (1 + np.exp(-(we @ x[t])))
+        got = util.bf16_to_f32(out[t]).astype(np.float64)
+        assert np.max(np.abs(got - want)) <= 0.03 * np.max(np.abs(want)), t

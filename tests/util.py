@@ -14,6 +14,7 @@ ORACLE_DIR = os.path.join(ROOT, "oracle")
 ORACLE_LIB = os.path.join(ORACLE_DIR, "liborc.so")
 
 Q4K, Q6K = 0, 1
+AFFINE4 = 2   # stacked experts in the 4-bit affine group-32 format riding in a k-matrix descriptor
 _orc = None
 
 
@@ -186,6 +187,13 @@ class HostKMat:
 
     @staticmethod
     def random(rng, kind, E, O, K, sigma=None):
+        if kind == AFFINE4:
+            # qs: codes two a byte (low nibble first); scales: bf16 scales; dm: bf16 biases, centred
+            w = rng.integers(0, 256, size=(E, O, K // 2), dtype=np.uint8)
+            s = (1.0 / (4.61 * np.sqrt(K))) * (0.5 + rng.random((E, O, K // 32)))
+            scales = f32_to_bf16(s.astype(np.float32))
+            biases = f32_to_bf16((-7.5 * bf16_to_f32(scales)).astype(np.float32))
+            return HostKMat(kind, E, O, K, (w, scales, biases))
         sigma = unit_sigma(kind, K) if sigma is None else sigma
         t = make_q4k(rng, E, O, K, d_sigma=sigma, centered=True) if kind == Q4K else make_q6k(rng, E, O, K, d_sigma=sigma)
         return HostKMat(kind, E, O, K, t)
@@ -266,6 +274,17 @@ class HostMoe:
 
     def __init__(self, rng, H=2048, E=256, I=512, top_k=8, gate_kind=Q4K, down_kind=Q6K, router_kind=Q6K):
         self.H, self.E, self.I, self.top_k = H, E, I, top_k
+        if gate_kind == AFFINE4:
+            # the published artifact's mix: 4-bit affine group 32 everywhere, the two gates 8-bit
+            self.router = HostLinear.affine8(rng, E, H)
+            self.ex_gate = HostKMat.random(rng, AFFINE4, E, I, H)
+            self.ex_up = HostKMat.random(rng, AFFINE4, E, I, H)
+            self.ex_down = HostKMat.random(rng, AFFINE4, E, H, I)
+            self.sh_gate = HostLinear.affine4(rng, I, H)
+            self.sh_up = HostLinear.affine4(rng, I, H)
+            self.sh_down = HostLinear.affine4(rng, H, I)
+            self.sh_egate = HostLinear.affine8(rng, 1, H)
+            return
         self.router = HostLinear.kq(rng, router_kind, E, H)
         self.ex_gate = HostKMat.random(rng, gate_kind, E, I, H)
         self.ex_up = HostKMat.random(rng, gate_kind, E, I, H)
