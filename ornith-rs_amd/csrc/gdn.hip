@@ -722,6 +722,12 @@ static void fill_front(FrontArgs& p, const void* d_conv_state, const void* d_qkv
   p.eps = eps;
 }
 
+// gdn_chunk.hip
+int gdn_chunked_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, const void* d_v, const float* d_g,
+                           const void* d_beta, const float* d_state_in, int T, int Hk, int Hv, int Dk, int Dv,
+                           void* d_y, float* d_state_out);
+constexpr int kChunkedRows = 128;  // from here a call's recurrence runs in 64-token chunks
+
 extern "C" {
 
 int ornith_gdn_step(ornith_ctx* ctx, const void* d_conv_state, const void* d_qkv, const void* d_cw,
@@ -821,6 +827,12 @@ int ornith_gdn_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, con
   RecArgs p{(const bf16_t*)d_q, (const bf16_t*)d_k, (const bf16_t*)d_v, d_g, (const bf16_t*)d_beta,
             d_state_in,         (bf16_t*)d_y,       d_snapshots,        T,   Hk, Hv, Dv,
             snapshot_every_token ? 1 : 0};
+  if (T >= kChunkedRows && !snapshot_every_token && ornith_option_gdn_chunked()) {
+    // long prompt chunks: the chunked form on the matrix cores (agrees to rounding)
+    const int rc = gdn_chunked_recurrence(ctx, d_q, d_k, d_v, d_g, d_beta, d_state_in, T, Hk, Hv, Dk, Dv, d_y,
+                                          d_snapshots);
+    if (rc != -1) return rc;
+  }
   if (T >= kPrefillRows && !snapshot_every_token) {
     // prompt chunks: the form with the short dependent chain (agrees to rounding)
     hipLaunchKernelGGL(gdn_recurrence_wide_kernel, dim3(Dv / 4, Hv), dim3(64), 0, ctx->stream, p);

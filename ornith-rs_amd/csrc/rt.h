@@ -108,6 +108,7 @@ int ornith_option_gemm_duo();  // 1: prefill GEMM with producer and consumer wav
 int ornith_option_kq_iters();      // output rows per wavefront pass of the mat-vec kernels; 0 = by shape
 int ornith_option_moe_up_iters();  // rows per wavefront of the fused gate+up kernel; 0 = by shape
 int ornith_option_moe_down_iters();  // column groups per workgroup of the expert down kernel; 0 = by shape
+int ornith_option_gdn_chunked();  // 1: the gated-delta recurrence of calls of 128 rows or more runs chunked on the matrix cores
 int ornith_option_fuse_moe_one();  // 1: the MoE block's router, up and down phases in one launch
 int ornith_option_ho_spins();      // polling rounds a hand-off wait inside a launch may take
 

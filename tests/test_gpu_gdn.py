@@ -121,11 +121,12 @@ def test_recurrence_small_heads_and_in_place(orn, ctx):
     for b in d + [yb]: b.free()
 
 
-@pytest.mark.parametrize("T,Hk,Hv", [(32, 2, 4), (77, 2, 4), (130, 16, 32)])
+@pytest.mark.parametrize("T,Hk,Hv", [(32, 2, 4), (77, 2, 4), (130, 16, 32), (128, 2, 4), (257, 2, 4), (1000, 4, 8)])
 def test_recurrence_at_prefill_width_close_to_exact(orn, ctx, T, Hk, Hv):
     """From 32 rows a call (only the final state wanted) the recurrence runs in its
-    short-dependent-chain form, which sums in another order: outputs within 0.5 % relative L2
-    of the oracle's exact recurrence per token, final state within 1e-4 relative L2."""
+    short-dependent-chain form, which sums in another order, and from 128 rows in 64-token
+    chunks on the matrix cores: outputs within 0.5 % relative L2 of the oracle's exact
+    recurrence per token, final state within 1e-4 relative L2."""
     rng = np.random.default_rng(T + Hv)
     q = util.bf16_normal(rng, (T, Hk, 128), 0.1); k = util.bf16_normal(rng, (T, Hk, 128), 0.1)
     v = util.bf16_normal(rng, (T, Hv, 128)); beta = util.f32_to_bf16(rng.random((T, Hv)).astype(np.float32))
@@ -143,3 +144,47 @@ def test_recurrence_at_prefill_width_close_to_exact(orn, ctx, T, Hk, Hv):
     assert err.max() < 5e-3, err.max()
     serr = np.linalg.norm(gs - wsnaps[-1]) / np.linalg.norm(wsnaps[-1])
     assert serr < 1e-4, serr
+
+
+@pytest.mark.parametrize("T,decay", [(192, "wide"), (300, "tiny"), (500, "mixed")])
+def test_chunked_recurrence_over_hard_decays(orn, ctx, T, decay):
+    """The chunked form keeps its decays as differences of running log sums: decays far from one,
+    decays that underflow to nothing (the state is forgotten mid-chunk) and beta = 0 / 1 rows
+    must come out like the exact walk. Same bounds as above; and with the chunked form switched
+    off the same call (the other prefill kernel) agrees with it too."""
+    rng = np.random.default_rng(T)
+    Hk, Hv = 2, 4
+    q = util.bf16_normal(rng, (T, Hk, 128), 0.1); k = util.bf16_normal(rng, (T, Hk, 128), 0.1)
+    v = util.bf16_normal(rng, (T, Hv, 128))
+    beta = rng.random((T, Hv)).astype(np.float32)
+    beta[rng.random((T, Hv)) < 0.1] = 0.0
+    beta[rng.random((T, Hv)) < 0.1] = 1.0
+    beta = util.f32_to_bf16(beta)
+    if decay == "wide":
+        g = (0.3 + 0.7 * rng.random((T, Hv))).astype(np.float32)
+    elif decay == "tiny":
+        g = (0.9 + 0.1 * rng.random((T, Hv))).astype(np.float32)
+        g[rng.random((T, Hv)) < 0.03] = 1e-30
+        g[7, 0] = 0.0
+    else:
+        g = np.exp(-np.exp(rng.normal(-3.0, 2.0, (T, Hv)))).astype(np.float32)
+    S0 = (rng.standard_normal((Hv, 128, 128)) * 0.1).astype(np.float32)
+    wy, wsnaps = util.orc_gdn_recurrence(q, k, v, g, beta, S0)
+    ry = util.bf16_to_f32(wy)
+    outs = {}
+    for chunked in (1, 0):
+        orn.set_option("gdn_chunked", chunked)
+        d = [ctx.to_device(a) for a in (q, k, v, g, beta, S0)]
+        y, fin = ctx.alloc(T * Hv * 128 * 2), ctx.alloc(Hv * 128 * 128 * 4)
+        ctx.gdn_recurrence(*d, T, Hk, Hv, 128, 128, y, fin, snap_all=False)
+        gy = util.bf16_to_f32(y.download(np.uint16, (T, Hv, 128)))
+        gs = fin.download(np.float32, (Hv, 128, 128))
+        for b in d + [y, fin]: b.free()
+        assert np.all(np.isfinite(gy)) and np.all(np.isfinite(gs))
+        err = np.linalg.norm((gy - ry).reshape(T, -1), axis=1) / (np.linalg.norm(ry.reshape(T, -1), axis=1) + 1e-30)
+        assert err.max() < 5e-3, (chunked, err.max())
+        serr = np.linalg.norm(gs - wsnaps[-1]) / np.linalg.norm(wsnaps[-1])
+        assert serr < 1e-4, (chunked, serr)
+        outs[chunked] = gy
+    orn.set_option("gdn_chunked", 1)
+    assert not np.array_equal(outs[0], outs[1])        # two different kernels did run
