@@ -49,6 +49,11 @@ struct ChunkArgs {
   bf16_t* pl;           //                  low part
   float* ell;           // [n, Hv, 64]
   bf16_t* kt;           // [n, Hk, 128, 64]  K transposed
+  bf16_t* qf;           // [n, Hk, 64, 128]  Q
+  // Everything the first kernel writes is laid out as the second kernel's wavefronts hold it: the
+  // 8 values of lane l for (16-row tile, 32-wide k slab) sit at ((tile * slabs + slab) * 64 + l) * 8,
+  // so that one load instruction of a wavefront is one contiguous KB (row-major, the same loads
+  // touch 16 half-used cache lines each and the L1's line rate bounds the scan).
   int T, Hk, Hv, Dv, nchunks;
 };
 
@@ -67,13 +72,16 @@ __device__ __forceinline__ f32x4_t mfma(bf16x8_t a, bf16x8_t b, f32x4_t c) {
 // holds A[m = l16][k = 8 lg ..+8], B^T[n = l16][k = 8 lg ..+8] of a 32-wide k slab and
 // D[m = 4 lg + r][n = l16], r < 4.
 __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
+  // A is kept as four planes, plane j % 4 holding A[i][j] at [i][j / 4] (rows of 16 + 4 pad, the
+  // planes 4 words apart in bank): the solve below reads a plane row by row, 16 bytes a read
+  constexpr int AROW = 20, APLANE = C * AROW + 4;
   __shared__ float lg_s[C], ell_s[C], bet_s[C];
   __shared__ __attribute__((aligned(16))) bf16_t Kt[DK][LDT];
   __shared__ __attribute__((aligned(16))) bf16_t Vt[DK][LDT];  // Dv <= 128 rows used
-  __shared__ __attribute__((aligned(16))) float Am[C][C + 8];  // A, later T in two bf16 parts
-  bf16_t(*Th)[LDT] = reinterpret_cast<bf16_t(*)[LDT]>(&Am[0][0]);
+  __shared__ __attribute__((aligned(16))) float Ap[4 * APLANE];  // A, later T in two bf16 parts
+  bf16_t(*Th)[LDT] = reinterpret_cast<bf16_t(*)[LDT]>(&Ap[0]);
   bf16_t(*Tl)[LDT] = Th + C;
-  static_assert(sizeof(float) * C * (C + 8) >= sizeof(bf16_t) * 2 * C * LDT, "T fits where A was");
+  static_assert(sizeof(float) * 4 * APLANE >= sizeof(bf16_t) * 2 * C * LDT, "T fits where A was");
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, lg = lane >> 4;
@@ -89,7 +97,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
     lg_s[tid] = live ? fmaxf(__logf(gv), -100.f) : 0.f;
     bet_s[tid] = live ? dm_bf2f(p.beta[(size_t)t * p.Hv + hv]) : 0.f;
   }
-  // K and V of the chunk, transposed into LDS: thread = (token tid / 4 + 64 pass.., 8-wide piece)
+  // K and V of the chunk, transposed into LDS: thread = (token, 8-wide piece)
   for (int idx = tid; idx < C * (DK / 8); idx += 256) {
     const int tok = idx / (DK / 8), pc = idx % (DK / 8);
     const int t = min(t0 + tok, p.T - 1);
@@ -113,113 +121,168 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
     ell_s[tid] = s;
     p.ell[ch * C + tid] = s;
   }
-  // K^T for the second kernel, once per key head
+  // K^T and Q for the second kernel, once per key head
   if (hv % (p.Hv / p.Hk) == 0) {
     bf16_t* dst = p.kt + ((size_t)chunk * p.Hk + hk) * DK * C;
     for (int idx = tid; idx < DK * (C / 8); idx += 256) {
-      const int r = idx / (C / 8), pc = idx % (C / 8);
-      *reinterpret_cast<bf16x8_t*>(dst + (size_t)r * C + 8 * pc) = ld8(&Kt[r][8 * pc]);
+      const int r = idx / (C / 8), pc = idx % (C / 8);  // row dk = r, tokens 8 pc ..
+      *reinterpret_cast<bf16x8_t*>(dst + ((size_t)((r >> 4) * 2 + (pc >> 2)) * 64 + (pc & 3) * 16 + (r & 15)) * 8) =
+          ld8(&Kt[r][8 * pc]);
+    }
+    bf16_t* qdst = p.qf + ((size_t)chunk * p.Hk + hk) * C * DK;
+    for (int idx = tid; idx < C * (DK / 8); idx += 256) {
+      const int tok = idx / (DK / 8), pc = idx % (DK / 8);  // row token, channels 8 pc ..
+      const int t = min(t0 + tok, p.T - 1);
+      *reinterpret_cast<bf16x8_t*>(qdst + ((size_t)((tok >> 4) * 4 + (pc >> 2)) * 64 + (pc & 3) * 16 + (tok & 15)) * 8) =
+          ld8(p.q + ((size_t)t * p.Hk + hk) * DK + 8 * pc);
     }
   }
   __syncthreads();
 
-  // ---- K K^T and Q K^T, rows 16 wave .. of the chunk; only the lower triangle is needed
+  // ---- K K^T and Q K^T for the chunk's tokens i = 16 wave + l16 (the n side of the product, so
+  // that a lane ends up with four consecutive j of one i: packed stores); lower triangle only
   {
     const int ti = min(t0 + 16 * wave + l16, p.T - 1);
-    bf16x8_t ak[4], aq[4];
+    bf16x8_t bki[4], bqi[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      ak[ks] = ld8(p.k + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
-      aq[ks] = ld8(p.q + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
+      bki[ks] = ld8(p.k + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
+      bqi[ks] = ld8(p.q + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
     }
-    bf16_t* pdst = p.pm + ch * C * C;
-    bf16_t* pdst_lo = p.pl + ch * C * C;
+    const int i = 16 * wave + l16;
+    const float ell_i = ell_s[i], bet_i = bet_s[i];
     for (int nt = 0; nt < 4; ++nt) {
       f32x4_t kk = {0.f, 0.f, 0.f, 0.f}, qk = {0.f, 0.f, 0.f, 0.f};
       if (nt <= wave) {
         const int tj = min(t0 + 16 * nt + l16, p.T - 1);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-          const bf16x8_t bk = ld8(p.k + ((size_t)tj * p.Hk + hk) * DK + 32 * ks + 8 * lg);
-          kk = mfma(ak[ks], bk, kk);
-          qk = mfma(aq[ks], bk, qk);
+          const bf16x8_t akj = ld8(p.k + ((size_t)tj * p.Hk + hk) * DK + 32 * ks + 8 * lg);
+          kk = mfma(akj, bki[ks], kk);  // [j][i]
+          qk = mfma(akj, bqi[ks], qk);
         }
       }
+      bf16_t ph[4], pl[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const int i = 16 * wave + 4 * lg + r, j = 16 * nt + l16;
-        const float e = j <= i ? __expf(ell_s[i] - ell_s[j]) : 0.f;
-        Am[i][j] = j < i ? bet_s[i] * e * kk[r] : 0.f;
-        split_bf16(e * qk[r], &pdst[(size_t)i * C + j], &pdst_lo[(size_t)i * C + j]);
+        const int j = 16 * nt + 4 * lg + r;
+        const float e = j <= i ? __expf(ell_i - ell_s[j]) : 0.f;
+        Ap[r * APLANE + i * AROW + 4 * nt + lg] = j < i ? bet_i * e * kk[r] : 0.f;
+        split_bf16(e * qk[r], &ph[r], &pl[r]);
       }
+      // element (i, j = 16 nt + 4 lg + r): tile i / 16, slab j / 32, lane (j % 32 / 8) * 16 + i % 16
+      const size_t po = ch * C * C + ((size_t)(wave * 2 + (nt >> 1)) * 64 + (2 * (nt & 1) + (lg >> 1)) * 16 + l16) * 8 + 4 * (lg & 1);
+      *reinterpret_cast<uint2*>(p.pm + po) = make_uint2(ph[0] | ((uint32_t)ph[1] << 16), ph[2] | ((uint32_t)ph[3] << 16));
+      *reinterpret_cast<uint2*>(p.pl + po) = make_uint2(pl[0] | ((uint32_t)pl[1] << 16), pl[2] | ((uint32_t)pl[3] << 16));
     }
   }
   __syncthreads();
 
-  // ---- T = (I + A)^-1 by forward substitution, one column a lane (first wavefront)
-  float t[C];
-  if (wave == 0) {
+  // ---- T = (I + A)^-1 by forward substitution. Thread (column c = tid / 4, part q4 = tid % 4)
+  // keeps T[j][c] for j = q4 mod 4; a row's sum over j is four partial sums met inside the quad.
+  const int col = tid >> 2, q4 = tid & 3;
+  float tq[C / 4];
+#pragma unroll
+  for (int m = 0; m < C / 4; ++m) tq[m] = 0.f;
+  {
+    const float* arow = &Ap[q4 * APLANE];
 #pragma unroll
     for (int i = 0; i < C; ++i) {
-      float acc = i == lane ? 1.f : 0.f;
+      float acc = 0.f;
 #pragma unroll
-      for (int j = 0; j < i; ++j) acc = dm_fma(-Am[i][j], t[j], acc);
-      t[i] = acc;
+      for (int m4 = 0; m4 < (i + 3) / 4; m4 += 4) {
+        const float4 a4 = *reinterpret_cast<const float4*>(arow + i * AROW + m4);
+        acc = dm_fma(a4.x, tq[m4], acc);
+        if (m4 + 1 < (i + 3) / 4) acc = dm_fma(a4.y, tq[m4 + 1], acc);
+        if (m4 + 2 < (i + 3) / 4) acc = dm_fma(a4.z, tq[m4 + 2], acc);
+        if (m4 + 3 < (i + 3) / 4) acc = dm_fma(a4.w, tq[m4 + 3], acc);
+      }
+      acc = acc + dm_xor_lane<1>(acc);
+      acc = acc + dm_xor_lane<2>(acc);
+      const float ti = (i == col ? 1.f : 0.f) - acc;
+      tq[i >> 2] = q4 == (i & 3) ? ti : tq[i >> 2];
     }
   }
   __syncthreads();  // A has been read; its memory becomes T
 
-  // two passes over T with its columns scaled: by beta e_j0 against K (W), by beta against V (U)
+  // two passes over T with its columns scaled: by beta e_j0 against K (W), by beta against V (U).
+  // The products are made transposed (K^T or V^T as the m side), so a lane holds four consecutive
+  // columns of one token's row and stores them in one piece.
   for (int pass = 0; pass < 2; ++pass) {
-    if (wave == 0) {
-      const float sc = pass == 0 ? bet_s[lane] * __expf(ell_s[lane]) : bet_s[lane];
+    {
+      const float sc = pass == 0 ? bet_s[col] * __expf(ell_s[col]) : bet_s[col];
 #pragma unroll
-      for (int i = 0; i < C; ++i) split_bf16(t[i] * sc, &Th[i][lane], &Tl[i][lane]);
+      for (int m = 0; m < C / 4; ++m) split_bf16(tq[m] * sc, &Th[4 * m + q4][col], &Tl[4 * m + q4][col]);
     }
     __syncthreads();
-    bf16x8_t ah[2], al[2];
+    const int i = 16 * wave + l16;
+    bf16x8_t bh[2], bl[2];
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      ah[ks] = ld8(&Th[16 * wave + l16][32 * ks + 8 * lg]);
-      al[ks] = ld8(&Tl[16 * wave + l16][32 * ks + 8 * lg]);
+      bh[ks] = ld8(&Th[i][32 * ks + 8 * lg]);
+      bl[ks] = ld8(&Tl[i][32 * ks + 8 * lg]);
     }
     const int ntiles = pass == 0 ? DK / 16 : Dv / 16;
     for (int nt = 0; nt < ntiles; ++nt) {
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
-        const bf16x8_t b = pass == 0 ? ld8(&Kt[16 * nt + l16][32 * ks + 8 * lg]) : ld8(&Vt[16 * nt + l16][32 * ks + 8 * lg]);
-        acc = mfma(ah[ks], b, acc);
-        acc = mfma(al[ks], b, acc);
-      }
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * wave + 4 * lg + r, n = 16 * nt + l16;
         if (pass == 0) {
-          bf16_t hi, lo;
-          split_bf16(-acc[r], &hi, &lo);
-          p.wh[(ch * C + i) * DK + n] = hi;
-          p.wl[(ch * C + i) * DK + n] = lo;
+          const bf16x8_t a = ld8(&Kt[16 * nt + l16][32 * ks + 8 * lg]);
+          acc = mfma(a, bh[ks], acc);  // [dk 16 nt + 4 lg + r][token i]
+          acc = mfma(a, bl[ks], acc);
         } else {
-          p.u[(ch * C + i) * Dv + n] = acc[r];
+          const bf16x8_t b = ld8(&Vt[16 * nt + l16][32 * ks + 8 * lg]);
+          acc = mfma(bh[ks], b, acc);  // [token 16 wave + 4 lg + r][dv 16 nt + l16]
+          acc = mfma(bl[ks], b, acc);
         }
+      }
+      if (pass == 0) {
+        bf16_t hi[4], lo[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) split_bf16(-acc[r], &hi[r], &lo[r]);
+        // element (i, dk = 16 nt + 4 lg + r): tile i / 16, slab dk / 32, lane (dk % 32 / 8) * 16 + i % 16
+        const size_t wo = ch * C * DK + ((size_t)(wave * 4 + (nt >> 1)) * 64 + (2 * (nt & 1) + (lg >> 1)) * 16 + l16) * 8 + 4 * (lg & 1);
+        *reinterpret_cast<uint2*>(p.wh + wo) = make_uint2(hi[0] | ((uint32_t)hi[1] << 16), hi[2] | ((uint32_t)hi[3] << 16));
+        *reinterpret_cast<uint2*>(p.wl + wo) = make_uint2(lo[0] | ((uint32_t)lo[1] << 16), lo[2] | ((uint32_t)lo[3] << 16));
+      } else {
+        // U is wanted as an accumulator tile [token][dv]: this product is made the other way round
+        // (T the m side), and a lane's four values are four tokens of one dv, one 16-byte store
+        *reinterpret_cast<float4*>(p.u + ch * C * Dv + ((size_t)(wave * (Dv / 16) + nt) * 64 + lane) * 4) =
+            make_float4(acc[0], acc[1], acc[2], acc[3]);
       }
     }
     __syncthreads();  // T's first scaling has been read before the second is written
   }
 }
 
+#ifdef ORN_TIMING
+// debug build only: phase time stamps (100 MHz wall clock) of chunk 10 of every workgroup
+__device__ long long g_chunk_marks[512][8];
+#define CH_MARK(i) do { if (threadIdx.x == 0 && chunk == 10 && blockIdx.x < 512) g_chunk_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_chunk(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_chunk_marks), sizeof(long long) * 512 * 8);
+}
+#else
+#define CH_MARK(i)
+#endif
+
 // ---- second kernel: the chunks of a head in order ------------------------------------------
-// grid (Dv / 16, Hv), 256 threads: a workgroup owns 16 rows of a head's state. Wavefront w owns
-// the chunk's tokens 16 w .. for D and Y, and the state columns 32 w .. for S.
+// 256 threads: a workgroup owns 16 rows of a head's state. Wavefront w owns the chunk's tokens
+// 16 w .. for D and Y, and the state columns 32 w .. for S. The Dv / 16 workgroups of a head read
+// the same W, P, Q, K^T, so they are placed on one XCD (workgroup ids go round the 8 XCDs, each
+// with its own L2): workgroup L sits on XCD L % 8 and takes head (L % 8) * heads_per_xcd + ...
 __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
   __shared__ __attribute__((aligned(16))) bf16_t S0h[16][LDS0], S0l[16][LDS0];
   __shared__ __attribute__((aligned(16))) bf16_t Dh[16][LDT], Dl[16][LDT], Fh[16][LDT], Fl[16][LDT];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, lg = lane >> 4;
-  const int dvb = blockIdx.x, hv = blockIdx.y, hk = hv / (p.Hv / p.Hk);
-  const int Dv = p.Dv, dv0 = dvb * 16;
+  const int Dv = p.Dv, nb = Dv / 16;
+  const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8, hpx = (p.Hv + 7) / 8;
+  const int hv = xcd * hpx + slot / nb, dvb = slot % nb;
+  if (slot / nb >= hpx || hv >= p.Hv) return;  // uniform over the workgroup
+  const int hk = hv / (p.Hv / p.Hk), dv0 = dvb * 16;
 
   f32x4_t s[2];
 #pragma unroll
@@ -228,35 +291,53 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
     for (int r = 0; r < 4; ++r)
       s[n2][r] = p.state_in[((size_t)hv * Dv + dv0 + 4 * lg + r) * DK + 16 * (2 * wave + n2) + l16];
 
-  for (int chunk = 0; chunk < p.nchunks; ++chunk) {
-    const int t0 = chunk * C;
-    const size_t ch = (size_t)chunk * p.Hv + hv;
-    const int row = 16 * wave + l16;  // this lane's token as an A-operand row
-    // operands that come straight from memory, asked for before anything waits
+  // A chunk's operands come straight from memory into registers, one chunk ahead of their use:
+  // the chunks of a head are a dependent chain, and a trip to memory inside a link would be
+  // most of its length.
+  struct Ops {
     bf16x8_t awh[4], awl[4], aq[4], ap[2], apl[2], bk[2][2];
-    const int tq = min(t0 + row, p.T - 1);
+    f32x4_t u, ellr;
+    float ell_c;
+  };
+  // in two halves, issued at different points of a chunk so that the memory pipe's work (82 KB
+  // a chunk and workgroup) runs beside the matrix products instead of ahead of them
+  auto fetch_a = [&](int chunk, Ops& o) {
+    const size_t ch = (size_t)chunk * p.Hv + hv, ck = (size_t)chunk * p.Hk + hk;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      awh[ks] = ld8(p.wh + (ch * C + row) * DK + 32 * ks + 8 * lg);
-      awl[ks] = ld8(p.wl + (ch * C + row) * DK + 32 * ks + 8 * lg);
-      aq[ks] = ld8(p.q + ((size_t)tq * p.Hk + hk) * DK + 32 * ks + 8 * lg);
+      o.awh[ks] = ld8(p.wh + ch * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
+      o.awl[ks] = ld8(p.wl + ch * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
+      o.aq[ks] = ld8(p.qf + ck * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
     }
+  };
+  auto fetch_b = [&](int chunk, Ops& o) {
+    const size_t ch = (size_t)chunk * p.Hv + hv, ck = (size_t)chunk * p.Hk + hk;
 #pragma unroll
     for (int k2 = 0; k2 < 2; ++k2) {
-      ap[k2] = ld8(p.pm + (ch * C + row) * C + 32 * k2 + 8 * lg);
-      apl[k2] = ld8(p.pl + (ch * C + row) * C + 32 * k2 + 8 * lg);
+      o.ap[k2] = ld8(p.pm + ch * C * C + ((size_t)(wave * 2 + k2) * 64 + lane) * 8);
+      o.apl[k2] = ld8(p.pl + ch * C * C + ((size_t)(wave * 2 + k2) * 64 + lane) * 8);
 #pragma unroll
       for (int n2 = 0; n2 < 2; ++n2)
-        bk[n2][k2] = ld8(p.kt + (((size_t)chunk * p.Hk + hk) * DK + 16 * (2 * wave + n2) + l16) * C + 32 * k2 + 8 * lg);
+        o.bk[n2][k2] = ld8(p.kt + ck * DK * C + ((size_t)((2 * wave + n2) * 2 + k2) * 64 + lane) * 8);
     }
-    f32x4_t d, ellr;
-    const float ell_c = p.ell[ch * C + C - 1];
+    o.ell_c = p.ell[ch * C + C - 1];
+    o.u = *reinterpret_cast<const f32x4_t*>(p.u + ch * C * Dv + ((size_t)(wave * nb + dvb) * 64 + lane) * 4);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int i = 16 * wave + 4 * lg + r;
-      d[r] = p.u[(ch * C + i) * Dv + dv0 + l16];
-      ellr[r] = p.ell[ch * C + i];
-    }
+    for (int r = 0; r < 4; ++r) o.ellr[r] = p.ell[ch * C + 16 * wave + 4 * lg + r];
+  };
+  Ops cur, nxt;
+  fetch_a(0, cur);
+  fetch_b(0, cur);
+  nxt = cur;
+  for (int chunk = 0; chunk < p.nchunks; ++chunk) {
+    const int t0 = chunk * C;
+    const bool more = chunk + 1 < p.nchunks;
+    CH_MARK(0);
+    const bf16x8_t(&awh)[4] = cur.awh, (&awl)[4] = cur.awl, (&aq)[4] = cur.aq, (&ap)[2] = cur.ap, (&apl)[2] = cur.apl;
+    const bf16x8_t(&bk)[2][2] = cur.bk;
+    f32x4_t d = cur.u;
+    const f32x4_t ellr = cur.ellr;
+    const float ell_c = cur.ell_c;
 
     // 1. the state as two bf16 parts
 #pragma unroll
@@ -265,18 +346,23 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
       for (int r = 0; r < 4; ++r)
         split_bf16(s[n2][r], &S0h[4 * lg + r][16 * (2 * wave + n2) + l16], &S0l[4 * lg + r][16 * (2 * wave + n2) + l16]);
     __syncthreads();
+    CH_MARK(1);
 
-    // 2. D = U + W S_0^T and the start of Y = diag(e_i0) Q S_0^T
-    f32x4_t yv = {0.f, 0.f, 0.f, 0.f};
+    // 2. D = U + W S_0^T and the start of Y = diag(e_i0) Q S_0^T; five accumulators, so that no
+    //    product waits for the one before it
+    if (more) fetch_a(chunk + 1, nxt);
+    f32x4_t yv = {0.f, 0.f, 0.f, 0.f}, d1 = yv, d2 = yv, y1 = yv;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       const bf16x8_t bh = ld8(&S0h[l16][32 * ks + 8 * lg]), bl = ld8(&S0l[l16][32 * ks + 8 * lg]);
       d = mfma(awh[ks], bh, d);
-      d = mfma(awh[ks], bl, d);
-      d = mfma(awl[ks], bh, d);
+      d1 = mfma(awh[ks], bl, d1);
+      d2 = mfma(awl[ks], bh, d2);
       yv = mfma(aq[ks], bh, yv);
-      yv = mfma(aq[ks], bl, yv);
+      y1 = mfma(aq[ks], bl, y1);
     }
+    d = d + (d1 + d2);
+    yv = yv + y1;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int i = 16 * wave + 4 * lg + r;
@@ -284,9 +370,12 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
       split_bf16(d[r] * __expf(ell_c - ellr[r]), &Fh[l16][i], &Fl[l16][i]);
       yv[r] *= __expf(ellr[r]);
     }
+    CH_MARK(2);
     __syncthreads();
+    CH_MARK(3);
 
     // 3. Y += P D
+    if (more) fetch_b(chunk + 1, nxt);
 #pragma unroll
     for (int k2 = 0; k2 < 2; ++k2) {
       const bf16x8_t dh = ld8(&Dh[l16][32 * k2 + 8 * lg]);
@@ -300,6 +389,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
       if (tk < p.T) p.y[((size_t)tk * p.Hv + hv) * Dv + dv0 + l16] = dm_f2bf(yv[r]);
     }
 
+    CH_MARK(4);
     // 4. S = e_C0 S + (diag(e_Cj) D)^T K
     const float gc = __expf(ell_c);
 #pragma unroll
@@ -312,7 +402,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
         s[n2] = mfma(ld8(&Fl[l16][32 * k2 + 8 * lg]), bk[n2][k2], s[n2]);
       }
     }
+    CH_MARK(5);
     __syncthreads();  // the tiles are rewritten by the next chunk
+    CH_MARK(6);
+    cur = nxt;
   }
 #pragma unroll
   for (int n2 = 0; n2 < 2; ++n2)
@@ -332,7 +425,7 @@ int gdn_chunked_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, co
   const size_t per = (size_t)n * Hv;
   void* base = nullptr;
   const size_t need = per * ((size_t)C * DK * 2 * 2 + (size_t)C * Dv * 4 + (size_t)C * C * 2 * 2 + C * 4) +
-                      (size_t)n * Hk * DK * C * 2 + 8 * 256;
+                      (size_t)n * Hk * DK * C * 2 * 2 + 10 * 256;
   int rc = ornith_scratch(ctx, need, &base);
   if (rc) return rc;
   ScratchCursor sc(base);
@@ -352,6 +445,7 @@ int gdn_chunked_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, co
   a.pl = sc.take<bf16_t>(per * C * C);
   a.ell = sc.take<float>(per * C);
   a.kt = sc.take<bf16_t>((size_t)n * Hk * DK * C);
+  a.qf = sc.take<bf16_t>((size_t)n * Hk * C * DK);
   a.T = T;
   a.Hk = Hk;
   a.Hv = Hv;
@@ -359,7 +453,7 @@ int gdn_chunked_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, co
   a.nchunks = n;
   hipLaunchKernelGGL(gdn_chunk_prep_kernel, dim3(n, Hv), dim3(256), 0, ctx->stream, a);
   ORN_LAUNCH_CHECK("gdn_chunk_prep_kernel");
-  hipLaunchKernelGGL(gdn_chunk_scan_kernel, dim3(Dv / 16, Hv), dim3(256), 0, ctx->stream, a);
+  hipLaunchKernelGGL(gdn_chunk_scan_kernel, dim3(8 * ((Hv + 7) / 8) * (Dv / 16)), dim3(256), 0, ctx->stream, a);
   ORN_LAUNCH_CHECK("gdn_chunk_scan_kernel");
   return ORNITH_OK;
 }
