@@ -48,11 +48,10 @@ struct MmArgs {
   const uint32_t* tile_start;  // [tiles] first pair
   const uint32_t* tile_count;  // [tiles] pairs in the tile (<= BM)
   const uint32_t* n_tiles;     // device scalar
+  int vec;                     // rows of y can be stored 16 bytes at a time
 };
 
-__device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)dm_f2bf(a) | ((uint32_t)dm_f2bf(b) << 16);
-}
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return dm_f2bf2(a, b); }
 
 // ---- weight slab pieces: loaded as codes into registers (so the loads of the next slab can
 // be in flight while the matrix cores work on this one), dequantized on the way into LDS ----
@@ -149,6 +148,60 @@ template <int KIND>
 struct BRegsOf { typedef BRegsQ4 type; };
 template <>
 struct BRegsOf<ORNITH_Q6K> { typedef BRegsQ6 type; };
+
+// ---- epilogue ------------------------------------------------------------------------------
+// The MFMA result has one output column per lane (D[row = 8*b + 4*(lane/32) + r][col = lane%32]
+// = acc[4*b + r]): stored from there, a tile row leaves in 2-byte pieces, 64 store instructions
+// per 32 x 32 tile. Each wavefront instead turns its own window of the tile around in LDS (the
+// slab buffers are free after the last barrier; no other wavefront touches the window, so no
+// barrier is needed) and stores 16 bytes a lane, eight lanes a 128-byte row piece. `vec`: the
+// rows of y are 16-byte aligned (O a multiple of 8); otherwise the direct 2-byte stores.
+template <int TM, int TN, bool GATHER>
+__device__ __forceinline__ void store_tile(const MmArgs& a, const f32x16_t (&acc)[TM][TN], bf16_t* cs, int row0,
+                                           int col0, int lane, int n0, int m0, int rows_here, const uint32_t* s_dst,
+                                           bool vec) {
+  constexpr int WTM = TM * 32, WTN = TN * 32, PPR = WTN / 8;
+  if (!vec) {
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int o = n0 + col0 + j * 32 + (lane & 31);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int r = row0 + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+          if (r < rows_here && o < a.O) {
+            const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
+            a.y[dst * a.O + o] = dm_f2bf(acc[i][j][e]);
+          }
+        }
+      }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      bf16_t* w = cs + (row0 + i * 32 + 4 * (lane >> 5)) * LDK + col0 + j * 32 + (lane & 31);
+#pragma unroll
+      for (int e = 0; e < 16; e += 2) {
+        const uint32_t pk = dm_f2bf2(acc[i][j][e], acc[i][j][e + 1]);
+        w[(8 * (e >> 2) + (e & 3)) * LDK] = (bf16_t)(pk & 0xffffu);
+        w[(8 * (e >> 2) + (e & 3) + 1) * LDK] = (bf16_t)(pk >> 16);
+      }
+    }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int p0 = 0; p0 < WTM * PPR; p0 += 64) {
+    const int p = p0 + lane, r = row0 + p / PPR, c = col0 + (p % PPR) * 8;
+    if (r < rows_here && n0 + c < a.O) {
+      const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
+      *reinterpret_cast<u32x4_t*>(a.y + dst * a.O + n0 + c) = *reinterpret_cast<const u32x4_t*>(cs + r * LDK + c);
+    }
+  }
+}
 
 // BM = 256: 2 x 2 wavefronts of 128 x 64; BM = 128: 2 x 2 of 64 x 64; BM = 64: 1 x 4 of 64 x 32
 template <int KIND, int BM, bool GATHER>
@@ -254,21 +307,7 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
     __syncthreads();
   }
 
-  // ---- epilogue: D[row = 8*b + 4*(lane/32) + r][col = lane%32] = acc[4*b + r]
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int o = n0 + wn * WTN + j * 32 + (lane & 31);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = wm * WTM + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-        if (r < rows_here && o < a.O) {
-          const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
-          a.y[dst * a.O + o] = dm_f2bf(acc[i][j][e]);
-        }
-      }
-    }
+  store_tile<TM, TN, GATHER>(a, acc, &As[0][0], wm * WTM, wn * WTN, lane, n0, m0, rows_here, s_dst, a.vec != 0);
 }
 
 // ---- the same GEMM with producers and consumers --------------------------------------------
@@ -499,21 +538,8 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
     __syncthreads();
   }
 
-  // ---- epilogue: D[row = 8*b + 4*(lane/32) + r][col = lane%32] = acc[4*b + r]
-#pragma unroll
-  for (int i = 0; i < TM; ++i)
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int o = n0 + wn * WTN + j * 32 + (lane & 31);
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int r = wm * WTM + i * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-        if (r < rows_here && o < a.O) {
-          const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
-          a.y[dst * a.O + o] = dm_f2bf(acc[i][j][e]);
-        }
-      }
-    }
+  static_assert(2 * LD2 >= LDK, "the tile does not fit over the slab buffers");
+  store_tile<TM, TN, GATHER>(a, acc, &As[0][0][0], wm * WTM, wn * WTN, lane, n0, m0, rows_here, s_dst, a.vec != 0);
 }
 
 // BM == 64 has two 32-row MFMA tiles per wavefront as well (TM = 2), one wavefront column
@@ -593,6 +619,7 @@ int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, 
   a.M = M;
   a.O = w->O;
   a.K = w->K;
+  a.vec = w->O % 8 == 0 && ((uintptr_t)d_y & 15) == 0;
   // 256-row tiles dequantize every weight tile half as often; 128-row tiles when that is what
   // it takes to give every compute unit a workgroup
   const int nx = (w->O + BN - 1) / BN;
@@ -660,6 +687,7 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   a.M = pairs;
   a.O = w->O;
   a.K = w->K;
+  a.vec = w->O % 8 == 0 && ((uintptr_t)d_y & 15) == 0;
   a.pair = pair;
   a.up_div = is_up ? top_k : 1;
   a.tile_expert = te;
