@@ -149,6 +149,22 @@ struct BRegsOf { typedef BRegsQ4 type; };
 template <>
 struct BRegsOf<ORNITH_Q6K> { typedef BRegsQ6 type; };
 
+#ifdef ORN_TIMING
+__device__ long long g_mm_marks[1024][8];
+__device__ long long g_mm_cyc[1024][2];
+#define MM_CYC(i) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y < 1024) g_mm_cyc[blockIdx.y][i] = clock64(); } while (0)
+extern "C" __attribute__((visibility("default"))) int ornith_debug_cyc_mm(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mm_cyc), sizeof(g_mm_cyc));
+}
+#define MM_MARK(i, cond) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y < 1024 && (cond)) g_mm_marks[blockIdx.y][i] = wall_clock64(); } while (0)
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_mm(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mm_marks), sizeof(g_mm_marks));
+}
+#else
+#define MM_MARK(i, cond)
+#define MM_CYC(i)
+#endif
+
 // ---- epilogue ------------------------------------------------------------------------------
 // The MFMA result has one output column per lane (D[row = 8*b + 4*(lane/32) + r][col = lane%32]
 // = acc[4*b + r]): stored from there, a tile row leaves in 2-byte pieces, 64 store instructions
@@ -159,7 +175,7 @@ struct BRegsOf<ORNITH_Q6K> { typedef BRegsQ6 type; };
 template <int TM, int TN, bool GATHER>
 __device__ __forceinline__ void store_tile(const MmArgs& a, const f32x16_t (&acc)[TM][TN], bf16_t* cs, int row0,
                                            int col0, int lane, int n0, int m0, int rows_here, const uint32_t* s_dst,
-                                           bool vec) {
+                                           bool vec, int ld = LDK) {
   constexpr int WTM = TM * 32, WTN = TN * 32, PPR = WTN / 8;
   if (!vec) {
 #pragma unroll
@@ -182,12 +198,12 @@ __device__ __forceinline__ void store_tile(const MmArgs& a, const f32x16_t (&acc
   for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      bf16_t* w = cs + (row0 + i * 32 + 4 * (lane >> 5)) * LDK + col0 + j * 32 + (lane & 31);
+      bf16_t* w = cs + (row0 + i * 32 + 4 * (lane >> 5)) * ld + col0 + j * 32 + (lane & 31);
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
         const uint32_t pk = dm_f2bf2(acc[i][j][e], acc[i][j][e + 1]);
-        w[(8 * (e >> 2) + (e & 3)) * LDK] = (bf16_t)(pk & 0xffffu);
-        w[(8 * (e >> 2) + (e & 3) + 1) * LDK] = (bf16_t)(pk >> 16);
+        w[(8 * (e >> 2) + (e & 3)) * ld] = (bf16_t)(pk & 0xffffu);
+        w[(8 * (e >> 2) + (e & 3) + 1) * ld] = (bf16_t)(pk >> 16);
       }
     }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -198,7 +214,7 @@ __device__ __forceinline__ void store_tile(const MmArgs& a, const f32x16_t (&acc
     const int p = p0 + lane, r = row0 + p / PPR, c = col0 + (p % PPR) * 8;
     if (r < rows_here && n0 + c < a.O) {
       const int64_t dst = GATHER ? (int64_t)s_dst[r] : (int64_t)(m0 + r);
-      *reinterpret_cast<u32x4_t*>(a.y + dst * a.O + n0 + c) = *reinterpret_cast<const u32x4_t*>(cs + r * LDK + c);
+      *reinterpret_cast<u32x4_t*>(a.y + dst * a.O + n0 + c) = *reinterpret_cast<const u32x4_t*>(cs + r * ld + c);
     }
   }
 }
@@ -542,6 +558,356 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
   store_tile<TM, TN, GATHER>(a, acc, &As[0][0][0], wm * WTM, wn * WTN, lane, n0, m0, rows_here, s_dst, a.vec != 0);
 }
 
+// ---- the gathered GEMM with the weights kept out of LDS -------------------------------------
+// A 64 x 64 wavefront tile reads 4 KB of fragments out of LDS for every four MFMAs: at the
+// matrix cores' full rate that is all the LDS bandwidth a compute unit has, so the kernels
+// above cannot pass half of the peak. Here a wavefront owns 64 output columns over ALL rows of
+// the tile (32 * TM, up to 192: an expert's whole share of a 4096-token chunk in one tile, so
+// its weights are dequantized once), and dequantizes the weights of its columns straight into
+// MFMA operand registers: a lane of v_mfma_f32_32x32x16_bf16 supplies 8 consecutive k of one
+// weight row, which is 4 bytes of Q4_K nibbles / Q6_K codes, and the order of the k steps
+// inside a slab is free as long as the activation fragments follow it. Only the activations go
+// through LDS (written once a slab, read by the four wavefronts: 32 * TM * 32 bytes per
+// 2 * TM MFMAs), and the vector work of the dequantization sits between the MFMAs of the same
+// wavefront. One wavefront a SIMD (the accumulators take 32 * TM registers), K slabs of 128.
+//
+// k step t (0..7) of a slab, lane half h: k = 32 * (t >> 1) + 16 * h + 8 * (t & 1) .. + 8.
+//   Q4_K: the slab is two 64-groups; the lane holds bytes 16h .. 16h + 16 of each (low nibbles:
+//         weights 16h + i, high nibbles: 32 + 16h + i).
+//   Q6_K: the slab is a 128-half; the lane holds positions 16h .. 16h + 16 (their weights l,
+//         l + 32, l + 64, l + 96 are quarters t >> 1 of the slab).
+struct RawQ4 {
+  u32x4_t q[2];
+  uint32_t s0, s1, s2, dmw;
+};
+struct RawQ6 {
+  u32x4_t qa, qb, qh;
+  uint32_t sc0, sc1, d;
+};
+template <int KIND>
+struct RawOf { typedef RawQ4 type; };
+template <>
+struct RawOf<ORNITH_Q6K> { typedef RawQ6 type; };
+
+// Every load of the main loop is a base the whole workgroup shares, moved from slab to slab by
+// scalar arithmetic, plus a 32-bit byte offset a lane computes once: no vector instruction is
+// spent on addresses between the MFMAs.
+struct RawOff {
+  uint32_t q, s, d;  // byte offsets of the lane's weight row in qs / scales / dm (+ 16 * h in q)
+};
+__device__ __forceinline__ RawOff raw_offsets(int kind, int64_t row, int nb, int h) {
+  RawOff o;
+  o.q = (uint32_t)(row * nb * (kind == ORNITH_Q4K ? 128 : 192) + 16 * h);
+  o.s = (uint32_t)(row * nb * (kind == ORNITH_Q4K ? 12 : 16));
+  o.d = (uint32_t)(row * nb * (kind == ORNITH_Q4K ? 4 : 2));
+  return o;
+}
+template <class V>
+__device__ __forceinline__ V ld_off(const uint8_t* base, uint32_t off) {
+  return *reinterpret_cast<const V*>(base + off);
+}
+__device__ __forceinline__ void raw_load(RawQ4& r, const MmArgs& a, const RawOff& o, int slab) {
+  const uint8_t* q = a.qs + slab * 64;
+  r.q[0] = ld_off<u32x4_t>(q, o.q);
+  r.q[1] = ld_off<u32x4_t>(q + 32, o.q);
+  const uint8_t* sc = a.scales + (slab >> 1) * 12;
+  r.s0 = ld_off<uint32_t>(sc, o.s);
+  r.s1 = ld_off<uint32_t>(sc + 4, o.s);
+  r.s2 = ld_off<uint32_t>(sc + 8, o.s);
+  r.dmw = ld_off<uint32_t>(reinterpret_cast<const uint8_t*>(a.dm) + (slab >> 1) * 4, o.d);
+}
+__device__ __forceinline__ void raw_load(RawQ6& r, const MmArgs& a, const RawOff& o, int slab) {
+  const int hh = slab & 1;
+  const uint8_t* base = a.qs + (slab >> 1) * 192;
+  r.qa = ld_off<u32x4_t>(base + 64 * hh, o.q);
+  r.qb = ld_off<u32x4_t>(base + 64 * hh + 32, o.q);
+  r.qh = ld_off<u32x4_t>(base + 128 + 32 * hh, o.q);
+  const uint8_t* sc = a.scales + slab * 8;
+  r.sc0 = ld_off<uint32_t>(sc, o.s);
+  r.sc1 = ld_off<uint32_t>(sc + 4, o.s);
+  r.d = ld_off<uint16_t>(reinterpret_cast<const uint8_t*>(a.dm) + (slab >> 1) * 2, o.d);
+}
+
+// scale and offset of the slab's four quarters (w = s * code + o)
+template <int HH>
+__device__ __forceinline__ void raw_scales(const RawQ4& r, int, float (&s)[4], float (&o)[4]) {
+  const float d = dm_h2f((f16_t)(r.dmw & 0xffffu)), dmin = dm_h2f((f16_t)(r.dmw >> 16));
+  // sub-blocks 4 * HH .. + 4: the 6-bit scales and mins, four to a word
+  uint32_t sc4, m4;
+  if constexpr (HH == 0) {
+    sc4 = r.s0 & 0x3f3f3f3fu;
+    m4 = r.s1 & 0x3f3f3f3fu;
+  } else {
+    sc4 = (r.s2 & 0x0f0f0f0fu) | ((r.s0 & 0xc0c0c0c0u) >> 2);
+    m4 = ((r.s2 >> 4) & 0x0f0f0f0fu) | ((r.s1 & 0xc0c0c0c0u) >> 2);
+  }
+  s[0] = d * dm_ubyte<0>(sc4);
+  s[1] = d * dm_ubyte<1>(sc4);
+  s[2] = d * dm_ubyte<2>(sc4);
+  s[3] = d * dm_ubyte<3>(sc4);
+  o[0] = -(dmin * dm_ubyte<0>(m4));
+  o[1] = -(dmin * dm_ubyte<1>(m4));
+  o[2] = -(dmin * dm_ubyte<2>(m4));
+  o[3] = -(dmin * dm_ubyte<3>(m4));
+}
+template <int HH>
+__device__ __forceinline__ void raw_scales(const RawQ6& r, int h, float (&s)[4], float (&o)[4]) {
+  const float d = dm_h2f((f16_t)r.d);
+  // the scale of quarter qd and lane half h is byte 2 * qd + h of the half's eight
+  const uint32_t w0 = r.sc0 >> (8 * h), w1 = r.sc1 >> (8 * h);
+  s[0] = d * (float)(int)(int8_t)(w0 & 0xffu);
+  s[1] = d * (float)(int)(int8_t)((w0 >> 16) & 0xffu);
+  s[2] = d * (float)(int)(int8_t)(w1 & 0xffu);
+  s[3] = d * (float)(int)(int8_t)((w1 >> 16) & 0xffu);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = -32.f * s[i];
+}
+
+// the two code words (four codes each) of k step T and the quarter they are scaled by
+template <int T>
+__device__ __forceinline__ void raw_codes(const RawQ4& r, uint32_t& c0, uint32_t& c1, int& quarter) {
+  constexpr int G = T >> 2, NIB = (T >> 1) & 1, W = 2 * (T & 1);
+  c0 = (r.q[G][W] >> (4 * NIB)) & 0x0f0f0f0fu;
+  c1 = (r.q[G][W + 1] >> (4 * NIB)) & 0x0f0f0f0fu;
+  quarter = 2 * G + NIB;
+}
+template <int T>
+__device__ __forceinline__ void raw_codes(const RawQ6& r, uint32_t& c0, uint32_t& c1, int& quarter) {
+  constexpr int QD = T >> 1, NIB = QD >> 1, W = 2 * (T & 1);
+  const u32x4_t& lo = (QD & 1) ? r.qb : r.qa;
+  c0 = ((lo[W] >> (4 * NIB)) & 0x0f0f0f0fu) | (((r.qh[W] >> (2 * QD)) & 0x03030303u) << 4);
+  c1 = ((lo[W + 1] >> (4 * NIB)) & 0x0f0f0f0fu) | (((r.qh[W + 1] >> (2 * QD)) & 0x03030303u) << 4);
+  quarter = QD;
+}
+template <int T, class Raw>
+__device__ __forceinline__ bf16x8_t raw_fragment(const Raw& r, const float (&s)[4], const float (&o)[4]) {
+  uint32_t c0, c1;
+  int qd;
+  raw_codes<T>(r, c0, c1, qd);
+  u32x4_t f;
+#ifdef ORN_NODEQ
+  f[0] = c0; f[1] = c1; f[2] = c0 ^ __float_as_uint(s[qd]); f[3] = c1 ^ __float_as_uint(o[qd]);
+  return __builtin_bit_cast(bf16x8_t, f);
+#endif
+  f[0] = pack2(dm_fma(s[qd], dm_ubyte<0>(c0), o[qd]), dm_fma(s[qd], dm_ubyte<1>(c0), o[qd]));
+  f[1] = pack2(dm_fma(s[qd], dm_ubyte<2>(c0), o[qd]), dm_fma(s[qd], dm_ubyte<3>(c0), o[qd]));
+  f[2] = pack2(dm_fma(s[qd], dm_ubyte<0>(c1), o[qd]), dm_fma(s[qd], dm_ubyte<1>(c1), o[qd]));
+  f[3] = pack2(dm_fma(s[qd], dm_ubyte<2>(c1), o[qd]), dm_fma(s[qd], dm_ubyte<3>(c1), o[qd]));
+  return __builtin_bit_cast(bf16x8_t, f);
+}
+
+constexpr int RN = 256;  // output columns of a workgroup of the register form
+
+constexpr int RM = 192;  // most rows of a tile of the register form
+
+// the main loop and the epilogue for a tile of up to 32 * TM rows
+template <int KIND, int TM, bool GATHER>
+__device__ __forceinline__ void reg_tile(const MmArgs& a, bf16_t (*As)[RM][LDK], const uint32_t* s_src,
+                                         const uint32_t* s_dst, int rows_here, int m0, int64_t wrow0) {
+  constexpr int BM = 32 * TM, TN = 2;
+  constexpr int NA = BM * 16 / 256;  // 16-byte pieces of an activation slab per thread
+  typedef typename RawOf<KIND>::type Raw;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, l32 = lane & 31, h = lane >> 5;
+  const int n0 = blockIdx.x * RN;
+  const int nb = a.K >> 8, nslab = a.K / BK;  // an even number of slabs
+  MM_MARK(5, true);
+  MM_CYC(0);
+
+  RawOff boff[TN];
+#pragma unroll
+  for (int j = 0; j < TN; ++j) boff[j] = raw_offsets(KIND, wrow0 + min(n0 + wave * 64 + j * 32 + l32, a.O - 1), nb, h);
+  uint32_t aoff[NA];
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    const int idx = tid + 256 * i, r = idx >> 4, c8 = idx & 15;
+    // rows past the end of the tile read a valid row: what they produce is never stored
+    const int64_t src = GATHER ? (int64_t)s_src[r] : (int64_t)min(m0 + r, a.M - 1);
+    aoff[i] = (uint32_t)((src * a.K + 8 * c8) * 2);
+  }
+  // Registers of a slab's way in: activations of slab k travel in areg[k & 1] (asked for two
+  // slabs ahead, written to LDS buffer k & 1 one slab ahead), codes in raw[k & 1] (asked for one
+  // slab ahead), scales in sc / of [k & 1].
+  u32x4_t areg[2][NA];
+  Raw raw[2][TN];
+  float sc[2][TN][4], of[2][TN][4];
+  auto fetch_a1 = [&](auto set, auto piece, int slab) {
+    constexpr int S = decltype(set)::value, I = decltype(piece)::value;
+    areg[S][I] = ld_off<u32x4_t>(reinterpret_cast<const uint8_t*>(a.x) + slab * (BK * 2), aoff[I]);
+  };
+  auto fetch_a = [&](auto set, int slab) {
+#define ORN_FETCH_A(I) if constexpr (NA > I) fetch_a1(set, std::integral_constant<int, (I < NA ? I : 0)>{}, slab)
+    ORN_FETCH_A(0); ORN_FETCH_A(1); ORN_FETCH_A(2); ORN_FETCH_A(3); ORN_FETCH_A(4); ORN_FETCH_A(5);
+    ORN_FETCH_A(6); ORN_FETCH_A(7); ORN_FETCH_A(8); ORN_FETCH_A(9); ORN_FETCH_A(10); ORN_FETCH_A(11);
+#undef ORN_FETCH_A
+  };
+  auto write_a = [&](auto set, auto piece) {
+    constexpr int S = decltype(set)::value, I = decltype(piece)::value;
+    const int idx = tid + 256 * I;
+    *reinterpret_cast<u32x4_t*>(&As[S][idx >> 4][8 * (idx & 15)]) = areg[S][I];
+  };
+  auto fetch_b = [&](auto set, int slab) {
+    constexpr int S = decltype(set)::value;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) raw_load(raw[S][j], a, boff[j], slab);
+  };
+  auto scales = [&](auto set) {
+    constexpr int S = decltype(set)::value;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) raw_scales<S>(raw[S][j], h, sc[S][j], of[S][j]);
+  };
+
+  f32x16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  bf16x8_t af[2][TM], bfr[2][TN];
+  // operands of k step T of the slab in set S into fragment set T & 1
+  auto frags = [&](auto set, auto tc) {
+    constexpr int S = decltype(set)::value, T = decltype(tc)::value;
+    const int kc = 32 * (T >> 1) + 16 * h + 8 * (T & 1);
+#pragma unroll
+    for (int i = 0; i < TM; ++i) af[T & 1][i] = *reinterpret_cast<const bf16x8_t*>(&As[S][i * 32 + l32][kc]);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bfr[T & 1][j] = raw_fragment<T>(raw[S][j], sc[S][j], of[S][j]);
+  };
+  auto mfmas = [&](auto tc) {
+    constexpr int T = decltype(tc)::value;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[T & 1][i], bfr[T & 1][j], acc[i][j], 0, 0, 0);
+  };
+  // issue order of a step: the LDS reads first, then every MFMA followed by its share of the
+  // step's other work (VALU: dequantization; LDS writes; global loads), which then runs in the
+  // shadow of the matrix core
+  auto order = [&](auto valu, auto dsw, auto vmem) {
+    __builtin_amdgcn_sched_group_barrier(0x100, TM, 0);
+#pragma unroll
+    for (int m = 0; m < TM * TN; ++m) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, decltype(valu)::value, 0);
+      if (m < decltype(dsw)::value) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      if (m < decltype(vmem)::value) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  using P0 = std::integral_constant<int, 0>;
+  using P1 = std::integral_constant<int, 1>;
+  constexpr int VQ = (52 + TM * TN - 1) / (TM * TN);  // vector instructions of a step's dequantization per MFMA
+
+  // slab s (parity: its LDS buffer and register sets). On entry fragment set 0 holds step 0.
+  auto slab = [&](auto par, int s) {
+    constexpr int HH = decltype(par)::value;
+    using Other = std::integral_constant<int, HH ^ 1>;
+    // (past the last slab the last one is asked for and written again, to no effect: loads and
+    // stores under a condition would make the compiler wait for everything in flight)
+    MM_MARK(0, s == 2);
+    // step 0: ask for the codes of slab s + 1
+    fetch_b(Other{}, min(s + 1, nslab - 1));
+    frags(par, std::integral_constant<int, 1>{});
+    mfmas(std::integral_constant<int, 0>{});
+    order(std::integral_constant<int, VQ>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, TM * TN>{});
+    MM_MARK(1, s == 2);
+    // steps 1 .. 6: the activations of slab s + 1 go from their registers to the other buffer,
+    // and those of slab s + 2 are asked for, a few pieces a step (all loads of a slab in one
+    // step fill the memory pipe's queue, and the wavefront stands still until it has drained)
+    const int s2 = min(s + 2, nslab - 1);
+    auto mid = [&](auto tc) {
+      constexpr int T = decltype(tc)::value;
+      constexpr int W0 = (T - 1) * NA / 6, W1 = T * NA / 6;
+      frags(par, std::integral_constant<int, T + 1>{});
+      mfmas(tc);
+      if constexpr (W1 - W0 >= 1) write_a(Other{}, std::integral_constant<int, W0>{});
+      if constexpr (W1 - W0 >= 2) write_a(Other{}, std::integral_constant<int, W0 + 1>{});
+      if constexpr (W1 - W0 >= 3) write_a(Other{}, std::integral_constant<int, W0 + 2>{});
+      if constexpr (W1 - W0 >= 1) fetch_a1(par, std::integral_constant<int, W0>{}, s2);
+      if constexpr (W1 - W0 >= 2) fetch_a1(par, std::integral_constant<int, W0 + 1>{}, s2);
+      if constexpr (W1 - W0 >= 3) fetch_a1(par, std::integral_constant<int, W0 + 2>{}, s2);
+      static_assert(W1 - W0 <= 3, "more activation pieces a step than written");
+      order(std::integral_constant<int, VQ>{}, std::integral_constant<int, W1 - W0>{}, std::integral_constant<int, W1 - W0>{});
+    };
+    mid(std::integral_constant<int, 1>{});
+    mid(std::integral_constant<int, 2>{});
+    mid(std::integral_constant<int, 3>{});
+    mid(std::integral_constant<int, 4>{});
+    mid(std::integral_constant<int, 5>{});
+    mid(std::integral_constant<int, 6>{});
+    MM_MARK(2, s == 2);
+    // every read of this slab's buffer has been issued, slab s + 1 is in the other one
+    __syncthreads();
+    MM_MARK(3, s == 2);
+    // step 7: scales and step 0 of slab s + 1
+    scales(Other{});
+    frags(Other{}, std::integral_constant<int, 0>{});
+    mfmas(std::integral_constant<int, 7>{});
+    order(std::integral_constant<int, (52 + 40 + TM * TN - 1) / (TM * TN)>{}, std::integral_constant<int, 0>{},
+          std::integral_constant<int, 0>{});
+    MM_MARK(4, s == 2);
+  };
+
+  fetch_a(P0{}, 0);
+  fetch_b(P0{}, 0);
+  fetch_a(P1{}, 1);
+#define ORN_WRITE_A(I) if constexpr (NA > I) write_a(P0{}, std::integral_constant<int, (I < NA ? I : 0)>{})
+  ORN_WRITE_A(0); ORN_WRITE_A(1); ORN_WRITE_A(2); ORN_WRITE_A(3); ORN_WRITE_A(4); ORN_WRITE_A(5);
+  ORN_WRITE_A(6); ORN_WRITE_A(7); ORN_WRITE_A(8); ORN_WRITE_A(9); ORN_WRITE_A(10); ORN_WRITE_A(11);
+#undef ORN_WRITE_A
+  static_assert(NA <= 12, "more activation pieces a thread than written");
+  __syncthreads();
+  scales(P0{});
+  frags(P0{}, std::integral_constant<int, 0>{});
+  __builtin_amdgcn_sched_barrier(0);
+  for (int s = 0; s < nslab; s += 2) {
+    slab(P0{}, s);
+    slab(P1{}, s + 1);
+  }
+  __syncthreads();  // the fragments of a slab past the end were read out of the buffers the output tile goes over
+  MM_MARK(6, true);
+  MM_CYC(1);
+  store_tile<TM, TN, GATHER>(a, acc, &As[0][0][0], 0, wave * 64, lane, n0, m0, rows_here, s_dst, a.vec != 0, RN + 8);
+  MM_MARK(7, true);
+}
+
+// One kernel for every tile height: a tile runs the loop compiled for the number of 32-row
+// MFMA tiles it really has (an expert with few pairs does not pay for the widest tile).
+template <int KIND, bool GATHER>
+__global__ __launch_bounds__(256) void kq_mm_reg_kernel(MmArgs a) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][RM][LDK];
+  __shared__ uint32_t s_src[RM], s_dst[RM];
+  static_assert(2 * LDK >= RN + 8, "the output tile does not fit over the slab buffers");
+  const int tid = threadIdx.x;
+  int rows_here, m0 = 0;
+  int64_t wrow0 = 0;
+  if constexpr (GATHER) {
+    if (blockIdx.y >= *a.n_tiles) return;
+    const uint32_t e = a.tile_expert[blockIdx.y], st = a.tile_start[blockIdx.y];
+    rows_here = min((int)a.tile_count[blockIdx.y], RM);
+    wrow0 = (int64_t)e * a.O;
+    for (int r = tid; r < RM; r += 256) {
+      const uint32_t p = r < rows_here ? a.pair[st + r] : 0u;
+      s_src[r] = p / (uint32_t)a.up_div;
+      s_dst[r] = p;
+    }
+    __syncthreads();
+  } else {
+    m0 = blockIdx.y * RM;
+    rows_here = min(RM, a.M - m0);
+  }
+  switch ((rows_here + 31) >> 5) {
+    case 1: reg_tile<KIND, 1, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
+    case 2: reg_tile<KIND, 2, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
+    case 3: reg_tile<KIND, 3, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
+    case 4: reg_tile<KIND, 4, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
+    case 5: reg_tile<KIND, 5, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
+    default: reg_tile<KIND, 6, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
+  }
+}
+
 // BM == 64 has two 32-row MFMA tiles per wavefront as well (TM = 2), one wavefront column
 static_assert(BN == 128 && BK == 128, "tile constants are baked into the index arithmetic");
 
@@ -669,10 +1035,20 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   uint32_t* ts = pc.take<uint32_t>(tiles_max);
   uint32_t* tc = pc.take<uint32_t>(tiles_max);
   uint32_t* nt = pc.take<uint32_t>(1);
-  // rows per tile: an expert's weight tile is dequantized once per tile, so with about 96 or
-  // more rows an expert on average the 128-row tile halves that work (the choice depends only
-  // on pairs and E, so the calls sharing a plan agree on it)
-  const int tile_rows = pairs / w->E >= 96 ? 128 : 64;
+  // rows per tile (the choice depends only on pairs and E, so the calls sharing a plan agree on
+  // it). Register form: the smallest of 96 / 128 / 160 / 192 rows that holds an expert's share
+  // of the pairs with 2.5 standard deviations to spare, so that nearly every expert is one
+  // tile and its weights are dequantized once. Below about 48 rows an expert, with offsets that
+  // do not fit 32 bits, and with the option off, the LDS form: 128-row tiles from 96 rows an
+  // expert on average, else 64.
+  const int avg = pairs / w->E;
+  int spare = 0;
+  while (4 * spare * spare < 25 * avg) ++spare;
+  const size_t x_bytes = (size_t)(is_up ? pairs / top_k : pairs) * w->K * 2;
+  const size_t q_bytes = (size_t)w->E * w->O * (w->K / 256) * (w->kind == ORNITH_Q4K ? 128 : 192);
+  const bool reg = ornith_option_gemm_reg() && avg >= 48 && x_bytes < (size_t(1) << 32) && q_bytes < (size_t(1) << 32);
+  const int need = avg + spare;
+  const int tile_rows = reg ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : avg >= 96 ? 128 : 64;
   if (rebuild_plan) {
     hipLaunchKernelGGL(moe_sort_pairs_kernel, dim3(1), dim3(1024), 0, ctx->stream, d_inds, pairs, w->E,
                        tile_rows, pair, te, ts, tc, nt);
@@ -694,6 +1070,15 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   a.tile_start = ts;
   a.tile_count = tc;
   a.n_tiles = nt;
+  if (reg) {
+    const dim3 rgrid((w->O + RN - 1) / RN, (unsigned)tiles_max);
+    if (w->kind == ORNITH_Q4K)
+      hipLaunchKernelGGL((kq_mm_reg_kernel<ORNITH_Q4K, true>), rgrid, dim3(256), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((kq_mm_reg_kernel<ORNITH_Q6K, true>), rgrid, dim3(256), 0, ctx->stream, a);
+    ORN_LAUNCH_CHECK("kq_mm_reg_kernel<gather>");
+    return ORNITH_OK;
+  }
   const dim3 grid((w->O + BN - 1) / BN, (unsigned)tiles_max);
   if (tile_rows == 128) {
     if (w->kind == ORNITH_Q4K)

@@ -104,6 +104,7 @@ int ornith_option_fuse_moe();
 int ornith_option_fuse_proj();
 int ornith_option_fuse_gdn();
 int ornith_option_fuse_norm();
+int ornith_option_gemm_reg();  // 1: expert-gathered prefill GEMM with the weights dequantized into MFMA operand registers; 0: through LDS
 int ornith_option_gemm_duo();  // 1: prefill GEMM with producer and consumer wavefronts; 0: every wavefront does both in turn
 int ornith_option_kq_iters();      // output rows per wavefront pass of the mat-vec kernels; 0 = by shape
 int ornith_option_moe_up_iters();  // rows per wavefront of the fused gate+up kernel; 0 = by shape
