@@ -174,6 +174,60 @@ __global__ void embedding4_kernel(const uint8_t* w, const bf16_t* scales, const 
   out[(size_t)r * K + i] = dm_f2bf(dm_rb(q * s) + b);
 }
 
+// ---- dense bf16 at prefill widths: a small GEMM on the matrix cores -------------------
+// y[M, O] = x[M, K] . W[O, K]^T for the narrow dense projections (the gated-delta a / b heads,
+// the shared expert's gate: O of 1 .. 64): as mat-vecs every activation row is read by O / 4
+// workgroups. One workgroup = 16 rows; its four wavefronts split K and add up through LDS; a
+// wavefront feeds v_mfma_f32_16x16x32_bf16 straight from global memory (A: 16 rows x 32
+// channels, B: 16 outputs x 32 channels, 16 bytes a lane each). grid.y covers O in 64s.
+typedef __bf16 dmm_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float dmm_f32x4_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void dense_mm_kernel(const bf16_t* w, const bf16_t* x, bf16_t* y, int M, int O,
+                                                       int K) {
+  __shared__ float red[3][4][64][4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l16 = lane & 15, lg = lane >> 4;
+  const int row0 = blockIdx.x * 16, o0 = blockIdx.y * 64;
+  const int kw = K / 4, k0 = wave * kw;  // K is a multiple of 128
+  const bf16_t* xp = x + (size_t)min(row0 + l16, M - 1) * K + k0 + 8 * lg;
+  const bf16_t* wp[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) wp[nt] = w + (size_t)min(o0 + nt * 16 + l16, O - 1) * K + k0 + 8 * lg;
+  const int nts = min(4, (O - o0 + 15) / 16);
+  dmm_f32x4_t acc[4];
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) acc[nt] = dmm_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+  for (int k = 0; k < kw; k += 32) {
+    const dmm_bf16x8_t a = *reinterpret_cast<const dmm_bf16x8_t*>(xp + k);
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+      if (nt < nts) {
+        const dmm_bf16x8_t b = *reinterpret_cast<const dmm_bf16x8_t*>(wp[nt] + k);
+        acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nt], 0, 0, 0);
+      }
+  }
+  if (wave > 0) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave - 1][nt][lane][r] = acc[nt][r];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  // D[m = 4 * lg + r][n = l16]
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int o = o0 + nt * 16 + l16;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int row = row0 + 4 * lg + r;
+      const float v = ((acc[nt][r] + red[0][nt][lane][r]) + red[1][nt][lane][r]) + red[2][nt][lane][r];
+      if (nt < nts && o < O && row < M) y[(size_t)row * O + o] = dm_f2bf(v);
+    }
+  }
+}
+
 template <bool GATHER>
 int launch_dense(ornith_ctx* ctx, const DenseSegs& s, const void* d_x, int K, int E, int x_rows,
                  const uint32_t* d_lhs, const uint32_t* d_rhs, int rows) {
@@ -242,6 +296,13 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
       ORN_REQUIRE(w->d_w, "linear_matmul: dense weight missing");
       ORN_REQUIRE(w->K % 8 == 0 && w->O >= 1 && M <= 65535, "linear_matmul: dense O=%d K=%d", w->O,
                   w->K);
+      // prefill widths (outside the exact window, like the k-quant GEMM): on the matrix cores
+      if (M >= kPrefillRows && w->K % 128 == 0 && ((uintptr_t)d_x & 15) == 0 && ((uintptr_t)w->d_w & 15) == 0) {
+        hipLaunchKernelGGL(dense_mm_kernel, dim3((M + 15) / 16, (w->O + 63) / 64), dim3(256), 0, ctx->stream,
+                           (const bf16_t*)w->d_w, (const bf16_t*)d_x, (bf16_t*)d_y, M, w->O, w->K);
+        ORN_LAUNCH_CHECK("dense_mm_kernel");
+        return ORNITH_OK;
+      }
       {
         DenseSegs s{};
         s.n = 1;

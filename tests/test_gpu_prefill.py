@@ -264,3 +264,26 @@ def test_model_forward_at_the_reference_chunk_width(orn, ctx):
     rel = np.linalg.norm(g - w, axis=1) / np.linalg.norm(w, axis=1)
     assert np.median(rel) < 0.003 and (rel <= 0.02).mean() >= 0.95, (float(np.median(rel)), float(rel.max()))
     for o in (a, b, model, ws): o.close()
+
+
+@pytest.mark.parametrize("O,K,M", [(32, 2048, 4096), (1, 2048, 300), (48, 256, 33), (130, 512, 77), (64, 128, 32)])
+def test_dense_matmul_vs_float64(orn, ctx, O, K, M):
+    """narrow dense bf16 projections at prefill widths run as a small matrix-core GEMM (rows split
+    over workgroups, K over a workgroup's wavefronts); reference: float64 over the same bf16 values"""
+    rng = np.random.default_rng(O + K + M)
+    hl = util.HostLinear.dense(rng, O, K)
+    lin = hl.dev(orn, ctx)
+    xb = util.bf16_normal(rng, (M, K))
+    dx, dy = ctx.to_device(xb), ctx.alloc(M * O * 2)
+    ctx.memset(dy, 0xFF, M * O * 2)
+    ctx.linear_matmul(lin, dx, M, dy)
+    got = dy.download(np.uint16, (M, O))
+    want = util.bf16_to_f32(xb).astype(np.float64) @ util.bf16_to_f32(hl.w).astype(np.float64).T
+    _check(got, want, K, (O, K, M))
+    # rows inside the exact window keep the mat-vec path: bit-equal to it row by row
+    dy1 = ctx.alloc(4 * O * 2)
+    ctx.linear_matmul(lin, dx, 4, dy1)
+    mv = util.bf16_to_f32(dy1.download(np.uint16, (4, O))).astype(np.float64)
+    assert np.max(np.abs(mv - util.bf16_to_f32(got[:4]).astype(np.float64))) <= 2.0 ** -7 * np.abs(mv).max() + 1e-3
+    for b in (dx, dy, dy1): b.free()
+    lin.free()
