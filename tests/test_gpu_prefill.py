@@ -100,7 +100,9 @@ def _rows_close(got_bits, want_bits, tol):
     return np.linalg.norm(g - w, axis=1) / (np.linalg.norm(w, axis=1) + 1e-30) <= tol
 
 
-@pytest.mark.parametrize("H,E,I,T", [(512, 64, 256, 48), (2048, 256, 512, 160)])
+@pytest.mark.parametrize("H,E,I,T", [(512, 64, 256, 48), (2048, 256, 512, 160),
+                                     # 64 and 150 rows an expert: the gathered GEMM's register form
+                                     (512, 64, 256, 512), (512, 64, 256, 1200)])
 def test_moe_block_prefill_width_close_to_exact_path(orn, ctx, H, E, I, T):
     """At prefill width the block runs as GEMMs. Against the oracle's exact path the rows agree
     to 2 % relative L2 (bf16 weights on the matrix cores, fp32 sums in another order); a row
