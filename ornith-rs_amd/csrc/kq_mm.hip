@@ -49,7 +49,33 @@ struct MmArgs {
   const uint32_t* tile_count;  // [tiles] pairs in the tile (<= BM)
   const uint32_t* n_tiles;     // device scalar
   int vec;                     // rows of y can be stored 16 bytes at a time
+  // further matrices of the same kind and K over the same activations (plain form): the
+  // workgroups from column block bx0 on belong to segment i
+  struct Seg {
+    const uint8_t* qs;
+    const uint8_t* scales;
+    const uint16_t* dm;
+    bf16_t* y;
+    int O, bx0;
+  } seg[3];
+  int nseg;
 };
+
+// the matrix a workgroup of the plain form works on; returns its column block there
+__device__ __forceinline__ int pick_segment(MmArgs& a) {
+  int bx = blockIdx.x;
+#pragma unroll
+  for (int i = 0; i < 3; ++i)
+    if (i < a.nseg && (int)blockIdx.x >= a.seg[i].bx0) {
+      a.qs = a.seg[i].qs;
+      a.scales = a.seg[i].scales;
+      a.dm = a.seg[i].dm;
+      a.y = a.seg[i].y;
+      a.O = a.seg[i].O;
+      bx = (int)blockIdx.x - a.seg[i].bx0;
+    }
+  return bx;
+}
 
 __device__ __forceinline__ uint32_t pack2(float a, float b) { return dm_f2bf2(a, b); }
 
@@ -232,7 +258,7 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-  const int n0 = blockIdx.x * BN;
+  const int n0 = (GATHER ? (int)blockIdx.x : pick_segment(a)) * BN;
   const int nb = a.K >> 8;
 
   int rows_here, m0 = 0;
@@ -420,7 +446,7 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
   __shared__ uint32_t s_src[BM], s_dst[BM];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * BN;
+  const int n0 = (GATHER ? (int)blockIdx.x : pick_segment(a)) * BN;
   const int nb = a.K >> 8;
   const int nslab = a.K / BK2;  // K is a multiple of 256: a multiple of four slabs
 
@@ -969,36 +995,52 @@ int check(const ornith_kmatrix* w, const char* who) {
 
 extern "C" {
 
-int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int M, void* d_y) {
-  ORN_REQUIRE(ctx && d_x && d_y, "kq_matmul: null argument");
-  int rc = check(w, "kq_matmul");
-  if (rc) return rc;
-  ORN_REQUIRE(w->E == 1, "kq_matmul: stacked matrix (use kq_gather_matmul)");
+// Up to four matrices of one kind and K over the same activations in one launch (the
+// projections that share an input: narrow ones alone leave compute units without a workgroup)
+int ornith_kq_matmul_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n, const void* d_x, int M,
+                           void* const* d_ys) {
+  ORN_REQUIRE(ctx && ws && d_x && d_ys && n >= 1 && n <= 4, "kq_matmul: bad argument");
   ORN_REQUIRE(M >= 1, "kq_matmul: M=%d", M);
   ORN_REQUIRE(((uintptr_t)d_x & 15) == 0, "kq_matmul: x must be 16-byte aligned");
   MmArgs a{};
-  a.qs = (const uint8_t*)w->d_qs;
-  a.scales = (const uint8_t*)w->d_scales;
-  a.dm = (const uint16_t*)w->d_dm;
+  int nx = 0;
+  a.vec = 1;
+  for (int i = 0; i < n; ++i) {
+    ORN_REQUIRE(ws[i] && d_ys[i], "kq_matmul: null entry %d", i);
+    int rc = check(ws[i], "kq_matmul");
+    if (rc) return rc;
+    ORN_REQUIRE(ws[i]->E == 1, "kq_matmul: stacked matrix (use kq_gather_matmul)");
+    ORN_REQUIRE(ws[i]->kind == ws[0]->kind && ws[i]->K == ws[0]->K, "kq_matmul: matrices of one launch differ in kind or K");
+    a.vec = a.vec && ws[i]->O % 8 == 0 && ((uintptr_t)d_ys[i] & 15) == 0;
+    if (i == 0) {
+      a.qs = (const uint8_t*)ws[0]->d_qs;
+      a.scales = (const uint8_t*)ws[0]->d_scales;
+      a.dm = (const uint16_t*)ws[0]->d_dm;
+      a.y = (bf16_t*)d_ys[0];
+      a.O = ws[0]->O;
+    } else {
+      a.seg[i - 1] = {(const uint8_t*)ws[i]->d_qs, (const uint8_t*)ws[i]->d_scales, (const uint16_t*)ws[i]->d_dm,
+                      (bf16_t*)d_ys[i], ws[i]->O, nx};
+    }
+    nx += (ws[i]->O + BN - 1) / BN;
+  }
+  a.nseg = n - 1;
   a.x = (const bf16_t*)d_x;
-  a.y = (bf16_t*)d_y;
   a.M = M;
-  a.O = w->O;
-  a.K = w->K;
-  a.vec = w->O % 8 == 0 && ((uintptr_t)d_y & 15) == 0;
+  a.K = ws[0]->K;
+  const int kind = ws[0]->kind;
   // 256-row tiles dequantize every weight tile half as often; 128-row tiles when that is what
   // it takes to give every compute unit a workgroup
-  const int nx = (w->O + BN - 1) / BN;
   const bool big = M >= 256 && (long)nx * ((M + 255) / 256) >= ctx->compute_units;
   const dim3 grid(nx, big ? (M + 255) / 256 : (M + 127) / 128);
   // the 256-row tile runs in its producer / consumer form (the smaller tiles measured no
   // faster that way: they have too few MFMAs a slab)
   if (big && ornith_option_gemm_duo()) {
-    if (w->kind == ORNITH_Q4K)
+    if (kind == ORNITH_Q4K)
       hipLaunchKernelGGL((kq_mm_duo_kernel<ORNITH_Q4K, 256, false>), grid, dim3(512), 0, ctx->stream, a);
     else
       hipLaunchKernelGGL((kq_mm_duo_kernel<ORNITH_Q6K, 256, false>), grid, dim3(512), 0, ctx->stream, a);
-  } else if (w->kind == ORNITH_Q4K) {
+  } else if (kind == ORNITH_Q4K) {
     if (big)
       hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 256, false>), grid, dim3(256), 0, ctx->stream, a);
     else
@@ -1011,6 +1053,11 @@ int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, 
   }
   ORN_LAUNCH_CHECK("kq_mm_kernel");
   return ORNITH_OK;
+}
+
+int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, int M, void* d_y) {
+  ORN_REQUIRE(w && d_y, "kq_matmul: null argument");
+  return ornith_kq_matmul_multi(ctx, &w, 1, d_x, M, &d_y);
 }
 
 // gather plan: expert-sorted pairs and the tile list, in caller-provided device memory

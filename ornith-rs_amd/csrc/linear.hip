@@ -341,9 +341,27 @@ int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, 
     }
     return launch_dense<false>(ctx, s, d_x, ws[0]->K, 1, M, nullptr, nullptr, M);
   }
-  for (int i = 0; i < n; ++i) {
-    int rc = ornith_linear_matmul(ctx, ws[i], d_x, M, d_ys[i]);
+  // prefill widths: runs of k-quant matrices of one kind and K share a GEMM launch
+  for (int i = 0; i < n;) {
+    int j = i + 1;
+    if (M >= kPrefillRows && ornith_option_fuse_proj() && ws[i]->mode == ORNITH_LIN_KQUANT) {
+      while (j < n && j - i < 4 && ws[j]->mode == ORNITH_LIN_KQUANT && ws[j]->km.kind == ws[i]->km.kind &&
+             ws[j]->K == ws[i]->K)
+        ++j;
+    }
+    int rc;
+    if (j - i >= 2) {
+      const ornith_kmatrix* kms[4];
+      for (int t = i; t < j; ++t) {
+        ORN_REQUIRE(ws[t]->km.O == ws[t]->O && ws[t]->km.K == ws[t]->K, "linear_matmul_multi: k-quant dims disagree");
+        kms[t - i] = &ws[t]->km;
+      }
+      rc = ornith_kq_matmul_multi(ctx, kms, j - i, d_x, M, d_ys + i);
+    } else {
+      rc = ornith_linear_matmul(ctx, ws[i], d_x, M, d_ys[i]);
+    }
     if (rc) return rc;
+    i = j;
   }
   return ORNITH_OK;
 }

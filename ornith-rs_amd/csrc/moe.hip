@@ -185,8 +185,11 @@ int moe_block_prefill(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
   TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
   TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
   TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
-  TRY(ornith_linear_matmul(ctx, &w->sh_gate, d_x, T, sg));
-  TRY(ornith_linear_matmul(ctx, &w->sh_up, d_x, T, su));
+  {
+    const ornith_linear* gu[2] = {&w->sh_gate, &w->sh_up};
+    void* ygu[2] = {sg, su};
+    TRY(ornith_linear_matmul_multi(ctx, gu, 2, d_x, T, ygu));
+  }
   TRY(ornith_swiglu(ctx, sg, su, (int64_t)T * SI, sact));
   TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
   TRY(ornith_kq_gather_matmul(ctx, &w->ex_gate, d_x, inds, pairs, k, 1, plan, 1, xg));

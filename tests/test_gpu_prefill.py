@@ -289,3 +289,25 @@ def test_dense_matmul_vs_float64(orn, ctx, O, K, M):
     assert np.max(np.abs(mv - util.bf16_to_f32(got[:4]).astype(np.float64))) <= 2.0 ** -7 * np.abs(mv).max() + 1e-3
     for b in (dx, dy, dy1): b.free()
     lin.free()
+
+
+@pytest.mark.parametrize("kind,Os,K,M", [(Q4K, (512, 512), 2048, 4096), (Q6K, (8192, 200, 512), 512, 300),
+                                         (Q4K, (256, 128, 384, 512), 256, 77)])
+def test_projections_sharing_an_input_share_a_gemm_launch(orn, ctx, kind, Os, K, M):
+    """linear_matmul_multi at prefill width: k-quant matrices of one kind and K run as column
+    ranges of one GEMM launch; every output equals the matrix's own launch bit for bit (an output
+    element is one dot product in a fixed k order, whatever tile computes it)"""
+    rng = np.random.default_rng(sum(Os) + K + M)
+    hls = [util.HostLinear.kq(rng, kind, O, K) for O in Os]
+    lins = [h.dev(orn, ctx) for h in hls]
+    xb = util.bf16_normal(rng, (M, K))
+    dx = ctx.to_device(xb)
+    ys = [ctx.alloc(M * O * 2) for O in Os]
+    for y, O in zip(ys, Os): ctx.memset(y, 0xFF, M * O * 2)
+    ctx.linear_matmul_multi(lins, dx, M, ys)
+    y1 = ctx.alloc(M * max(Os) * 2)
+    for lin, y, O in zip(lins, ys, Os):
+        ctx.linear_matmul(lin, dx, M, y1)
+        assert np.array_equal(y.download(np.uint16, (M, O)), y1.download(np.uint16, (M, O))), O
+    for b in [dx, y1] + ys: b.free()
+    for l in lins: l.free()
