@@ -35,7 +35,7 @@ struct FaArgs {
 
 #ifdef ORN_TIMING
 __device__ long long g_fa_marks[1024][8];
-#define FA_MARK(i) do { if (threadIdx.x == 0 && blockIdx.y == 3 && blockIdx.x < 1024 && kb == 5) g_fa_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+#define FA_MARK(i) do { if (threadIdx.x == 0 && blockIdx.y == 3 && blockIdx.x < 1024 && kb == 40) g_fa_marks[blockIdx.x][i] = wall_clock64(); } while (0)
 extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_fa(long long* out) {
   return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_fa_marks), sizeof(g_fa_marks));
 }
@@ -57,9 +57,11 @@ __global__ __launch_bounds__(256) void sdpa_prefill_kernel(FaArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, lg = lane >> 4;
-  const int h = blockIdx.y, hk = h / (p.Hq / p.Hkv);
-  // the longest workgroups (last rows of a causal chunk) start first
-  const int qb = (int)gridDim.x - 1 - (int)blockIdx.x;
+  // workgroups start in the order of their number: the longest (last rows of a causal chunk)
+  // first, over all heads, and the heads of one KV group next to each other
+  const int wg = (int)blockIdx.x + (int)gridDim.x * (int)blockIdx.y;
+  const int h = wg % p.Hq, hk = h / (p.Hq / p.Hkv);
+  const int qb = (int)gridDim.x - 1 - wg / p.Hq;
   const int q0 = qb * BQ * G, r0 = q0 + 16 * G * wave;  // group g: rows r0 + 16 * g + l16
   const int last_row = min(p.T, q0 + BQ * G) - 1;
   const int n_kb = (p.offset + last_row) / BKV + 1;
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(256) void sdpa_prefill_kernel(FaArgs p) {
   for (int g = 0; g < G; ++g)
 #pragma unroll
     for (int t = 0; t < HD / 16; ++t) o[g][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  // base-2 logarithms: scores are scaled by scale * log2(e) once, exp is then one instruction
+  // base-2 exponentials: exp(scale * (s - m)) = exp2(s * c2 - m * c2) with c2 = scale * log2(e)
   constexpr float kNone = -1e30f;
   const float c2 = p.scale * 1.44269504088896340736f;
   float m_i[G], l_i[G];  // l_i: this lane's share of the row sum
@@ -194,32 +196,47 @@ __global__ __launch_bounds__(256) void sdpa_prefill_kernel(FaArgs p) {
       for (int nt = 0; nt < BKV / 16; ++nt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float v = st[g][nt][r] * c2;
-          if (diag && kb * BKV + nt * 16 + 4 * lg + r > pos) v = kNone;
-          st[g][nt][r] = v;
-          mx = fmaxf(mx, v);
+          if (diag && kb * BKV + nt * 16 + 4 * lg + r > pos) st[g][nt][r] = kNone;
+          mx = fmaxf(mx, st[g][nt][r]);
         }
       mx = fmaxf(mx, dm_xor_lane<16>(mx));
       mx = fmaxf(mx, dm_xor_lane<32>(mx));
-      const float m_new = fmaxf(m_i[g], mx);
-      const float alpha = __builtin_amdgcn_exp2f(m_i[g] - m_new);
+      // the maximum is kept unscaled (scale > 0): a probability is then one fma and one exp2
+      // The reference point of a row's exponentials only moves when the maximum has grown by
+      // more than 8 binary orders: until then probabilities up to 2^8 are accumulated (harmless
+      // in fp32 sums and bf16 operands, and the final division by the row sum takes it out
+      // again), and the running output needs no rescaling, which costs three instructions an
+      // accumulator register.
+      const bool grow = (mx - m_i[g]) * c2 > 8.f;
+      const float m_new = grow ? mx : m_i[g];
+      const float alpha = grow ? __builtin_amdgcn_exp2f((m_i[g] - m_new) * c2) : 1.f;
       m_i[g] = m_new;
+      const float mc = -(m_new * c2);
       float rs = 0.f;
 #pragma unroll
       for (int nt = 0; nt < BKV / 16; ++nt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const float pv = __builtin_amdgcn_exp2f(st[g][nt][r] - m_new);
+          const float pv = __builtin_amdgcn_exp2f(dm_fma(st[g][nt][r], c2, mc));
           st[g][nt][r] = pv;
           rs += pv;
         }
       l_i[g] = l_i[g] * alpha + rs;
       // the running output only needs rescaling when some row's maximum moved
+      // (the accumulators live in accumulation registers, which vector arithmetic cannot read:
+      // written out by hand so that the moves to a vector register and back stay inside this
+      // rarely taken branch; left to the compiler they are made on both paths)
       if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
         for (int t = 0; t < HD / 16; ++t)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) o[g][t][r] *= alpha;
+          for (int r = 0; r < 4; ++r) {
+            float x = o[g][t][r], tmp;
+            asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 %0, %1"
+                         : "+a"(x), "=&v"(tmp)
+                         : "v"(alpha));
+            o[g][t][r] = x;
+          }
       }
 #pragma unroll
       for (int k2 = 0; k2 < BKV / 32; ++k2) {
