@@ -938,48 +938,78 @@ __global__ __launch_bounds__(256) void kq_mm_reg_kernel(MmArgs a) {
 static_assert(BN == 128 && BK == 128, "tile constants are baked into the index arithmetic");
 
 // ---- expert-sorted pair list for the gathered form -----------------------------------
-// inds [pairs] (expert of pair p; pair p = token * k + slot). One workgroup:
-// counts per expert, exclusive scan, scatter, then the tile list.
+// inds [pairs] (expert of pair p; pair p = token * k + slot). One workgroup: counts per expert,
+// exclusive scan, scatter, then the tile list, fullest tiles first (the GEMM's workgroups start
+// in the order of the list, and one that starts late with many rows would be the tail).
+constexpr int kSortTilesMax = 2048;  // tile lists up to this length are ordered
+
 __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* inds, int pairs, int E,
                                                               int bm, uint32_t* pair, uint32_t* tile_expert,
                                                               uint32_t* tile_start, uint32_t* tile_count,
                                                               uint32_t* n_tiles) {
-  __shared__ uint32_t cnt[1024], start[1025], tiles_before[1025];
+  __shared__ uint32_t cnt[1024], fill[1024];
+  __shared__ unsigned long long scan[2][1024];  // pairs before an expert (low 40 bits) and tiles before it
+  __shared__ uint32_t t_expert[kSortTilesMax], t_start[kSortTilesMax], t_count[kSortTilesMax];
   const int tid = threadIdx.x;
-  if (tid < 1024) cnt[tid] = 0;
+  cnt[tid] = 0;
+  fill[tid] = 0;
   __syncthreads();
   for (int p = tid; p < pairs; p += 1024) atomicAdd(&cnt[min(inds[p], (uint32_t)(E - 1))], 1u);
   __syncthreads();
-  if (tid == 0) {
-    uint32_t s = 0, t = 0;
-    for (int e = 0; e < E; ++e) {
-      start[e] = s;
-      tiles_before[e] = t;
-      s += cnt[e];
-      t += (cnt[e] + bm - 1) / bm;
-    }
-    start[E] = s;
-    tiles_before[E] = t;
-    *n_tiles = t;
+  // inclusive scan over the 1024 slots (experts past E hold zero), ten doubling steps
+  const uint32_t mine = cnt[tid];
+  scan[0][tid] = (unsigned long long)mine | ((unsigned long long)((mine + bm - 1) / bm) << 40);
+  __syncthreads();
+  int cur = 0;
+  for (int d = 1; d < 1024; d <<= 1) {
+    const unsigned long long v = scan[cur][tid] + (tid >= d ? scan[cur][tid - d] : 0ull);
+    scan[cur ^ 1][tid] = v;
+    cur ^= 1;
+    __syncthreads();
   }
+  const unsigned long long incl = scan[cur][tid];
+  const uint32_t my_tiles = (mine + bm - 1) / bm;
+  const uint32_t start = (uint32_t)(incl & ((1ull << 40) - 1)) - mine;
+  const uint32_t tiles_before = (uint32_t)(incl >> 40) - my_tiles;
+  const uint32_t total_tiles = (uint32_t)(scan[cur][1023] >> 40);
+  if (tid == 0) *n_tiles = total_tiles;
+  __syncthreads();
+  scan[0][tid] = start;  // (reused: where an expert's run of pairs begins)
   __syncthreads();
   // placement: a pair takes the next free place of its expert. The order inside an expert's
   // run depends on the scheduling of the atomics, the results do not: every output row is one
   // dot product over k in a fixed order, whichever tile row computes it.
-  __shared__ uint32_t fill[1024];
-  fill[tid] = 0;
-  __syncthreads();
   for (int p = tid; p < pairs; p += 1024) {
     const uint32_t e = min(inds[p], (uint32_t)(E - 1));
-    pair[start[e] + atomicAdd(&fill[e], 1u)] = (uint32_t)p;
+    pair[(uint32_t)scan[0][e] + atomicAdd(&fill[e], 1u)] = (uint32_t)p;
   }
-  for (int e = tid; e < E; e += 1024) {
-    const uint32_t nt = (cnt[e] + bm - 1) / bm;
-    for (uint32_t t = 0; t < nt; ++t) {
-      tile_expert[tiles_before[e] + t] = e;
-      tile_start[tiles_before[e] + t] = start[e] + t * bm;
-      tile_count[tiles_before[e] + t] = min((uint32_t)bm, cnt[e] - t * bm);
+  const bool ordered = total_tiles <= (uint32_t)kSortTilesMax;
+  if (tid < E)
+    for (uint32_t t = 0; t < my_tiles; ++t) {
+      const uint32_t i = tiles_before + t, st = start + t * bm, c = min((uint32_t)bm, mine - t * bm);
+      if (ordered) {
+        t_expert[i] = tid;
+        t_start[i] = st;
+        t_count[i] = c;
+      } else {
+        tile_expert[i] = tid;
+        tile_start[i] = st;
+        tile_count[i] = c;
+      }
     }
+  __syncthreads();
+  if (!ordered) return;
+  // rank of a tile: the tiles with more rows, and of those with as many the earlier ones
+  for (uint32_t i = tid; i < total_tiles; i += 1024) {
+    const uint32_t c = t_count[i];
+    uint32_t rank = 0;
+    for (uint32_t j = 0; j < total_tiles; ++j) {
+      const uint32_t cj = t_count[j];
+      rank += (cj > c || (cj == c && j < i)) ? 1u : 0u;
+    }
+    tile_expert[rank] = t_expert[i];
+    tile_start[rank] = t_start[i];
+    tile_count[rank] = c;
   }
 }
 
