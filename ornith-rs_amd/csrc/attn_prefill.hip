@@ -318,8 +318,8 @@ extern "C" int ornith_sdpa_prefill_gated(ornith_ctx* ctx, const void* d_q_rot, c
               offset + T, cap);
   FaArgs p{(const bf16_t*)d_q_rot, (const bf16_t*)d_k_cache, (const bf16_t*)d_v_cache, (const bf16_t*)d_qg,
            (bf16_t*)d_out, T, Hq, Hkv, offset, cap, scale};
-  // 128-row workgroups once they still give every compute unit two
-  if ((long)((T + 2 * BQ - 1) / (2 * BQ)) * Hq >= 2L * ctx->compute_units && getenv("ORN_FA_G1") == nullptr)
+  // 128-row workgroups once there is one for every compute unit
+  if ((long)((T + 2 * BQ - 1) / (2 * BQ)) * Hq >= (long)ctx->compute_units)
     hipLaunchKernelGGL(sdpa_prefill_kernel<2>, dim3((T + 2 * BQ - 1) / (2 * BQ), Hq), dim3(256), 0, ctx->stream, p);
   else
     hipLaunchKernelGGL(sdpa_prefill_kernel<1>, dim3((T + BQ - 1) / BQ, Hq), dim3(256), 0, ctx->stream, p);

@@ -954,7 +954,16 @@ __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* in
   cnt[tid] = 0;
   fill[tid] = 0;
   __syncthreads();
-  for (int p = tid; p < pairs; p += 1024) atomicAdd(&cnt[min(inds[p], (uint32_t)(E - 1))], 1u);
+  // (eight loads in flight a thread: one after the other, each pass over the pairs is 32 memory
+  // latencies long for a 4096-token chunk)
+  for (int p0 = tid; p0 < pairs; p0 += 8 * 1024) {
+    uint32_t e[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) e[u] = p0 + 1024 * u < pairs ? inds[p0 + 1024 * u] : 0u;
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (p0 + 1024 * u < pairs) atomicAdd(&cnt[min(e[u], (uint32_t)(E - 1))], 1u);
+  }
   __syncthreads();
   // inclusive scan over the 1024 slots (experts past E hold zero), ten doubling steps
   const uint32_t mine = cnt[tid];
@@ -979,9 +988,13 @@ __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* in
   // placement: a pair takes the next free place of its expert. The order inside an expert's
   // run depends on the scheduling of the atomics, the results do not: every output row is one
   // dot product over k in a fixed order, whichever tile row computes it.
-  for (int p = tid; p < pairs; p += 1024) {
-    const uint32_t e = min(inds[p], (uint32_t)(E - 1));
-    pair[(uint32_t)scan[0][e] + atomicAdd(&fill[e], 1u)] = (uint32_t)p;
+  for (int p0 = tid; p0 < pairs; p0 += 8 * 1024) {
+    uint32_t e[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) e[u] = p0 + 1024 * u < pairs ? min(inds[p0 + 1024 * u], (uint32_t)(E - 1)) : 0u;
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (p0 + 1024 * u < pairs) pair[(uint32_t)scan[0][e[u]] + atomicAdd(&fill[e[u]], 1u)] = (uint32_t)(p0 + 1024 * u);
   }
   const bool ordered = total_tiles <= (uint32_t)kSortTilesMax;
   if (tid < E)
@@ -1011,6 +1024,95 @@ __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* in
     tile_start[rank] = t_start[i];
     tile_count[rank] = c;
   }
+}
+
+// ---- the same plan from many workgroups -----------------------------------------------
+// A pass over the pairs is one LDS atomic a pair, about a cycle each in one workgroup: 33 us
+// for the 32768 pairs of a 4096-token chunk. From 8192 pairs on, kSortParts workgroups count
+// their slices of the pairs side by side, one workgroup turns the counts into places (per
+// expert, then per slice inside an expert's run) and writes the tile list, and the slices
+// scatter side by side.
+constexpr int kSortParts = 32;
+
+__global__ __launch_bounds__(256) void moe_sort_count_kernel(const uint32_t* inds, int pairs, int E, uint32_t* part_cnt) {
+  __shared__ uint32_t cnt[1024];
+  for (int e = threadIdx.x; e < E; e += 256) cnt[e] = 0;
+  __syncthreads();
+  const int per = (pairs + kSortParts - 1) / kSortParts, a = blockIdx.x * per, b = min(pairs, a + per);
+  for (int p = a + threadIdx.x; p < b; p += 256) atomicAdd(&cnt[min(inds[p], (uint32_t)(E - 1))], 1u);
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += 256) part_cnt[blockIdx.x * E + e] = cnt[e];
+}
+
+// part_cnt [parts, E] in: pairs of expert e in slice b; out: where slice b's pairs of expert e begin
+__global__ __launch_bounds__(1024) void moe_sort_plan_kernel(int E, int bm, uint32_t* part_cnt, uint32_t* tile_expert,
+                                                             uint32_t* tile_start, uint32_t* tile_count,
+                                                             uint32_t* n_tiles) {
+  __shared__ unsigned long long scan[2][1024];
+  __shared__ uint32_t t_expert[kSortTilesMax], t_start[kSortTilesMax], t_count[kSortTilesMax];
+  const int tid = threadIdx.x;
+  uint32_t mine = 0;
+  if (tid < E)
+    for (int b = 0; b < kSortParts; ++b) mine += part_cnt[b * E + tid];
+  const uint32_t my_tiles = (mine + bm - 1) / bm;
+  scan[0][tid] = (unsigned long long)mine | ((unsigned long long)my_tiles << 40);
+  __syncthreads();
+  int cur = 0;
+  for (int d = 1; d < 1024; d <<= 1) {
+    const unsigned long long v = scan[cur][tid] + (tid >= d ? scan[cur][tid - d] : 0ull);
+    scan[cur ^ 1][tid] = v;
+    cur ^= 1;
+    __syncthreads();
+  }
+  const unsigned long long incl = scan[cur][tid];
+  const uint32_t start = (uint32_t)(incl & ((1ull << 40) - 1)) - mine;
+  const uint32_t tiles_before = (uint32_t)(incl >> 40) - my_tiles;
+  const uint32_t total_tiles = (uint32_t)(scan[cur][1023] >> 40);
+  if (tid == 0) *n_tiles = total_tiles;
+  if (tid < E) {
+    uint32_t at = start;
+    for (int b = 0; b < kSortParts; ++b) {
+      const uint32_t c = part_cnt[b * E + tid];
+      part_cnt[b * E + tid] = at;
+      at += c;
+    }
+  }
+  const bool ordered = total_tiles <= (uint32_t)kSortTilesMax;
+  if (tid < E)
+    for (uint32_t t = 0; t < my_tiles; ++t) {
+      const uint32_t i = tiles_before + t, st = start + t * bm, c = min((uint32_t)bm, mine - t * bm);
+      if (ordered) {
+        t_expert[i] = tid;
+        t_start[i] = st;
+        t_count[i] = c;
+      } else {
+        tile_expert[i] = tid;
+        tile_start[i] = st;
+        tile_count[i] = c;
+      }
+    }
+  __syncthreads();
+  if (!ordered) return;
+  for (uint32_t i = tid; i < total_tiles; i += 1024) {
+    const uint32_t c = t_count[i];
+    uint32_t rank = 0;
+    for (uint32_t j = 0; j < total_tiles; ++j) {
+      const uint32_t cj = t_count[j];
+      rank += (cj > c || (cj == c && j < i)) ? 1u : 0u;
+    }
+    tile_expert[rank] = t_expert[i];
+    tile_start[rank] = t_start[i];
+    tile_count[rank] = c;
+  }
+}
+
+__global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const uint32_t* inds, int pairs, int E,
+                                                               const uint32_t* part_at, uint32_t* pair) {
+  __shared__ uint32_t at[1024];
+  for (int e = threadIdx.x; e < E; e += 256) at[e] = part_at[blockIdx.x * E + e];
+  __syncthreads();
+  const int per = (pairs + kSortParts - 1) / kSortParts, a = blockIdx.x * per, b = min(pairs, a + per);
+  for (int p = a + threadIdx.x; p < b; p += 256) pair[atomicAdd(&at[min(inds[p], (uint32_t)(E - 1))], 1u)] = (uint32_t)p;
 }
 
 int check(const ornith_kmatrix* w, const char* who) {
@@ -1094,7 +1196,7 @@ int ornith_kq_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x, 
 // (ornith_kq_gather_plan_bytes(pairs, E) bytes)
 size_t ornith_kq_gather_plan_bytes(int pairs, int E) {
   const size_t tiles = (size_t)pairs / 64 + (size_t)E + 1;
-  return ((size_t)pairs + tiles * 3 + 1) * 4 + 5 * 256;
+  return ((size_t)pairs + tiles * 3 + 1 + (size_t)kSortParts * E) * 4 + 6 * 256;
 }
 
 int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d_x,
@@ -1112,6 +1214,7 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   uint32_t* ts = pc.take<uint32_t>(tiles_max);
   uint32_t* tc = pc.take<uint32_t>(tiles_max);
   uint32_t* nt = pc.take<uint32_t>(1);
+  uint32_t* parts = pc.take<uint32_t>((size_t)kSortParts * w->E);
   // rows per tile (the choice depends only on pairs and E, so the calls sharing a plan agree on
   // it). Register form: the smallest of 96 / 128 / 160 / 192 rows that holds an expert's share
   // of the pairs with 2.5 standard deviations to spare, so that nearly every expert is one
@@ -1126,7 +1229,13 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   const bool reg = ornith_option_gemm_reg() && avg >= 48 && x_bytes < (size_t(1) << 32) && q_bytes < (size_t(1) << 32);
   const int need = avg + spare;
   const int tile_rows = reg ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : avg >= 96 ? 128 : 64;
-  if (rebuild_plan) {
+  if (rebuild_plan && pairs >= 8192) {
+    hipLaunchKernelGGL(moe_sort_count_kernel, dim3(kSortParts), dim3(256), 0, ctx->stream, d_inds, pairs, w->E, parts);
+    hipLaunchKernelGGL(moe_sort_plan_kernel, dim3(1), dim3(1024), 0, ctx->stream, w->E, tile_rows, parts, te, ts, tc, nt);
+    hipLaunchKernelGGL(moe_sort_scatter_kernel, dim3(kSortParts), dim3(256), 0, ctx->stream, d_inds, pairs, w->E,
+                       parts, pair);
+    ORN_LAUNCH_CHECK("moe_sort_*_kernel");
+  } else if (rebuild_plan) {
     hipLaunchKernelGGL(moe_sort_pairs_kernel, dim3(1), dim3(1024), 0, ctx->stream, d_inds, pairs, w->E,
                        tile_rows, pair, te, ts, tc, nt);
     ORN_LAUNCH_CHECK("moe_sort_pairs_kernel");
