@@ -1226,7 +1226,10 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   while (4 * spare * spare < 25 * avg) ++spare;
   const size_t x_bytes = (size_t)(is_up ? pairs / top_k : pairs) * w->K * 2;
   const size_t q_bytes = (size_t)w->E * w->O * (w->K / 256) * (w->kind == ORNITH_Q4K ? 128 : 192);
-  const bool reg = ornith_option_gemm_reg() && avg >= 48 && x_bytes < (size_t(1) << 32) && q_bytes < (size_t(1) << 32);
+  // (with few K slabs a workgroup's way in and out, which nothing overlaps at one workgroup a
+  // compute unit, outweighs what the register form saves: K >= 1024 only)
+  const bool reg = ornith_option_gemm_reg() && avg >= 48 && w->K >= 1024 && x_bytes < (size_t(1) << 32) &&
+                   q_bytes < (size_t(1) << 32);
   const int need = avg + spare;
   const int tile_rows = reg ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : avg >= 96 ? 128 : 64;
   if (rebuild_plan && pairs >= 8192) {
