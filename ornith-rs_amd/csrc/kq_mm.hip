@@ -1220,7 +1220,8 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   // of the pairs with 2.5 standard deviations to spare, so that nearly every expert is one
   // tile and its weights are dequantized once. Below about 48 rows an expert, with offsets that
   // do not fit 32 bits, and with the option off, the LDS form: 128-row tiles from 96 rows an
-  // expert on average, else 64.
+  // expert on average (and K >= 1024: with few slabs a tile, three 64-row workgroups a compute
+  // unit hide more than 128-row tiles save), else 64.
   const int avg = pairs / w->E;
   int spare = 0;
   while (4 * spare * spare < 25 * avg) ++spare;
@@ -1231,7 +1232,7 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   const bool reg = ornith_option_gemm_reg() && avg >= 48 && w->K >= 1024 && x_bytes < (size_t(1) << 32) &&
                    q_bytes < (size_t(1) << 32);
   const int need = avg + spare;
-  const int tile_rows = reg ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : avg >= 96 ? 128 : 64;
+  const int tile_rows = reg ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : (avg >= 96 && w->K >= 1024) ? 128 : 64;
   if (rebuild_plan && pairs >= 8192) {
     hipLaunchKernelGGL(moe_sort_count_kernel, dim3(kSortParts), dim3(256), 0, ctx->stream, d_inds, pairs, w->E, parts);
     hipLaunchKernelGGL(moe_sort_plan_kernel, dim3(1), dim3(1024), 0, ctx->stream, w->E, tile_rows, parts, te, ts, tc, nt);
