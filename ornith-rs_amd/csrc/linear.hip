@@ -183,17 +183,40 @@ __global__ void embedding4_kernel(const uint8_t* w, const bf16_t* scales, const 
 typedef __bf16 dmm_bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float dmm_f32x4_t __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(256) void dense_mm_kernel(const bf16_t* w, const bf16_t* x, bf16_t* y, int M, int O,
-                                                       int K) {
+struct DenseMmSegs {
+  const bf16_t* w[4];
+  bf16_t* y[4];
+  int O[4];
+  int n;
+};
+
+__global__ __launch_bounds__(256) void dense_mm_kernel(DenseMmSegs s, const bf16_t* x, int M, int K) {
   __shared__ float red[3][4][64][4];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l16 = lane & 15, lg = lane >> 4;
-  const int row0 = blockIdx.x * 16, o0 = blockIdx.y * 64;
+  const int row0 = blockIdx.x * 16;
   const int kw = K / 4, k0 = wave * kw;  // K is a multiple of 128
   const bf16_t* xp = x + (size_t)min(row0 + l16, M - 1) * K + k0 + 8 * lg;
+  // the four 16-output tiles of this workgroup: tile 4 * blockIdx.y + nt of the segments' tiles
+  // laid end to end (a segment's last tile may be ragged)
   const bf16_t* wp[4];
+  bf16_t* yp[4];
+  int ocol[4], oend[4], ostride[4];
 #pragma unroll
-  for (int nt = 0; nt < 4; ++nt) wp[nt] = w + (size_t)min(o0 + nt * 16 + l16, O - 1) * K + k0 + 8 * lg;
-  const int nts = min(4, (O - o0 + 15) / 16);
+  for (int nt = 0; nt < 4; ++nt) {
+    int t = 4 * blockIdx.y + nt, seg = -1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (seg < 0 && i < s.n) {
+        const int tiles = (s.O[i] + 15) / 16;
+        if (t < tiles) seg = i; else t -= tiles;
+      }
+    const int sg = seg < 0 ? 0 : seg;
+    ocol[nt] = 16 * t + l16;
+    oend[nt] = seg < 0 ? 0 : s.O[sg];
+    ostride[nt] = s.O[sg];
+    yp[nt] = s.y[sg];
+    wp[nt] = s.w[sg] + (size_t)min(ocol[nt], s.O[sg] - 1) * K + k0 + 8 * lg;
+  }
   dmm_f32x4_t acc[4];
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) acc[nt] = dmm_f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -202,7 +225,7 @@ __global__ __launch_bounds__(256) void dense_mm_kernel(const bf16_t* w, const bf
     const dmm_bf16x8_t a = *reinterpret_cast<const dmm_bf16x8_t*>(xp + k);
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt)
-      if (nt < nts) {
+      if (oend[nt] > 0) {  // (the same for every lane of the wavefront)
         const dmm_bf16x8_t b = *reinterpret_cast<const dmm_bf16x8_t*>(wp[nt] + k);
         acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[nt], 0, 0, 0);
       }
@@ -218,14 +241,35 @@ __global__ __launch_bounds__(256) void dense_mm_kernel(const bf16_t* w, const bf
   // D[m = 4 * lg + r][n = l16]
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
-    const int o = o0 + nt * 16 + l16;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int row = row0 + 4 * lg + r;
       const float v = ((acc[nt][r] + red[0][nt][lane][r]) + red[1][nt][lane][r]) + red[2][nt][lane][r];
-      if (nt < nts && o < O && row < M) y[(size_t)row * O + o] = dm_f2bf(v);
+      if (ocol[nt] < oend[nt] && row < M) yp[nt][(size_t)row * ostride[nt] + ocol[nt]] = dm_f2bf(v);
     }
   }
+}
+
+// up to four dense matrices of one K over the same activations at prefill width; false when
+// the shapes do not allow it
+static bool launch_dense_mm(ornith_ctx* ctx, const ornith_linear* const* ws, int n, const void* d_x, int M,
+                            void* const* d_ys) {
+  if (n < 1 || n > 4 || ((uintptr_t)d_x & 15) != 0) return false;
+  DenseMmSegs s{};
+  s.n = n;
+  int tiles = 0;
+  for (int i = 0; i < n; ++i) {
+    if (ws[i]->mode != ORNITH_LIN_DENSE || !ws[i]->d_w || ws[i]->K != ws[0]->K || ws[i]->K % 128 != 0 || ws[i]->O < 1 ||
+        ((uintptr_t)ws[i]->d_w & 15) != 0)
+      return false;
+    s.w[i] = (const bf16_t*)ws[i]->d_w;
+    s.y[i] = (bf16_t*)d_ys[i];
+    s.O[i] = ws[i]->O;
+    tiles += (ws[i]->O + 15) / 16;
+  }
+  hipLaunchKernelGGL(dense_mm_kernel, dim3((M + 15) / 16, (tiles + 3) / 4), dim3(256), 0, ctx->stream, s,
+                     (const bf16_t*)d_x, M, ws[0]->K);
+  return true;
 }
 
 template <bool GATHER>
@@ -297,9 +341,7 @@ int ornith_linear_matmul(ornith_ctx* ctx, const ornith_linear* w, const void* d_
       ORN_REQUIRE(w->K % 8 == 0 && w->O >= 1 && M <= 65535, "linear_matmul: dense O=%d K=%d", w->O,
                   w->K);
       // prefill widths (outside the exact window, like the k-quant GEMM): on the matrix cores
-      if (M >= kPrefillRows && w->K % 128 == 0 && ((uintptr_t)d_x & 15) == 0 && ((uintptr_t)w->d_w & 15) == 0) {
-        hipLaunchKernelGGL(dense_mm_kernel, dim3((M + 15) / 16, (w->O + 63) / 64), dim3(256), 0, ctx->stream,
-                           (const bf16_t*)w->d_w, (const bf16_t*)d_x, (bf16_t*)d_y, M, w->O, w->K);
+      if (M >= kPrefillRows && launch_dense_mm(ctx, &w, 1, d_x, M, &d_y)) {
         ORN_LAUNCH_CHECK("dense_mm_kernel");
         return ORNITH_OK;
       }
@@ -340,6 +382,11 @@ int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, 
       s.O[i] = ws[i]->O;
     }
     return launch_dense<false>(ctx, s, d_x, ws[0]->K, 1, M, nullptr, nullptr, M);
+  }
+  // prefill widths: dense matrices of one K share a launch
+  if (M >= kPrefillRows && ornith_option_fuse_proj() && n >= 2 && launch_dense_mm(ctx, ws, n, d_x, M, d_ys)) {
+    ORN_LAUNCH_CHECK("dense_mm_kernel");
+    return ORNITH_OK;
   }
   // prefill widths: runs of k-quant matrices of one kind and K share a GEMM launch
   for (int i = 0; i < n;) {

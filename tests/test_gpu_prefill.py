@@ -311,3 +311,23 @@ def test_projections_sharing_an_input_share_a_gemm_launch(orn, ctx, kind, Os, K,
         assert np.array_equal(y.download(np.uint16, (M, O)), y1.download(np.uint16, (M, O))), O
     for b in [dx, y1] + ys: b.free()
     for l in lins: l.free()
+
+
+@pytest.mark.parametrize("Os,K,M", [((32, 32), 2048, 4096), ((1, 40, 16), 256, 77)])
+def test_dense_projections_sharing_an_input_share_a_launch(orn, ctx, Os, K, M):
+    """linear_matmul_multi over dense matrices at prefill width: their 16-output tiles laid end to
+    end in one launch; every output equals the matrix's own launch bit for bit"""
+    rng = np.random.default_rng(sum(Os) + K + M)
+    hls = [util.HostLinear.dense(rng, O, K) for O in Os]
+    lins = [h.dev(orn, ctx) for h in hls]
+    xb = util.bf16_normal(rng, (M, K))
+    dx = ctx.to_device(xb)
+    ys = [ctx.alloc(M * O * 2) for O in Os]
+    for y, O in zip(ys, Os): ctx.memset(y, 0xFF, M * O * 2)
+    ctx.linear_matmul_multi(lins, dx, M, ys)
+    y1 = ctx.alloc(M * max(Os) * 2)
+    for lin, y, O in zip(lins, ys, Os):
+        ctx.linear_matmul(lin, dx, M, y1)
+        assert np.array_equal(y.download(np.uint16, (M, O)), y1.download(np.uint16, (M, O))), O
+    for b in [dx, y1] + ys: b.free()
+    for l in lins: l.free()
