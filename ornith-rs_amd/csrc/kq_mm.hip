@@ -943,6 +943,36 @@ static_assert(BN == 128 && BK == 128, "tile constants are baked into the index a
 // in the order of the list, and one that starts late with many rows would be the tail).
 constexpr int kSortTilesMax = 2048;  // tile lists up to this length are ordered
 
+// Writes the tile list fullest first: a counting sort over the tile heights (a tile has 1 .. bm
+// <= 256 rows; tiles of one height land in the order their atomics are served, which changes
+// the order workgroups start in and nothing else). All 1024 threads of the workgroup call it.
+__device__ __forceinline__ void order_tiles(uint32_t total_tiles, int bm, const uint32_t* t_expert, const uint32_t* t_start,
+                                            const uint32_t* t_count, uint32_t* tile_expert, uint32_t* tile_start,
+                                            uint32_t* tile_count) {
+  __shared__ uint32_t bin[257];
+  const int tid = threadIdx.x;
+  if (tid < 257) bin[tid] = 0;
+  __syncthreads();
+  for (uint32_t i = tid; i < total_tiles; i += 1024) atomicAdd(&bin[min(t_count[i], 256u)], 1u);
+  __syncthreads();
+  if (tid == 0) {  // places of the heights, tallest first
+    uint32_t at = 0;
+    for (int c = min(bm, 256); c >= 0; --c) {
+      const uint32_t n = bin[c];
+      bin[c] = at;
+      at += n;
+    }
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < total_tiles; i += 1024) {
+    const uint32_t c = t_count[i], at = atomicAdd(&bin[min(c, 256u)], 1u);
+    tile_expert[at] = t_expert[i];
+    tile_start[at] = t_start[i];
+    tile_count[at] = c;
+  }
+}
+
+
 __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* inds, int pairs, int E,
                                                               int bm, uint32_t* pair, uint32_t* tile_expert,
                                                               uint32_t* tile_start, uint32_t* tile_count,
@@ -1012,18 +1042,7 @@ __global__ __launch_bounds__(1024) void moe_sort_pairs_kernel(const uint32_t* in
     }
   __syncthreads();
   if (!ordered) return;
-  // rank of a tile: the tiles with more rows, and of those with as many the earlier ones
-  for (uint32_t i = tid; i < total_tiles; i += 1024) {
-    const uint32_t c = t_count[i];
-    uint32_t rank = 0;
-    for (uint32_t j = 0; j < total_tiles; ++j) {
-      const uint32_t cj = t_count[j];
-      rank += (cj > c || (cj == c && j < i)) ? 1u : 0u;
-    }
-    tile_expert[rank] = t_expert[i];
-    tile_start[rank] = t_start[i];
-    tile_count[rank] = c;
-  }
+  order_tiles(total_tiles, bm, t_expert, t_start, t_count, tile_expert, tile_start, tile_count);
 }
 
 // ---- the same plan from many workgroups -----------------------------------------------
@@ -1093,17 +1112,7 @@ __global__ __launch_bounds__(1024) void moe_sort_plan_kernel(int E, int bm, uint
     }
   __syncthreads();
   if (!ordered) return;
-  for (uint32_t i = tid; i < total_tiles; i += 1024) {
-    const uint32_t c = t_count[i];
-    uint32_t rank = 0;
-    for (uint32_t j = 0; j < total_tiles; ++j) {
-      const uint32_t cj = t_count[j];
-      rank += (cj > c || (cj == c && j < i)) ? 1u : 0u;
-    }
-    tile_expert[rank] = t_expert[i];
-    tile_start[rank] = t_start[i];
-    tile_count[rank] = c;
-  }
+  order_tiles(total_tiles, bm, t_expert, t_start, t_count, tile_expert, tile_start, tile_count);
 }
 
 __global__ __launch_bounds__(256) void moe_sort_scatter_kernel(const uint32_t* inds, int pairs, int E,
