@@ -85,6 +85,13 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *   "gemm_duo"  (ORNITH_GEMM_DUO, default 1): the 256-row tile of the prefill GEMM runs with
  *               producer and consumer wavefronts (0: every wavefront dequantizes, then
  *               multiplies); same results either way
+ *   "gemm_reg"  (ORNITH_GEMM_REG, default 1): the expert-gathered prefill GEMM dequantizes the
+ *               weights into MFMA operand registers where the shape suits it (48 rows an expert
+ *               or more, K >= 1024; 0: always through LDS); results agree to the order of the
+ *               fp32 sums
+ *   "gdn_chunked" (ORNITH_GDN_CHUNKED, default 1): the gated-delta recurrence of calls of 128
+ *               rows or more (without per-token snapshots) runs in 64-token chunks on the
+ *               matrix cores (0: token by token); results agree to rounding
  *   "fuse_moe_one" (ORNITH_FUSE_MOE_ONE, default 0): the MoE block's phases as ranges of
  *               workgroups of ONE launch that hand their intermediates over through memory
  *               (1: router + up + down, 2: up + down after a router launch). Bit-identical,

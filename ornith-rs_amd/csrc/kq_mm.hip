@@ -6,16 +6,18 @@
 // the expert-gathered form where each tile's rows belong to one routed expert.
 //
 // This is the one GEMM-shaped piece of the path (81 % of a prefill chunk in the
-// reference, /root/reference/src/bin/arithmetic.rs:4-7), so it runs on MFMA:
-// v_mfma_f32_32x32x16_bf16, a workgroup tile of BM x 128 outputs over K slabs of 128.
-//   * A (activations, bf16) goes global -> LDS as is.
-//   * B (weights) is read as k-quant codes (the 144 / 210 bytes per 256 weights that HBM
-//     holds), dequantized with the arithmetic of kquant::dequantize (d*sc*q - dmin*m,
-//     resp. d*sc*q) and rounded to bf16 into LDS: HBM traffic stays at the quantized size.
-//   * LDS rows are padded by 8 elements so the 16-byte fragment reads of 32 consecutive
-//     rows spread over the banks.
-//   * Four wavefronts: 2 x 2 of 64 x 64 outputs each for BM = 128, 1 x 4 of 64 x 32 for
-//     BM = 64 (used when an expert's share of the tokens is small).
+// reference, /root/reference/src/bin/arithmetic.rs:4-7), so it runs on MFMA
+// (v_mfma_f32_32x32x16_bf16). Three forms, all reading the weights as k-quant codes (the 144 /
+// 210 bytes per 256 weights that HBM holds) and dequantizing them with the arithmetic of
+// kquant::dequantize (d*sc*q - dmin*m, resp. d*sc*q), rounded to bf16:
+//   * kq_mm_kernel: a workgroup tile of BM x 128 outputs over K slabs of 128; activations go
+//     global -> LDS as they are, weights are dequantized on the way into LDS; LDS rows padded by
+//     8 elements so the 16-byte fragment reads of 32 consecutive rows spread over the banks;
+//     four wavefronts: 2 x 2 of 64 x 64 outputs each for BM = 128, 1 x 4 of 64 x 32 for BM = 64.
+//   * kq_mm_duo_kernel: the 256-row tile with producer and consumer wavefronts.
+//   * kq_mm_reg_kernel: expert-gathered tiles of up to 192 rows with the weights dequantized
+//     straight into MFMA operand registers (only activations through LDS).
+// Up to four matrices of one kind and K over the same activations share a launch.
 //
 // Prefill is exempt from the "row r of a batch == row r alone" rule in the reference too
 // (src/ops/invariant.rs:140-168): results agree with the mat-vec path to bf16 rounding of
@@ -107,8 +109,9 @@ __device__ __forceinline__ BRegsQ4 load_q4k(const MmArgs& a, int64_t row, int nb
 }
 
 // 64 weights as bf16 into dst[0..64): d*sc*q - dmin*m (kquant::dequantize, q4k.metal:64-96).
-// About three vector instructions a weight (byte -> float, one fma, half a bf16 pack): the
-// dequantization shares the wavefront with the MFMAs it feeds, so its length is GEMM time.
+// Two and a half vector instructions a weight (byte -> float, one fma, half a two-value bf16
+// conversion): the dequantization shares the wavefront with the MFMAs it feeds, so its length
+// is GEMM time.
 __device__ __forceinline__ void dequant_q4k(const BRegsQ4& r, int grp, bf16_t* dst) {
   // the 6-bit scale and min of sub-blocks 2*grp and 2*grp + 1, two bytes each way
   const int sh16 = (grp & 1) * 16;
@@ -177,18 +180,8 @@ struct BRegsOf<ORNITH_Q6K> { typedef BRegsQ6 type; };
 
 #ifdef ORN_TIMING
 __device__ long long g_mm_marks[1024][8];
-__device__ long long g_mm_cyc[1024][2];
-#define MM_CYC(i) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y < 1024) g_mm_cyc[blockIdx.y][i] = clock64(); } while (0)
-extern "C" __attribute__((visibility("default"))) int ornith_debug_cyc_mm(long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mm_cyc), sizeof(g_mm_cyc));
-}
-#define MM_MARK(i, cond) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y < 1024 && (cond)) g_mm_marks[blockIdx.y][i] = wall_clock64(); } while (0)
-extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_mm(long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mm_marks), sizeof(g_mm_marks));
-}
 #else
 #define MM_MARK(i, cond)
-#define MM_CYC(i)
 #endif
 
 // ---- epilogue ------------------------------------------------------------------------------
@@ -711,10 +704,6 @@ __device__ __forceinline__ bf16x8_t raw_fragment(const Raw& r, const float (&s)[
   int qd;
   raw_codes<T>(r, c0, c1, qd);
   u32x4_t f;
-#ifdef ORN_NODEQ
-  f[0] = c0; f[1] = c1; f[2] = c0 ^ __float_as_uint(s[qd]); f[3] = c1 ^ __float_as_uint(o[qd]);
-  return __builtin_bit_cast(bf16x8_t, f);
-#endif
   f[0] = pack2(dm_fma(s[qd], dm_ubyte<0>(c0), o[qd]), dm_fma(s[qd], dm_ubyte<1>(c0), o[qd]));
   f[1] = pack2(dm_fma(s[qd], dm_ubyte<2>(c0), o[qd]), dm_fma(s[qd], dm_ubyte<3>(c0), o[qd]));
   f[2] = pack2(dm_fma(s[qd], dm_ubyte<0>(c1), o[qd]), dm_fma(s[qd], dm_ubyte<1>(c1), o[qd]));
@@ -737,7 +726,6 @@ __device__ __forceinline__ void reg_tile(const MmArgs& a, bf16_t (*As)[RM][LDK],
   const int n0 = blockIdx.x * RN;
   const int nb = a.K >> 8, nslab = a.K / BK;  // an even number of slabs
   MM_MARK(5, true);
-  MM_CYC(0);
 
   RawOff boff[TN];
 #pragma unroll
@@ -894,7 +882,6 @@ __device__ __forceinline__ void reg_tile(const MmArgs& a, bf16_t (*As)[RM][LDK],
   }
   __syncthreads();  // the fragments of a slab past the end were read out of the buffers the output tile goes over
   MM_MARK(6, true);
-  MM_CYC(1);
   store_tile<TM, TN, GATHER>(a, acc, &As[0][0][0], 0, wave * 64, lane, n0, m0, rows_here, s_dst, a.vec != 0, RN + 8);
   MM_MARK(7, true);
 }
