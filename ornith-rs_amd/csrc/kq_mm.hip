@@ -58,9 +58,10 @@ struct MmArgs {
     const uint8_t* scales;
     const uint16_t* dm;
     bf16_t* y;
-    int O, bx0;
+    int O, bx0, kind;
   } seg[3];
   int nseg;
+  int kind;  // of the first matrix (read by the kernel instance for matrices of both kinds)
 };
 
 // the matrix a workgroup of the plain form works on; returns its column block there
@@ -74,6 +75,7 @@ __device__ __forceinline__ int pick_segment(MmArgs& a) {
       a.dm = a.seg[i].dm;
       a.y = a.seg[i].y;
       a.O = a.seg[i].O;
+      a.kind = a.seg[i].kind;
       bx = (int)blockIdx.x - a.seg[i].bx0;
     }
   return bx;
@@ -180,6 +182,10 @@ struct BRegsOf<ORNITH_Q6K> { typedef BRegsQ6 type; };
 
 #ifdef ORN_TIMING
 __device__ long long g_mm_marks[1024][8];
+#define MM_MARK(i, cond) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y < 1024 && (cond)) g_mm_marks[blockIdx.y][i] = wall_clock64(); } while (0)
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_mm(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mm_marks), sizeof(g_mm_marks));
+}
 #else
 #define MM_MARK(i, cond)
 #endif
@@ -238,7 +244,9 @@ __device__ __forceinline__ void store_tile(const MmArgs& a, const f32x16_t (&acc
   }
 }
 
-// BM = 256: 2 x 2 wavefronts of 128 x 64; BM = 128: 2 x 2 of 64 x 64; BM = 64: 1 x 4 of 64 x 32
+// BM = 256: 2 x 2 wavefronts of 128 x 64; BM = 128: 2 x 2 of 64 x 64; BM = 64: 1 x 4 of 64 x 32.
+// KIND = kMixed: the matrices of the launch differ in kind (a workgroup asks its own).
+constexpr int kMixed = 2;
 template <int KIND, int BM, bool GATHER>
 __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
   constexpr int WM = BM >= 128 ? 2 : 1, WN = 4 / WM;
@@ -285,15 +293,17 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
     asrc[i] = a.x + src * a.K + 8 * c8;
   }
   u32x4_t areg[NA];
-  typename BRegsOf<KIND>::type breg;
+  BRegsQ4 breg4;
+  BRegsQ6 breg6;
+  const bool q4 = KIND == kMixed ? a.kind == ORNITH_Q4K : KIND == ORNITH_Q4K;
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < NA; ++i)
       areg[i] = *reinterpret_cast<const u32x4_t*>(asrc[i] + k0);
-    if constexpr (KIND == ORNITH_Q4K)
-      breg = load_q4k(a, brow, nb, k0 >> 8, ((k0 & 255) >> 6) + bpart);
+    if (q4)
+      breg4 = load_q4k(a, brow, nb, k0 >> 8, ((k0 & 255) >> 6) + bpart);
     else
-      breg = load_q6k(a, brow, nb, k0 >> 8, (k0 & 255) >> 7, bpart);
+      breg6 = load_q6k(a, brow, nb, k0 >> 8, (k0 & 255) >> 7, bpart);
   };
 
   f32x16_t acc[TM][TN];
@@ -311,10 +321,10 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
       const int idx = tid + 256 * i;
       *reinterpret_cast<u32x4_t*>(&As[idx >> 4][8 * (idx & 15)]) = areg[i];
     }
-    if constexpr (KIND == ORNITH_Q4K)
-      dequant_q4k(breg, ((k0 & 255) >> 6) + bpart, &Bs[br][64 * bpart]);
+    if (q4)
+      dequant_q4k(breg4, ((k0 & 255) >> 6) + bpart, &Bs[br][64 * bpart]);
     else
-      dequant_q6k(breg, bpart, &Bs[br][0]);
+      dequant_q6k(breg6, bpart, &Bs[br][0]);
     __syncthreads();
     if (k0 + BK < a.K) fetch(k0 + BK);  // in flight while the matrix cores run
     // fragments of step kk + 1 leave LDS while the matrix cores work on step kk
@@ -1123,8 +1133,9 @@ int check(const ornith_kmatrix* w, const char* who) {
 
 extern "C" {
 
-// Up to four matrices of one kind and K over the same activations in one launch (the
-// projections that share an input: narrow ones alone leave compute units without a workgroup)
+// Up to four matrices of one K over the same activations in one launch (the projections that
+// share an input: narrow ones alone leave compute units without a workgroup). Matrices of one
+// kind take the tile the whole launch's size calls for; a mix of kinds takes 128-row tiles.
 int ornith_kq_matmul_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n, const void* d_x, int M,
                            void* const* d_ys) {
   ORN_REQUIRE(ctx && ws && d_x && d_ys && n >= 1 && n <= 4, "kq_matmul: bad argument");
@@ -1132,13 +1143,15 @@ int ornith_kq_matmul_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int
   ORN_REQUIRE(((uintptr_t)d_x & 15) == 0, "kq_matmul: x must be 16-byte aligned");
   MmArgs a{};
   int nx = 0;
+  bool mixed = false;
   a.vec = 1;
   for (int i = 0; i < n; ++i) {
     ORN_REQUIRE(ws[i] && d_ys[i], "kq_matmul: null entry %d", i);
     int rc = check(ws[i], "kq_matmul");
     if (rc) return rc;
     ORN_REQUIRE(ws[i]->E == 1, "kq_matmul: stacked matrix (use kq_gather_matmul)");
-    ORN_REQUIRE(ws[i]->kind == ws[0]->kind && ws[i]->K == ws[0]->K, "kq_matmul: matrices of one launch differ in kind or K");
+    ORN_REQUIRE(ws[i]->K == ws[0]->K, "kq_matmul: matrices of one launch differ in K");
+    mixed = mixed || ws[i]->kind != ws[0]->kind;
     a.vec = a.vec && ws[i]->O % 8 == 0 && ((uintptr_t)d_ys[i] & 15) == 0;
     if (i == 0) {
       a.qs = (const uint8_t*)ws[0]->d_qs;
@@ -1148,7 +1161,7 @@ int ornith_kq_matmul_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int
       a.O = ws[0]->O;
     } else {
       a.seg[i - 1] = {(const uint8_t*)ws[i]->d_qs, (const uint8_t*)ws[i]->d_scales, (const uint16_t*)ws[i]->d_dm,
-                      (bf16_t*)d_ys[i], ws[i]->O, nx};
+                      (bf16_t*)d_ys[i], ws[i]->O, nx, ws[i]->kind};
     }
     nx += (ws[i]->O + BN - 1) / BN;
   }
@@ -1157,6 +1170,12 @@ int ornith_kq_matmul_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int
   a.M = M;
   a.K = ws[0]->K;
   const int kind = ws[0]->kind;
+  a.kind = kind;
+  if (mixed) {  // matrices of both kinds: the 128-row tile, every workgroup asking its matrix's kind
+    hipLaunchKernelGGL((kq_mm_kernel<kMixed, 128, false>), dim3(nx, (M + 127) / 128), dim3(256), 0, ctx->stream, a);
+    ORN_LAUNCH_CHECK("kq_mm_kernel<mixed>");
+    return ORNITH_OK;
+  }
   // 256-row tiles dequantize every weight tile half as often; 128-row tiles when that is what
   // it takes to give every compute unit a workgroup
   const bool big = M >= 256 && (long)nx * ((M + 255) / 256) >= ctx->compute_units;

@@ -388,13 +388,21 @@ int ornith_linear_matmul_multi(ornith_ctx* ctx, const ornith_linear* const* ws, 
     ORN_LAUNCH_CHECK("dense_mm_kernel");
     return ORNITH_OK;
   }
-  // prefill widths: runs of k-quant matrices of one kind and K share a GEMM launch
+  // prefill widths: runs of k-quant matrices of one K share a GEMM launch. A run of one kind may
+  // be large (it picks its tile by size); a matrix of the other kind joins a run only while the
+  // run is narrow (a mixed launch takes 128-row tiles, which wide matrices should not pay for).
   for (int i = 0; i < n;) {
     int j = i + 1;
     if (M >= kPrefillRows && ornith_option_fuse_proj() && ws[i]->mode == ORNITH_LIN_KQUANT) {
-      while (j < n && j - i < 4 && ws[j]->mode == ORNITH_LIN_KQUANT && ws[j]->km.kind == ws[i]->km.kind &&
-             ws[j]->K == ws[i]->K)
+      int cols = ws[i]->O;
+      bool mixed = false;
+      while (j < n && j - i < 4 && ws[j]->mode == ORNITH_LIN_KQUANT && ws[j]->K == ws[i]->K) {
+        const bool other = ws[j]->km.kind != ws[i]->km.kind;
+        if ((other || mixed) && cols + ws[j]->O > 2048) break;
+        mixed = mixed || other;
+        cols += ws[j]->O;
         ++j;
+      }
     }
     int rc;
     if (j - i >= 2) {

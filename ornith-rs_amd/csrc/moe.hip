@@ -182,14 +182,15 @@ int moe_block_prefill(ornith_ctx* ctx, const ornith_moe_weights* w, const void* 
     rc = (e);           \
     if (rc) return rc;  \
   } while (0)
-  TRY(ornith_linear_matmul(ctx, &w->router, d_x, T, gates));
+  {
+    // the router and the shared expert's gate / up read the same rows: one launch where their
+    // formats allow (alone, the 256-column router is 64 workgroups)
+    const ornith_linear* in3[3] = {&w->router, &w->sh_gate, &w->sh_up};
+    void* y3[3] = {gates, sg, su};
+    TRY(ornith_linear_matmul_multi(ctx, in3, 3, d_x, T, y3));
+  }
   TRY(ornith_linear_matmul(ctx, &w->sh_egate, d_x, T, eg));
   TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
-  {
-    const ornith_linear* gu[2] = {&w->sh_gate, &w->sh_up};
-    void* ygu[2] = {sg, su};
-    TRY(ornith_linear_matmul_multi(ctx, gu, 2, d_x, T, ygu));
-  }
   TRY(ornith_swiglu(ctx, sg, su, (int64_t)T * SI, sact));
   TRY(ornith_linear_matmul(ctx, &w->sh_down, sact, T, sy));
   TRY(ornith_kq_gather_matmul(ctx, &w->ex_gate, d_x, inds, pairs, k, 1, plan, 1, xg));

@@ -292,13 +292,16 @@ def test_dense_matmul_vs_float64(orn, ctx, O, K, M):
 
 
 @pytest.mark.parametrize("kind,Os,K,M", [(Q4K, (512, 512), 2048, 4096), (Q6K, (8192, 200, 512), 512, 300),
-                                         (Q4K, (256, 128, 384, 512), 256, 77)])
+                                         (Q4K, (256, 128, 384, 512), 256, 77),
+                                         # both kinds in one launch: the MoE block's router with the shared expert's gate / up
+                                         ((Q6K, Q4K, Q4K), (256, 512, 512), 2048, 4096), ((Q4K, Q6K), (100, 300), 512, 130)])
 def test_projections_sharing_an_input_share_a_gemm_launch(orn, ctx, kind, Os, K, M):
-    """linear_matmul_multi at prefill width: k-quant matrices of one kind and K run as column
-    ranges of one GEMM launch; every output equals the matrix's own launch bit for bit (an output
-    element is one dot product in a fixed k order, whatever tile computes it)"""
+    """linear_matmul_multi at prefill width: k-quant matrices of one K run as column ranges of
+    one GEMM launch; every output equals the matrix's own launch bit for bit (an output element
+    is one dot product in a fixed k order, whatever tile computes it)"""
     rng = np.random.default_rng(sum(Os) + K + M)
-    hls = [util.HostLinear.kq(rng, kind, O, K) for O in Os]
+    kinds = kind if isinstance(kind, tuple) else (kind,) * len(Os)
+    hls = [util.HostLinear.kq(rng, kd, O, K) for kd, O in zip(kinds, Os)]
     lins = [h.dev(orn, ctx) for h in hls]
     xb = util.bf16_normal(rng, (M, K))
     dx = ctx.to_device(xb)
