@@ -368,8 +368,9 @@ def main():
                     help="with --config5: probability-ratio (rejection-sampling) acceptance, or the reference's token equality")
     ap.add_argument("--rng", choices=("philox", "threefry"), default="philox",
                     help="with --config5: the sampler's random stream")
-    ap.add_argument("--prefill-chunk", type=int, default=4096,
-                    help="rows per prefill call with --config5 (the reference's prefill_step_size is 2048; up to 4096 here)")
+    ap.add_argument("--prefill-chunk", type=int, default=8192,
+                    help="rows per prefill call with --config5 (the reference's prefill_step_size is 2048; up to 8192 "
+                         "here: by default the 6621-token prompt is one call)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="with --config5: stop after the first generated token (a short run for "
                          "profiling the matrix-core prefill kernels)")

@@ -504,8 +504,8 @@ ORNITH_API int ornith_text_config_load(const char* model_dir, ornith_text_config
 ORNITH_API int ornith_model_destroy(ornith_model* m);
 /* Rows one forward call may carry (default 16: decode, verify, short prompt chunks). The
  * reference prefills in chunks of prefill_step_size (2048, src/generate.rs:90-136); raise
- * this before creating caches to prefill in chunks that wide. From 32 rows up the
- * k-quant projections and the MoE experts run as matrix-core GEMMs. */
+ * this before creating caches to prefill in chunks that wide (16 .. 8192 rows). From 32
+ * rows up the k-quant projections and the MoE experts run as matrix-core GEMMs. */
 ORNITH_API int ornith_model_set_max_rows(ornith_model* m, int rows);
 /* The MoE block of decoder layer `layer` as the model holds it (pointers into the weight
  * store, valid while the model lives): lets a caller run or time ornith_moe_block /

@@ -345,7 +345,7 @@ int ornith_model_moe_weights(const ornith_model* m, int layer, ornith_moe_weight
 
 int ornith_model_set_max_rows(ornith_model* m, int rows) {
   ORN_REQUIRE(m, "model_set_max_rows: null model");
-  ORN_REQUIRE(rows >= kMaxRows && rows <= 4096, "model_set_max_rows: rows=%d (%d..4096)", rows, kMaxRows);
+  ORN_REQUIRE(rows >= kMaxRows && rows <= 8192, "model_set_max_rows: rows=%d (%d..8192)", rows, kMaxRows);
   if (rows == m->max_rows) return ORNITH_OK;
   TRY(ornith_sync(m->ctx));
   void* buf = nullptr;

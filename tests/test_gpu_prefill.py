@@ -207,14 +207,15 @@ def test_prefill_attention_close_to_exact_kernel(orn, ctx, T, Hq, Hkv, cap, offs
     for b in (dq, dk, dv, dg, dout): b.free()
 
 
-def test_prefill_attention_at_the_long_context_sizes(orn, ctx):
-    """The sampled configuration's sizes: a 4096-row prompt chunk behind 4096 cached rows in a
-    16384-row cache, 16 query heads over 2 KV heads of 256. Checked on 96 sampled (row, head)
-    pairs (first and last rows included) against a float64 softmax attention of the same bf16
-    operands, and for chunk invariance: the same rows in eight 512-row calls agree with the one
-    call to rounding."""
-    T, Hq, Hkv, hd, cap, offset = 4096, 16, 2, 256, 16384, 4096
-    rng = np.random.default_rng(55)
+@pytest.mark.parametrize("T,offset", [(4096, 4096), (6621, 0)])
+def test_prefill_attention_at_the_long_context_sizes(orn, ctx, T, offset):
+    """The sampled configuration's sizes: a 4096-row prompt chunk behind 4096 cached rows, and
+    the whole 6621-row prompt in one call, in a 16384-row cache, 16 query heads over 2 KV heads
+    of 256. Checked on 96 sampled (row, head) pairs (first and last rows included) against a
+    float64 softmax attention of the same bf16 operands, and for chunk invariance: the same rows
+    in 512-row calls agree with the one call to rounding."""
+    Hq, Hkv, hd, cap = 16, 2, 256, 16384
+    rng = np.random.default_rng(55 + offset)
     q = util.bf16_normal(rng, (T, Hq, hd)); qg = util.bf16_normal(rng, (T, Hq, 2 * hd))
     kc = np.full((Hkv, cap, hd), 0x7FC0, np.uint16); vc = np.full((Hkv, cap, hd), 0x7FC0, np.uint16)
     kc[:, :offset + T] = util.bf16_normal(rng, (Hkv, offset + T, hd)); vc[:, :offset + T] = util.bf16_normal(rng, (Hkv, offset + T, hd))
@@ -265,6 +266,31 @@ def test_model_forward_at_the_reference_chunk_width(orn, ctx):
     assert np.isfinite(g).all()
     rel = np.linalg.norm(g - w, axis=1) / np.linalg.norm(w, axis=1)
     assert np.median(rel) < 0.003 and (rel <= 0.02).mean() >= 0.95, (float(np.median(rel)), float(rel.max()))
+    for o in (a, b, model, ws): o.close()
+
+
+def test_model_forward_of_a_whole_long_prompt_in_one_call(orn, ctx):
+    """6621 rows (the sampled configuration's prompt) in one call, ragged against every tile
+    (6621 = 103 * 64 + 29): with bf16-exact weights the result agrees with 512-row calls to
+    summation-order noise, and the cache ends at the same length."""
+    import synth
+    s = synth.SynthModel(synth.TINY, seed=11, with_mtp=False)
+    _make_weights_bf16_exact(s)
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    model.set_max_rows(8192)
+    T = 6621
+    toks = np.random.default_rng(2).integers(0, s.cfg["vocab_size"], T).astype(np.uint32)
+    a, b = model.make_cache(6700, 2), model.make_cache(6700, 2)
+    h1 = model.forward(a, toks)
+    hc = np.concatenate([model.forward(b, toks[i:i + 512]) for i in range(0, T, 512)])
+    assert a.offset == b.offset == T
+    g = util.bf16_to_f32(h1).astype(np.float64); w = util.bf16_to_f32(hc).astype(np.float64)
+    assert np.isfinite(g).all()
+    rel = np.linalg.norm(g - w, axis=1) / np.linalg.norm(w, axis=1)
+    assert np.median(rel) < 0.003 and (rel <= 0.02).mean() >= 0.95, (float(np.median(rel)), float(rel.max()))
+    with pytest.raises(orn.OrnithError, match="rows"):
+        model.set_max_rows(8193)
     for o in (a, b, model, ws): o.close()
 
 
