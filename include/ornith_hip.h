@@ -92,6 +92,9 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *   "gdn_chunked" (ORNITH_GDN_CHUNKED, default 1): the gated-delta recurrence of calls of 128
  *               rows or more (without per-token snapshots) runs in 64-token chunks on the
  *               matrix cores (0: token by token); results agree to rounding
+ *   "gdn_block_chunks" (ORNITH_GDN_BLOCK_CHUNKS, default 64): chunks one prepare / scan launch
+ *               pair of that recurrence covers (longer calls go block by block so that the
+ *               block's operands stay in the last-level cache); same results for any value
  *   "fuse_moe_one" (ORNITH_FUSE_MOE_ONE, default 0): the MoE block's phases as ranges of
  *               workgroups of ONE launch that hand their intermediates over through memory
  *               (1: router + up + down, 2: up + down after a router launch). Bit-identical,

@@ -50,6 +50,7 @@ struct MmArgs {
   const uint32_t* tile_start;  // [tiles] first pair
   const uint32_t* tile_count;  // [tiles] pairs in the tile (<= BM)
   const uint32_t* n_tiles;     // device scalar
+  int sub;                     // workgroups a plan tile takes (plan tiles may be taller than the kernel's)
   int vec;                     // rows of y can be stored 16 bytes at a time
   // further matrices of the same kind and K over the same activations (plain form): the
   // workgroups from column block bx0 on belong to segment i
@@ -265,9 +266,12 @@ __global__ __launch_bounds__(256) void kq_mm_kernel(MmArgs a) {
   int rows_here, m0 = 0;
   int64_t wrow0 = 0;  // first weight row of this tile's matrix
   if constexpr (GATHER) {
-    if (blockIdx.y >= *a.n_tiles) return;
-    const uint32_t e = a.tile_expert[blockIdx.y], st = a.tile_start[blockIdx.y];
-    rows_here = (int)a.tile_count[blockIdx.y];
+    // a plan tile of more rows than BM is worked on by a.sub workgroups, BM rows each
+    const uint32_t tile = blockIdx.y / (uint32_t)a.sub, part = blockIdx.y % (uint32_t)a.sub;
+    if (tile >= *a.n_tiles) return;
+    const uint32_t e = a.tile_expert[tile], st = a.tile_start[tile] + part * BM;
+    rows_here = min((int)a.tile_count[tile] - (int)(part * BM), BM);
+    if (rows_here <= 0) return;
     wrow0 = (int64_t)e * a.O;
     for (int r = tid; r < BM; r += 256) {
       const uint32_t p = r < rows_here ? a.pair[st + r] : 0u;
@@ -1230,24 +1234,27 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   uint32_t* tc = pc.take<uint32_t>(tiles_max);
   uint32_t* nt = pc.take<uint32_t>(1);
   uint32_t* parts = pc.take<uint32_t>((size_t)kSortParts * w->E);
-  // rows per tile (the choice depends only on pairs and E, so the calls sharing a plan agree on
-  // it). Register form: the smallest of 96 / 128 / 160 / 192 rows that holds an expert's share
-  // of the pairs with 2.5 standard deviations to spare, so that nearly every expert is one
-  // tile and its weights are dequantized once. Below about 48 rows an expert, with offsets that
-  // do not fit 32 bits, and with the option off, the LDS form: 128-row tiles from 96 rows an
-  // expert on average (and K >= 1024: with few slabs a tile, three 64-row workgroups a compute
-  // unit hide more than 128-row tiles save), else 64.
+  // Rows per plan tile: the choice depends only on pairs and E (and the option), so the calls
+  // sharing a plan agree on it. With 48 rows an expert or more: the smallest of 96 / 128 / 160 /
+  // 192 rows that holds an expert's share of the pairs with 2.5 standard deviations to spare, so
+  // that nearly every expert is one tile (the register form dequantizes its weights once).
+  // Otherwise 128-row tiles from 96 rows an expert on average, else 64.
   const int avg = pairs / w->E;
   int spare = 0;
   while (4 * spare * spare < 25 * avg) ++spare;
+  const int need = avg + spare;
+  const bool tall = ornith_option_gemm_reg() && avg >= 48;
+  const int tile_rows = tall ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : avg >= 96 ? 128 : 64;
+  // The kernel for this matrix: the register form for tall plans when K >= 1024 (with few K
+  // slabs a workgroup's way in and out, which nothing overlaps at one workgroup a compute unit,
+  // outweighs what that form saves) and its 32-bit offsets reach; otherwise the LDS form, 128
+  // rows a workgroup under the same two conditions on size, else 64 (three 64-row workgroups a
+  // compute unit hide more than 128-row tiles save when a tile has few slabs). A plan tile
+  // taller than that is split over several workgroups.
   const size_t x_bytes = (size_t)(is_up ? pairs / top_k : pairs) * w->K * 2;
   const size_t q_bytes = (size_t)w->E * w->O * (w->K / 256) * (w->kind == ORNITH_Q4K ? 128 : 192);
-  // (with few K slabs a workgroup's way in and out, which nothing overlaps at one workgroup a
-  // compute unit, outweighs what the register form saves: K >= 1024 only)
-  const bool reg = ornith_option_gemm_reg() && avg >= 48 && w->K >= 1024 && x_bytes < (size_t(1) << 32) &&
-                   q_bytes < (size_t(1) << 32);
-  const int need = avg + spare;
-  const int tile_rows = reg ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : (avg >= 96 && w->K >= 1024) ? 128 : 64;
+  const bool reg = tall && w->K >= 1024 && x_bytes < (size_t(1) << 32) && q_bytes < (size_t(1) << 32);
+  const int lds_rows = (avg >= 96 && w->K >= 1024) ? 128 : 64;
   if (rebuild_plan && pairs >= 8192) {
     hipLaunchKernelGGL(moe_sort_count_kernel, dim3(kSortParts), dim3(256), 0, ctx->stream, d_inds, pairs, w->E, parts);
     hipLaunchKernelGGL(moe_sort_plan_kernel, dim3(1), dim3(1024), 0, ctx->stream, w->E, tile_rows, parts, te, ts, tc, nt);
@@ -1284,8 +1291,9 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
     ORN_LAUNCH_CHECK("kq_mm_reg_kernel<gather>");
     return ORNITH_OK;
   }
-  const dim3 grid((w->O + BN - 1) / BN, (unsigned)tiles_max);
-  if (tile_rows == 128) {
+  a.sub = (tile_rows + lds_rows - 1) / lds_rows;
+  const dim3 grid((w->O + BN - 1) / BN, (unsigned)(tiles_max * a.sub));
+  if (lds_rows == 128) {
     if (w->kind == ORNITH_Q4K)
       hipLaunchKernelGGL((kq_mm_kernel<ORNITH_Q4K, 128, true>), grid, dim3(256), 0, ctx->stream, a);
     else

@@ -188,3 +188,30 @@ def test_chunked_recurrence_over_hard_decays(orn, ctx, T, decay):
         outs[chunked] = gy
     orn.set_option("gdn_chunked", 1)
     assert not np.array_equal(outs[0], outs[1])        # two different kernels did run
+
+
+def test_chunked_recurrence_block_by_block_is_the_same_recurrence(orn, ctx):
+    """Long calls of the chunked form go through the prepare / scan kernels in blocks of chunks
+    with the state handed on: blocks of 2 chunks, of 3 (a ragged last block) and one block give
+    the same outputs and final state bit for bit (a chunk's arithmetic does not depend on the
+    block it is launched in)."""
+    rng = np.random.default_rng(77)
+    T, Hk, Hv = 531, 2, 4
+    q = util.bf16_normal(rng, (T, Hk, 128), 0.1); k = util.bf16_normal(rng, (T, Hk, 128), 0.1)
+    v = util.bf16_normal(rng, (T, Hv, 128))
+    beta = util.f32_to_bf16(rng.random((T, Hv)).astype(np.float32))
+    g = (0.9 + 0.1 * rng.random((T, Hv))).astype(np.float32)
+    S0 = (rng.standard_normal((Hv, 128, 128)) * 0.1).astype(np.float32)
+    outs = []
+    try:
+        for blk in (64, 2, 3):
+            orn.set_option("gdn_block_chunks", blk)
+            d = [ctx.to_device(a) for a in (q, k, v, g, beta, S0)]
+            y, fin = ctx.alloc(T * Hv * 128 * 2), ctx.alloc(Hv * 128 * 128 * 4)
+            ctx.gdn_recurrence(*d, T, Hk, Hv, 128, 128, y, fin, snap_all=False)
+            outs.append((y.download(np.uint16, (T, Hv, 128)), fin.download(np.float32, (Hv, 128, 128))))
+            for b in d + [y, fin]: b.free()
+    finally:
+        orn.set_option("gdn_block_chunks", 64)
+    for gy, gs in outs[1:]:
+        assert np.array_equal(gy, outs[0][0]) and np.array_equal(gs, outs[0][1])

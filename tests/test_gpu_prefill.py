@@ -101,8 +101,10 @@ def _rows_close(got_bits, want_bits, tol):
 
 
 @pytest.mark.parametrize("H,E,I,T", [(512, 64, 256, 48), (2048, 256, 512, 160),
-                                     # 64 and 150 rows an expert: the gathered GEMM's register form
-                                     (512, 64, 256, 512), (512, 64, 256, 1200)])
+                                     # 64 and 150 rows an expert: tall plan tiles, split over 64-row workgroups
+                                     (512, 64, 256, 512), (512, 64, 256, 1200),
+                                     # gate / up in the register form (K = 1024), down on the same plan in 64-row workgroups
+                                     (1024, 64, 256, 512), (1024, 64, 256, 1300)])
 def test_moe_block_prefill_width_close_to_exact_path(orn, ctx, H, E, I, T):
     """At prefill width the block runs as GEMMs. Against the oracle's exact path the rows agree
     to 2 % relative L2 (bf16 weights on the matrix cores, fp32 sums in another order); a row
