@@ -362,3 +362,30 @@ def test_dense_projections_sharing_an_input_share_a_launch(orn, ctx, Os, K, M):
         assert np.array_equal(y.download(np.uint16, (M, O)), y1.download(np.uint16, (M, O))), O
     for b in [dx, y1] + ys: b.free()
     for l in lins: l.free()
+
+
+def test_gathered_matmuls_of_different_depth_share_a_plan(orn, ctx):
+    """The MoE block builds the pair plan with its gate projection (K = 1024 here: tall tiles,
+    register form) and runs the down projection (K = 256: 64-row workgroups) on the same plan
+    without rebuilding it: every pair's row must be computed, whatever the kernel's own tile
+    height (outputs poisoned beforehand)."""
+    rng = np.random.default_rng(12)
+    E, T, k, Kg, Og, Kd, Od = 64, 700, 8, 1024, 256, 256, 384
+    pairs = T * k
+    tg, td = util.make_kq(Q4K, rng, E, Og, Kg), util.make_kq(Q6K, rng, E, Od, Kd)
+    wg, wd = orn.KMatrix(ctx, Q4K, *tg, E, Og, Kg), orn.KMatrix(ctx, Q6K, *td, E, Od, Kd)
+    inds = np.stack([rng.permutation(E)[:k] for _ in range(T)]).astype(np.uint32)
+    plan = ctx.alloc(orn.kq_gather_plan_bytes(pairs, E)); di = ctx.to_device(inds.reshape(-1))
+    xb = util.bf16_normal(rng, (T, Kg)); ab = util.bf16_normal(rng, (pairs, Kd))
+    dx, da = ctx.to_device(xb), ctx.to_device(ab)
+    dyg, dyd = ctx.alloc(pairs * Og * 2), ctx.alloc(pairs * Od * 2)
+    ctx.memset(dyg, 0xFF, pairs * Og * 2); ctx.memset(dyd, 0xFF, pairs * Od * 2)
+    orn.kq_gather_matmul(ctx, wg, dx, di, pairs, k, True, plan, True, dyg)
+    orn.kq_gather_matmul(ctx, wd, da, di, pairs, k, False, plan, False, dyd)
+    flat = inds.reshape(-1)
+    dg, dd = _deq_bf16(Q4K, tg, E, Og, Kg), _deq_bf16(Q6K, td, E, Od, Kd)
+    xf, af = util.bf16_to_f32(xb).astype(np.float64), util.bf16_to_f32(ab).astype(np.float64)
+    _check(dyg.download(np.uint16, (pairs, Og)), np.stack([xf[p // k] @ dg[flat[p]].T for p in range(pairs)]), Kg, "gate")
+    _check(dyd.download(np.uint16, (pairs, Od)), np.stack([af[p] @ dd[flat[p]].T for p in range(pairs)]), Kd, "down")
+    for b in (plan, di, dx, da, dyg, dyd): b.free()
+    wg.free(); wd.free()
