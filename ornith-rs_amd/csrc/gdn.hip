@@ -135,8 +135,16 @@ __global__ __launch_bounds__(64) void gdn_front_run_kernel(FrontArgs p) {
   }
   const bool is_qk = slot < 2 * p.Hk, is_q = slot < p.Hk;
   const float sc = is_q ? p.q_scale : p.k_scale;
-  for (int t = t0; t < t1; ++t) {
-    win[S] = input(t + S);  // = qkv[t]
+  // the run's inputs are asked for together (one after the other, every token would wait out a
+  // memory latency of its own); rows past the end of the call read the last row, unused
+  uint32_t in[kFrontRun];
+#pragma unroll
+  for (int u = 0; u < kFrontRun; ++u) in[u] = input(min(t0 + u, p.T - 1) + S);
+#pragma unroll
+  for (int u = 0; u < kFrontRun; ++u) {
+    const int t = t0 + u;
+    if (t >= t1) break;
+    win[S] = in[u];  // = qkv[t]
     float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
     for (int i = 0; i < K; ++i) {
