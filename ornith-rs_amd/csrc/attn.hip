@@ -19,6 +19,8 @@
 // A query row only ever sees keys at or before its own position, and blocks are
 // aligned to absolute positions, so row r of a T-row verify call is bit-identical
 // to a one-row call at that position.
+#include <type_traits>
+
 #include "dmath.h"
 #include "rt.h"
 
@@ -293,91 +295,187 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
 }
 
 // The same partial sums when there are many blocks to work through (long contexts): 256
-// threads and little LDS a block, so that several blocks are resident per compute unit and
-// hide each other's trips to memory. Thread `tid` owns key `tid` for the scores and channel
-// `tid` for the values and runs the chains of 64 one after the other.
-// grid (nblk, Hq, T), 256 threads.
-template <int HD>
+// threads a block, several blocks resident per compute unit. A workgroup takes NH query heads
+// of one KV group (four when the group allows it): the key and value block is then read once
+// for the four instead of once a head (with one head a workgroup the L2 delivered every block
+// 32 times for 8 heads a group and 4 rows, 440 MB a call at a 6.6 k context, and that, not
+// HBM or the arithmetic, set the time). Thread `tid` owns key `tid` for the scores and runs
+// the chains of 64 channels one after the other; the key block reaches it through LDS, 64
+// channels at a time, so that the global loads are whole 128-byte pieces of a row. For the
+// values a thread owns four channels of one 64-key chain (8-byte loads, a wavefront reads 512
+// contiguous bytes a key); the four chains of a channel meet in LDS. Every sum of every head
+// keeps its order. grid (nblk, Hq / NH, T), 256 threads.
+template <int HD, int NH>
 __global__ __launch_bounds__(256) void sdpa_partial_many_kernel(SdpaArgs p) {
-  const int b = blockIdx.x, hq = blockIdx.y, t = blockIdx.z, tid = threadIdx.x;
+  const int b = blockIdx.x, hq0 = blockIdx.y * NH, t = blockIdx.z, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int offset = p.d_offset ? *p.d_offset : p.offset;
   const int last = min(offset + t, p.cap - 1);
   if (b * ATT_KB > last) return;
-  const int hk = hq / (p.Hq / p.Hkv);
-  constexpr int NKC = HD / 64, NVB = ATT_KB / 64;
+  const int hk = hq0 / (p.Hq / p.Hkv);  // the NH heads share it
+  constexpr int NKC = HD / 64, NVB = ATT_KB / 64, KLD = 64 + 8;
+  static_assert(ATT_KB == 256, "one key per thread");
+  static_assert(NKC == 2 || NKC == 4, "head widths of 128 and 256");
 
-  __shared__ __align__(16) float qs[HD];
-  __shared__ float pr[ATT_KB];
-  __shared__ float red[4];
+  __shared__ __align__(16) bf16_t ks[ATT_KB][KLD];
+  __shared__ __align__(16) float qs[NH][HD];
+  __shared__ float pr[NH][ATT_KB];
+  __shared__ float red[NH][4];
+  __shared__ float part[NH][NVB * HD];
 
   const int key = b * ATT_KB + tid;
   const bool valid = key <= last;
   const int nvalid = min(ATT_KB, last - b * ATT_KB + 1);
-  const bf16_t* krow = p.k_cache + ((size_t)hk * p.cap + (valid ? key : last)) * HD;
+  const bf16_t* kblk = p.k_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD;
 
-  for (int d = tid; d < HD; d += 256) qs[d] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq) * HD + d]);
-  __syncthreads();
-  float cpart[NKC];
+  // 64-channel panel c of the key block: 2048 16-byte pieces, eight a thread (rows past the
+  // last key read the last key's: their scores are masked). Two panels travel in registers
+  // ahead of their use, and so do the first 32 keys of this thread's value chain: a block is a
+  // chain of memory latencies otherwise.
+  u32x4 kreg[2][8];
+  auto fetch_panel = [&](auto set, int c) {
+    constexpr int S = decltype(set)::value;
 #pragma unroll
-  for (int c = 0; c < NKC; ++c) {
-    float a = 0.f;
-#pragma unroll 4
-    for (int dc = 8 * c; dc < 8 * c + 8; ++dc) {
-      const uint4 kw = *reinterpret_cast<const uint4*>(krow + 8 * dc);
-      const float4 q0 = *reinterpret_cast<const float4*>(&qs[8 * dc]);
-      const float4 q1 = *reinterpret_cast<const float4*>(&qs[8 * dc + 4]);
-      a = dm_fma(q0.x, dm_bf2f_lo(kw.x), a);
-      a = dm_fma(q0.y, dm_bf2f_hi(kw.x), a);
-      a = dm_fma(q0.z, dm_bf2f_lo(kw.y), a);
-      a = dm_fma(q0.w, dm_bf2f_hi(kw.y), a);
-      a = dm_fma(q1.x, dm_bf2f_lo(kw.z), a);
-      a = dm_fma(q1.y, dm_bf2f_hi(kw.z), a);
-      a = dm_fma(q1.z, dm_bf2f_lo(kw.w), a);
-      a = dm_fma(q1.w, dm_bf2f_hi(kw.w), a);
+    for (int u = 0; u < 8; ++u) {
+      const int idx = tid + 256 * u, r = min(idx >> 3, nvalid - 1), part8 = idx & 7;
+      kreg[S][u] = *reinterpret_cast<const u32x4*>(kblk + (size_t)r * HD + 64 * c + 8 * part8);
     }
-    cpart[c] = a;
+  };
+  using S0 = std::integral_constant<int, 0>;
+  using S1 = std::integral_constant<int, 1>;
+  fetch_panel(S0{}, 0);
+  fetch_panel(S1{}, 1);
+  constexpr int TPC = HD / 4;  // threads a value chain
+  const int vg = tid / TPC, vcg = tid % TPC;
+  const bf16_t* vcol = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB + 64 * vg) * HD + 4 * vcg;
+  const int vn = min(64, nvalid - 64 * vg);  // keys of this thread's chain that exist (may be <= 0)
+  uint2 vreg[2][16];
+  auto fetch_values = [&](auto set, int i0) {
+    constexpr int S = decltype(set)::value;
+    if (tid < HD) {
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        vreg[S][u] = *reinterpret_cast<const uint2*>(vcol + (size_t)min(i0 + u, max(vn - 1, 0)) * HD);
+    }
+  };
+  fetch_values(S0{}, 0);
+  fetch_values(S1{}, 16);
+  for (int i = tid; i < NH * HD; i += 256)
+    qs[i / HD][i % HD] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq0 + i / HD) * HD + i % HD]);
+  float cpart[NH][NKC];
+  auto panel = [&](auto set, auto cc) {
+    constexpr int S = decltype(set)::value, c = decltype(cc)::value;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int idx = tid + 256 * u;
+      *reinterpret_cast<u32x4*>(&ks[idx >> 3][8 * (idx & 7)]) = kreg[S][u];
+    }
+    __syncthreads();
+    if constexpr (c + 2 < NKC) fetch_panel(set, c + 2);
+    float a[NH];
+#pragma unroll
+    for (int j = 0; j < NH; ++j) a[j] = 0.f;
+#pragma unroll
+    for (int dc = 0; dc < 8; ++dc) {
+      const uint4 kw = *reinterpret_cast<const uint4*>(&ks[tid][8 * dc]);
+      const float k0 = dm_bf2f_lo(kw.x), k1 = dm_bf2f_hi(kw.x), k2 = dm_bf2f_lo(kw.y), k3 = dm_bf2f_hi(kw.y);
+      const float k4 = dm_bf2f_lo(kw.z), k5 = dm_bf2f_hi(kw.z), k6 = dm_bf2f_lo(kw.w), k7 = dm_bf2f_hi(kw.w);
+#pragma unroll
+      for (int j = 0; j < NH; ++j) {
+        const float4 q0 = *reinterpret_cast<const float4*>(&qs[j][64 * c + 8 * dc]);
+        const float4 q1 = *reinterpret_cast<const float4*>(&qs[j][64 * c + 8 * dc + 4]);
+        a[j] = dm_fma(q0.x, k0, a[j]);
+        a[j] = dm_fma(q0.y, k1, a[j]);
+        a[j] = dm_fma(q0.z, k2, a[j]);
+        a[j] = dm_fma(q0.w, k3, a[j]);
+        a[j] = dm_fma(q1.x, k4, a[j]);
+        a[j] = dm_fma(q1.y, k5, a[j]);
+        a[j] = dm_fma(q1.z, k6, a[j]);
+        a[j] = dm_fma(q1.w, k7, a[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NH; ++j) cpart[j][c] = a[j];
+    __syncthreads();
+  };
+  panel(S0{}, std::integral_constant<int, 0>{});
+  panel(S1{}, std::integral_constant<int, 1>{});
+  if constexpr (NKC > 2) {
+    panel(S0{}, std::integral_constant<int, 2>{});
+    panel(S1{}, std::integral_constant<int, 3>{});
   }
-  const float sc = sdpa_pair_tree<NKC>(cpart, 1);
-  // block max
-  {
-    const float m = dm_wave_max<64>(valid ? sc : -DM_INF);
-    if (lane == 0) red[wave] = m;
+  float sc[NH], mg[NH];
+#pragma unroll
+  for (int j = 0; j < NH; ++j) {
+    sc[j] = sdpa_pair_tree<NKC>(cpart[j], 1);
+    const float m = dm_wave_max<64>(valid ? sc[j] : -DM_INF);  // block max
+    if (lane == 0) red[j][wave] = m;
   }
   __syncthreads();
-  float mg = red[0];
-  mg = red[1] > mg ? red[1] : mg;
-  mg = red[2] > mg ? red[2] : mg;
-  mg = red[3] > mg ? red[3] : mg;
+#pragma unroll
+  for (int j = 0; j < NH; ++j) {
+    float m = red[j][0];
+    m = red[j][1] > m ? red[j][1] : m;
+    m = red[j][2] > m ? red[j][2] : m;
+    m = red[j][3] > m ? red[j][3] : m;
+    mg[j] = m;
+  }
   __syncthreads();
-  {
-    const float pv = valid ? dm_exp(sc - mg) : 0.f;
-    pr[tid] = pv;
+#pragma unroll
+  for (int j = 0; j < NH; ++j) {
+    const float pv = valid ? dm_exp(sc[j] - mg[j]) : 0.f;
+    pr[j][tid] = pv;
     const float ws = dm_wave_sum<64>(pv);
-    if (lane == 0) red[wave] = ws;
+    if (lane == 0) red[j][wave] = ws;
   }
   __syncthreads();
-  // values: channel `tid`, one chain per 64 keys
-  const size_t pi = ((size_t)t * p.Hq + hq) * p.nblk + b;
+  // values: chain vg = keys 64 * vg .. + 64, channels 4 * vcg .. + 4, for every head
   if (tid < HD) {
-    const bf16_t* vcol = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + tid;
-    float opart[NVB];
+    float o[NH][4];
 #pragma unroll
-    for (int g = 0; g < NVB; ++g) {
-      float o = 0.f;
-      const int end = min(64 * g + 64, nvalid);
-#pragma unroll 8
-      for (int i = 64 * g; i < end; ++i) o = dm_fma(pr[i], dm_bf2f(vcol[(size_t)i * HD]), o);
-      opart[g] = o;
-    }
-    p.part_o[pi * HD + tid] = sdpa_pair_tree<NVB>(opart, 1);
+    for (int j = 0; j < NH; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[j][e] = 0.f;
+    auto batch = [&](auto set, int i0) {
+      constexpr int S = decltype(set)::value;
+#pragma unroll
+      for (int u = 0; u < 16; ++u)
+        if (i0 + u < vn) {
+          const float v0 = dm_bf2f_lo(vreg[S][u].x), v1 = dm_bf2f_hi(vreg[S][u].x);
+          const float v2 = dm_bf2f_lo(vreg[S][u].y), v3 = dm_bf2f_hi(vreg[S][u].y);
+#pragma unroll
+          for (int j = 0; j < NH; ++j) {
+            const float pw = pr[j][64 * vg + i0 + u];
+            o[j][0] = dm_fma(pw, v0, o[j][0]);
+            o[j][1] = dm_fma(pw, v1, o[j][1]);
+            o[j][2] = dm_fma(pw, v2, o[j][2]);
+            o[j][3] = dm_fma(pw, v3, o[j][3]);
+          }
+        }
+    };
+    batch(S0{}, 0);
+    fetch_values(S0{}, 32);
+    batch(S1{}, 16);
+    fetch_values(S1{}, 48);
+    batch(S0{}, 32);
+    batch(S1{}, 48);
+#pragma unroll
+    for (int j = 0; j < NH; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) part[j][vg * HD + 4 * vcg + e] = o[j][e];
   }
-  if (tid == 0) {
-    float l = red[0] + red[1];
-    l = l + red[2];
-    l = l + red[3];
-    p.part_m[pi] = mg;
-    p.part_l[pi] = l;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < NH; ++j) {
+    const size_t pi = ((size_t)t * p.Hq + hq0 + j) * p.nblk + b;
+    if (tid < HD) p.part_o[pi * HD + tid] = sdpa_pair_tree<NVB>(part[j] + tid, HD);
+    if (tid == 0) {
+      float l = red[j][0] + red[j][1];
+      l = l + red[j][2];
+      l = l + red[j][3];
+      p.part_m[pi] = mg[j];
+      p.part_l[pi] = l;
+    }
   }
 }
 
@@ -392,10 +490,23 @@ __global__ __launch_bounds__(HD) void sdpa_merge_kernel(SdpaArgs p) {
   float M = -DM_INF;
   for (int b = 0; b < nb; ++b) M = p.part_m[pi + b] > M ? p.part_m[pi + b] : M;
   float L = 0.f, O = 0.f;
-  for (int b = 0; b < nb; ++b) {
-    const float w = dm_exp(p.part_m[pi + b] - M);
-    L = dm_fma(p.part_l[pi + b], w, L);
-    O = dm_fma(p.part_o[(pi + b) * HD + d], w, O);
+  // eight blocks' partial sums are asked for together (the sums keep their ascending order)
+  for (int b0 = 0; b0 < nb; b0 += 8) {
+    float pm[8], pl[8], po[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int b = min(b0 + u, nb - 1);
+      pm[u] = p.part_m[pi + b];
+      pl[u] = p.part_l[pi + b];
+      po[u] = p.part_o[(pi + b) * HD + d];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (b0 + u < nb) {
+        const float w = dm_exp(pm[u] - M);
+        L = dm_fma(pl[u], w, L);
+        O = dm_fma(po[u], w, O);
+      }
   }
   const float att = dm_rb(O / L);
   const float g = dm_sigmoid_bf16(dm_bf2f(p.qg[((size_t)t * p.Hq + h) * 2 * HD + HD + d]));
@@ -522,11 +633,19 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   const long live = (long)(last_max / ATT_KB + 1) * Hq * T;
   // one key block for every row (and the kernel form that knows how): no merge launch
   p.finish = (last_max < ATT_KB && live <= 2L * ctx->compute_units) ? 1 : 0;
-  if (live > 2L * ctx->compute_units) {
-    if (hd == 256)
-      hipLaunchKernelGGL((sdpa_partial_many_kernel<256>), grid, dim3(256), 0, ctx->stream, p);
-    else
-      hipLaunchKernelGGL((sdpa_partial_many_kernel<128>), grid, dim3(256), 0, ctx->stream, p);
+  // four heads of a KV group a workgroup (the key / value block read once for the four) from a
+  // workgroup for every fourth compute unit on: 25.6 us against 35.4 for one row at a 6.6 k
+  // context (108 workgroups), 22.4 against 14.3 at 3 k (48)
+  const bool four = (Hq / Hkv) % 4 == 0 && live / 4 >= ctx->compute_units / 4;
+  if (live > 2L * ctx->compute_units || four) {
+    const dim3 g4(nblk, Hq / 4, T);
+    if (hd == 256) {
+      if (four) hipLaunchKernelGGL((sdpa_partial_many_kernel<256, 4>), g4, dim3(256), 0, ctx->stream, p);
+      else hipLaunchKernelGGL((sdpa_partial_many_kernel<256, 1>), grid, dim3(256), 0, ctx->stream, p);
+    } else {
+      if (four) hipLaunchKernelGGL((sdpa_partial_many_kernel<128, 4>), g4, dim3(256), 0, ctx->stream, p);
+      else hipLaunchKernelGGL((sdpa_partial_many_kernel<128, 1>), grid, dim3(256), 0, ctx->stream, p);
+    }
   } else if (hd == 256) {
     // 150 KB of LDS a block (the whole key block staged at once): asked for once per kernel
     static bool lds_set = false;

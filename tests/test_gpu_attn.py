@@ -23,6 +23,8 @@ def _mk(rng, T, Hq, Hkv, hd, cap, offset):
     (3, 4, 1, 256, 512, 0), (2, 4, 2, 128, 768, 300), (1, 2, 2, 256, 256, 7),
     # many live key blocks: the launch switches to its 256-thread form (same sums)
     (4, 16, 2, 256, 4096, 4000), (4, 16, 2, 128, 4096, 3000),
+    # ... with one head a workgroup (KV groups of three heads) and four (groups of eight, ragged last block)
+    (8, 6, 2, 256, 8192, 8000), (3, 16, 2, 256, 8192, 7000),
     # the long-context configuration: a depth-3 verify window at the end of a 16384-row cache
     (4, 16, 2, 256, 16384, 16380), (1, 16, 2, 256, 16384, 6621)])
 def test_attention_bit_exact(orn, ctx, T, Hq, Hkv, hd, cap, offset):
