@@ -361,14 +361,15 @@ int launch_m(ornith_ctx* ctx, KqArgs& a, int M) {
 // rows each wavefront walks: the kernels are bound by VALU issue and by latency, not by
 // HBM, so the converted activations are amortised over as many rows as still leaves
 // about three workgroups per compute unit (measured optimum on 256 CUs for 0.4..55 MB).
-int pick_iters(const ornith_ctx* ctx, int kind, int K, long total_rows, int grid_y) {
+int pick_iters(const ornith_ctx* ctx, int kind, int K, long total_rows, int grid_y, int M = 1) {
   if (const int forced = ornith_option_kq_iters()) return forced > 8 ? 8 : forced;
   const int nch = (K >> 8) * (kind == ORNITH_Q4K ? 8 : 4);
   const int lpr = nch >= 64 ? 64 : nch;
   const int ks = nch > 64 ? 2 : 1;
   const int rows_per_pass = (64 / lpr) * (4 / ks);  // rows a block covers per iteration
   const long blocks_at_1 = (total_rows + rows_per_pass - 1) / rows_per_pass * grid_y;
-  const long want = (long)ctx->compute_units * 3;
+  // (three or four activation rows: twice the conversion work to spread, half the workgroups)
+  const long want = M >= 3 ? (long)ctx->compute_units * 3 / 2 : (long)ctx->compute_units * 3;
   int iters = (int)(blocks_at_1 / want);
   if (iters < 1) iters = 1;
   if (iters > 8) iters = 8;
@@ -454,7 +455,7 @@ int kq_qmv_multi_prenorm(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n
   a.nseg = n;
   a.K = kPreN;
   a.y_bf16 = 1;
-  a.iters = pick_iters(ctx, ws[0]->kind, kPreN, total, 1);
+  a.iters = pick_iters(ctx, ws[0]->kind, kPreN, total, 1, M);
   for (int s = 0; s < n; ++s) {
     a.seg[s].qs = (const uint8_t*)ws[s]->d_qs;
     a.seg[s].scales = (const uint8_t*)ws[s]->d_scales;
@@ -490,7 +491,7 @@ int ornith_kq_qmv_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n,
   a.nseg = n;
   a.K = K;
   a.y_bf16 = y_dtype == ORNITH_BF16;
-  a.iters = pick_iters(ctx, kind, K, total, 1);
+  a.iters = pick_iters(ctx, kind, K, total, 1, M < 4 ? M : 4);
   for (int m0 = 0; m0 < M; m0 += 4) {
     const int mw = M - m0 < 4 ? M - m0 : 4;
     a.x = (const char*)d_x + (size_t)m0 * K * xs;
