@@ -631,13 +631,15 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   // soonest; many: the 256-thread form keeps more blocks in flight. Same sums either way.
   const int last_max = (d_offset ? cap - 1 : (offset + T - 1 < cap - 1 ? offset + T - 1 : cap - 1));
   const long live = (long)(last_max / ATT_KB + 1) * Hq * T;
-  // one key block for every row (and the kernel form that knows how): no merge launch
-  p.finish = (last_max < ATT_KB && live <= 2L * ctx->compute_units) ? 1 : 0;
   // four heads of a KV group a workgroup (the key / value block read once for the four) from a
   // workgroup for every fourth compute unit on: 25.6 us against 35.4 for one row at a 6.6 k
   // context (108 workgroups), 22.4 against 14.3 at 3 k (48)
-  const bool four = (Hq / Hkv) % 4 == 0 && live / 4 >= ctx->compute_units / 4;
-  if (live > 2L * ctx->compute_units || four) {
+  // (inside the first key block the finishing form is one launch instead of two)
+  const bool four = (Hq / Hkv) % 4 == 0 && live / 4 >= ctx->compute_units / 4 && last_max >= ATT_KB;
+  const bool many = live > 2L * ctx->compute_units || four;
+  // one key block for every row, in the kernel form that knows how to finish: no merge launch
+  p.finish = (last_max < ATT_KB && !many) ? 1 : 0;
+  if (many) {
     const dim3 g4(nblk, Hq / 4, T);
     if (hd == 256) {
       if (four) hipLaunchKernelGGL((sdpa_partial_many_kernel<256, 4>), g4, dim3(256), 0, ctx->stream, p);

@@ -25,6 +25,9 @@ def _mk(rng, T, Hq, Hkv, hd, cap, offset):
     (4, 16, 2, 256, 4096, 4000), (4, 16, 2, 128, 4096, 3000),
     # ... with one head a workgroup (KV groups of three heads) and four (groups of eight, ragged last block)
     (8, 6, 2, 256, 8192, 8000), (3, 16, 2, 256, 8192, 7000),
+    # 16-row prompt chunks inside the first key block (one finishing launch) and across its end
+    # (enough rows for the four-head form, which leaves the finishing to the merge launch)
+    (16, 16, 2, 256, 4096, 35), (16, 16, 2, 128, 4096, 0), (16, 16, 2, 256, 4096, 250),
     # the long-context configuration: a depth-3 verify window at the end of a 16384-row cache
     (4, 16, 2, 256, 16384, 16380), (1, 16, 2, 256, 16384, 6621)])
 def test_attention_bit_exact(orn, ctx, T, Hq, Hkv, hd, cap, offset):
