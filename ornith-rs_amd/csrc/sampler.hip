@@ -101,14 +101,15 @@ __global__ __launch_bounds__(RB) void radix_hist_kernel(const bf16_t* x, int neg
 
 // in-place exclusive scan of m counters by one workgroup, in tiles of 1024 consecutive
 // counters (coalesced). Up to 64 tiles are fetched into registers before the first is
-// scanned, so the walk over the tiles never waits on memory.
+// scanned, so the walk over the tiles never waits on memory. One barrier a tile: the
+// wavefront totals of consecutive tiles alternate between two LDS rows, and every thread keeps
+// the running total itself.
 __global__ __launch_bounds__(RB) void radix_scan_kernel(uint32_t* table, int m) {
-  __shared__ uint32_t wtot[RB / 64];
-  __shared__ uint32_t s_carry;
+  constexpr int NW = RB / 64;
+  __shared__ uint32_t wtot[2][NW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) s_carry = 0;
-  __syncthreads();
   constexpr int G = 64;
+  uint32_t carry = 0;
   for (int t0 = 0; t0 * RB < m; t0 += G) {
     uint32_t v[G];
 #pragma unroll
@@ -126,16 +127,20 @@ __global__ __launch_bounds__(RB) void radix_scan_kernel(uint32_t* table, int m) 
         const uint32_t o = __shfl_up(x, d, 64);
         if (lane >= d) x += o;
       }
-      if (lane == 63) wtot[wave] = x;
+      if (lane == 63) wtot[t & 1][wave] = x;
       __syncthreads();
-      uint32_t before = s_carry;
-      for (int w = 0; w < wave; ++w) before += wtot[w];
+      uint32_t before = carry, total = 0;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const uint32_t c = wtot[t & 1][w];
+        before += w < wave ? c : 0u;
+        total += c;
+      }
       const int j = (t0 + t) * RB + tid;
       if (j < m) table[j] = before + x - v[t];
-      __syncthreads();
-      if (tid == RB - 1) s_carry = before + x;
-      __syncthreads();
+      carry += total;
     }
+    __syncthreads();  // (G is even: the next round starts on row 0 again, which tile G - 2 used)
   }
 }
 
