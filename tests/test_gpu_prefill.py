@@ -389,3 +389,36 @@ def test_gathered_matmuls_of_different_depth_share_a_plan(orn, ctx):
     _check(dyd.download(np.uint16, (pairs, Od)), np.stack([af[p] @ dd[flat[p]].T for p in range(pairs)]), Kd, "down")
     for b in (plan, di, dx, da, dyg, dyd): b.free()
     wg.free(); wd.free()
+
+
+def test_prefill_paths_are_repeatable(orn, ctx):
+    """The same MoE block call and the same model forward twice give the same bits: the expert
+    plan is built with atomics (the order of an expert's pairs changes from run to run), so a row
+    that depended on its place in a tile, or a tile row left uncomputed, shows up here as a
+    difference between runs."""
+    import synth
+    rng = np.random.default_rng(21)
+    moe = util.HostMoe(rng, H=1024, E=64, I=256, top_k=8, gate_kind=Q4K, down_kind=Q6K, router_kind=Q6K)
+    dw = moe.dev(orn, ctx)
+    T = 1300
+    xb = util.bf16_normal(rng, (T, 1024))
+    dx, dout = ctx.to_device(xb), ctx.alloc(T * 1024 * 2)
+    outs = []
+    for fill in (0x00, 0xFF, 0x5A):
+        ctx.memset(dout, fill, T * 1024 * 2)
+        ctx.moe_block(dw, dx, T, dout)
+        outs.append(dout.download(np.uint16, (T, 1024)))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    dx.free(); dout.free(); moe.free()
+    s = synth.SynthModel(synth.TINY, seed=13, with_mtp=False)
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    model.set_max_rows(2048)
+    toks = np.random.default_rng(3).integers(0, s.cfg["vocab_size"], 1500).astype(np.uint32)
+    cache = model.make_cache(1600, 2)
+    hs = []
+    for _ in range(3):
+        cache.reset()
+        hs.append(model.forward(cache, toks))
+    assert np.array_equal(hs[0], hs[1]) and np.array_equal(hs[0], hs[2])
+    for o in (cache, model, ws): o.close()
