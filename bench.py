@@ -294,6 +294,45 @@ def moe_ab(orn, ctx, model, np, n_layers):
     print(json.dumps({"moe_block_launch_structure": rows}), flush=True)
 
 
+def warm_cold(orn, ctx, np):
+    """What a mat-vec gains when its weights were read just before by another kernel (they then
+    sit in the memory-side cache, not in the L2 of the die that needs them), against weights
+    nobody read (cycling over > 600 MB of copies) and against one matrix re-used by every launch
+    (warm in its own dies' L2). The read before is `ornith_copy` of the code bytes; the setting
+    `other` runs the same copy on a matrix that is not used next, so `other` - `touch` is the gain
+    and `none` shows what the copy itself costs in this loop. Prints a JSON table."""
+    import util
+    rng = np.random.default_rng(0)
+    scratch = ctx.alloc(64 << 20)
+    rows = []
+    for name, kind, O, K in (("in_proj 12288x2048 Q4_K", util.Q4K, 12288, 2048), ("out_proj 2048x4096 Q4_K", util.Q4K, 2048, 4096),
+                             ("q_proj 8192x2048 Q6_K", util.Q6K, 8192, 2048)):
+        t = util.make_kq(kind, rng, 1, O, K)
+        ncopy = int(600e6 // sum(a.nbytes for a in t)) + 1
+        mats = [orn.KMatrix(ctx, kind, *t, 1, O, K) for _ in range(ncopy)]
+        qbytes = t[0].nbytes
+        for M in (1, 2):
+            x = ctx.to_device(util.bf16_normal(rng, (M, K)))
+            y = ctx.alloc(M * O * 2)
+
+            def run(i, mode):
+                m = mats[0] if mode == "same" else mats[i % ncopy]
+                if mode == "touch":
+                    ctx.copy(scratch, m.bufs[0], qbytes)
+                elif mode == "other":
+                    ctx.copy(scratch, mats[(i + ncopy // 2) % ncopy].bufs[0], qbytes)
+                ctx.kq_qmv(m, x, orn.BF16, M, y, orn.BF16)
+
+            row = {"matrix": name, "M": M}
+            for mode in ("same", "none", "other", "touch"):
+                row[mode + "_us"] = round(_time_loop(ctx, lambda i: run(i, mode), 600, 50), 2)
+            rows.append(row)
+            x.free(); y.free()
+        for m in mats:
+            m.free()
+    print(json.dumps({"matvec_warm_cold": rows}), flush=True)
+
+
 def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
     """BASELINE config 5: sampled speculative decode at depth 3 after a long prefill."""
     depth, n_prompt, n_gen, cap = 3, 6621, (1 if args.prefill_only else 256), 16384
@@ -379,6 +418,8 @@ def main():
                          "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--moe-ab", action="store_true",
                     help="only the A/B of the MoE block's launch structure (option fuse_moe_one = 0, 1, 2)")
+    ap.add_argument("--warm-cold", action="store_true",
+                    help="only the mat-vec timings on re-used, unread and just-read weights")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (one process, one stream); "
@@ -391,6 +432,8 @@ def main():
     dev_name, cus, mem = ctx.device_info()
     log(f"device: {dev_name}, {cus} CUs, {mem / 2**30:.0f} GiB")
 
+    if args.warm_cold:
+        return warm_cold(orn, ctx, np)
     cfg = dict(synth.FULL, num_hidden_layers=args.layers)
     t0 = time.time()
     sm = synth.SynthModel(cfg, seed=2025)
