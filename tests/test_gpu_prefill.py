@@ -60,7 +60,12 @@ def test_kq_matmul_vs_float64(orn, ctx, kind, O, K, M):
 @pytest.mark.parametrize("kind,E,O,K,T,k", [(Q4K, 8, 256, 512, 40, 2), (Q4K, 256, 512, 2048, 300, 8),
                                              (Q6K, 256, 2048, 512, 300, 8), (Q6K, 16, 128, 256, 5, 4),
                                              # about 100 rows an expert and more: 128-row tiles
-                                             (Q4K, 8, 256, 512, 400, 2), (Q6K, 16, 128, 256, 500, 4)])
+                                             (Q4K, 8, 256, 512, 400, 2), (Q6K, 16, 128, 256, 500, 4),
+                                             # more than 8192 pairs (the plan made by three launches), a few
+                                             # hundred rows an expert and one crowded expert: tall tiles, the
+                                             # register form for K >= 1024 and its split over shorter workgroups
+                                             (Q4K, 32, 512, 2048, 1100, 8), (Q6K, 32, 256, 1024, 1100, 8),
+                                             (Q6K, 32, 1024, 512, 1100, 8)])
 def test_kq_gather_matmul_vs_float64(orn, ctx, kind, E, O, K, T, k):
     rng = np.random.default_rng(E + O + K + T)
     t = util.make_kq(kind, rng, E, O, K)
@@ -79,7 +84,16 @@ def test_kq_gather_matmul_vs_float64(orn, ctx, kind, E, O, K, T, k):
     orn.kq_gather_matmul(ctx, w, dx, di, pairs, k, True, plan, True, dy)
     got = dy.download(np.uint16, (pairs, O))
     xf = util.bf16_to_f32(xb).astype(np.float64)
-    want = np.stack([xf[p // k] @ deq[inds.reshape(-1)[p]].T for p in range(pairs)])
+    flat = inds.reshape(-1)
+
+    def by_expert(rows_in):       # want[p] = rows_in[p] @ deq[flat[p]].T, one product an expert
+        out = np.empty((pairs, O))
+        for e in np.unique(flat):
+            sel = np.nonzero(flat == e)[0]
+            out[sel] = rows_in[sel] @ deq[e].T
+        return out
+
+    want = by_expert(xf[np.arange(pairs) // k])
     _check(got, want, K, "up")
     # down form on the same plan: pair p reads row p
     ab = util.bf16_normal(rng, (pairs, K))
@@ -87,7 +101,7 @@ def test_kq_gather_matmul_vs_float64(orn, ctx, kind, E, O, K, T, k):
     orn.kq_gather_matmul(ctx, w, da, di, pairs, k, False, plan, False, dy)
     got = dy.download(np.uint16, (pairs, O))
     af = util.bf16_to_f32(ab).astype(np.float64)
-    want = np.stack([af[p] @ deq[inds.reshape(-1)[p]].T for p in range(pairs)])
+    want = by_expert(af)
     _check(got, want, K, "down")
     for b in (plan, di, dx, dy, da): b.free()
     w.free()
