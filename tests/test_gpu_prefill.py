@@ -436,3 +436,25 @@ def test_prefill_paths_are_repeatable(orn, ctx):
         hs.append(model.forward(cache, toks))
     assert np.array_equal(hs[0], hs[1]) and np.array_equal(hs[0], hs[2])
     for o in (cache, model, ws): o.close()
+
+
+@pytest.mark.parametrize("kind,E,O,K,T", [(Q4K, 8, 256, 1024, 3000), (Q6K, 8, 256, 512, 700)])
+def test_kq_gather_matmul_every_pair_on_one_expert(orn, ctx, kind, E, O, K, T):
+    """The other experts have no rows and no tiles; the one expert's rows fill tile after tile
+    (the last one ragged). k = 1: a pair is a token."""
+    rng = np.random.default_rng(T)
+    t = util.make_kq(kind, rng, E, O, K)
+    w = orn.KMatrix(ctx, kind, *t, E, O, K)
+    inds = np.full(T, 5, np.uint32)
+    deq = _deq_bf16(kind, t, E, O, K)
+    plan = ctx.alloc(orn.kq_gather_plan_bytes(T, E))
+    di = ctx.to_device(inds)
+    xb = util.bf16_normal(rng, (T, K))
+    dx, dy = ctx.to_device(xb), ctx.alloc(T * O * 2)
+    want = util.bf16_to_f32(xb).astype(np.float64) @ deq[5].T
+    for make_plan, gate_form in ((True, True), (False, False)):
+        ctx.memset(dy, 0xFF, T * O * 2)
+        orn.kq_gather_matmul(ctx, w, dx, di, T, 1, gate_form, plan, make_plan, dy)
+        _check(dy.download(np.uint16, (T, O)), want, K, "one expert")
+    for b in (plan, di, dx, dy): b.free()
+    w.free()
