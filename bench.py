@@ -45,13 +45,20 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 HBM_PEAK_GBS = 8000.0
 EXPERT_BYTES = 2 * 589_824 + 860_160       # gate + up (Q4_K 512x2048) + down (Q6_K 2048x512)
 
-# HBM bytes per launch of the up kernel at verify width 2 with 17 experts, from two
-# `rocprofv3 --pmc` runs (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch) recorded in
-# profiles/moe_up_T2_pmc.md, each scaled by what the same counter reads for a 256 MiB device
-# copy (fetch x 2.0, write x 1.0). Counters cannot be read from inside this script: the figure
-# is carried from that profile and labelled so.
-PROFILE_TRAFFIC = {"bytes": int(round((9866.6 * 2.0 + 36.0 * 1.0) * 1024)), "algorithmic_bytes": 20_080_704,
-                   "kernel": "moe_up_kernel (T = 2, 17 experts)", "source": "profiles/moe_up_T2_pmc.md"}
+# HBM bytes per launch from two `rocprofv3 --pmc` runs of `bench.py --roofline-only` (FETCH_SIZE,
+# then WRITE_SIZE, KiB per dispatch) recorded in profiles/moe_up_T2_pmc.md, each scaled by what
+# the same counter reads for a 256 MiB device copy (fetch x 2.0, write x 1.0): the up + down pair
+# as the model launches it at verify width 2 (the router's own picks, 15.4 distinct experts on
+# average; its algorithmic bytes are the `bytes_per_pair` of that loop) and the up kernel alone
+# with 17 given experts. Counters cannot be read from inside this script: the figures are
+# carried from that profile and labelled so.
+_KIB = 1024
+PROFILE_TRAFFIC = {
+    "pair": {"bytes": int(round(((9583.2 + 7092.6) * 2.0 + (36.2 + 8.0) * 1.0) * _KIB)), "algorithmic_bytes": 33_557_094,
+             "kernel": "moe_up_kernel<0, 64, 2, true> + moe_down_kernel<1, 8, 2> (T = 2, the router's picks)"},
+    "up_alone": {"bytes": int(round((9866.6 * 2.0 + 36.0 * 1.0) * _KIB)), "algorithmic_bytes": 20_080_704,
+                 "kernel": "moe_up_kernel<0, 64, 2, false> (T = 2, 17 experts)"},
+    "source": "profiles/moe_up_T2_pmc.md (rocprofv3 --pmc runs of `bench.py --roofline-only`, not read in this run)"}
 
 
 def log(*a):
@@ -522,8 +529,8 @@ def main():
     by_width = [expert_roofline(orn, ctx, model, np, args.layers, T) for T in (1, 2, 4)]
     main_w = next(w for w in by_width if w["verify_width"] == 2)
     roof = {"bound": "hbm", "achieved": main_w["achieved"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": main_w["frac"],
-            "traffic": None, "traffic_from_profile": PROFILE_TRAFFIC,
-            "kernel": "moe_up_kernel<Q4_K, 64, 2, routing made in the launch> + moe_down_kernel<Q6_K, 8, 1>: the expert "
+            "traffic": PROFILE_TRAFFIC["pair"]["bytes"], "traffic_from_profile": PROFILE_TRAFFIC,
+            "kernel": "moe_up_kernel<Q4_K, 64, 2, routing made in the launch> + moe_down_kernel<Q6_K, 8, 2>: the expert "
                       "gather-GEMV of one MoE block as the model launches it (gate + up + swiglu, down + combine), "
                       "verify width 2, the router's own picks",
             "us_per_launch": main_w["us_per_pair"], "launches_per_unit": 2, "bytes_per_launch": main_w["bytes_per_pair"],
