@@ -67,6 +67,24 @@ __device__ __forceinline__ f32x4_t mfma(bf16x8_t a, bf16x8_t b, f32x4_t c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+#ifdef ORN_TIMING
+// debug build only: phase time stamps (100 MHz wall clock) of chunk 10 of every workgroup of the
+// scan, and of the prep workgroups of head 5
+__device__ long long g_chunk_marks[512][8];
+__device__ long long g_prep_marks[512][8];
+#define CH_MARK(i) do { if (threadIdx.x == 0 && chunk == 10 && blockIdx.x < 512) g_chunk_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+#define PR_MARK(i) do { if (threadIdx.x == 0 && blockIdx.y == 5 && blockIdx.x < 512) g_prep_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_chunk(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_chunk_marks), sizeof(long long) * 512 * 8);
+}
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_prep(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_prep_marks), sizeof(long long) * 512 * 8);
+}
+#else
+#define CH_MARK(i)
+#define PR_MARK(i)
+#endif
+
 // ---- first kernel: everything of a chunk that does not depend on the state --------------
 // grid (nchunks, Hv), 256 threads. Operand layout of v_mfma_f32_16x16x32_bf16: lane (l16, lg)
 // holds A[m = l16][k = 8 lg ..+8], B^T[n = l16][k = 8 lg ..+8] of a 32-wide k slab and
@@ -89,6 +107,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
   const int t0 = chunk * C, Dv = p.Dv;
   const size_t ch = (size_t)chunk * p.Hv + hv;
 
+  PR_MARK(0);
   // decay logs and beta of the chunk's tokens; tokens past the end leave the state alone
   if (tid < C) {
     const int t = t0 + tid;
@@ -97,24 +116,60 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
     lg_s[tid] = live ? fmaxf(__logf(gv), -100.f) : 0.f;
     bet_s[tid] = live ? dm_bf2f(p.beta[(size_t)t * p.Hv + hv]) : 0.f;
   }
-  // K and V of the chunk, transposed into LDS: thread = (token, 8-wide piece)
-  for (int idx = tid; idx < C * (DK / 8); idx += 256) {
-    const int tok = idx / (DK / 8), pc = idx % (DK / 8);
-    const int t = min(t0 + tok, p.T - 1);
-    const uint4 kv8 = *reinterpret_cast<const uint4*>(p.k + ((size_t)t * p.Hk + hk) * DK + 8 * pc);
-    const uint32_t kw[4] = {kv8.x, kv8.y, kv8.z, kv8.w};
+  // Operand fragments of the K K^T / Q K^T products below, asked for now (they depend on
+  // nothing made here): tokens i = 16 wave + l16 as the n side, tokens j of the tiles nt < wave as
+  // the m side (tile nt = wave has the same rows as the n side).
+  bf16x8_t bki[4], bqi[4], akj[3][4];
+  {
+    const int ti = min(t0 + 16 * wave + l16, p.T - 1);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) Kt[8 * pc + e][tok] = (bf16_t)(kw[e >> 1] >> (16 * (e & 1)));
+    for (int ks = 0; ks < 4; ++ks) {
+      bki[ks] = ld8(p.k + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
+      bqi[ks] = ld8(p.q + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
+    }
+#pragma unroll
+    for (int nt = 0; nt < 3; ++nt) {
+      if (nt < wave) {
+        const int tj = min(t0 + 16 * nt + l16, p.T - 1);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) akj[nt][ks] = ld8(p.k + ((size_t)tj * p.Hk + hk) * DK + 32 * ks + 8 * lg);
+      }
+    }
   }
-  for (int idx = tid; idx < C * (Dv / 8); idx += 256) {
-    const int tok = idx / (Dv / 8), pc = idx % (Dv / 8);
-    const int t = min(t0 + tok, p.T - 1);
-    const uint4 vv8 = *reinterpret_cast<const uint4*>(p.v + ((size_t)t * p.Hv + hv) * Dv + 8 * pc);
-    const uint32_t vw[4] = {vv8.x, vv8.y, vv8.z, vv8.w};
+  // K and V of the chunk, transposed into LDS: thread = (token pair, 8-wide piece); the two
+  // tokens' values of a channel are one 4-byte write, and a wavefront's 64 writes of a channel
+  // (32 pairs of two pieces) fall on 64 different banks. All loads first, then the writes.
+  {
+    uint4 kr[2][2], vr[2][2];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) Vt[8 * pc + e][tok] = (bf16_t)(vw[e >> 1] >> (16 * (e & 1)));
+    for (int it = 0; it < 2; ++it) {
+      const int idx = tid + 256 * it, tp = idx & 31, pc = idx >> 5;
+      const int ta = min(t0 + 2 * tp, p.T - 1), tb = min(t0 + 2 * tp + 1, p.T - 1);
+      kr[it][0] = *reinterpret_cast<const uint4*>(p.k + ((size_t)ta * p.Hk + hk) * DK + 8 * pc);
+      kr[it][1] = *reinterpret_cast<const uint4*>(p.k + ((size_t)tb * p.Hk + hk) * DK + 8 * pc);
+      if (8 * pc < Dv) {
+        vr[it][0] = *reinterpret_cast<const uint4*>(p.v + ((size_t)ta * p.Hv + hv) * Dv + 8 * pc);
+        vr[it][1] = *reinterpret_cast<const uint4*>(p.v + ((size_t)tb * p.Hv + hv) * Dv + 8 * pc);
+      }
+    }
+    auto put = [&](bf16_t(*dst)[LDT], const uint4& a, const uint4& b, int pc, int tp) {
+      const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t w = (e & 1) ? ((aw[e >> 1] >> 16) | (bw[e >> 1] & 0xffff0000u))
+                                   : ((aw[e >> 1] & 0xffffu) | (bw[e >> 1] << 16));
+        *reinterpret_cast<uint32_t*>(&dst[8 * pc + e][2 * tp]) = w;
+      }
+    };
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int idx = tid + 256 * it, tp = idx & 31, pc = idx >> 5;
+      put(Kt, kr[it][0], kr[it][1], pc, tp);
+      if (8 * pc < Dv) put(Vt, vr[it][0], vr[it][1], pc, tp);
+    }
   }
   __syncthreads();
+  PR_MARK(1);
   if (tid < C) {
     float s = 0.f;
     for (int j = 0; j <= tid; ++j) s += lg_s[j];
@@ -138,28 +193,22 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
     }
   }
   __syncthreads();
+  PR_MARK(2);
 
   // ---- K K^T and Q K^T for the chunk's tokens i = 16 wave + l16 (the n side of the product, so
   // that a lane ends up with four consecutive j of one i: packed stores); lower triangle only
   {
-    const int ti = min(t0 + 16 * wave + l16, p.T - 1);
-    bf16x8_t bki[4], bqi[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      bki[ks] = ld8(p.k + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
-      bqi[ks] = ld8(p.q + ((size_t)ti * p.Hk + hk) * DK + 32 * ks + 8 * lg);
-    }
     const int i = 16 * wave + l16;
     const float ell_i = ell_s[i], bet_i = bet_s[i];
+#pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
       f32x4_t kk = {0.f, 0.f, 0.f, 0.f}, qk = {0.f, 0.f, 0.f, 0.f};
       if (nt <= wave) {
-        const int tj = min(t0 + 16 * nt + l16, p.T - 1);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-          const bf16x8_t akj = ld8(p.k + ((size_t)tj * p.Hk + hk) * DK + 32 * ks + 8 * lg);
-          kk = mfma(akj, bki[ks], kk);  // [j][i]
-          qk = mfma(akj, bqi[ks], qk);
+          const bf16x8_t a = nt < wave ? akj[nt < 3 ? nt : 0][ks] : bki[ks];
+          kk = mfma(a, bki[ks], kk);  // [j][i]
+          qk = mfma(a, bqi[ks], qk);
         }
       }
       bf16_t ph[4], pl[4];
@@ -177,6 +226,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
     }
   }
   __syncthreads();
+  PR_MARK(3);
 
   // ---- T = (I + A)^-1 by forward substitution. Thread (column c = tid / 4, part q4 = tid % 4)
   // keeps T[j][c] for j = q4 mod 4; a row's sum over j is four partial sums met inside the quad.
@@ -204,6 +254,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
     }
   }
   __syncthreads();  // A has been read; its memory becomes T
+  PR_MARK(4);
 
   // two passes over T with its columns scaled: by beta e_j0 against K (W), by beta against V (U).
   // The products are made transposed (K^T or V^T as the m side), so a lane holds four consecutive
@@ -253,19 +304,10 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
       }
     }
     __syncthreads();  // T's first scaling has been read before the second is written
+    PR_MARK(5 + pass);
   }
 }
 
-#ifdef ORN_TIMING
-// debug build only: phase time stamps (100 MHz wall clock) of chunk 10 of every workgroup
-__device__ long long g_chunk_marks[512][8];
-#define CH_MARK(i) do { if (threadIdx.x == 0 && chunk == 10 && blockIdx.x < 512) g_chunk_marks[blockIdx.x][i] = wall_clock64(); } while (0)
-extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_chunk(long long* out) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_chunk_marks), sizeof(long long) * 512 * 8);
-}
-#else
-#define CH_MARK(i)
-#endif
 
 // ---- second kernel: the chunks of a head in order ------------------------------------------
 // 256 threads: a workgroup owns 16 rows of a head's state. Wavefront w owns the chunk's tokens
