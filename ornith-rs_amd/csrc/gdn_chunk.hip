@@ -73,7 +73,7 @@ __device__ __forceinline__ f32x4_t mfma(bf16x8_t a, bf16x8_t b, f32x4_t c) {
 __device__ long long g_chunk_marks[512][8];
 __device__ long long g_prep_marks[512][8];
 #define CH_MARK(i) do { if (threadIdx.x == 0 && chunk == 10 && blockIdx.x < 512) g_chunk_marks[blockIdx.x][i] = wall_clock64(); } while (0)
-#define PR_MARK(i) do { if (threadIdx.x == 0 && blockIdx.y == 5 && blockIdx.x < 512) g_prep_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+#define PR_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x == 5 && blockIdx.y < 512) g_prep_marks[blockIdx.y][i] = wall_clock64(); } while (0)
 extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_chunk(long long* out) {
   return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_chunk_marks), sizeof(long long) * 512 * 8);
 }
@@ -86,7 +86,8 @@ extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_prep(lo
 #endif
 
 // ---- first kernel: everything of a chunk that does not depend on the state --------------
-// grid (nchunks, Hv), 256 threads. Operand layout of v_mfma_f32_16x16x32_bf16: lane (l16, lg)
+// grid (Hv, nchunks), 256 threads (the heads of a chunk start together: they read neighbouring
+// pieces of the same token rows and write neighbouring operand blocks). Operand layout of v_mfma_f32_16x16x32_bf16: lane (l16, lg)
 // holds A[m = l16][k = 8 lg ..+8], B^T[n = l16][k = 8 lg ..+8] of a 32-wide k slab and
 // D[m = 4 lg + r][n = l16], r < 4.
 __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l16 = lane & 15, lg = lane >> 4;
-  const int chunk = blockIdx.x, hv = blockIdx.y, hk = hv / (p.Hv / p.Hk);
+  const int chunk = blockIdx.y, hv = blockIdx.x, hk = hv / (p.Hv / p.Hk);
   const int t0 = chunk * C, Dv = p.Dv;
   const size_t ch = (size_t)chunk * p.Hv + hv;
 
@@ -500,7 +501,7 @@ int gdn_chunked_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, co
     a.state_in = t0 == 0 ? d_state_in : d_state_out;
     a.T = rows;
     a.nchunks = n;
-    hipLaunchKernelGGL(gdn_chunk_prep_kernel, dim3(n, Hv), dim3(256), 0, ctx->stream, a);
+    hipLaunchKernelGGL(gdn_chunk_prep_kernel, dim3(Hv, n), dim3(256), 0, ctx->stream, a);
     ORN_LAUNCH_CHECK("gdn_chunk_prep_kernel");
     hipLaunchKernelGGL(gdn_chunk_scan_kernel, dim3(8 * ((Hv + 7) / 8) * (Dv / 16)), dim3(256), 0, ctx->stream, a);
     ORN_LAUNCH_CHECK("gdn_chunk_scan_kernel");
