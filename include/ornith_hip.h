@@ -87,8 +87,8 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *               multiplies); same results either way
  *   "gemm_reg"  (ORNITH_GEMM_REG, default 1): the expert-gathered prefill GEMM dequantizes the
  *               weights into MFMA operand registers where the shape suits it (48 rows an expert
- *               or more, K >= 1024; 0: always through LDS); results agree to the order of the
- *               fp32 sums
+ *               or more: a workgroup a tile for K >= 1024, 64-row workgroups for fewer K slabs;
+ *               0: always through LDS); results agree to the order of the fp32 sums
  *   "gdn_chunked" (ORNITH_GDN_CHUNKED, default 1): the gated-delta recurrence of calls of 128
  *               rows or more (without per-token snapshots) runs in 64-token chunks on the
  *               matrix cores (0: token by token); results agree to rounding

@@ -730,8 +730,8 @@ constexpr int RN = 256;  // output columns of a workgroup of the register form
 constexpr int RM = 192;  // most rows of a tile of the register form
 
 // the main loop and the epilogue for a tile of up to 32 * TM rows
-template <int KIND, int TM, bool GATHER>
-__device__ __forceinline__ void reg_tile(const MmArgs& a, bf16_t (*As)[RM][LDK], const uint32_t* s_src,
+template <int KIND, int TM, bool GATHER, int ROWS>
+__device__ __forceinline__ void reg_tile(const MmArgs& a, bf16_t (*As)[ROWS][LDK], const uint32_t* s_src,
                                          const uint32_t* s_dst, int rows_here, int m0, int64_t wrow0) {
   constexpr int BM = 32 * TM, TN = 2;
   constexpr int NA = BM * 16 / 256;  // 16-byte pieces of an activation slab per thread
@@ -902,37 +902,54 @@ __device__ __forceinline__ void reg_tile(const MmArgs& a, bf16_t (*As)[RM][LDK],
 
 // One kernel for every tile height: a tile runs the loop compiled for the number of 32-row
 // MFMA tiles it really has (an expert with few pairs does not pay for the widest tile).
-template <int KIND, bool GATHER>
-__global__ __launch_bounds__(256) void kq_mm_reg_kernel(MmArgs a) {
-  __shared__ __attribute__((aligned(16))) bf16_t As[2][RM][LDK];
-  __shared__ uint32_t s_src[RM], s_dst[RM];
-  static_assert(2 * LDK >= RN + 8, "the output tile does not fit over the slab buffers");
+template <int KIND, bool GATHER, int ROWS>
+__device__ __forceinline__ void reg_body(const MmArgs& a) {
+  __shared__ __attribute__((aligned(16))) bf16_t As[2][ROWS][LDK];
+  __shared__ uint32_t s_src[ROWS], s_dst[ROWS];
+  static_assert(2 * LDK >= RN + 8 && ROWS % 32 == 0 && ROWS <= RM, "the output tile does not fit over the slab buffers");
   const int tid = threadIdx.x;
   int rows_here, m0 = 0;
   int64_t wrow0 = 0;
   if constexpr (GATHER) {
-    if (blockIdx.y >= *a.n_tiles) return;
-    const uint32_t e = a.tile_expert[blockIdx.y], st = a.tile_start[blockIdx.y];
-    rows_here = min((int)a.tile_count[blockIdx.y], RM);
+    // a plan tile of more rows than ROWS is worked on by a.sub workgroups, ROWS rows each
+    const uint32_t tile = blockIdx.y / (uint32_t)a.sub, part = blockIdx.y % (uint32_t)a.sub;
+    if (tile >= *a.n_tiles) return;
+    const uint32_t e = a.tile_expert[tile], st = a.tile_start[tile] + part * ROWS;
+    rows_here = min((int)a.tile_count[tile] - (int)(part * ROWS), ROWS);
+    if (rows_here <= 0) return;
     wrow0 = (int64_t)e * a.O;
-    for (int r = tid; r < RM; r += 256) {
+    for (int r = tid; r < ROWS; r += 256) {
       const uint32_t p = r < rows_here ? a.pair[st + r] : 0u;
       s_src[r] = p / (uint32_t)a.up_div;
       s_dst[r] = p;
     }
     __syncthreads();
   } else {
-    m0 = blockIdx.y * RM;
-    rows_here = min(RM, a.M - m0);
+    m0 = blockIdx.y * ROWS;
+    rows_here = min(ROWS, a.M - m0);
   }
-  switch ((rows_here + 31) >> 5) {
-    case 1: reg_tile<KIND, 1, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
-    case 2: reg_tile<KIND, 2, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
-    case 3: reg_tile<KIND, 3, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
-    case 4: reg_tile<KIND, 4, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
-    case 5: reg_tile<KIND, 5, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
-    default: reg_tile<KIND, 6, GATHER>(a, As, s_src, s_dst, rows_here, m0, wrow0); break;
-  }
+  // a tile runs the loop compiled for the number of 32-row MFMA tiles it really has (an expert
+  // with few pairs does not pay for the widest tile)
+  const int groups = (rows_here + 31) >> 5;
+#define ORN_REG_TILE(N) reg_tile<KIND, (N <= ROWS / 32 ? N : 1), GATHER, ROWS>(a, As, s_src, s_dst, rows_here, m0, wrow0)
+  if (groups <= 1) ORN_REG_TILE(1);
+  else if (groups == 2 || ROWS / 32 == 2) ORN_REG_TILE(2);
+  else if (groups == 3 || ROWS / 32 == 3) ORN_REG_TILE(3);
+  else if (groups == 4 || ROWS / 32 == 4) ORN_REG_TILE(4);
+  else if (groups == 5 || ROWS / 32 == 5) ORN_REG_TILE(5);
+  else ORN_REG_TILE(6);
+#undef ORN_REG_TILE
+}
+
+template <int KIND, bool GATHER>
+__global__ __launch_bounds__(256) void kq_mm_reg_kernel(MmArgs a) {
+  reg_body<KIND, GATHER, RM>(a);
+}
+// 64 rows a workgroup, two workgroups a compute unit: one's way in and out runs beside the
+// other's main loop (matrices of few K slabs)
+template <int KIND, bool GATHER>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void kq_mm_reg64_kernel(MmArgs a) {
+  reg_body<KIND, GATHER, 64>(a);
 }
 
 // BM == 64 has two 32-row MFMA tiles per wavefront as well (TM = 2), one wavefront column
@@ -1245,12 +1262,13 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   const int need = avg + spare;
   const bool tall = ornith_option_gemm_reg() && avg >= 48;
   const int tile_rows = tall ? (need <= 96 ? 96 : need <= 128 ? 128 : need <= 160 ? 160 : 192) : avg >= 96 ? 128 : 64;
-  // The kernel for this matrix: the register form for tall plans when K >= 1024 (with few K
-  // slabs a workgroup's way in and out, which nothing overlaps at one workgroup a compute unit,
-  // outweighs what that form saves) and its 32-bit offsets reach; otherwise the LDS form, 128
-  // rows a workgroup under the same two conditions on size, else 64 (three 64-row workgroups a
-  // compute unit hide more than 128-row tiles save when a tile has few slabs). A plan tile
-  // taller than that is split over several workgroups.
+  // The kernel for this matrix. Tall plans take the register form when its 32-bit offsets reach:
+  // for K >= 1024 a workgroup a plan tile (one a compute unit), for fewer K slabs 64-row
+  // workgroups, two a compute unit (a workgroup's way in and out, which weighs more the fewer
+  // slabs there are, then runs beside the other's main loop; the weights still bypass LDS, which
+  // is what bounds the LDS form at 64 rows). Otherwise the LDS form: 128 rows a workgroup from 96
+  // rows an expert on and K >= 1024, else 64. A plan tile taller than its kernel's workgroups is
+  // split over several of them.
   const size_t x_bytes = (size_t)(is_up ? pairs / top_k : pairs) * w->K * 2;
   const size_t q_bytes = (size_t)w->E * w->O * (w->K / 256) * (w->kind == ORNITH_Q4K ? 128 : 192);
   const bool reg = tall && w->K >= 1024 && x_bytes < (size_t(1) << 32) && q_bytes < (size_t(1) << 32);
@@ -1283,12 +1301,23 @@ int ornith_kq_gather_matmul(ornith_ctx* ctx, const ornith_kmatrix* w, const void
   a.tile_count = tc;
   a.n_tiles = nt;
   if (reg) {
+    a.sub = 1;
     const dim3 rgrid((w->O + RN - 1) / RN, (unsigned)tiles_max);
     if (w->kind == ORNITH_Q4K)
       hipLaunchKernelGGL((kq_mm_reg_kernel<ORNITH_Q4K, true>), rgrid, dim3(256), 0, ctx->stream, a);
     else
       hipLaunchKernelGGL((kq_mm_reg_kernel<ORNITH_Q6K, true>), rgrid, dim3(256), 0, ctx->stream, a);
     ORN_LAUNCH_CHECK("kq_mm_reg_kernel<gather>");
+    return ORNITH_OK;
+  }
+  if (tall && w->K % 256 == 0 && x_bytes < (size_t(1) << 32) && q_bytes < (size_t(1) << 32)) {
+    a.sub = (tile_rows + 63) / 64;
+    const dim3 rgrid((w->O + RN - 1) / RN, (unsigned)(tiles_max * a.sub));
+    if (w->kind == ORNITH_Q4K)
+      hipLaunchKernelGGL((kq_mm_reg64_kernel<ORNITH_Q4K, true>), rgrid, dim3(256), 0, ctx->stream, a);
+    else
+      hipLaunchKernelGGL((kq_mm_reg64_kernel<ORNITH_Q6K, true>), rgrid, dim3(256), 0, ctx->stream, a);
+    ORN_LAUNCH_CHECK("kq_mm_reg64_kernel<gather>");
     return ORNITH_OK;
   }
   a.sub = (tile_rows + lds_rows - 1) / lds_rows;
