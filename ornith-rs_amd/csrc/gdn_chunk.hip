@@ -311,15 +311,21 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
 
 
 // ---- second kernel: the chunks of a head in order ------------------------------------------
-// 256 threads: a workgroup owns 16 rows of a head's state. Wavefront w owns the chunk's tokens
-// 16 w .. for D and Y, and the state columns 32 w .. for S. The Dv / 16 workgroups of a head read
-// the same W, P, Q, K^T, so they are placed on one XCD (workgroup ids go round the 8 XCDs, each
-// with its own L2): workgroup L sits on XCD L % 8 and takes head (L % 8) * heads_per_xcd + ...
-__global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
+// 512 threads: a workgroup owns 16 rows of a head's state. Only D and the state are links of the
+// chain from chunk to chunk; Y is not. So the eight wavefronts have two roles, and a SIMD runs
+// one of each:
+//   chain  (wavefronts 0..3)  D = U + W S_0^T for the tokens 16 w .., then the state columns 32 w ..
+//   output (wavefronts 4..7)  Y = diag(e_i0) Q S_0^T + P D for the tokens 16 w .., stored as y
+// Both read the state as two bf16 parts (S0h, S0l) and D (Dh, Dl) from LDS; two barriers a chunk.
+// The Dv / 16 workgroups of a head read the same W, P, Q, K^T, so they are placed on one XCD
+// (workgroup ids go round the 8 XCDs, each with its own L2): workgroup L sits on XCD L % 8 and
+// takes head (L % 8) * heads_per_xcd + ...
+__global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
   __shared__ __attribute__((aligned(16))) bf16_t S0h[16][LDS0], S0l[16][LDS0];
   __shared__ __attribute__((aligned(16))) bf16_t Dh[16][LDT], Dl[16][LDT], Fh[16][LDT], Fl[16][LDT];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = (tid >> 6) & 3;
+  const bool chain = tid < 256;
   const int l16 = lane & 15, lg = lane >> 4;
   const int Dv = p.Dv, nb = Dv / 16;
   const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8, hpx = (p.Hv + 7) / 8;
@@ -327,134 +333,163 @@ __global__ __launch_bounds__(256) void gdn_chunk_scan_kernel(ChunkArgs p) {
   if (slot / nb >= hpx || hv >= p.Hv) return;  // uniform over the workgroup
   const int hk = hv / (p.Hv / p.Hk), dv0 = dvb * 16;
 
-  f32x4_t s[2];
-#pragma unroll
-  for (int n2 = 0; n2 < 2; ++n2)
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      s[n2][r] = p.state_in[((size_t)hv * Dv + dv0 + 4 * lg + r) * DK + 16 * (2 * wave + n2) + l16];
-
   // A chunk's operands come straight from memory into registers, one chunk ahead of their use:
   // the chunks of a head are a dependent chain, and a trip to memory inside a link would be
   // most of its length.
-  struct Ops {
-    bf16x8_t awh[4], awl[4], aq[4], ap[2], apl[2], bk[2][2];
-    f32x4_t u, ellr;
-    float ell_c;
-  };
-  // in two halves, issued at different points of a chunk so that the memory pipe's work (82 KB
-  // a chunk and workgroup) runs beside the matrix products instead of ahead of them
-  auto fetch_a = [&](int chunk, Ops& o) {
-    const size_t ch = (size_t)chunk * p.Hv + hv, ck = (size_t)chunk * p.Hk + hk;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      o.awh[ks] = ld8(p.wh + ch * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
-      o.awl[ks] = ld8(p.wl + ch * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
-      o.aq[ks] = ld8(p.qf + ck * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
-    }
-  };
-  auto fetch_b = [&](int chunk, Ops& o) {
-    const size_t ch = (size_t)chunk * p.Hv + hv, ck = (size_t)chunk * p.Hk + hk;
-#pragma unroll
-    for (int k2 = 0; k2 < 2; ++k2) {
-      o.ap[k2] = ld8(p.pm + ch * C * C + ((size_t)(wave * 2 + k2) * 64 + lane) * 8);
-      o.apl[k2] = ld8(p.pl + ch * C * C + ((size_t)(wave * 2 + k2) * 64 + lane) * 8);
-#pragma unroll
-      for (int n2 = 0; n2 < 2; ++n2)
-        o.bk[n2][k2] = ld8(p.kt + ck * DK * C + ((size_t)((2 * wave + n2) * 2 + k2) * 64 + lane) * 8);
-    }
-    o.ell_c = p.ell[ch * C + C - 1];
-    o.u = *reinterpret_cast<const f32x4_t*>(p.u + ch * C * Dv + ((size_t)(wave * nb + dvb) * 64 + lane) * 4);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) o.ellr[r] = p.ell[ch * C + 16 * wave + 4 * lg + r];
-  };
-  Ops cur, nxt;
-  fetch_a(0, cur);
-  fetch_b(0, cur);
-  nxt = cur;
-  for (int chunk = 0; chunk < p.nchunks; ++chunk) {
-    const int t0 = chunk * C;
-    const bool more = chunk + 1 < p.nchunks;
-    CH_MARK(0);
-    const bf16x8_t(&awh)[4] = cur.awh, (&awl)[4] = cur.awl, (&aq)[4] = cur.aq, (&ap)[2] = cur.ap, (&apl)[2] = cur.apl;
-    const bf16x8_t(&bk)[2][2] = cur.bk;
-    f32x4_t d = cur.u;
-    const f32x4_t ellr = cur.ellr;
-    const float ell_c = cur.ell_c;
-
-    // 1. the state as two bf16 parts
+  if (chain) {
+    f32x4_t s[2];
 #pragma unroll
     for (int n2 = 0; n2 < 2; ++n2)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        split_bf16(s[n2][r], &S0h[4 * lg + r][16 * (2 * wave + n2) + l16], &S0l[4 * lg + r][16 * (2 * wave + n2) + l16]);
-    __syncthreads();
-    CH_MARK(1);
+        s[n2][r] = p.state_in[((size_t)hv * Dv + dv0 + 4 * lg + r) * DK + 16 * (2 * wave + n2) + l16];
+    struct Ops {
+      bf16x8_t awh[4], awl[4], bk[2][2];
+      f32x4_t u, ellr;
+      float ell_c;
+    };
+    // in two halves, issued at different points of a chunk so that the memory pipe's work runs
+    // beside the matrix products instead of ahead of them
+    auto fetch_a = [&](int chunk, Ops& o) {
+      const size_t ch = (size_t)chunk * p.Hv + hv;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        o.awh[ks] = ld8(p.wh + ch * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
+        o.awl[ks] = ld8(p.wl + ch * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
+      }
+      o.u = *reinterpret_cast<const f32x4_t*>(p.u + ch * C * Dv + ((size_t)(wave * nb + dvb) * 64 + lane) * 4);
+    };
+    auto fetch_b = [&](int chunk, Ops& o) {
+      const size_t ch = (size_t)chunk * p.Hv + hv, ck = (size_t)chunk * p.Hk + hk;
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+        for (int n2 = 0; n2 < 2; ++n2)
+          o.bk[n2][k2] = ld8(p.kt + ck * DK * C + ((size_t)((2 * wave + n2) * 2 + k2) * 64 + lane) * 8);
+      o.ell_c = p.ell[ch * C + C - 1];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o.ellr[r] = p.ell[ch * C + 16 * wave + 4 * lg + r];
+    };
+    Ops cur, nxt;
+    fetch_a(0, cur);
+    fetch_b(0, cur);
+    nxt = cur;
+    for (int chunk = 0; chunk < p.nchunks; ++chunk) {
+      const bool more = chunk + 1 < p.nchunks;
+      CH_MARK(0);
+      const bf16x8_t(&awh)[4] = cur.awh, (&awl)[4] = cur.awl;
+      const bf16x8_t(&bk)[2][2] = cur.bk;
+      f32x4_t d = cur.u;
+      const f32x4_t ellr = cur.ellr;
+      const float ell_c = cur.ell_c;
 
-    // 2. D = U + W S_0^T and the start of Y = diag(e_i0) Q S_0^T; five accumulators, so that no
-    //    product waits for the one before it
-    if (more) fetch_a(chunk + 1, nxt);
-    f32x4_t yv = {0.f, 0.f, 0.f, 0.f}, d1 = yv, d2 = yv, y1 = yv;
+      // 1. the state as two bf16 parts
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const bf16x8_t bh = ld8(&S0h[l16][32 * ks + 8 * lg]), bl = ld8(&S0l[l16][32 * ks + 8 * lg]);
-      d = mfma(awh[ks], bh, d);
-      d1 = mfma(awh[ks], bl, d1);
-      d2 = mfma(awl[ks], bh, d2);
-      yv = mfma(aq[ks], bh, yv);
-      y1 = mfma(aq[ks], bl, y1);
-    }
-    d = d + (d1 + d2);
-    yv = yv + y1;
+      for (int n2 = 0; n2 < 2; ++n2)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int i = 16 * wave + 4 * lg + r;
-      split_bf16(d[r], &Dh[l16][i], &Dl[l16][i]);
-      split_bf16(d[r] * __expf(ell_c - ellr[r]), &Fh[l16][i], &Fl[l16][i]);
-      yv[r] *= __expf(ellr[r]);
-    }
-    CH_MARK(2);
-    __syncthreads();
-    CH_MARK(3);
+        for (int r = 0; r < 4; ++r)
+          split_bf16(s[n2][r], &S0h[4 * lg + r][16 * (2 * wave + n2) + l16], &S0l[4 * lg + r][16 * (2 * wave + n2) + l16]);
+      __syncthreads();
+      CH_MARK(1);
 
-    // 3. Y += P D
-    if (more) fetch_b(chunk + 1, nxt);
+      // 2. D = U + W S_0^T; three accumulators, so that no product waits for the one before it
+      if (more) fetch_a(chunk + 1, nxt);
+      f32x4_t d1 = {0.f, 0.f, 0.f, 0.f}, d2 = d1;
 #pragma unroll
-    for (int k2 = 0; k2 < 2; ++k2) {
-      const bf16x8_t dh = ld8(&Dh[l16][32 * k2 + 8 * lg]);
-      yv = mfma(ap[k2], dh, yv);
-      yv = mfma(ap[k2], ld8(&Dl[l16][32 * k2 + 8 * lg]), yv);
-      yv = mfma(apl[k2], dh, yv);
-    }
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8_t bh = ld8(&S0h[l16][32 * ks + 8 * lg]), bl = ld8(&S0l[l16][32 * ks + 8 * lg]);
+        d = mfma(awh[ks], bh, d);
+        d1 = mfma(awh[ks], bl, d1);
+        d2 = mfma(awl[ks], bh, d2);
+      }
+      d = d + (d1 + d2);
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int tk = t0 + 16 * wave + 4 * lg + r;
-      if (tk < p.T) p.y[((size_t)tk * p.Hv + hv) * Dv + dv0 + l16] = dm_f2bf(yv[r]);
-    }
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * wave + 4 * lg + r;
+        split_bf16(d[r], &Dh[l16][i], &Dl[l16][i]);
+        split_bf16(d[r] * __expf(ell_c - ellr[r]), &Fh[l16][i], &Fl[l16][i]);
+      }
+      CH_MARK(2);
+      __syncthreads();
+      CH_MARK(3);
 
-    CH_MARK(4);
-    // 4. S = e_C0 S + (diag(e_Cj) D)^T K
-    const float gc = __expf(ell_c);
+      // 3. S = e_C0 S + (diag(e_Cj) D)^T K
+      if (more) fetch_b(chunk + 1, nxt);
+      CH_MARK(4);
+      const float gc = __expf(ell_c);
 #pragma unroll
-    for (int n2 = 0; n2 < 2; ++n2) {
+      for (int n2 = 0; n2 < 2; ++n2) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) s[n2][r] *= gc;
+        for (int r = 0; r < 4; ++r) s[n2][r] *= gc;
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2) {
+          s[n2] = mfma(ld8(&Fh[l16][32 * k2 + 8 * lg]), bk[n2][k2], s[n2]);
+          s[n2] = mfma(ld8(&Fl[l16][32 * k2 + 8 * lg]), bk[n2][k2], s[n2]);
+        }
+      }
+      CH_MARK(5);
+      // the tiles read here are rewritten behind the next chunk's first barrier, the state tiles
+      // behind the barrier above
+      CH_MARK(6);
+      cur = nxt;
+    }
+#pragma unroll
+    for (int n2 = 0; n2 < 2; ++n2)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        p.state_out[((size_t)hv * Dv + dv0 + 4 * lg + r) * DK + 16 * (2 * wave + n2) + l16] = s[n2][r];
+  } else {
+    struct Ops {
+      bf16x8_t aq[4], ap[2], apl[2];
+      f32x4_t ellr;
+    };
+    auto fetch = [&](int chunk, Ops& o) {
+      const size_t ch = (size_t)chunk * p.Hv + hv, ck = (size_t)chunk * p.Hk + hk;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) o.aq[ks] = ld8(p.qf + ck * C * DK + ((size_t)(wave * 4 + ks) * 64 + lane) * 8);
 #pragma unroll
       for (int k2 = 0; k2 < 2; ++k2) {
-        s[n2] = mfma(ld8(&Fh[l16][32 * k2 + 8 * lg]), bk[n2][k2], s[n2]);
-        s[n2] = mfma(ld8(&Fl[l16][32 * k2 + 8 * lg]), bk[n2][k2], s[n2]);
+        o.ap[k2] = ld8(p.pm + ch * C * C + ((size_t)(wave * 2 + k2) * 64 + lane) * 8);
+        o.apl[k2] = ld8(p.pl + ch * C * C + ((size_t)(wave * 2 + k2) * 64 + lane) * 8);
       }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o.ellr[r] = p.ell[ch * C + 16 * wave + 4 * lg + r];
+    };
+    Ops cur, nxt;
+    fetch(0, cur);
+    nxt = cur;
+    for (int chunk = 0; chunk < p.nchunks; ++chunk) {
+      const int t0 = chunk * C;
+      __syncthreads();  // the state's two parts are in LDS
+      if (chunk + 1 < p.nchunks) fetch(chunk + 1, nxt);
+      // the start of Y = diag(e_i0) Q S_0^T, two accumulators
+      f32x4_t yv = {0.f, 0.f, 0.f, 0.f}, y1 = yv;
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8_t bh = ld8(&S0h[l16][32 * ks + 8 * lg]), bl = ld8(&S0l[l16][32 * ks + 8 * lg]);
+        yv = mfma(cur.aq[ks], bh, yv);
+        y1 = mfma(cur.aq[ks], bl, y1);
+      }
+      yv = yv + y1;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) yv[r] *= __expf(cur.ellr[r]);
+      __syncthreads();  // D is in LDS (and the state's parts have been read)
+      // Y += P D
+#pragma unroll
+      for (int k2 = 0; k2 < 2; ++k2) {
+        const bf16x8_t dh = ld8(&Dh[l16][32 * k2 + 8 * lg]);
+        yv = mfma(cur.ap[k2], dh, yv);
+        yv = mfma(cur.ap[k2], ld8(&Dl[l16][32 * k2 + 8 * lg]), yv);
+        yv = mfma(cur.apl[k2], dh, yv);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int tk = t0 + 16 * wave + 4 * lg + r;
+        if (tk < p.T) p.y[((size_t)tk * p.Hv + hv) * Dv + dv0 + l16] = dm_f2bf(yv[r]);
+      }
+      cur = nxt;
     }
-    CH_MARK(5);
-    __syncthreads();  // the tiles are rewritten by the next chunk
-    CH_MARK(6);
-    cur = nxt;
   }
-#pragma unroll
-  for (int n2 = 0; n2 < 2; ++n2)
-#pragma unroll
-    for (int r = 0; r < 4; ++r)
-      p.state_out[((size_t)hv * Dv + dv0 + 4 * lg + r) * DK + 16 * (2 * wave + n2) + l16] = s[n2][r];
 }
 
 }  // namespace
@@ -503,7 +538,7 @@ int gdn_chunked_recurrence(ornith_ctx* ctx, const void* d_q, const void* d_k, co
     a.nchunks = n;
     hipLaunchKernelGGL(gdn_chunk_prep_kernel, dim3(Hv, n), dim3(256), 0, ctx->stream, a);
     ORN_LAUNCH_CHECK("gdn_chunk_prep_kernel");
-    hipLaunchKernelGGL(gdn_chunk_scan_kernel, dim3(8 * ((Hv + 7) / 8) * (Dv / 16)), dim3(256), 0, ctx->stream, a);
+    hipLaunchKernelGGL(gdn_chunk_scan_kernel, dim3(8 * ((Hv + 7) / 8) * (Dv / 16)), dim3(512), 0, ctx->stream, a);
     ORN_LAUNCH_CHECK("gdn_chunk_scan_kernel");
   }
   return ORNITH_OK;
