@@ -370,12 +370,10 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) o.ellr[r] = p.ell[ch * C + 16 * wave + 4 * lg + r];
     };
-    Ops cur, nxt;
-    fetch_a(0, cur);
-    fetch_b(0, cur);
-    nxt = cur;
-    for (int chunk = 0; chunk < p.nchunks; ++chunk) {
-      const bool more = chunk + 1 < p.nchunks;
+    // three operand sets in turn, asked for two chunks ahead of their use (one chunk of a chain
+    // this short is less than a trip to memory); the sets are named, not indexed or copied
+    auto link = [&](int chunk, const Ops& cur, Ops& fill) {
+      const bool more = chunk + 2 < p.nchunks;
       CH_MARK(0);
       const bf16x8_t(&awh)[4] = cur.awh, (&awl)[4] = cur.awl;
       const bf16x8_t(&bk)[2][2] = cur.bk;
@@ -393,7 +391,7 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
       CH_MARK(1);
 
       // 2. D = U + W S_0^T; three accumulators, so that no product waits for the one before it
-      if (more) fetch_a(chunk + 1, nxt);
+      if (more) fetch_a(chunk + 2, fill);
       f32x4_t d1 = {0.f, 0.f, 0.f, 0.f}, d2 = d1;
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
@@ -414,7 +412,7 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
       CH_MARK(3);
 
       // 3. S = e_C0 S + (diag(e_Cj) D)^T K
-      if (more) fetch_b(chunk + 1, nxt);
+      if (more) fetch_b(chunk + 2, fill);
       CH_MARK(4);
       const float gc = __expf(ell_c);
 #pragma unroll
@@ -431,7 +429,18 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
       // the tiles read here are rewritten behind the next chunk's first barrier, the state tiles
       // behind the barrier above
       CH_MARK(6);
-      cur = nxt;
+    };
+    Ops o0, o1, o2;
+    fetch_a(0, o0);
+    fetch_b(0, o0);
+    if (p.nchunks > 1) {
+      fetch_a(1, o1);
+      fetch_b(1, o1);
+    }
+    for (int chunk = 0; chunk < p.nchunks; chunk += 3) {
+      link(chunk, o0, o2);
+      if (chunk + 1 < p.nchunks) link(chunk + 1, o1, o0);
+      if (chunk + 2 < p.nchunks) link(chunk + 2, o2, o1);
     }
 #pragma unroll
     for (int n2 = 0; n2 < 2; ++n2)
@@ -455,13 +464,10 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) o.ellr[r] = p.ell[ch * C + 16 * wave + 4 * lg + r];
     };
-    Ops cur, nxt;
-    fetch(0, cur);
-    nxt = cur;
-    for (int chunk = 0; chunk < p.nchunks; ++chunk) {
+    auto link = [&](int chunk, const Ops& cur, Ops& fill) {
       const int t0 = chunk * C;
       __syncthreads();  // the state's two parts are in LDS
-      if (chunk + 1 < p.nchunks) fetch(chunk + 1, nxt);
+      if (chunk + 2 < p.nchunks) fetch(chunk + 2, fill);
       // the start of Y = diag(e_i0) Q S_0^T, two accumulators
       f32x4_t yv = {0.f, 0.f, 0.f, 0.f}, y1 = yv;
 #pragma unroll
@@ -487,7 +493,14 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
         const int tk = t0 + 16 * wave + 4 * lg + r;
         if (tk < p.T) p.y[((size_t)tk * p.Hv + hv) * Dv + dv0 + l16] = dm_f2bf(yv[r]);
       }
-      cur = nxt;
+    };
+    Ops o0, o1, o2;
+    fetch(0, o0);
+    if (p.nchunks > 1) fetch(1, o1);
+    for (int chunk = 0; chunk < p.nchunks; chunk += 3) {
+      link(chunk, o0, o2);
+      if (chunk + 1 < p.nchunks) link(chunk + 1, o1, o0);
+      if (chunk + 2 < p.nchunks) link(chunk + 2, o2, o1);
     }
   }
 }
