@@ -310,6 +310,15 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
 }
 
 
+// four fp32 values as their high and low bf16 parts, each quad one 8-byte LDS write
+__device__ __forceinline__ void split4_bf16(const f32x4_t& v, bf16_t* hi, bf16_t* lo) {
+  bf16_t h[4], l[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) split_bf16(v[r], &h[r], &l[r]);
+  *reinterpret_cast<uint2*>(hi) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
+  *reinterpret_cast<uint2*>(lo) = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
+}
+
 // ---- second kernel: the chunks of a head in order ------------------------------------------
 // 512 threads: a workgroup owns 16 rows of a head's state. Only D and the state are links of the
 // chain from chunk to chunk; Y is not. So the eight wavefronts have two roles, and a SIMD runs
@@ -337,12 +346,13 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
   // the chunks of a head are a dependent chain, and a trip to memory inside a link would be
   // most of its length.
   if (chain) {
+    // The state products are made transposed (K^T the m side), so that a lane holds four
+    // consecutive key channels of one state row: s[n2][r] = S[dv0 + l16][16 (2 w + n2) + 4 lg + r],
+    // 16 bytes in memory and 8 bytes of each bf16 part in LDS.
     f32x4_t s[2];
 #pragma unroll
     for (int n2 = 0; n2 < 2; ++n2)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        s[n2][r] = p.state_in[((size_t)hv * Dv + dv0 + 4 * lg + r) * DK + 16 * (2 * wave + n2) + l16];
+      s[n2] = *reinterpret_cast<const f32x4_t*>(p.state_in + ((size_t)hv * Dv + dv0 + l16) * DK + 16 * (2 * wave + n2) + 4 * lg);
     struct Ops {
       bf16x8_t awh[4], awl[4], bk[2][2];
       f32x4_t u, ellr;
@@ -384,9 +394,7 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
       // 1. the state as two bf16 parts
 #pragma unroll
       for (int n2 = 0; n2 < 2; ++n2)
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          split_bf16(s[n2][r], &S0h[4 * lg + r][16 * (2 * wave + n2) + l16], &S0l[4 * lg + r][16 * (2 * wave + n2) + l16]);
+        split4_bf16(s[n2], &S0h[l16][16 * (2 * wave + n2) + 4 * lg], &S0l[l16][16 * (2 * wave + n2) + 4 * lg]);
       __syncthreads();
       CH_MARK(1);
 
@@ -401,12 +409,11 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
         d2 = mfma(awl[ks], bh, d2);
       }
       d = d + (d1 + d2);
+      f32x4_t f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * wave + 4 * lg + r;
-        split_bf16(d[r], &Dh[l16][i], &Dl[l16][i]);
-        split_bf16(d[r] * __expf(ell_c - ellr[r]), &Fh[l16][i], &Fl[l16][i]);
-      }
+      for (int r = 0; r < 4; ++r) f[r] = d[r] * __expf(ell_c - ellr[r]);
+      split4_bf16(d, &Dh[l16][16 * wave + 4 * lg], &Dl[l16][16 * wave + 4 * lg]);
+      split4_bf16(f, &Fh[l16][16 * wave + 4 * lg], &Fl[l16][16 * wave + 4 * lg]);
       CH_MARK(2);
       __syncthreads();
       CH_MARK(3);
@@ -421,8 +428,8 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
         for (int r = 0; r < 4; ++r) s[n2][r] *= gc;
 #pragma unroll
         for (int k2 = 0; k2 < 2; ++k2) {
-          s[n2] = mfma(ld8(&Fh[l16][32 * k2 + 8 * lg]), bk[n2][k2], s[n2]);
-          s[n2] = mfma(ld8(&Fl[l16][32 * k2 + 8 * lg]), bk[n2][k2], s[n2]);
+          s[n2] = mfma(bk[n2][k2], ld8(&Fh[l16][32 * k2 + 8 * lg]), s[n2]);  // [dk][dv]
+          s[n2] = mfma(bk[n2][k2], ld8(&Fl[l16][32 * k2 + 8 * lg]), s[n2]);
         }
       }
       CH_MARK(5);
@@ -444,9 +451,7 @@ __global__ __launch_bounds__(512) void gdn_chunk_scan_kernel(ChunkArgs p) {
     }
 #pragma unroll
     for (int n2 = 0; n2 < 2; ++n2)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        p.state_out[((size_t)hv * Dv + dv0 + 4 * lg + r) * DK + 16 * (2 * wave + n2) + l16] = s[n2][r];
+      *reinterpret_cast<f32x4_t*>(p.state_out + ((size_t)hv * Dv + dv0 + l16) * DK + 16 * (2 * wave + n2) + 4 * lg) = s[n2];
   } else {
     struct Ops {
       bf16x8_t aq[4], ap[2], apl[2];
