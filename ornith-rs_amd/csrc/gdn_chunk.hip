@@ -312,11 +312,11 @@ __global__ __launch_bounds__(256) void gdn_chunk_prep_kernel(ChunkArgs p) {
 
 // four fp32 values as their high and low bf16 parts, each quad one 8-byte LDS write
 __device__ __forceinline__ void split4_bf16(const f32x4_t& v, bf16_t* hi, bf16_t* lo) {
-  bf16_t h[4], l[4];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) split_bf16(v[r], &h[r], &l[r]);
-  *reinterpret_cast<uint2*>(hi) = make_uint2(h[0] | ((uint32_t)h[1] << 16), h[2] | ((uint32_t)h[3] << 16));
-  *reinterpret_cast<uint2*>(lo) = make_uint2(l[0] | ((uint32_t)l[1] << 16), l[2] | ((uint32_t)l[3] << 16));
+  const uint32_t h01 = dm_f2bf2(v[0], v[1]), h23 = dm_f2bf2(v[2], v[3]);  // two conversions an instruction
+  const uint32_t l01 = dm_f2bf2(v[0] - dm_bf2f_lo(h01), v[1] - dm_bf2f_hi(h01));
+  const uint32_t l23 = dm_f2bf2(v[2] - dm_bf2f_lo(h23), v[3] - dm_bf2f_hi(h23));
+  *reinterpret_cast<uint2*>(hi) = make_uint2(h01, h23);
+  *reinterpret_cast<uint2*>(lo) = make_uint2(l01, l23);
 }
 
 // ---- second kernel: the chunks of a head in order ------------------------------------------
