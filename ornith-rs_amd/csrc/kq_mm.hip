@@ -184,11 +184,13 @@ struct BRegsOf<ORNITH_Q6K> { typedef BRegsQ6 type; };
 #ifdef ORN_TIMING
 __device__ long long g_mm_marks[1024][8];
 #define MM_MARK(i, cond) do { if (threadIdx.x == 0 && blockIdx.x == 0 && blockIdx.y < 1024 && (cond)) g_mm_marks[blockIdx.y][i] = wall_clock64(); } while (0)
+#define MM_MARK_P(i, cond) do { if (threadIdx.x == 256 && blockIdx.x == 0 && blockIdx.y < 1024 && (cond)) g_mm_marks[blockIdx.y][i] = wall_clock64(); } while (0)
 extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_mm(long long* out) {
   return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_mm_marks), sizeof(g_mm_marks));
 }
 #else
 #define MM_MARK(i, cond)
+#define MM_MARK_P(i, cond)
 #endif
 
 // ---- epilogue ------------------------------------------------------------------------------
@@ -534,9 +536,13 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
     // while the consumers work on slab s + u: slab s + u + 1 into the other buffer, then its
     // register set asks for the slab four further on
     auto step = [&](auto set, int k) {
+      MM_MARK_P(3, k == 9);
       if (k < nslab) write(set, k * BK2);
+      MM_MARK_P(4, k == 9);
       if (k + 4 < nslab) fetch(set, (k + 4) * BK2);
+      MM_MARK_P(5, k == 9);
       __syncthreads();
+      MM_MARK_P(6, k == 9);
     };
     for (int s = 0; s < nslab; s += 4) {
       step(Set1{}, s + 1);
@@ -581,8 +587,11 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
   };
   __syncthreads();  // slab 0 is in buffer 0
   for (int s = 0; s < nslab; s += 2) {  // (the producers count the same barriers, four a turn)
+    MM_MARK(0, s == 8);
     slab(0);
+    MM_MARK(1, s == 8);
     __syncthreads();
+    MM_MARK(2, s == 8);
     slab(1);
     __syncthreads();
   }
