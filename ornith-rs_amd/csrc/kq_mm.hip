@@ -514,6 +514,7 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
         const int idx = ptid + 256 * i;
         *reinterpret_cast<u32x4_t*>(&As[BUF][idx >> 3][8 * (idx & 7)]) = areg[SET][i];
       }
+      MM_MARK_P(7, k0 == 9 * BK2);
       if constexpr (KIND == ORNITH_Q4K) {
         const PipeQ4 pp = pipe_prepare(breg[SET], (k0 & 255) >> 6, bpart);
 #pragma unroll
