@@ -449,7 +449,11 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
   constexpr int WM = BM >= 128 ? 2 : 1, WN = 4 / WM;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int NA = BM * 8 / 256;  // 16-byte pieces of an activation slab per producer thread
+  constexpr int NA = BM * 8 / 256;  // 16-byte pieces of an activation slab per thread of one role
+  // The producers set the pace (activations and weights into LDS, the loads asked for), the
+  // consumers wait a third of a slab at its barrier: the consumers carry the upper half of the
+  // activation rows into LDS themselves (asked for two slabs ahead, written before the slab's MFMAs).
+  constexpr int NAP = NA / 2, NAC = NA - NAP;
   __shared__ __attribute__((aligned(16))) bf16_t As[2][BM][LD2];
   __shared__ __attribute__((aligned(16))) bf16_t Bs[2][BN][LD2];
   __shared__ uint32_t s_src[BM], s_dst[BM];
@@ -484,9 +488,9 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
     const int ptid = tid - 256;
     const int br = ptid >> 1, bpart = ptid & 1;
     const int64_t brow = wrow0 + min(n0 + br, a.O - 1);
-    const bf16_t* asrc[NA];
+    const bf16_t* asrc[NAP];
 #pragma unroll
-    for (int i = 0; i < NA; ++i) {
+    for (int i = 0; i < NAP; ++i) {
       const int idx = ptid + 256 * i, r = idx >> 3, c8 = idx & 7;
       // rows past the end of the tile read a valid row: what they produce is never stored
       const int64_t src = GATHER ? (int64_t)s_src[r] : (int64_t)min(m0 + r, a.M - 1);
@@ -496,12 +500,12 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
     // written to LDS buffer k & 1, so a load has about four slab times to arrive. (Sets and
     // buffers are picked by constants: an index known only at run time would put the arrays
     // in scratch memory.)
-    u32x4_t areg[4][NA];
+    u32x4_t areg[4][NAP];
     typename BRegsOf<KIND>::type breg[4];
     auto fetch = [&](auto set, int k0) {
       constexpr int SET = decltype(set)::value;
 #pragma unroll
-      for (int i = 0; i < NA; ++i) areg[SET][i] = *reinterpret_cast<const u32x4_t*>(asrc[i] + k0);
+      for (int i = 0; i < NAP; ++i) areg[SET][i] = *reinterpret_cast<const u32x4_t*>(asrc[i] + k0);
       if constexpr (KIND == ORNITH_Q4K)
         breg[SET] = load_q4k(a, brow, nb, k0 >> 8, (k0 & 255) >> 6);
       else
@@ -510,7 +514,7 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
     auto write = [&](auto set, int k0) {
       constexpr int SET = decltype(set)::value, BUF = SET & 1;
 #pragma unroll
-      for (int i = 0; i < NA; ++i) {
+      for (int i = 0; i < NAP; ++i) {
         const int idx = ptid + 256 * i;
         *reinterpret_cast<u32x4_t*>(&As[BUF][idx >> 3][8 * (idx & 7)]) = areg[SET][i];
       }
@@ -563,6 +567,33 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
     for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  // the consumers' share of the activation slab: pieces NAP .. NA of the same index scheme; slab
+  // k travels in register set k & 1 into LDS buffer k & 1
+  const bf16_t* csrc[NAC];
+#pragma unroll
+  for (int i = 0; i < NAC; ++i) {
+    const int idx = tid + 256 * (NAP + i), r = idx >> 3, c8 = idx & 7;
+    const int64_t src = GATHER ? (int64_t)s_src[r] : (int64_t)min(m0 + r, a.M - 1);
+    csrc[i] = a.x + src * a.K + 8 * c8;
+  }
+  u32x4_t creg[2][NAC];
+  auto cfetch = [&](auto set, int k) {
+    constexpr int SET = decltype(set)::value;
+    if (k < nslab) {
+#pragma unroll
+      for (int i = 0; i < NAC; ++i) creg[SET][i] = *reinterpret_cast<const u32x4_t*>(csrc[i] + k * BK2);
+    }
+  };
+  auto cwrite = [&](auto set, int k) {
+    constexpr int SET = decltype(set)::value;
+    if (k < nslab) {
+#pragma unroll
+      for (int i = 0; i < NAC; ++i) {
+        const int idx = tid + 256 * (NAP + i);
+        *reinterpret_cast<u32x4_t*>(&As[SET][idx >> 3][8 * (idx & 7)]) = creg[SET][i];
+      }
+    }
+  };
   auto frags = [&](int buf, int kk, bf16x8_t (&fa)[TM], bf16x8_t (&fb)[TN]) {
     const int kc = kk * 16 + 8 * (lane >> 5);
 #pragma unroll
@@ -586,13 +617,21 @@ __global__ __launch_bounds__(512) void kq_mm_duo_kernel(MmArgs a) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[kk & 1][i], bfr[kk & 1][j], acc[i][j], 0, 0, 0);
     }
   };
+  cfetch(Set0{}, 0);
+  cfetch(Set1{}, 1);
+  cwrite(Set0{}, 0);
+  cfetch(Set0{}, 2);
   __syncthreads();  // slab 0 is in buffer 0
   for (int s = 0; s < nslab; s += 2) {  // (the producers count the same barriers, four a turn)
     MM_MARK(0, s == 8);
+    cwrite(Set1{}, s + 1);  // into the buffer the MFMAs below do not read
+    cfetch(Set1{}, s + 3);
     slab(0);
     MM_MARK(1, s == 8);
     __syncthreads();
     MM_MARK(2, s == 8);
+    cwrite(Set0{}, s + 2);
+    cfetch(Set0{}, s + 4);
     slab(1);
     __syncthreads();
   }
