@@ -340,8 +340,113 @@ def warm_cold(orn, ctx, np):
     print(json.dumps({"matvec_warm_cold": rows}), flush=True)
 
 
+def ceiling(orn, ctx, np):
+    """What the machine allows a decode launch, measured with the library's probe kernels
+    (csrc/probe.hip): the cost of a launch that does nothing, of launches of the expert kernels'
+    shapes that only stream their bytes (cold: cycling over > 1 GiB), of a long read, where
+    workgroups land, and how long a word stored by one workgroup takes to reach another on the
+    same die and on another. Prints one JSON object."""
+    lib = orn.lib()
+    res = {}
+    sink = ctx.alloc(256)
+
+    def probe(rc, what):
+        if rc != 0:
+            raise orn.OrnithError(f"{what}: {lib.ornith_last_error().decode()}")
+
+    # -- launches that do nothing, back to back. The host enqueues 1000 launches per call: if
+    #    the figure does not grow with the grid it is the host's enqueue rate, not the device's.
+    rows = []
+    for wgs, thr, args_ in ((1, 64, 0), (1152, 256, 0), (1152, 256, 1), (512, 576, 1)):
+        probe(lib.ornith_probe_empty(ctx.h, wgs, thr, args_, 200), "probe_empty")
+        ctx.sync()
+        ctx.timer_begin()
+        probe(lib.ornith_probe_empty(ctx.h, wgs, thr, args_, 2000), "probe_empty")
+        us = ctx.timer_end() * 1000.0 / 2000
+        ms = C.c_float()
+        probe(lib.ornith_probe_empty_graph(ctx.h, wgs, thr, args_, 2000, C.byref(ms)), "probe_empty_graph")
+        rows.append({"workgroups": wgs, "threads": thr, "argument_block": bool(args_), "us_per_launch": round(us, 2),
+                     "us_per_launch_in_a_graph": round(ms.value * 1000.0 / 2000, 2)})
+    res["empty_launch"] = rows
+
+    # -- launches of the expert kernels' shapes with the arithmetic taken out
+    big = 2 << 30
+    buf = ctx.alloc(big)
+    lib.ornith_memset(ctx.h, buf.ptr, 1, C.c_size_t(big))
+    rows = []
+    shapes = (("expert up at T=2: 1152 x 256 threads, 4 x 16 B a thread, contiguous 4 KB a wavefront (18.9 MB)", 1152, 4, 1024),
+              ("expert up at T=2, a wavefront's four pieces 1152 B apart as Q4_K rows lie (18.9 MB)", 1152, 4, 1152),
+              ("expert down at T=2: 512 x 256 threads, 7 x 16 B a thread (14.7 MB)", 512, 7, 1024),
+              ("expert up at T=1: 576 workgroups (9.4 MB)", 576, 4, 1024),
+              ("one 4 KB piece a wavefront over 4608 workgroups (75 MB)", 4608, 4, 1024),
+              ("lm_head-sized: 17,460 workgroups x 16 KB (286 MB)", 17460, 4, 1024))
+    for name, wgs, per, stride in shapes:
+        span = ((wgs * 4 * per - 1) * stride + 1024 + 4095) & ~4095
+        nslots = max(1, min(64, big // span))
+
+        def run(i):
+            off = (i % nslots) * span
+            probe(lib.ornith_probe_stream(ctx.h, C.c_void_p(buf.ptr.value + off), C.c_size_t(span), wgs, per,
+                                          C.c_size_t(stride), sink.ptr), "probe_stream")
+
+        n = 400 if span < (64 << 20) else 60
+        us = _time_loop(ctx, run, n, nslots)
+        nbytes = wgs * 256 * per * 16
+        rows.append({"shape": name, "bytes": nbytes, "us_per_launch": round(us, 2),
+                     "GB_s": round(nbytes / (us * 1e-6) / 1e9, 1), "frac_of_8TBs": round(nbytes / (us * 1e-6) / 8e12, 3)})
+    res["stream_only_launch"] = rows
+
+    # -- one long read
+    rows = []
+    for mib in (64, 256, 1024, 2048):
+        n = mib << 20
+        us = _time_loop(ctx, lambda i: probe(lib.ornith_probe_read(ctx.h, buf.ptr, C.c_size_t(n), sink.ptr), "probe_read"), 20, 3)
+        rows.append({"MiB": mib, "us": round(us, 1), "GB_s": round(n / (us * 1e-6) / 1e9, 1), "frac_of_8TBs": round(n / (us * 1e-6) / 8e12, 3)})
+    res["long_read"] = rows
+    buf.free()
+
+    # -- where workgroups land
+    n = 2048
+    xo = ctx.alloc(n * 4)
+    agree = 0
+    for rep in range(20):
+        probe(lib.ornith_probe_xcc(ctx.h, n, xo.ptr), "probe_xcc")
+        ids = xo.download(np.uint32, (n,))
+        if rep == 0:
+            first = ids[:16].tolist()
+            shift = int((ids[0] - 0) % 8)
+        agree += int(np.array_equal(ids, (np.arange(n) + shift) % 8))
+    res["workgroup_to_xcc"] = {"first_16": first, "rule": f"xcc = (workgroup + {shift}) mod 8", "launches_following_the_rule": agree, "of": 20}
+    xo.free()
+
+    # -- a word from one workgroup to another (workgroups 0 and 8 share a die, 0 and 1 do not)
+    flag, out4 = ctx.alloc(4096 * 256), ctx.alloc(64)
+    flag.zero()
+    rows = []
+    slot = 0
+    for place, cons in (("same XCC", 8), ("another XCC", 1)):
+        for mode, mname in ((0, "plain store, agent-scope (sc1) loads"), (1, "sc1 store, sc1 loads"), (2, "plain store, plain loads")):
+            lat, xcc = [], None
+            for rep in range(9):
+                probe(lib.ornith_probe_handoff(ctx.h, C.c_void_p(flag.ptr.value + 256 * slot), out4.ptr, 0, cons, mode), "probe_handoff")
+                slot += 1
+                o = out4.download(np.int64, (4,))
+                xcc = (int(o[2]), int(o[3]))
+                lat.append((o[1] - o[0]) / 100.0 if o[1] else None)
+            seen = [v for v in lat if v is not None]
+            rows.append({"where": place, "how": mname, "xcc_ids": xcc, "seen": len(seen), "of": len(lat),
+                         "us_min": round(min(seen), 2) if seen else None, "us_median": round(float(np.median(seen)), 2) if seen else None,
+                         "us_max": round(max(seen), 2) if seen else None})
+    res["word_between_workgroups"] = rows
+    for b in (flag, out4, sink):
+        b.free()
+    print(json.dumps({"ceiling": res}), flush=True)
+
+
 def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
-    """BASELINE config 5: sampled speculative decode at depth 3 after a long prefill."""
+    """BASELINE config 5: sampled speculative decode at depth 3 after a long prefill. Runs the
+    whole sequence twice (the second run is the one reported; the two must give the same tokens)
+    and returns its figures."""
     depth, n_prompt, n_gen, cap = 3, 6621, (1 if args.prefill_only else 256), 16384
     model.set_max_rows(args.prefill_chunk)
     caches = model.make_cache(cap, depth + 1)
@@ -393,7 +498,9 @@ def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
             "accepted": int(st.accepted), "accepted_tokens_per_verify_step": round(int(st.accepted) / max(1, int(st.cycles)), 4),
             "tokens_per_verify_step": round(n_gen / max(1, int(st.cycles)), 3),
             "repeatable": True, "device": dev_name, "data": "synthetic"}
-    print(json.dumps(line), flush=True)
+    for o in (fr, head, caches):
+        o.close()
+    return line
 
 
 def main():
@@ -425,6 +532,9 @@ def main():
                          "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--moe-ab", action="store_true",
                     help="only the A/B of the MoE block's launch structure (option fuse_moe_one = 0, 1, 2)")
+    ap.add_argument("--ceiling", action="store_true",
+                    help="only the machine probes: empty launches, stream-only launches of the expert kernels' shapes, "
+                         "a long read, the workgroup-to-die rule, the latency of a word between workgroups")
     ap.add_argument("--warm-cold", action="store_true",
                     help="only the mat-vec timings on re-used, unread and just-read weights")
     args = ap.parse_args()
@@ -439,6 +549,8 @@ def main():
     dev_name, cus, mem = ctx.device_info()
     log(f"device: {dev_name}, {cus} CUs, {mem / 2**30:.0f} GiB")
 
+    if args.ceiling:
+        return ceiling(orn, ctx, np)
     if args.warm_cold:
         return warm_cold(orn, ctx, np)
     cfg = dict(synth.FULL, num_hidden_layers=args.layers)
@@ -460,7 +572,8 @@ def main():
     if args.moe_ab:
         return moe_ab(orn, ctx, model, np, args.layers)
     if args.config5:
-        return config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name)
+        print(json.dumps(config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name)), flush=True)
+        return
     rng = np.random.default_rng(51)
     prompt = rng.integers(0, cfg["vocab_size"], 51).astype(np.uint32)
     cap = 4096
@@ -537,7 +650,36 @@ def main():
             "distinct_experts": main_w["distinct_experts_mean"], "verify_width": 2, "by_width": by_width}
     log("roofline:", roof)
 
+    # Whole-step figures: the algorithmic bytes one decode step has to read (and the recurrent
+    # state it writes) against the time the step takes. Dense projections of 30 gated-delta and
+    # 10 attention layers, per MoE block the router + (distinct routed + 1) experts, the output
+    # head (all 248,320 rows of Q4_K), 2 MiB of recurrent state a gated-delta layer read once and
+    # written once per row, the KV rows of a context of about 150 tokens. The depth-1 cycle adds
+    # the draft: the bf16 head layer (129 MB) and the 32,768-row pruned output head.
+    dense = 30 * 19_202_048 + 10 * 22_364_160
+    head_full, head_pruned, mtp_layer = 286_064_640, 37_748_736, 129_000_000
+    state = 30 * 2_097_152
+    kv = 10 * 2 * 2 * 150 * 256 * 2
+
+    def step_bytes(T, U):
+        return dense + 40 * ((U + 1) * EXPERT_BYTES + 430_080) + head_full + state * (1 + T) + kv
+
+    u1 = next(w for w in by_width if w["verify_width"] == 1)["distinct_experts_mean"]
+    u2 = main_w["distinct_experts_mean"]
+    plain_ms = ar_s / len(ar) * 1e3
+    cycle_ms = total_s / len(times) / max(1, int(stats.cycles)) * 1e3
+    b_plain, b_cycle = step_bytes(1, u1), step_bytes(2, u2) + mtp_layer + head_pruned
+    step_roof = {"plain_greedy": {"bytes_per_token": int(b_plain), "ms_per_token": round(plain_ms, 4),
+                                  "GB_s": round(b_plain / plain_ms / 1e6, 1), "frac_of_hbm_peak": round(b_plain / plain_ms / 1e6 / HBM_PEAK_GBS, 4)},
+                 "mtp_depth1_cycle": {"bytes_per_cycle": int(b_cycle), "ms_per_cycle": round(cycle_ms, 4),
+                                      "GB_s": round(b_cycle / cycle_ms / 1e6, 1), "frac_of_hbm_peak": round(b_cycle / cycle_ms / 1e6 / HBM_PEAK_GBS, 4)}}
+    log("step_roofline:", step_roof)
+
     configs = per_config(orn, ctx, np, with_cpu=not args.no_cpu)
+    # config 5 (sampled depth-3 decode behind a 6621-token matrix-core prefill) on the same model
+    for o in (fr, head, caches):
+        o.close()
+    configs["config5"] = config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name)
     log("per_config:", configs)
 
     cpu = None
@@ -564,6 +706,7 @@ def main():
                    "cycles": int(stats.cycles), "accepted": int(stats.accepted), "drafted": int(stats.drafted),
                    "weights_GB": round(ws.stats()[1] / 1e9, 2), "device": dev_name},
         "roofline": roof,
+        "step_roofline": step_roof,
         "per_config": configs,
         "cpu_baseline": cpu,
     }

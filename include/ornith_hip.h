@@ -799,6 +799,33 @@ ORNITH_API int ornith_json_dumps(const char* json, size_t len, char* out, size_t
 #define ORNITH_FN_XOR_LANE 9
 ORNITH_API int ornith_selftest_unary(ornith_ctx* ctx, int fn, const float* d_in, float* d_out, int64_t n);
 
+/* ---- machine probes (`bench.py --ceiling`) ------------------------------------------
+ * No reference counterpart (the reference times its own dispatches from the host,
+ * src/bin/dispatch.rs, Q4K.md:479-484); nothing on the decode path calls these. They price a
+ * decode launch against the machine: all are enqueued on the context's stream and timed by
+ * the caller with ornith_timer_begin / ornith_timer_end.
+ * probe_empty: `launches` launches of a kernel that does nothing (with_args: it carries an
+ * argument block the size of the expert kernel's). probe_stream: one launch of `workgroups`
+ * x 256 threads in which every thread reads `per_thread` (1..16) 16-byte pieces, a wavefront's
+ * pieces 1 KB contiguous each and `stride_bytes` apart, all requested before any is used: the
+ * expert launch's shape with none of its arithmetic. probe_read: one grid-stride read of the
+ * whole buffer. probe_xcc: the XCC (die) id each of `workgroups` workgroups ran on, in launch
+ * order. probe_handoff: workgroup `producer` writes a word 4 us into the launch, workgroup
+ * `consumer` polls it (mode 0: plain store, agent-scope loads; 1: agent-scope store and loads;
+ * 2: plain store and plain loads, which never see it); d_out4 receives four 64-bit words:
+ * the 100 MHz clock at the store, at the observation (0: the bounded poll ran out), and the
+ * two workgroups' XCC ids. d_flag must be zeroed by the caller. */
+ORNITH_API int ornith_probe_empty(ornith_ctx* ctx, int workgroups, int threads, int with_args, int launches);
+/* the same launches recorded into a HIP graph and replayed as one submission; *ms_out = the
+ * replay's duration (the device's own launch-after-launch rate, no host enqueue in it) */
+ORNITH_API int ornith_probe_empty_graph(ornith_ctx* ctx, int workgroups, int threads, int with_args, int launches,
+                                        float* ms_out);
+ORNITH_API int ornith_probe_stream(ornith_ctx* ctx, const void* d_src, size_t bytes, int workgroups, int per_thread,
+                                   size_t stride_bytes, void* d_sink);
+ORNITH_API int ornith_probe_read(ornith_ctx* ctx, const void* d_src, size_t bytes, void* d_sink);
+ORNITH_API int ornith_probe_xcc(ornith_ctx* ctx, int workgroups, uint32_t* d_out);
+ORNITH_API int ornith_probe_handoff(ornith_ctx* ctx, void* d_flag, void* d_out4, int producer, int consumer, int mode);
+
 #ifdef __cplusplus
 }
 #endif

@@ -136,3 +136,39 @@ def test_sampled_loop_with_ratio_acceptance_matches_oracle(orn, ctx, tiny_small_
     finally:
         oracle().orc_set_sampler(0, C.c_double(1.0), C.c_double(1.0), 0, C.c_uint64(0))
         fr.close(); head.close(); caches.close()
+
+
+def test_config5_sequence_on_the_tiny_model(orn, ctx):
+    """The sampled configuration end to end at its cache size: a 700-token prompt through the
+    matrix-core prefill path (256-row calls), then sampled depth-3 decode with probability-ratio
+    acceptance and the Philox stream into a 16384-row cache. The prefill path is a tolerance
+    path (its sums run in another order than the oracle's), so what is pinned here is what the
+    configuration promises: the same seed gives the same tokens and counts on every run, another
+    seed gives another sequence, the counts are consistent and the caches end where the loop's
+    contract says (prompt + tokens shown)."""
+    s = synth.SynthModel(dict(synth.TINY, vocab_size=512), seed=21)
+    ws = s.upload(orn, ctx)
+    model = orn.TextModel(ctx, ws, s.text_config(orn))
+    model.set_max_rows(256)
+    V = s.cfg["vocab_size"]
+    n_prompt, n_tok, cap, depth = 700, 48, 16384, 3
+    prompt = np.random.default_rng(3).integers(0, V, n_prompt).astype(np.uint32)
+    fr = orn.FrSpec(model, ids=synth.zipf_frspec_ids(V, 128, seed=1))
+    caches = model.make_cache(cap, depth + 1)
+    head = orn.MtpHead(model, ws, cap)
+    runs = []
+    try:
+        for seed in (2025, 2025, 7):
+            caches.reset()
+            smp = orn.Sampler(1, 0.8, 0.95, 0, seed, orn.ACCEPT_RATIO, orn.RNG_PHILOX)
+            toks, st = orn.generate_step_mtp(model, head, fr, caches, prompt, depth, n_tok, sampler=smp,
+                                             prefill_step=256, policy=orn.HISTORY_COMMITTED)
+            assert len(toks) == n_tok and caches.offset == n_prompt + n_tok
+            assert 0 <= st.accepted <= st.drafted <= depth * st.cycles and st.cycles >= n_tok // (depth + 1)
+            assert st.accepted + st.cycles >= n_tok - 1
+            runs.append((toks, (int(st.cycles), int(st.drafted), int(st.accepted))))
+        assert runs[0] == runs[1], "same seed, different sampled sequence"
+        assert runs[0][0] != runs[2][0], "another seed gave the same 48 sampled tokens"
+    finally:
+        for o in (fr, head, caches, model, ws):
+            o.close()
