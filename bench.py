@@ -381,19 +381,19 @@ def ceiling(orn, ctx, np):
               ("one 4 KB piece a wavefront over 4608 workgroups (75 MB)", 4608, 4, 1024),
               ("lm_head-sized: 17,460 workgroups x 16 KB (286 MB)", 17460, 4, 1024))
     for name, wgs, per, stride in shapes:
-        span = ((wgs * 4 * per - 1) * stride + 1024 + 4095) & ~4095
-        nslots = max(1, min(64, big // span))
-
-        def run(i):
-            off = (i % nslots) * span
-            probe(lib.ornith_probe_stream(ctx.h, C.c_void_p(buf.ptr.value + off), C.c_size_t(span), wgs, per,
-                                          C.c_size_t(stride), sink.ptr), "probe_stream")
-
-        n = 400 if span < (64 << 20) else 60
-        us = _time_loop(ctx, run, n, nslots)
         nbytes = wgs * 256 * per * 16
-        rows.append({"shape": name, "bytes": nbytes, "us_per_launch": round(us, 2),
-                     "GB_s": round(nbytes / (us * 1e-6) / 1e9, 1), "frac_of_8TBs": round(nbytes / (us * 1e-6) / 8e12, 3)})
+        n = 400 if nbytes < (64 << 20) else 60
+        best = 1e30
+        for rep in range(4):   # the first pass also warms the launch path; the best of the rest is reported
+            ctx.sync()
+            ctx.timer_begin()
+            probe(lib.ornith_probe_stream(ctx.h, buf.ptr, C.c_size_t(big), wgs, per, C.c_size_t(stride), sink.ptr, n),
+                  "probe_stream")
+            us = ctx.timer_end() * 1000.0 / n
+            if rep:
+                best = min(best, us)
+        rows.append({"shape": name, "bytes": nbytes, "us_per_launch": round(best, 2),
+                     "GB_s": round(nbytes / (best * 1e-6) / 1e9, 1), "frac_of_8TBs": round(nbytes / (best * 1e-6) / 8e12, 3)})
     res["stream_only_launch"] = rows
 
     # -- one long read

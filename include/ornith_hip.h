@@ -516,10 +516,20 @@ ORNITH_API int ornith_model_set_max_rows(ornith_model* m, int rows);
  * model.layers[i].mlp, src/model/qwen3_5.rs:261-283). */
 ORNITH_API int ornith_model_moe_weights(const ornith_model* m, int layer, ornith_moe_weights* out);
 /* make_cache: one KvCache (bf16 [Hkv, capacity, hd] x2) or GdnCache (conv window +
- * fp32 state with max_window snapshot slots) per layer. capacity bounds prompt +
- * generated tokens (the reference grows in steps of 256; here it is fixed up front). */
+ * fp32 state with max_window snapshot slots) per layer. `capacity` is where the KV tensors
+ * start; a forward that needs more rows grows them, as KvCache::update_and_fetch does
+ * (src/model/cache.rs:38-79): to a multiple of 256 rows, at least half as large again as
+ * before, rows [0, offset) carried over (the stream is synchronised and device memory is
+ * allocated and freed at that moment). A caller that must not allocate inside its loop
+ * reserves up front (ornith_caches_reserve) or fixes the capacity
+ * (ornith_caches_set_growable(c, 0)): ornith_generate / ornith_mtp_generate then refuse, before
+ * any token is handed out, a run whose prompt + max_tokens (+ depth) rows cannot fit, and a
+ * forward past the capacity is an error. */
 ORNITH_API int ornith_caches_create(ornith_model* m, int capacity, int max_window,
                                     ornith_caches** out);
+ORNITH_API int ornith_caches_reserve(ornith_caches* c, int rows);
+ORNITH_API int ornith_caches_set_growable(ornith_caches* c, int growable);
+ORNITH_API int ornith_caches_capacity(const ornith_caches* c, int* capacity_out);
 ORNITH_API int ornith_caches_reset(ornith_caches* c);
 ORNITH_API int ornith_caches_destroy(ornith_caches* c);
 ORNITH_API int ornith_caches_offset(const ornith_caches* c, int* offset_out);
@@ -584,6 +594,9 @@ ORNITH_API int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspe
                                   const void* d_trunk_hidden, const uint32_t* d_next_ids, int T,
                                   void* d_hidden_out, void* d_logits);
 ORNITH_API int ornith_mtp_cache_set_offset(ornith_mtp_head* h, int offset);
+/* the head's one-layer KV cache grows like the trunk's (see ornith_caches_create) */
+ORNITH_API int ornith_mtp_cache_reserve(ornith_mtp_head* h, int rows);
+ORNITH_API int ornith_mtp_cache_set_growable(ornith_mtp_head* h, int growable);
 ORNITH_API int ornith_mtp_cache_offset(const ornith_mtp_head* h, int* offset_out);
 /* Measurement aid, no counterpart in the reference: a host list g[0..n) of the tokens a run
  * is known to produce (g[0] = the first token after the prompt, e.g. the plain greedy output).
@@ -805,10 +818,11 @@ ORNITH_API int ornith_selftest_unary(ornith_ctx* ctx, int fn, const float* d_in,
  * decode launch against the machine: all are enqueued on the context's stream and timed by
  * the caller with ornith_timer_begin / ornith_timer_end.
  * probe_empty: `launches` launches of a kernel that does nothing (with_args: it carries an
- * argument block the size of the expert kernel's). probe_stream: one launch of `workgroups`
- * x 256 threads in which every thread reads `per_thread` (1..16) 16-byte pieces, a wavefront's
- * pieces 1 KB contiguous each and `stride_bytes` apart, all requested before any is used: the
- * expert launch's shape with none of its arithmetic. probe_read: one grid-stride read of the
+ * argument block the size of the expert kernel's). probe_stream: `launches` launches of
+ * `workgroups` x 256 threads in which every thread reads `per_thread` (1..16) 16-byte pieces, a
+ * wavefront's pieces 1 KB contiguous each and `stride_bytes` apart, all requested before any is
+ * used: the expert launch's shape with none of its arithmetic; successive launches walk through
+ * the buffer so that none finds its bytes cached. probe_read: one grid-stride read of the
  * whole buffer. probe_xcc: the XCC (die) id each of `workgroups` workgroups ran on, in launch
  * order. probe_handoff: workgroup `producer` writes a word 4 us into the launch, workgroup
  * `consumer` polls it (mode 0: plain store, agent-scope loads; 1: agent-scope store and loads;
@@ -821,7 +835,7 @@ ORNITH_API int ornith_probe_empty(ornith_ctx* ctx, int workgroups, int threads, 
 ORNITH_API int ornith_probe_empty_graph(ornith_ctx* ctx, int workgroups, int threads, int with_args, int launches,
                                         float* ms_out);
 ORNITH_API int ornith_probe_stream(ornith_ctx* ctx, const void* d_src, size_t bytes, int workgroups, int per_thread,
-                                   size_t stride_bytes, void* d_sink);
+                                   size_t stride_bytes, void* d_sink, int launches);
 ORNITH_API int ornith_probe_read(ornith_ctx* ctx, const void* d_src, size_t bytes, void* d_sink);
 ORNITH_API int ornith_probe_xcc(ornith_ctx* ctx, int workgroups, uint32_t* d_out);
 ORNITH_API int ornith_probe_handoff(ornith_ctx* ctx, void* d_flag, void* d_out4, int producer, int consumer, int mode);

@@ -650,19 +650,17 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
     }
   } else if (hd == 256) {
     // 150 KB of LDS a block (the whole key block staged at once): asked for once per kernel
-    static bool lds_set = false;
-    if (!lds_set) {
+    if (!(ctx->lds_attr_set & 1)) {
       ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<256>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<256>()));
-      lds_set = true;
+      ctx->lds_attr_set |= 1;
     }
     hipLaunchKernelGGL((sdpa_partial_kernel<256>), grid, dim3(SDPA_NT), sdpa_stage_bytes<256>(), ctx->stream, p);
   } else {
-    static bool lds_set = false;
-    if (!lds_set) {
+    if (!(ctx->lds_attr_set & 2)) {
       ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<128>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<128>()));
-      lds_set = true;
+      ctx->lds_attr_set |= 2;
     }
     hipLaunchKernelGGL((sdpa_partial_kernel<128>), grid, dim3(SDPA_NT), sdpa_stage_bytes<128>(), ctx->stream, p);
   }

@@ -100,9 +100,9 @@ int ornith_generate(ornith_model* m, ornith_caches* c, const uint32_t* prompt, s
                     ornith_progress_cb progress, ornith_token_cb on_token, void* user) {
   ORN_REQUIRE(m && c && prompt && on_token, "generate: null argument");
   ORN_REQUIRE(n_prompt >= 1, "generate_step needs a prompt");
-  // the caches are of fixed capacity (the reference's grow in steps of 256): refuse a run that
-  // cannot finish before any token has been handed out
-  ORN_REQUIRE((size_t)c->offset + n_prompt + max_tokens <= (size_t)c->capacity,
+  // caches whose capacity has been fixed (ornith_caches_set_growable(c, 0)): refuse a run that
+  // cannot finish before any token has been handed out; growable ones grow as the rows arrive
+  ORN_REQUIRE(caches_fit(c, (size_t)c->offset + n_prompt + max_tokens),
               "generate: %d cached + %zu prompt + %zu new tokens exceed cache capacity %d", c->offset, n_prompt,
               max_tokens, c->capacity);
   ornith_ctx* ctx = m->ctx;
@@ -160,13 +160,14 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
               "mtp_generate: unknown history policy %d", policy);
   ORN_REQUIRE(head->m == m && (!frspec || frspec->m == m), "mtp_generate: head / frspec of another model");
   if (stats_out) *stats_out = ornith_mtp_stats{};  // defined on every return, error returns included
-  // fixed-capacity caches: a verify window holds up to `depth` rows beyond the committed ones;
-  // the head's own cache holds one row per committed token under Committed, a cycle's rows under
-  // Cycle. Refuse up front rather than fail between two tokens already handed out.
-  ORN_REQUIRE((size_t)c->offset + n_prompt + max_tokens + (size_t)depth <= (size_t)c->capacity,
+  // a verify window holds up to `depth` rows beyond the committed ones; the head's own cache
+  // holds one row per committed token under Committed, a cycle's rows under Cycle. With caches
+  // of fixed capacity a run that cannot fit is refused up front rather than failing between two
+  // tokens already handed out; growable caches grow as the rows arrive.
+  ORN_REQUIRE(caches_fit(c, (size_t)c->offset + n_prompt + max_tokens + (size_t)depth),
               "mtp_generate: %d cached + %zu prompt + %zu new tokens + a %d-row window exceed cache capacity %d",
               c->offset, n_prompt, max_tokens, depth, c->capacity);
-  ORN_REQUIRE((size_t)head->capacity >= (policy == ORNITH_HISTORY_COMMITTED ? max_tokens + (size_t)depth : (size_t)depth),
+  ORN_REQUIRE(mtp_cache_fits(head, policy == ORNITH_HISTORY_COMMITTED ? max_tokens + (size_t)depth : (size_t)depth),
               "mtp_generate: the head's cache of %d rows is too small for %zu tokens at depth %d under this "
               "history policy", head->capacity, max_tokens, depth);
   ornith_ctx* ctx = m->ctx;
@@ -335,6 +336,7 @@ int ornith_mtp_generate(ornith_model* m, ornith_mtp_head* head, const ornith_frs
     if (policy == ORNITH_HISTORY_COMMITTED) {
       // keep the level-1 row (it drafted from the trunk's hidden), rebuild the rest
       // from what the verify pass actually saw
+      TRY(ornith_mtp_cache_reserve(head, cycle_mtp_offset + 1 + k));
       TRY(ornith_mtp_cache_set_offset(head, std::min(cycle_mtp_offset + 1, head->capacity)));
       if (k > 0) TRY(ornith_mtp_forward(head, nullptr, d_hidden, d_window + 1, k, d_scratch_h, nullptr));
     }

@@ -367,6 +367,67 @@ int ornith_model_destroy(ornith_model* m) {
   return ORNITH_OK;
 }
 
+// KvCache::update_and_fetch's growth (/root/reference/src/model/cache.rs:38-79): a KV pair
+// [Hkv, cap, hd] that must hold `need` rows moves to tensors of a larger capacity, a multiple of
+// 256 rows as the reference's steps are and at least half as large again as before (so a long
+// generation copies its cache a logarithmic number of times, not once per 256 tokens). Rows
+// [0, offset) of every head are carried over; what lies past them was never committed.
+static int kv_new_capacity(int capacity, int need) {
+  const long grown = (long)capacity + capacity / 2;
+  const long want = need > grown ? need : grown;
+  return (int)((want + 255) / 256 * 256);
+}
+
+static int kv_move(ornith_model* m, void** buf, int old_cap, int new_cap, int offset) {
+  const auto& c = m->cfg;
+  const size_t row = (size_t)c.head_dim * 2;
+  void* nb = nullptr;
+  TRY(ornith_alloc(m->ctx, (size_t)c.num_key_value_heads * new_cap * row, &nb));
+  if (offset > 0) {
+    hipError_t e = hipMemcpy2DAsync(nb, (size_t)new_cap * row, *buf, (size_t)old_cap * row, (size_t)offset * row,
+                                    c.num_key_value_heads, hipMemcpyDeviceToDevice, m->ctx->stream);
+    if (e != hipSuccess) {
+      ornith_free(m->ctx, nb);
+      return ornith_fail(ORNITH_ERR_HIP, "growing a KV cache: %s", hipGetErrorString(e));
+    }
+  }
+  const int rc = ornith_sync(m->ctx);  // the old tensor is freed next: everything that reads it has run
+  if (rc) {
+    ornith_free(m->ctx, nb);
+    return rc;
+  }
+  ornith_free(m->ctx, *buf);
+  *buf = nb;
+  return ORNITH_OK;
+}
+
+int ornith_caches_reserve(ornith_caches* cc, int rows) {
+  ORN_REQUIRE(cc && rows >= 0, "caches_reserve: bad argument");
+  if (rows <= cc->capacity) return ORNITH_OK;
+  ornith_model* m = cc->m;
+  const int ncap = kv_new_capacity(cc->capacity, rows);
+  TRY(model_ensure_rope(m, ncap));
+  for (size_t i = 0; i < cc->layers.size(); ++i) {
+    if (m->layers[i].linear) continue;
+    TRY(kv_move(m, &cc->layers[i].k, cc->capacity, ncap, cc->offset));
+    TRY(kv_move(m, &cc->layers[i].v, cc->capacity, ncap, cc->offset));
+  }
+  cc->capacity = ncap;
+  return ORNITH_OK;
+}
+
+int ornith_caches_set_growable(ornith_caches* cc, int growable) {
+  ORN_REQUIRE(cc, "caches_set_growable: null caches");
+  cc->growable = growable != 0;
+  return ORNITH_OK;
+}
+
+int ornith_caches_capacity(const ornith_caches* cc, int* capacity_out) {
+  ORN_REQUIRE(cc && capacity_out, "caches_capacity: null argument");
+  *capacity_out = cc->capacity;
+  return ORNITH_OK;
+}
+
 int ornith_caches_create(ornith_model* m, int capacity, int max_window, ornith_caches** out) {
   ORN_REQUIRE(m && out, "caches_create: null argument");
   ORN_REQUIRE(capacity >= 1 && max_window >= 1 && max_window <= kMaxRows,
@@ -452,8 +513,9 @@ int ornith_model_forward(ornith_model* m, ornith_caches* cc, const uint32_t* d_t
               cc->conv_rows - (m->cfg.linear_conv_kernel_dim - 1));
   ORN_REQUIRE(!capture || T <= cc->max_window, "model_forward: capture of %d rows, window is %d", T,
               cc->max_window);
-  ORN_REQUIRE(cc->offset + T <= cc->capacity, "model_forward: %d + %d rows exceed cache capacity %d",
+  ORN_REQUIRE(cc->growable || cc->offset + T <= cc->capacity, "model_forward: %d + %d rows exceed cache capacity %d",
               cc->offset, T, cc->capacity);
+  TRY(ornith_caches_reserve(cc, cc->offset + T));
   return forward_rows(m, cc, d_tokens, T, capture != 0, d_hidden_out);
 }
 
@@ -649,6 +711,23 @@ int ornith_mtp_force_drafts(ornith_mtp_head* h, const uint32_t* tokens, size_t n
   return ORNITH_OK;
 }
 
+int ornith_mtp_cache_reserve(ornith_mtp_head* h, int rows) {
+  ORN_REQUIRE(h && rows >= 0, "mtp_cache_reserve: bad argument");
+  if (rows <= h->capacity) return ORNITH_OK;
+  const int ncap = kv_new_capacity(h->capacity, rows);
+  TRY(model_ensure_rope(h->m, ncap));
+  TRY(kv_move(h->m, &h->k, h->capacity, ncap, h->offset));
+  TRY(kv_move(h->m, &h->v, h->capacity, ncap, h->offset));
+  h->capacity = ncap;
+  return ORNITH_OK;
+}
+
+int ornith_mtp_cache_set_growable(ornith_mtp_head* h, int growable) {
+  ORN_REQUIRE(h, "mtp_cache_set_growable: null head");
+  h->growable = growable != 0;
+  return ORNITH_OK;
+}
+
 int ornith_mtp_cache_set_offset(ornith_mtp_head* h, int offset) {
   ORN_REQUIRE(h && offset >= 0 && offset <= h->capacity, "mtp_cache_set_offset: offset=%d", offset);
   h->offset = offset;
@@ -665,8 +744,9 @@ int ornith_mtp_forward(ornith_mtp_head* h, const ornith_frspec* frspec, const vo
                        const uint32_t* d_next_ids, int T, void* d_hidden_out, void* d_logits) {
   ORN_REQUIRE(h && d_trunk_hidden && d_next_ids && d_hidden_out, "mtp_forward: null argument");
   ORN_REQUIRE(T >= 1 && T <= h->max_rows, "mtp_forward: T=%d", T);
-  ORN_REQUIRE(h->offset + T <= h->capacity, "mtp_forward: %d + %d rows exceed the head's cache (%d)",
+  ORN_REQUIRE(h->growable || h->offset + T <= h->capacity, "mtp_forward: %d + %d rows exceed the head's cache (%d)",
               h->offset, T, h->capacity);
+  TRY(ornith_mtp_cache_reserve(h, h->offset + T));
   ornith_model* m = h->m;
   ornith_ctx* ctx = m->ctx;
   const auto& c = m->cfg;

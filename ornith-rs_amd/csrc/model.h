@@ -79,6 +79,17 @@ struct ornith_weights {
     }                                                                \
   } while (0)
 
+// After lookups that may legitimately come back null (an optional tensor): a failed copy-in
+// is reported as itself rather than read as "the tensor is absent".
+#define ORN_RETURN_FAULT(ws)               \
+  do {                                     \
+    if ((ws)->fault_rc) {                  \
+      const int rc__ = (ws)->fault_rc;     \
+      (ws)->fault_rc = 0;                  \
+      return rc__;                         \
+    }                                      \
+  } while (0)
+
 // Resolves module `path` into a Linear by the tensors present (k-quant / affine8 / dense).
 int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* out);
 // A routed k-quant module [E, O, K].
@@ -138,6 +149,7 @@ struct LayerCache {
 struct ornith_caches {
   ornith_model* m = nullptr;
   int capacity = 0, max_window = 0, conv_rows = 0;
+  bool growable = true;  // a forward past the capacity grows the KV tensors (else it is refused)
   std::vector<LayerCache> layers;
   // one set of cursors serves every layer: they all advance together
   int offset = 0;     // tokens held
@@ -166,6 +178,7 @@ struct ornith_mtp_head {
   // one-layer KV cache
   void *k = nullptr, *v = nullptr;
   int capacity = 0, offset = 0;
+  bool growable = true;
   void* buf = nullptr;  // step buffers
   int max_rows = 0;
   // tokens that replace the drafts (ornith_mtp_force_drafts), indexed by output position
@@ -175,3 +188,7 @@ struct ornith_mtp_head {
 
 // grows the model's RoPE tables to cover `npos` positions
 int model_ensure_rope(ornith_model* m, int npos);
+// What a loop asks before it starts: `rows` rows must fit. Growable caches always say yes (they
+// grow as the rows arrive); fixed ones are checked against their capacity.
+inline bool caches_fit(const ornith_caches* c, size_t rows) { return c->growable || rows <= (size_t)c->capacity; }
+inline bool mtp_cache_fits(const ornith_mtp_head* h, size_t rows) { return h->growable || rows <= (size_t)h->capacity; }

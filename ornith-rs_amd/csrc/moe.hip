@@ -304,7 +304,19 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
     ORN_REQUIRE(!d_inds_out && !d_scores_out, "moe_block: index outputs are a decode-width feature");
     return moe_block_prefill(ctx, w, d_x, T, d_out);
   }
-  ORN_REQUIRE(T <= 64, "moe_block: T=%d with dense or 4-bit affine experts (decode/verify widths only)", T);
+  if (T > 64) {
+    // dense and 4-bit affine experts have no prefill-width form: the operator path takes the
+    // rows in blocks of 64 (rows are independent of each other, so the result is the same)
+    for (int t0 = 0; t0 < T; t0 += 64) {
+      const int n = T - t0 < 64 ? T - t0 : 64;
+      const int rcb = moe_block_impl(ctx, w, static_cast<const bf16_t*>(d_x) + (size_t)t0 * H, n,
+                                     static_cast<bf16_t*>(d_out) + (size_t)t0 * H,
+                                     d_inds_out ? d_inds_out + (size_t)t0 * k : nullptr,
+                                     d_scores_out ? static_cast<bf16_t*>(d_scores_out) + (size_t)t0 * k : nullptr, nullptr);
+      if (rcb) return rcb;
+    }
+    return ORNITH_OK;
+  }
 
   const size_t need = 2 * ((size_t)T * E * 2 + (size_t)T * SI * 3 + (size_t)T * H + T +
                            (size_t)(T * k + T) * (2 * I + I + SI + H + 1)) +

@@ -152,14 +152,19 @@ int ornith_probe_empty_graph(ornith_ctx* ctx, int workgroups, int threads, int w
 }
 
 int ornith_probe_stream(ornith_ctx* ctx, const void* d_src, size_t bytes, int workgroups, int per_thread,
-                        size_t stride_bytes, void* d_sink) {
-  ORN_REQUIRE(ctx && d_src && d_sink && workgroups >= 1 && per_thread >= 1 && per_thread <= 16,
+                        size_t stride_bytes, void* d_sink, int launches) {
+  ORN_REQUIRE(ctx && d_src && d_sink && workgroups >= 1 && per_thread >= 1 && per_thread <= 16 && launches >= 1,
               "probe_stream: bad argument");
   ORN_REQUIRE(stride_bytes >= 1024 && stride_bytes % 16 == 0, "probe_stream: stride of %zu bytes", stride_bytes);
-  const size_t need = ((size_t)workgroups * 4 * per_thread - 1) * stride_bytes + 1024;
-  ORN_REQUIRE(need <= bytes, "probe_stream: the launch reads %zu bytes, the buffer has %zu", need, bytes);
-  hipLaunchKernelGGL(probe_stream_kernel, dim3(workgroups), dim3(256), 0, ctx->stream, (const uint4*)d_src,
-                     per_thread, stride_bytes / 16, (uint32_t*)d_sink);
+  // one launch reads `span` bytes; launch i starts (i mod slots) spans into the buffer, so that
+  // no launch finds its bytes in a cache when the buffer holds many spans
+  const size_t span = ((((size_t)workgroups * 4 * per_thread - 1) * stride_bytes + 1024) + 4095) & ~size_t(4095);
+  ORN_REQUIRE(span <= bytes, "probe_stream: a launch reads %zu bytes, the buffer has %zu", span, bytes);
+  const size_t slots = bytes / span;
+  for (int i = 0; i < launches; ++i)
+    hipLaunchKernelGGL(probe_stream_kernel, dim3(workgroups), dim3(256), 0, ctx->stream,
+                       (const uint4*)(static_cast<const char*>(d_src) + (i % slots) * span), per_thread,
+                       stride_bytes / 16, (uint32_t*)d_sink);
   ORN_LAUNCH_CHECK("probe_stream_kernel");
   return ORNITH_OK;
 }

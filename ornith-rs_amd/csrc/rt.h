@@ -31,6 +31,11 @@ struct ornith_ctx {
   uint32_t ho_epoch = 0;
   volatile uint32_t* ho_err = nullptr;
   uint32_t* ho_err_dev = nullptr;
+  // kernels whose dynamic LDS limit has been raised for this context's device (a function
+  // attribute is per device; a context is used from one thread at a time)
+  unsigned lds_attr_set = 0;
+  // this device's copy of the greedy selection's fixed scratch array (sample.hip)
+  void* na_scratch = nullptr;
 };
 
 // After the stream has been synchronised: fails if a hand-off wait inside a launch gave up.
@@ -69,8 +74,8 @@ int ornith_greedy_rows_ws(ornith_ctx* ctx, const void* d_logits, int rows, int V
                           void* d_lse, ScratchCursor& sc);
 
 // Resolves the device address of the greedy selection's fixed scratch array on `device`
-// (which must be current); ornith_ctx_create calls it once per device.
-int ornith_sample_init_device(int device);
+// (which must be current) once per device; ornith_ctx_create keeps it in the context.
+int ornith_sample_init_device(int device, void** ptr_out);
 
 // Records the message for ornith_last_error() and returns `code`.
 int ornith_fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));

@@ -136,35 +136,46 @@ int ornith_ctx_create(int device, ornith_ctx** out) {
     return ornith_fail(ORNITH_ERR_UNSUPPORTED,
                        "ornith_ctx_create: device %d is %s; this library is built for gfx950 only",
                        device, prop.gcnArchName);
-  if (int rc = ornith_sample_init_device(device)) return rc;
+  void* na_scratch = nullptr;
+  if (int rc = ornith_sample_init_device(device, &na_scratch)) return rc;
   ornith_ctx* c = new ornith_ctx();
   c->device = device;
+  c->na_scratch = na_scratch;
   c->compute_units = prop.multiProcessorCount;
-  ORN_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
-  ORN_HIP(hipEventCreate(&c->ev0));
-  ORN_HIP(hipEventCreate(&c->ev1));
-  ORN_HIP(hipHostMalloc(&c->pinned, ornith_ctx::kPinnedBytes, hipHostMallocDefault));
-  ORN_HIP(hipMalloc((void**)&c->ho_flags, sizeof(uint32_t) * ornith_ctx::kHoFlagWords));
-  ORN_HIP(hipMemset(c->ho_flags, 0, sizeof(uint32_t) * ornith_ctx::kHoFlagWords));
-  void* err_host = nullptr;
-  ORN_HIP(hipHostMalloc(&err_host, 256, hipHostMallocDefault));
-  memset(err_host, 0, 256);
-  c->ho_err = static_cast<volatile uint32_t*>(err_host);
-  ORN_HIP(hipHostGetDevicePointer((void**)&c->ho_err_dev, err_host, 0));
+  // every step below can fail: one way out, which releases whatever the steps before it made
+  const int rc = [&]() -> int {
+    ORN_HIP(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+    ORN_HIP(hipEventCreate(&c->ev0));
+    ORN_HIP(hipEventCreate(&c->ev1));
+    ORN_HIP(hipHostMalloc(&c->pinned, ornith_ctx::kPinnedBytes, hipHostMallocDefault));
+    ORN_HIP(hipMalloc((void**)&c->ho_flags, sizeof(uint32_t) * ornith_ctx::kHoFlagWords));
+    ORN_HIP(hipMemset(c->ho_flags, 0, sizeof(uint32_t) * ornith_ctx::kHoFlagWords));
+    void* err_host = nullptr;
+    ORN_HIP(hipHostMalloc(&err_host, 256, hipHostMallocDefault));
+    memset(err_host, 0, 256);
+    c->ho_err = static_cast<volatile uint32_t*>(err_host);
+    ORN_HIP(hipHostGetDevicePointer((void**)&c->ho_err_dev, err_host, 0));
+    return ORNITH_OK;
+  }();
+  if (rc) {
+    ornith_ctx_destroy(c);
+    return rc;
+  }
   *out = c;
   return ORNITH_OK;
 }
 
 int ornith_ctx_destroy(ornith_ctx* ctx) {
   if (!ctx) return ORNITH_OK;
-  (void)hipStreamSynchronize(ctx->stream);
+  // also the way out of a context that was only partly made: every member is checked
+  if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
   if (ctx->scratch) (void)hipFree(ctx->scratch);
   if (ctx->pinned) (void)hipHostFree(ctx->pinned);
   if (ctx->ho_flags) (void)hipFree(ctx->ho_flags);
   if (ctx->ho_err) (void)hipHostFree(const_cast<uint32_t*>(ctx->ho_err));
-  (void)hipEventDestroy(ctx->ev0);
-  (void)hipEventDestroy(ctx->ev1);
-  (void)hipStreamDestroy(ctx->stream);
+  if (ctx->ev0) (void)hipEventDestroy(ctx->ev0);
+  if (ctx->ev1) (void)hipEventDestroy(ctx->ev1);
+  if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
   delete ctx;
   return ORNITH_OK;
 }

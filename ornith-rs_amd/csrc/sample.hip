@@ -33,7 +33,8 @@ constexpr size_t NA_BYTES = 4 * NA_ARRAY_BYTES;
 static __device__ __align__(256) unsigned char scratch[NA_BYTES];
 
 // `scratch` names a host-side stand-in here; the array's device address differs per GPU
-// and is asked for once per device (ornith_sample_init_device) and kept in this table.
+// and is asked for once per device (ornith_sample_init_device, under the lock) and kept in this
+// table; a context carries its device's address, so no call reads the table afterwards.
 constexpr int NA_MAX_DEVICES = 64;
 void* g_scratch_ptr[NA_MAX_DEVICES] = {};
 std::mutex g_scratch_mu;
@@ -202,15 +203,18 @@ int run(ornith_ctx* ctx, const void* d_logits, int rows, int V, uint32_t* d_toke
 }  // namespace
 
 // Called by ornith_ctx_create with `device` current: resolves this GPU's copy of `scratch`.
-int ornith_sample_init_device(int device) {
+int ornith_sample_init_device(int device, void** ptr_out) {
   ORN_REQUIRE(device >= 0 && device < NA_MAX_DEVICES, "device %d is beyond the %d this library tracks", device,
               NA_MAX_DEVICES);
+  ORN_REQUIRE(ptr_out, "sample_init_device: null argument");
   std::lock_guard<std::mutex> lock(g_scratch_mu);
-  if (g_scratch_ptr[device]) return ORNITH_OK;
-  void* ptr = nullptr;
-  ORN_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-  ORN_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null address for the fixed scratch array");
-  g_scratch_ptr[device] = ptr;
+  if (!g_scratch_ptr[device]) {
+    void* ptr = nullptr;
+    ORN_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    ORN_REQUIRE(ptr != nullptr, "hipGetSymbolAddress returned a null address for the fixed scratch array");
+    g_scratch_ptr[device] = ptr;
+  }
+  *ptr_out = g_scratch_ptr[device];
   return ORNITH_OK;
 }
 
@@ -246,7 +250,7 @@ int ornith_greedy_rows_noalloc(ornith_ctx* ctx, const void* d_logits, int rows, 
   ORN_REQUIRE(V >= 1 && V <= NA_MAX_V,
               "greedy_rows_noalloc: %d logits a row; the fixed scratch array holds at most %d (use "
               "ornith_greedy_rows)", V, NA_MAX_V);
-  void* ptr = (ctx->device >= 0 && ctx->device < NA_MAX_DEVICES) ? g_scratch_ptr[ctx->device] : nullptr;
+  void* ptr = ctx->na_scratch;  // resolved for this context's device when the context was made
   ORN_REQUIRE(ptr != nullptr, "greedy_rows_noalloc: the fixed scratch array of device %d was never resolved",
               ctx->device);
   // every partial is written by the pass before the one that reads it, for exactly the

@@ -35,9 +35,11 @@ static int check_mode(const ornith_weights* ws, const std::string& path, bool is
 
 static int kq_from(const ornith_weights* ws, const std::string& path, bool routed,
                    ornith_kmatrix* out) {
+  ws->fault_rc = 0;
   const Tensor* w = ws->find(path + ".weight");
   const Tensor* s = ws->find(path + ".scales");
   const Tensor* d = ws->find(path + ".dm");
+  ORN_RETURN_FAULT(ws);
   if (routed && w && s && !d && ornith_weights_has(ws, (path + ".biases").c_str())) {
     // stacked experts in the 4-bit affine group-32 format (the published artifact's switch_mlp)
     const Tensor* b = ws->find(path + ".biases");
@@ -93,6 +95,7 @@ int ws_kmatrix(const ornith_weights* ws, const std::string& path, ornith_kmatrix
 
 int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* out) {
   memset(out, 0, sizeof *out);
+  ws->fault_rc = 0;
   const Tensor* w = ws->find(path + ".weight");
   ORN_REQUIRE_TENSOR(ws, w, "%s.weight: no such tensor", path.c_str());
   if (ornith_weights_has(ws, (path + ".dm").c_str())) {
@@ -105,9 +108,11 @@ int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* 
   }
   int rc = check_mode(ws, path, false, 0);
   if (rc) return rc;
-  if (const Tensor* b = ws->find(path + ".biases")) {
+  const Tensor* b = ws->find(path + ".biases");
+  ORN_RETURN_FAULT(ws);  // a .biases that exists but could not be copied in is not a dense module
+  if (b) {
     const Tensor* s = ws->find(path + ".scales");
-    ORN_REQUIRE(s, "%s: affine module needs .scales", path.c_str());
+    ORN_REQUIRE_TENSOR(ws, s, "%s: affine module needs .scales", path.c_str());
     ORN_REQUIRE(s->dtype == ORNITH_DT_BF16 && b->dtype == ORNITH_DT_BF16,
                 "%s: affine scales/biases must be bfloat16", path.c_str());
     ORN_REQUIRE(w->dtype == ORNITH_DT_U32 || w->dtype == ORNITH_DT_U8, "%s.weight must be uint32",
@@ -149,6 +154,7 @@ int ws_linear(const ornith_weights* ws, const std::string& path, ornith_linear* 
 
 int ws_tensor(const ornith_weights* ws, const std::string& name, int dtype, int64_t numel,
               const void** out) {
+  ws->fault_rc = 0;
   const Tensor* t = ws->find(name);
   ORN_REQUIRE_TENSOR(ws, t, "%s: no such tensor", name.c_str());
   ORN_REQUIRE(t->dtype == dtype, "%s: dtype %d, expected %d", name.c_str(), t->dtype, dtype);

@@ -228,6 +228,20 @@ class Caches:
     def reset(self):
         _check(lib().ornith_caches_reset(self.h), "caches_reset")
 
+    def reserve(self, rows):
+        """Grow the KV tensors now so that `rows` rows fit (they grow by themselves otherwise)."""
+        _check(lib().ornith_caches_reserve(self.h, rows), "caches_reserve")
+
+    def set_growable(self, growable):
+        """False: the capacity is fixed; loops refuse up front what cannot fit."""
+        _check(lib().ornith_caches_set_growable(self.h, int(growable)), "caches_set_growable")
+
+    @property
+    def capacity(self):
+        o = C.c_int()
+        _check(lib().ornith_caches_capacity(self.h, C.byref(o)), "caches_capacity")
+        return o.value
+
     @property
     def offset(self):
         o = C.c_int()
@@ -347,6 +361,13 @@ class MtpHead:
             for b in (dh, di, do, dl):
                 if b:
                     b.free()
+
+    def set_growable(self, growable):
+        """False: the head's cache keeps its capacity; a run that cannot fit is refused."""
+        _check(lib().ornith_mtp_cache_set_growable(self.h, int(growable)), "mtp_cache_set_growable")
+
+    def reserve(self, rows):
+        _check(lib().ornith_mtp_cache_reserve(self.h, rows), "mtp_cache_reserve")
 
     def set_offset(self, off):
         _check(lib().ornith_mtp_cache_set_offset(self.h, off), "mtp_cache_set_offset")

@@ -71,10 +71,11 @@ def test_model_with_4bit_affine_modules_matches_oracle(orn, ctx):
         head.close(); caches.close(); model.close(); ws.close()
 
 
-@pytest.mark.parametrize("T", [1, 2, 4, 9])
+@pytest.mark.parametrize("T", [1, 2, 4, 9, 150])
 def test_moe_block_with_4bit_affine_experts_bit_exact(orn, ctx, T):
     """The published artifact's block: routed and shared experts 4-bit affine group 32, router and
-    shared gate 8-bit. Expert ids, scores and output by bits against the oracle."""
+    shared gate 8-bit. Expert ids, scores and output by bits against the oracle. 150 rows: a
+    prompt chunk wider than the operator path's 64 rows, taken in blocks."""
     rng = np.random.default_rng(40 + T)
     moe = util.HostMoe(rng, H=1024, E=64, I=256, top_k=8, gate_kind=util.AFFINE4)
     xb = util.bf16_normal(rng, (T, 1024))

@@ -237,6 +237,7 @@ def test_stop_callback_and_errors(orn, ctx, tiny):
     assert len(seen) == 3 and caches.offset == 5 + 3   # the stopping token is in the caches too
     head = orn.MtpHead(model, ws, 32)
     caches.reset()
+    caches.set_growable(False)      # fixed capacity: what cannot fit is refused
     with pytest.raises(orn.OrnithError, match="capture window"):
         orn.generate_step_mtp(model, head, None, caches, prompt, 3, 5)
     with pytest.raises(orn.OrnithError, match="exceed cache capacity"):
@@ -249,6 +250,7 @@ def test_stop_callback_and_errors(orn, ctx, tiny):
     with pytest.raises(orn.OrnithError, match="exceed cache capacity"):
         orn.generate_step_mtp(model, head, None, caches, prompt, 1, 27, on_token=lambda t: (seen.append(t), True)[1])
     small_head = orn.MtpHead(model, ws, 4)
+    small_head.set_growable(False)
     with pytest.raises(orn.OrnithError, match="head's cache"):
         orn.generate_step_mtp(model, small_head, None, caches, prompt, 1, 10, on_token=lambda t: (seen.append(t), True)[1])
     toks, _ = orn.generate_step_mtp(model, small_head, None, caches, prompt, 1, 10, policy=orn.HISTORY_CYCLE)
@@ -260,6 +262,39 @@ def test_stop_callback_and_errors(orn, ctx, tiny):
     with pytest.raises(orn.OrnithError, match="temp"):
         orn.generate_step(model, caches, prompt, 2, sampler=orn.Sampler(1, 0.0, 0.95, 0, 1))
     head.close(); caches.close()
+
+
+def test_caches_grow_like_the_reference_and_change_nothing(orn, ctx, tiny):
+    """KvCache::update_and_fetch grows its tensors when a step does not fit
+    (/root/reference/src/model/cache.rs:38-79). Caches that start at 8 rows and grow under both
+    loops give the tokens, the counts and the hidden rows of caches that were large from the
+    start; the capacity moves in multiples of 256 rows; reserve() grows ahead of time."""
+    s, ws, model = tiny
+    rng = np.random.default_rng(17)
+    prompt = rng.integers(0, s.cfg["vocab_size"], 300).astype(np.uint32)   # past one 256-row step in the prefill
+    n = 40
+    big, small = model.make_cache(1024, 3), model.make_cache(8, 3)
+    hb, hs = orn.MtpHead(model, ws, 1024), orn.MtpHead(model, ws, 2)
+    try:
+        want = orn.generate_step(model, big, prompt, n, prefill_step=16)
+        got = orn.generate_step(model, small, prompt, n, prefill_step=16)
+        assert got == want and small.offset == big.offset == 300 + n
+        assert small.capacity % 256 == 0 and 300 + n <= small.capacity < 1024
+        # the rows a grown cache holds are the rows a large one holds: continue from both
+        nxt = rng.integers(0, s.cfg["vocab_size"], 5).astype(np.uint32)
+        assert np.array_equal(model.forward(small, nxt), model.forward(big, nxt))
+        big.reset(); small.close()
+        small = model.make_cache(8, 3)
+        wt, wst = orn.generate_step_mtp(model, hb, None, big, prompt, 2, n, prefill_step=16, policy=orn.HISTORY_COMMITTED)
+        gt, gst = orn.generate_step_mtp(model, hs, None, small, prompt, 2, n, prefill_step=16, policy=orn.HISTORY_COMMITTED)
+        assert gt == wt == want
+        assert (gst.cycles, gst.drafted, gst.accepted) == (wst.cycles, wst.drafted, wst.accepted)
+        assert hs.offset == hb.offset
+        small.reserve(5000)
+        assert small.capacity >= 5000 and small.capacity % 256 == 0 and small.offset == 300 + n
+        assert np.array_equal(model.forward(small, nxt), model.forward(big, nxt))
+    finally:
+        for o in (hb, hs, big, small): o.close()
 
 
 @pytest.mark.parametrize("temp,top_p,top_k", [(0.8, 0.95, 0), (0.6, 0.95, 20), (1.0, 1.0, 0)])

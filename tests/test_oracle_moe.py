@@ -137,3 +137,28 @@ def test_moe_block_matches_numpy_float64_composition():
         got = util.bf16_to_f32(out[t]).astype(np.float64)
         scale = np.max(np.abs(want))
         assert np.max(np.abs(got - want)) <= 0.03 * scale, (t, np.max(np.abs(got - want)), scale)
+
+
+def test_dense_gather_mv_against_float64_and_its_index_roles():
+    """out[r] = x[lhs[r]] . W[rhs[r]]^T over stacked bf16 experts: every row within one bf16 ulp
+    of the float64 product of the row lhs names with the expert rhs names; with the two index
+    lists exchanged (a transposed-operand mistake) the result must be far off."""
+    rng = np.random.default_rng(11)
+    E, O, K, X, R = 6, 24, 256, 4, 9
+    w = util.f32_to_bf16(rng.standard_normal((E, O, K)).astype(np.float32))
+    xb = util.f32_to_bf16(rng.standard_normal((X, K)).astype(np.float32))
+    lhs = np.array([0, 1, 2, 3, 3, 2, 1, 0, 2], np.uint32)
+    rhs = np.array([5, 4, 3, 2, 1, 0, 5, 3, 4], np.uint32)
+    y = np.empty((R, O), np.uint16)
+    oracle().orc_dense_gather_mv(p(w), O, K, p(xb), p(lhs), p(rhs), R, p(y))
+    w64, x64 = util.bf16_to_f32(w).astype(np.float64), util.bf16_to_f32(xb).astype(np.float64)
+    want = np.stack([w64[rhs[r]] @ x64[lhs[r]] for r in range(R)])
+    got = util.bf16_to_f32(y).astype(np.float64)
+    assert np.all(np.abs(got - want) <= 2.0 ** -8 * np.abs(want) + 1e-5)
+    # the roles of the lists: lhs indexes activation rows (< X), rhs experts (< E)
+    swapped = np.stack([w64[lhs[r]] @ x64[rhs[r] % X] for r in range(R)])
+    assert np.max(np.abs(got - swapped)) > 1.0
+    # and a gathered row is the plain mat-vec of that expert's slice on that activation row
+    y1 = np.empty((1, O), np.uint16)
+    oracle().orc_dense_gemv(p(np.ascontiguousarray(w[rhs[4]])), O, K, p(np.ascontiguousarray(xb[lhs[4]:lhs[4] + 1])), 1, p(y1))
+    assert np.array_equal(y1[0], y[4])

@@ -148,3 +148,44 @@ def test_sampled_loop_with_ratio_acceptance():
         assert runs[(0, 1, False)][0] != runs[(1, 1, False)][0]  # the generators differ
     finally:
         synth.util.oracle().orc_set_sampler(0, C.c_double(1.0), C.c_double(1.0), 0, C.c_uint64(0))
+
+
+def test_sampler_weights_against_float64():
+    """orc_sampler_weights (the unnormalised distribution both sides of the acceptance ratio
+    use): w_i = exp((lp_i - max) / T) over the filtered log-probabilities, 0 for a filtered-out
+    token, and the returned total is their sum. Checked against float64 on the surviving set
+    the oracle's own (separately pinned) top-p / top-k stages name; the temperature enters as
+    the bf16-rounded 1/T and the scaled log-probability is rounded to bf16 before the exponential,
+    as the reference's categorical draw does, so the comparison allows that rounding."""
+    f = oracle().orc_sampler_weights
+    f.restype = C.c_float
+    rng = np.random.default_rng(4)
+    V = 300
+    for temp, top_p, top_k in ((0.8, 0.95, 0), (1.0, 1.0, 0), (0.6, 0.9, 20), (1.3, 0.5, 0)):
+        logits = util.bf16_normal(rng, (V,), 2.5)
+        w = np.empty(V, np.float32)
+        total = f(p(logits), V, C.c_double(temp), C.c_double(top_p), top_k, p(w))
+        # the filtered log-probabilities, from the stages pinned in test_oracle_sampler.py
+        lp = np.empty(V, np.uint16)
+        oracle().orc_logprobs_row(p(logits), V, p(lp))
+        if 0.0 < top_p < 1.0:
+            b = np.empty(V, np.uint16)
+            oracle().orc_apply_top_p(p(lp), V, C.c_double(top_p), p(b))
+            lp = b
+        if top_k > 0:
+            b = np.empty(V, np.uint16)
+            oracle().orc_apply_top_k(p(lp), V, top_k, p(b))
+            lp = b
+        lpf = util.bf16_to_f32(lp).astype(np.float64)
+        keep = np.isfinite(lpf)
+        assert 0 < keep.sum() <= V and (top_k == 0 or keep.sum() <= top_k)
+        assert np.all(w[~keep] == 0.0) and np.all(w[keep] > 0.0)
+        inv_t = float(util.bf16_to_f32(util.f32_to_bf16(np.array([1.0 / temp], np.float32)))[0])
+        z = lpf[keep] * inv_t
+        want = np.exp(z - z.max())
+        # z is rounded to bf16 (relative 2^-9 of |z|) before the exponential: an absolute error of
+        # up to 2^-9 |z| in the exponent, i.e. that much relative error in w
+        tol = 2.0 ** -8 * np.maximum(np.abs(z), np.abs(z.max())) + 1e-6
+        assert np.all(np.abs(w[keep] / want - 1.0) <= tol), float(np.max(np.abs(w[keep] / want - 1.0) / tol))
+        assert w[keep].max() == 1.0            # the most likely token has weight exp(0)
+        assert abs(float(total) - float(np.sum(w.astype(np.float64)))) <= 1e-5 * float(total)

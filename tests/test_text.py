@@ -355,3 +355,69 @@ def test_rendered_prompt_round_trips_through_the_tokenizer(tk):
     assert ids[0] == tk.id("<|im_start|>") and ids.count(tk.id("<|im_end|>")) == 2
     assert tk.id("<think>") in ids and tk.id("</think>") in ids
     assert tk.decode(ids) == prompt
+
+
+# ---- against the reference's own Unicode 16 tables (this container only) ------------------
+_REF_TABLES = "/root/reference/src/tokenizer/tables.rs"
+
+
+def _ref_table(src, name, width):
+    import re
+    body = re.search(r"pub static %s: &\[\((?:u32|u8)(?:, (?:u32|u8))*\)\] = &\[(.*?)\];" % name, src, re.S).group(1)
+    nums = [int(x, 0) for x in re.findall(r"0x[0-9A-Fa-f]+|\d+", body)]
+    assert len(nums) % width == 0
+    return [tuple(nums[i:i + width]) for i in range(0, len(nums), width)]
+
+
+@pytest.mark.skipif(not os.path.exists(_REF_TABLES), reason="the reference's tables are only present where it is mounted")
+def test_tables_against_the_reference_unicode_16_tables():
+    """The reference's tokenizer tables are Unicode 16 data (src/tokenizer/tables.rs, read here as
+    text); this library's are Unicode 13 (what this image's Python can generate). For every code
+    point Unicode 13 assigns, the character class equals the one the reference's LETTER / MARK /
+    NUMBER / WHITE_SPACE ranges give, a code point outside its NFC_UNSAFE ranges is left alone
+    by nfc(), and every primary composite of its COMPOSE table made of such code points
+    composes. What differs is exactly the code points assigned since Unicode 13 that the
+    reference classes as letter, mark or number: here they are class 0 (their count is
+    printed); text containing them splits differently, and that stays parity-unpinned."""
+    src = open(_REF_TABLES).read()
+    want = bytearray(0x110000)
+    for name, cls in (("WHITE_SPACE", 3), ("NUMBER", 2), ("MARK", 1), ("LETTER", 1)):
+        for a, b in _ref_table(src, name, 2):
+            for c in range(a, b + 1):
+                want[c] = cls
+    unsafe = bytearray(0x110000)
+    for a, b in _ref_table(src, "NFC_UNSAFE", 2):
+        for c in range(a, b + 1):
+            unsafe[c] = 1
+    bad, newer, changed = [], 0, []
+    for c in range(0x110000):
+        if 0xD800 <= c <= 0xDFFF:
+            continue
+        got = text.char_class(c)
+        if ud.category(chr(c)) == "Cn":
+            # not assigned in Unicode 13: this library knows nothing about it
+            assert got == 0, hex(c)
+            newer += want[c] != 0
+            continue
+        if got != want[c]:
+            bad.append((hex(c), got, want[c]))
+    # a handful of assigned code points changed general category between the two versions
+    for h, got, w in bad:
+        changed.append(h)
+    print("classes: %d code points newer than Unicode 13 are letters / marks / numbers in the reference's tables "
+          "and class 0 here; %d assigned code points differ: %s" % (newer, len(bad), changed[:12]))
+    assert len(bad) <= 8, bad[:20]
+    assert 5000 < newer < 12000
+    # NFC: what the reference calls safe is left alone (sampled: every 7th code point, all of the BMP's first 0x3000)
+    for c in list(range(0x3000)) + list(range(0x3000, 0x110000, 7)):
+        if 0xD800 <= c <= 0xDFFF or ud.category(chr(c)) == "Cn" or unsafe[c]:
+            continue
+        assert text.nfc(chr(c)) == chr(c), hex(c)
+    # and its primary composites compose (those whose three code points Unicode 13 has)
+    n = 0
+    for first, second, composed in _ref_table(src, "COMPOSE", 3):
+        if any(ud.category(chr(x)) == "Cn" for x in (first, second, composed)):
+            continue
+        assert text.nfc(chr(first) + chr(second)) == chr(composed), (hex(first), hex(second))
+        n += 1
+    assert n > 900
