@@ -124,6 +124,44 @@ def expert_roofline(orn, ctx, model, np, n_layers, T, pairs=400):
                               "frac": round(up_bytes / (us_up * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)}}
 
 
+def expert_overlap(orn, ctx, model, np, n_layers, cases=("distinct", "same8"), widths=(2, 4), pairs=400):
+    """Verify rows of real text share experts; random-init routing does not (U = 15.4 of 16 at
+    T = 2). This leg gives the up + down pair routing in which all T tokens pick the same 8
+    experts (`same8`) beside routing with 8 T distinct ones (`distinct`), ids given, cycling the
+    layers' resident weights so that nothing is warm from an earlier launch. The kernels take a
+    (token, expert) row per workgroup column, but a grid x of 64 puts the workgroups that read
+    the same weight rows for different tokens on the same die, so the second token's reads are
+    L2 hits: `bytes_distinct` is what memory has to deliver."""
+    rng = np.random.default_rng(321)
+    H, I, E, k = 2048, 512, 256, 8
+    moes = [model.moe_weights(i) for i in range(n_layers)]
+    rows = []
+    for T in widths:
+        x = ctx.to_device(orn.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32)))
+        scores = ctx.to_device(orn.f32_to_bf16((rng.random((T, k)) + 0.1).astype(np.float32)))
+        egate = ctx.to_device(orn.f32_to_bf16(rng.standard_normal((T,)).astype(np.float32)))
+        act, out = ctx.alloc((T * k + T) * I * 2), ctx.alloc(T * H * 2)
+        for case in cases:
+            ids = []
+            for _ in range(n_layers):
+                if case == "same8":
+                    v = np.tile(rng.permutation(E)[:k], T)
+                else:
+                    v = rng.permutation(E)[:k * T]
+                ids.append(ctx.to_device(v.astype(np.uint32)))
+            us = _time_loop(ctx, lambda i: orn.moe_experts(ctx, moes[i % n_layers], x, T, ids[i % n_layers], scores, egate,
+                                                           act, out, 3), pairs, n_layers)
+            U = k if case == "same8" else k * T
+            nbytes = (U + 1) * EXPERT_BYTES + T * H * 2 * 2 + 2 * (T * k + T) * I * 2
+            rows.append({"verify_width": T, "routing": case, "distinct_experts": U, "us_per_pair": round(us, 3),
+                         "bytes_distinct": int(nbytes), "GB_s": round(nbytes / (us * 1e-6) / 1e9, 1)})
+            for b in ids:
+                b.free()
+        for b in (x, scores, egate, act, out):
+            b.free()
+    return rows
+
+
 def per_config(orn, ctx, np, with_cpu):
     """BASELINE configs 1-3 on their own seeded tensors: GPU time from HIP events over chained
     launches; CPU time of the oracle's restatement of the same operator (best of 5)."""
@@ -530,6 +568,9 @@ def main():
     ap.add_argument("--roofline-only", action="store_true",
                     help="only the expert-kernel timing loops plus three 256 MiB device copies "
                          "(the known-size reference for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--overlap", choices=("distinct", "same8"), default=None,
+                    help="only the expert pair under the named routing at T = 2 (all tokens on the same 8 experts, "
+                         "or on 16 distinct ones), then three 256 MiB device copies: one rocprofv3 --pmc run a case")
     ap.add_argument("--moe-ab", action="store_true",
                     help="only the A/B of the MoE block's launch structure (option fuse_moe_one = 0, 1, 2)")
     ap.add_argument("--ceiling", action="store_true",
@@ -568,6 +609,14 @@ def main():
             ctx.copy(a, b, 256 << 20)
         ctx.sync()
         print(json.dumps({"roofline": roof}), flush=True)
+        return
+    if args.overlap:
+        rows = expert_overlap(orn, ctx, model, np, args.layers, cases=(args.overlap,), widths=(2,), pairs=200)
+        a, b = ctx.alloc(256 << 20), ctx.alloc(256 << 20)
+        for _ in range(3):
+            ctx.copy(a, b, 256 << 20)
+        ctx.sync()
+        print(json.dumps({"overlapping_routing": rows}), flush=True)
         return
     if args.moe_ab:
         return moe_ab(orn, ctx, model, np, args.layers)
@@ -647,7 +696,8 @@ def main():
                       "gather-GEMV of one MoE block as the model launches it (gate + up + swiglu, down + combine), "
                       "verify width 2, the router's own picks",
             "us_per_launch": main_w["us_per_pair"], "launches_per_unit": 2, "bytes_per_launch": main_w["bytes_per_pair"],
-            "distinct_experts": main_w["distinct_experts_mean"], "verify_width": 2, "by_width": by_width}
+            "distinct_experts": main_w["distinct_experts_mean"], "verify_width": 2, "by_width": by_width,
+            "overlapping_routing": expert_overlap(orn, ctx, model, np, args.layers)}
     log("roofline:", roof)
 
     # Whole-step figures: the algorithmic bytes one decode step has to read (and the recurrent

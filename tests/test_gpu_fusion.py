@@ -235,3 +235,62 @@ def test_norm_inside_router_launch_equals_separate(orn, ctx):
     finally:
         orn.set_option("fuse_norm", 1)
         wn.free(); moe.free()
+
+
+@pytest.mark.parametrize("H,E,I,gk,dk", [(2048, 256, 512, Q4K, Q6K), (512, 64, 256, Q6K, Q4K)])
+def test_expert_kernels_under_overlapping_routing(orn, ctx, H, E, I, gk, dk):
+    """Verify rows of real text share experts. With routing that overlaps fully (every token on
+    the same 8 experts), with the same experts in other slots, partly, and not at all: every
+    (token, slot) row of the up launch equals that row computed alone (T = 1 with that expert),
+    the block's output equals the per-token outputs, rows of one input on the same experts
+    equal each other, and whole blocks (routing made in the launch) on duplicated input rows
+    equal the oracle."""
+    rng = np.random.default_rng(H + I)
+    moe = util.HostMoe(rng, H=H, E=E, I=I, top_k=8, gate_kind=gk, down_kind=dk, router_kind=Q6K)
+    dw = moe.dev(orn, ctx)
+    k = 8
+    try:
+        for T in (2, 3, 4):
+            base = rng.permutation(E)[:k].astype(np.uint32)
+            others = [rng.permutation(E)[:k].astype(np.uint32) for _ in range(T)]
+            part = np.stack(others)
+            for t in range(1, T):       # tokens 1.. take three of token 0's experts, in other slots
+                take = part[0, [5, 6, 7]]
+                rest = np.array([e for e in part[t] if e not in set(take.tolist())], np.uint32)[:k - 3]
+                part[t] = np.concatenate([take[::-1], rest]) if t % 2 else np.concatenate([rest, take])
+            cases = {"none": np.stack(others), "full": np.stack([base] * T),
+                     "rotated": np.stack([np.roll(base, t) for t in range(T)]), "partial": part}
+            for inds in cases.values():
+                for t in range(T):
+                    assert len(set(inds[t].tolist())) == k
+            xb = util.bf16_normal(rng, (T, H))
+            xb[1] = xb[0]              # tokens 0 and 1 are the same input row
+            scores = util.f32_to_bf16(rng.random((T, k)).astype(np.float32) + 0.1)
+            eg = util.bf16_normal(rng, (T,))
+            dx, ds, de = ctx.to_device(xb), ctx.to_device(scores), ctx.to_device(eg)
+            act, out = ctx.alloc((T * k + T) * I * 2), ctx.alloc(T * H * 2)
+            act1, out1 = ctx.alloc((k + 1) * I * 2), ctx.alloc(H * 2)
+            for name, inds in cases.items():
+                di = ctx.to_device(np.ascontiguousarray(inds, dtype=np.uint32))
+                orn.moe_experts(ctx, dw, dx, T, di, ds, de, act, out, 3)
+                a, o = act.download(np.uint16, (T * k + T, I)), out.download(np.uint16, (T, H))
+                for t in range(T):     # the same token alone
+                    d1 = [ctx.to_device(np.ascontiguousarray(v)) for v in (xb[t:t + 1], inds[t], scores[t], eg[t:t + 1])]
+                    orn.moe_experts(ctx, dw, d1[0], 1, d1[1], d1[2], d1[3], act1, out1, 3)
+                    a1 = act1.download(np.uint16, (k + 1, I))
+                    assert np.array_equal(a[t * k:(t + 1) * k], a1[:k]) and np.array_equal(a[T * k + t], a1[k]), (T, name, t)
+                    assert np.array_equal(o[t], out1.download(np.uint16, (H,))), (T, name, t)
+                    for b in d1: b.free()
+                if name == "full":
+                    assert np.array_equal(a[0:k], a[k:2 * k]) and np.array_equal(a[T * k], a[T * k + 1])
+                di.free()
+            for b in (dx, ds, de, act, out, act1, out1): b.free()
+            # whole blocks on duplicated rows (identical routing by construction) against the oracle
+            xd = util.bf16_normal(rng, (T, H))
+            xd[T - 1] = xd[0]
+            want_out, want_inds, _, _ = util.orc_moe_block(moe, xd, T)
+            got_out, got_inds, _ = _block(orn, ctx, moe, dw, xd, T)
+            assert np.array_equal(got_inds, want_inds) and np.array_equal(got_inds[0], got_inds[T - 1])
+            assert np.array_equal(got_out, want_out)
+    finally:
+        moe.free()
