@@ -10,6 +10,15 @@
 
 #include "dmath.h"
 
+// swiglu of one gate / up pair as the separate operators leave it: both mat-vec outputs rounded
+// to bf16, silu and the product in bf16 steps
+// (/root/reference/kernels/ornith_elementwise.metal:97-105)
+__device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
+  const float gb = dm_rb(g), ub = dm_rb(u);
+  const float s = dm_rb(gb * dm_sigmoid_bf16(gb));
+  return dm_f2bf(s * ub);
+}
+
 template <int S>
 __device__ __forceinline__ uint32_t dm_xor_lane_u32(uint32_t v) {
   return __builtin_bit_cast(uint32_t, dm_xor_lane<S>(__builtin_bit_cast(float, v)));

@@ -52,12 +52,6 @@ struct UpArgs {
   bf16_t* scores_out;    // [T*k]
 };
 
-__device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
-  const float gb = dm_rb(g), ub = dm_rb(u);
-  const float s = dm_rb(gb * dm_sigmoid_bf16(gb));
-  return dm_f2bf(s * ub);
-}
-
 // grid (ceil(I / (RPW * 4 * ITERS)), T*k + T), 256 threads
 #ifdef ORN_TIMING
 // debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch

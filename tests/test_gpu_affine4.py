@@ -84,11 +84,16 @@ def test_moe_block_with_4bit_affine_experts_bit_exact(orn, ctx, T):
     dx = ctx.to_device(xb)
     out, inds, scores = ctx.alloc(T * 1024 * 2), ctx.alloc(T * 8 * 4), ctx.alloc(T * 8 * 2)
     try:
-        ctx.moe_block(w, dx, T, out, inds, scores)
-        assert np.array_equal(inds.download(np.uint32, (T, 8)), winds)
-        assert np.array_equal(scores.download(np.uint16, (T, 8)), wscores)
-        assert np.array_equal(out.download(np.uint16, (T, 1024)), want)
+        # the two fused expert launches (the default), then one launch per operator
+        for fuse in (1, 0):
+            orn.set_option("fuse_moe", fuse)
+            for b in (out, inds, scores): b.zero()
+            ctx.moe_block(w, dx, T, out, inds, scores)
+            assert np.array_equal(inds.download(np.uint32, (T, 8)), winds), fuse
+            assert np.array_equal(scores.download(np.uint16, (T, 8)), wscores), fuse
+            assert np.array_equal(out.download(np.uint16, (T, 1024)), want), fuse
     finally:
+        orn.set_option("fuse_moe", 1)
         for b in (dx, out, inds, scores): b.free()
         moe.free()
 
