@@ -4,8 +4,8 @@
 
 hipcc cross-compiles without a GPU. Every translation unit is compiled with
 -ffp-contract=off (the only fused multiply-adds are the explicit ones, so results
-do not depend on what the optimiser chooses to contract) and with packed-fp32
-instruction selection disabled.
+do not depend on what the optimiser chooses to contract), with packed-fp32
+instruction selection disabled, and with kernel-argument preloading on.
 """
 import concurrent.futures
 import os
@@ -23,6 +23,9 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-fno-fast-math", "-fvisibility=hidden", "-Wall", "-Wno-unused-function",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the first 14 dwords of a kernel's flat (non-struct) arguments arrive in scalar registers
+    # with the wavefront instead of through a scalar load (gfx950 kernel-argument preloading)
+    "-mllvm", "-amdgpu-kernarg-preload-count=14",
     "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument", "-Wno-pass-failed",
 ]
 

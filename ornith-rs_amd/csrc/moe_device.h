@@ -91,18 +91,28 @@ __device__ __forceinline__ void router_topk_wave(const bf16_t* gates_row, int k,
     // a NaN probability (NaN gates) never wins
     key[i] = (pb & 0x7fffu) > 0x7f80u ? 0u : ((((uint32_t)(pb & 0x7fffu)) << 16) | (uint32_t)(lane * PER + i)) + 1u;
   }
-  for (int r = 0; r < k; ++r) {
-    uint32_t best = 0;
+  // the lane's keys in descending order (odd-even transposition), so that a round's candidate is
+  // key[0] and the lane that wins shifts its list up by one
 #pragma unroll
-    for (int i = 0; i < PER; ++i) best = key[i] > best ? key[i] : best;
-    const uint32_t win = dm_wave_max_u32(best);
+  for (int pass = 0; pass < PER; ++pass)
 #pragma unroll
-    for (int i = 0; i < PER; ++i)
-      if (key[i] == win) key[i] = 0;
-    if (lane == 0) {
-      const uint32_t w = win - 1u;  // win == 0 only if every entry is NaN / taken: id wraps, clamped by users
-      inds_row[k - 1 - r] = win ? (w & 0xffffu) : 0xffffffffu;
-      scores_row[k - 1 - r] = win ? (bf16_t)(w >> 16) : (bf16_t)0;
+    for (int i = pass & 1; i + 1 < PER; i += 2) {
+      const uint32_t hi = max(key[i], key[i + 1]), lo = min(key[i], key[i + 1]);
+      key[i] = hi;
+      key[i + 1] = lo;
     }
+  uint32_t mine = 0;  // lane r keeps round r's winner; one store after the rounds
+  for (int r = 0; r < k; ++r) {
+    const uint32_t win = dm_wave_max_u32(key[0]);
+    const bool won = key[0] == win;  // keys are distinct (the index is in them) unless 0
+#pragma unroll
+    for (int i = 0; i + 1 < PER; ++i) key[i] = won ? key[i + 1] : key[i];
+    key[PER - 1] = won ? 0u : key[PER - 1];
+    mine = lane == r ? win : mine;
+  }
+  if (lane < k) {
+    const uint32_t w = mine - 1u;  // mine == 0 only if every entry is NaN / taken: id wraps, clamped by users
+    inds_row[k - 1 - lane] = mine ? (w & 0xffffu) : 0xffffffffu;
+    scores_row[k - 1 - lane] = mine ? (bf16_t)(w >> 16) : (bf16_t)0;
   }
 }

@@ -45,7 +45,7 @@ struct UpArgs {
   bf16_t* act;           // [T*k + T, I]
   int T, k, E, I, K;
   // gates != null: the routing is not read but made -- every workgroup of a routed row runs
-  // softmax + top-k over its token's gates (one wavefront, ~400 instructions) and the first
+  // softmax + top-k over its token's gates (one wavefront, ~300 instructions) and the first
   // workgroup of each token stores inds / scores for the down kernel
   const bf16_t* gates;   // [T, E]
   uint32_t* inds_out;    // [T*k]
@@ -57,13 +57,20 @@ struct UpArgs {
 // debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch
 __device__ long long g_up_marks[2048][8];
 #define UP_MARK(i) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if (threadIdx.x == 0 && bl__ < 2048) g_up_marks[bl__][i] = wall_clock64(); } while (0)
+__device__ long long g_down_marks[1024][8];
+#define DOWN_MARK(i) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if ((threadIdx.x & 63) == 0 && (threadIdx.x >> 6) == (i >> 3) && bl__ < 1024) g_down_marks[bl__][i & 7] = wall_clock64(); } while (0)
 #else
 #define UP_MARK(i)
+#define DOWN_MARK(i)
 #endif
 
 // ROUTE: the routing is made in the head of the launch (a.gates) instead of read (a.inds)
+// The leading flat arguments repeat what decides a workgroup's expert (the library is built with
+// kernel-argument preloading: they are in scalar registers when the wavefront starts, so the
+// gates / ids are asked for while the argument block is still being fetched).
 template <int KIND, int LPR, int ITERS, bool ROUTE>
-__global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
+__global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* h_gates, const uint32_t* h_inds, int h_T, int h_k,
+                                                     int h_E, UpArgs a) {
   UP_MARK(0);
   using KL = KqLane<KIND, 1>;
   constexpr int RPW = 64 / LPR;
@@ -71,10 +78,37 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
   const int slot = lane / LPR, c = lane % LPR;
   const int nb = a.K >> 8;
   const int r = blockIdx.y;
-  const int routed = a.T * a.k;
-  int token;
-  int64_t row0;
-  KqPtr wg, wu;
+  const int routed = h_T * h_k;
+  const bool is_routed = r < routed;  // the same for the whole workgroup
+  const int token = is_routed ? r / h_k : r - routed;
+  // the expert first: its chain (gates -> softmax + top-k, or the id) starts from the preloaded
+  // arguments alone
+  uint32_t e = 0;
+  if constexpr (ROUTE) {
+    __shared__ uint32_t s_inds[16];
+    __shared__ bf16_t s_scores[16];
+    if (is_routed) {
+      if (wave == 0) {
+        const bf16_t* g = h_gates + (size_t)token * h_E;
+        switch (h_E / 64) {
+          case 1: router_topk_wave<1>(g, h_k, s_inds, s_scores, nullptr, lane); break;
+          case 2: router_topk_wave<2>(g, h_k, s_inds, s_scores, nullptr, lane); break;
+          case 4: router_topk_wave<4>(g, h_k, s_inds, s_scores, nullptr, lane); break;
+          case 8: router_topk_wave<8>(g, h_k, s_inds, s_scores, nullptr, lane); break;
+          default: router_topk_wave<16>(g, h_k, s_inds, s_scores, nullptr, lane); break;
+        }
+      }
+      __syncthreads();
+      UP_MARK(5);
+      e = s_inds[r - token * h_k];
+      if (blockIdx.x == 0 && r == token * h_k && threadIdx.x < h_k) {
+        a.inds_out[r + threadIdx.x] = s_inds[threadIdx.x];
+        a.scores_out[r + threadIdx.x] = s_scores[threadIdx.x];
+      }
+    }
+  } else {
+    if (is_routed) e = h_inds[r];
+  }
   // both sets of weight pointers as values in scalar registers before the choice is made:
   // chosen by address instead, the pointers would be loaded in a second trip after the first
   KqPtr pin[4] = {a.gate, a.up, a.sgate, a.sup};
@@ -86,40 +120,8 @@ __global__ __launch_bounds__(256) void moe_up_kernel(UpArgs a) {
     pin[i].scales = dm_global_ptr<const uint8_t>(sc);
     pin[i].dm = dm_global_ptr<const uint16_t>(d);
   }
-  if (r < routed) {
-    token = r / a.k;
-    uint32_t e;
-    if constexpr (ROUTE) {
-      __shared__ uint32_t s_inds[16];
-      __shared__ bf16_t s_scores[16];
-      if (wave == 0) {
-        const bf16_t* g = a.gates + (size_t)token * a.E;
-        switch (a.E / 64) {
-          case 1: router_topk_wave<1>(g, a.k, s_inds, s_scores, nullptr, lane); break;
-          case 2: router_topk_wave<2>(g, a.k, s_inds, s_scores, nullptr, lane); break;
-          case 4: router_topk_wave<4>(g, a.k, s_inds, s_scores, nullptr, lane); break;
-          case 8: router_topk_wave<8>(g, a.k, s_inds, s_scores, nullptr, lane); break;
-          default: router_topk_wave<16>(g, a.k, s_inds, s_scores, nullptr, lane); break;
-        }
-      }
-      __syncthreads();
-      e = s_inds[r - token * a.k];
-      if (blockIdx.x == 0 && r == token * a.k && threadIdx.x < a.k) {
-        a.inds_out[r + threadIdx.x] = s_inds[threadIdx.x];
-        a.scores_out[r + threadIdx.x] = s_scores[threadIdx.x];
-      }
-    } else {
-      e = a.inds[r];
-    }
-    row0 = (int64_t)min(e, (uint32_t)(a.E - 1)) * a.I;
-    wg = pin[0];
-    wu = pin[1];
-  } else {
-    token = r - routed;
-    row0 = 0;
-    wg = pin[2];
-    wu = pin[3];
-  }
+  const int64_t row0 = is_routed ? (int64_t)min(e, (uint32_t)(h_E - 1)) * a.I : 0;
+  const KqPtr wg = is_routed ? pin[0] : pin[2], wu = is_routed ? pin[1] : pin[3];
   typename KL::Lane L;
   L.set_chunk(c);
   const int base = (blockIdx.x * 4 + wave) * (RPW * ITERS);
@@ -184,15 +186,21 @@ struct DownArgs {
 constexpr int kMaxK = 8;
 
 // grid (ceil(H / (RPW * ITERS)), T), 64 * (k + 1) threads
+// The leading flat arguments repeat what a routed wavefront needs for its first weight request
+// (the library is built with kernel-argument preloading: they are in scalar registers when the
+// wavefront starts, while the argument block is still being fetched).
 template <int KIND, int LPR, int ITERS>
-__global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) {
+__global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(const uint8_t* h_qs, const uint8_t* h_scales,
+                                                                    const uint16_t* h_dm, const uint32_t* h_inds,
+                                                                    int h_k, int h_E, int h_H, int h_I, DownArgs a) {
   using KL = KqLane<KIND, 1>;
   constexpr int RPW = 64 / LPR, COLS = RPW * ITERS;
   const int lane = threadIdx.x & 63, j = threadIdx.x >> 6;  // j: expert slot, k = shared
   const int slot = lane / LPR, c = lane % LPR;
-  const int nb = a.I >> 8;
-  const int t = blockIdx.y, k = a.k;
+  const int nb = h_I >> 8;
+  const int t = blockIdx.y, k = h_k;
   const int c0 = blockIdx.x * COLS;
+  DOWN_MARK(0);
 
   __shared__ float yl[kMaxK + 1][COLS];
   __shared__ float wj[kMaxK];
@@ -200,19 +208,21 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) 
 
   const bool shared = j == k;
   const int arow = shared ? a.T * k + t : t * k + j;
-  const KqPtr w = shared ? a.sdown : a.down;
-  const int64_t row0 = shared ? 0 : (int64_t)min(a.inds[t * k + j], (uint32_t)(a.E - 1)) * a.H;
+  const KqPtr w = shared ? a.sdown : KqPtr{h_qs, h_scales, h_dm};
+  const int64_t row0 = shared ? 0 : (int64_t)min(h_inds[t * k + j], (uint32_t)(h_E - 1)) * h_H;
   typename KL::Lane L;
   L.set_chunk(c);
   typename KL::Row rr[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     const int o = c0 + it * RPW + slot;
-    rr[it] = KL::load(w.qs, w.scales, w.dm, row0 + (o < a.H ? o : a.H - 1), nb, L);
+    rr[it] = KL::load(w.qs, w.scales, w.dm, row0 + (o < h_H ? o : h_H - 1), nb, L);
   }
   __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  DOWN_MARK(1);
   const void* xrow[1] = {a.act + (size_t)arow * a.I};
   L.template load_x<false>(xrow, c);
+  DOWN_MARK(2);
 
   if (j == 0) {
     // the router weights of this token: denom = ((0+s0)+s1)..., w_j = bf16(s_j / denom)
@@ -230,7 +240,9 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) 
     const float v = dm_wave_sum<LPR>(acc[0]);
     if (c == 0) yl[j][it * RPW + slot] = dm_rb(v);  // expert outputs are bf16 in the unfused path
   }
+  DOWN_MARK(3);
   __syncthreads();
+  DOWN_MARK(4);
   const int col = threadIdx.x;
   if (col < COLS && c0 + col < a.H) {
     float acc = 0.f;
@@ -241,6 +253,7 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(DownArgs a) 
     const float gated = dm_rb(gsig * yl[k][col]);
     a.out[(size_t)t * a.H + c0 + col] = dm_f2bf(acc + gated);
   }
+  DOWN_MARK(5);
 }
 
 // ---- router: the gates mat-vec and, in one extra workgroup, the shared expert's scalar
@@ -297,13 +310,18 @@ __device__ __forceinline__ float egate_row_dot(const RouterArgs& a, const bf16_t
 }
 
 // grid ceil(E / (RPW * 4)) + 1, 256 threads, M <= 4 tokens
+// The leading flat arguments repeat what the first loads need (the norm's inputs and the router's
+// rows): preloaded into scalar registers, they let those loads leave while the argument block is
+// still being fetched.
 template <int KIND, int LPR, int M>
-__global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
+__global__ __launch_bounds__(256) void moe_router_kernel(const bf16_t* h_res, const bf16_t* h_y, const bf16_t* h_w,
+                                                         const uint8_t* h_qs, const uint8_t* h_scales,
+                                                         const uint16_t* h_dm, int h_E, int h_K, RouterArgs a) {
   using KL = KqLane<KIND, M>;
   constexpr int RPW = 64 / LPR;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   __shared__ PreNormLds<M> pn;
-  const bool pre = a.pre.res != nullptr;
+  const bool pre = h_res != nullptr;
   if (blockIdx.x == gridDim.x - 1) {
     if (pre) prenorm_rows<M>(a.pre, false, pn);
     if (wave < M) {
@@ -313,16 +331,22 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
     return;
   }
   const int slot = lane / LPR, c = lane % LPR;
-  const int nb = a.K >> 8;
+  const int nb = h_K >> 8;
   typename KL::Lane L;
   L.set_chunk(c);
   const int o = (blockIdx.x * 4 + wave) * RPW + slot;
   // the norm's inputs first (cached, back early), the weight row right behind them: loads
   // return in issue order
   PreNormRegs<M> pg;
-  if (pre) prenorm_issue<M>(a.pre, pg);
+  if (pre) {
+    PreNorm ph{};
+    ph.res = h_res;
+    ph.y = h_y;
+    ph.w = h_w;
+    prenorm_issue<M>(ph, pg);
+  }
   __builtin_amdgcn_sched_barrier(0);
-  const typename KL::Row row = KL::load(a.w.qs, a.w.scales, a.w.dm, o < a.E ? o : a.E - 1, nb, L);
+  const typename KL::Row row = KL::load(h_qs, h_scales, h_dm, o < h_E ? o : h_E - 1, nb, L);
   __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of everything that follows
   if (pre) prenorm_finish<M>(a.pre, pg, blockIdx.x == 0, pn);
   const void* xrow[M];
@@ -340,15 +364,16 @@ __global__ __launch_bounds__(256) void moe_router_kernel(RouterArgs a) {
   }
 }
 
+#define ORN_ROUTER_HEAD(a) (a).pre.res, (a).pre.y, (a).pre.w, (a).w.qs, (a).w.scales, (a).w.dm, (a).E, (a).K
 template <int KIND, int LPR>
 void launch_router_fused(ornith_ctx* ctx, const RouterArgs& a, int M) {
   constexpr int RPW = 64 / LPR;
   dim3 grid((a.E + RPW * 4 - 1) / (RPW * 4) + 1);
   switch (M) {
-    case 1: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 1>), grid, dim3(256), 0, ctx->stream, a); break;
-    case 2: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 2>), grid, dim3(256), 0, ctx->stream, a); break;
-    case 3: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 3>), grid, dim3(256), 0, ctx->stream, a); break;
-    default: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 4>), grid, dim3(256), 0, ctx->stream, a); break;
+    case 1: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 1>), grid, dim3(256), 0, ctx->stream, ORN_ROUTER_HEAD(a), a); break;
+    case 2: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 2>), grid, dim3(256), 0, ctx->stream, ORN_ROUTER_HEAD(a), a); break;
+    case 3: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 3>), grid, dim3(256), 0, ctx->stream, ORN_ROUTER_HEAD(a), a); break;
+    default: hipLaunchKernelGGL((moe_router_kernel<KIND, LPR, 4>), grid, dim3(256), 0, ctx->stream, ORN_ROUTER_HEAD(a), a); break;
   }
 }
 
@@ -621,6 +646,7 @@ __device__ __forceinline__ void one_down(const OneArgs& o, int dd, char* lds) {
     const float gated = dm_rb(*gsig * yl[k][col]);
     a.out[(size_t)t * a.H + c0 + col] = dm_f2bf(acc + gated);
   }
+  DOWN_MARK(5);
 }
 
 template <int M>
@@ -671,15 +697,19 @@ void launch_up(ornith_ctx* ctx, const UpArgs& a, int rows_y) {
   if (ornith_option_moe_up_iters() == 4) {
     dim3 grid((a.I + RPW * 4 * 4 - 1) / (RPW * 4 * 4), rows_y);
     if (a.gates)
-      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4, true>), grid, dim3(256), 0, ctx->stream, a);
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4, true>), grid, dim3(256), 0, ctx->stream, a.gates, a.inds, a.T,
+                         a.k, a.E, a);
     else
-      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4, false>), grid, dim3(256), 0, ctx->stream, a);
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 4, false>), grid, dim3(256), 0, ctx->stream, a.gates, a.inds, a.T,
+                         a.k, a.E, a);
   } else {
     dim3 grid((a.I + RPW * 4 * 2 - 1) / (RPW * 4 * 2), rows_y);
     if (a.gates)
-      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2, true>), grid, dim3(256), 0, ctx->stream, a);
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2, true>), grid, dim3(256), 0, ctx->stream, a.gates, a.inds, a.T,
+                         a.k, a.E, a);
     else
-      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2, false>), grid, dim3(256), 0, ctx->stream, a);
+      hipLaunchKernelGGL((moe_up_kernel<KIND, LPR, 2, false>), grid, dim3(256), 0, ctx->stream, a.gates, a.inds, a.T,
+                         a.k, a.E, a);
   }
 }
 
@@ -696,13 +726,16 @@ void launch_down(ornith_ctx* ctx, const DownArgs& a) {
   const int iters = forced ? forced : groups1 >= 3 * cu ? 4 : groups1 >= 2 * cu ? 2 : 1;
   if (iters >= 4) {
     dim3 grid((a.H + RPW * 4 - 1) / (RPW * 4), a.T);
-    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 4>), grid, block, 0, ctx->stream, a);
+    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 4>), grid, block, 0, ctx->stream, a.down.qs, a.down.scales,
+                       a.down.dm, a.inds, a.k, a.E, a.H, a.I, a);
   } else if (iters == 2) {
     dim3 grid((a.H + RPW * 2 - 1) / (RPW * 2), a.T);
-    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 2>), grid, block, 0, ctx->stream, a);
+    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 2>), grid, block, 0, ctx->stream, a.down.qs, a.down.scales,
+                       a.down.dm, a.inds, a.k, a.E, a.H, a.I, a);
   } else {
     dim3 grid((a.H + RPW - 1) / RPW, a.T);
-    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 1>), grid, block, 0, ctx->stream, a);
+    hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 1>), grid, block, 0, ctx->stream, a.down.qs, a.down.scales,
+                       a.down.dm, a.inds, a.k, a.E, a.H, a.I, a);
   }
 }
 
@@ -711,6 +744,9 @@ void launch_down(ornith_ctx* ctx, const DownArgs& a) {
 #ifdef ORN_TIMING
 extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_up(long long* out) {
   return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_up_marks), sizeof(long long) * 2048 * 8);
+}
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_down(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_down_marks), sizeof(long long) * 1024 * 8);
 }
 #endif
 
