@@ -108,8 +108,15 @@ ORC_API void orc_moe_combine(const bf16_t* scores, const bf16_t* y, const bf16_t
 /* ---- 8-bit affine, group 64: y = sum_g (s_g * sum x q + b_g * sum x) ---------
  * w u8[O,K], scales/biases bf16[O,K/64]. Lane l owns 8-element chunks
  * j = l + 64c; per chunk p = fma(sum_x, bias, scale * accum); tree64. */
+extern int orc_row_order; /* orc_ref_order.c: > 0 selects the reference's 32-lane schedule */
+float orc_affine4_row_dot_ref32(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K, const float* x,
+                                int fma, int tree);
+float orc_affine8_row_dot_ref32(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K, const float* x,
+                                int fma, int tree);
+
 float orc_affine8_row_dot(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K,
                           const float* x) {
+  if (orc_row_order > 0) return orc_affine8_row_dot_ref32(w, scales, biases, K, x, (orc_row_order - 1) / 3, (orc_row_order - 1) % 3);
   float lanes[64];
   for (int l = 0; l < 64; ++l) lanes[l] = 0.f;
   for (int j = 0; j < K / 8; ++j) {
@@ -147,6 +154,7 @@ ORC_API void orc_affine8_qmv(const uint8_t* w, const bf16_t* scales, const bf16_
  * scale * accum); tree64. */
 float orc_affine4_row_dot(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K,
                           const float* x) {
+  if (orc_row_order > 0) return orc_affine4_row_dot_ref32(w, scales, biases, K, x, (orc_row_order - 1) / 3, (orc_row_order - 1) % 3);
   float lanes[64];
   for (int l = 0; l < 64; ++l) lanes[l] = 0.f;
   for (int j = 0; j < K / 16; ++j) {

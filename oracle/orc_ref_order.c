@@ -19,6 +19,16 @@
  *        2: lane order;   fma 0: every product rounded, 1: accumulations and sums of
  *        products contracted where the source has the shape a * b + c.
  * None of the six variants is "the" reference; the spread over them is the measurement.
+ *
+ * The mlx affine formats (4-bit group 32, 8-bit group 64) in the reference's schedule as well:
+ *   vendored kernels/mlx/mlx/backend/metal/kernels/quantized.h:757-821 (qmv_fast_impl), :62-70 and
+ *   :98-101 (load_vector), :235-244 and :282-288 (qdot): lane l of 32 takes values_per_thread
+ *   = 16 (4-bit) or 8 (8-bit) consecutive values of every block of 512 / 256; 4-bit: the
+ *   activations are summed four at a time (sum += x0 + x1 + x2 + x3) and pre-divided by 1, 16,
+ *   256, 4096 against the unshifted nibble masks (exact: the products are those of x and the
+ *   nibble), the four products of a 16-bit word are added up and then added to the accumulator;
+ *   8-bit: accum += x * w one value at a time; a lane's block result scale * accum + sum * bias is
+ *   added to its running result; then simd_sum. The same two parameters apply.
  */
 #include "orc_common.h"
 
@@ -139,8 +149,59 @@ float orc_q6k_row_dot_ref32(const uint8_t* w, const uint8_t* scales, const f16_t
   return fold32(lanes, tree);
 }
 
+float orc_affine4_row_dot_ref32(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K, const float* x,
+                                int fma, int tree) {
+  float lanes[32];
+  for (int lane = 0; lane < 32; ++lane) {
+    float result = 0.f;
+    for (int k = 0; k + 16 * lane < K; k += 512) {
+      const int e0 = k + 16 * lane; /* K % 16 == 0: a lane's 16 values are inside the row or not at all */
+      const float* xv = x + e0;
+      float xt[16], sum = 0.f;
+      for (int i = 0; i < 16; i += 4) {
+        sum = sum + (((xv[i] + xv[i + 1]) + xv[i + 2]) + xv[i + 3]);
+        xt[i] = xv[i];
+        xt[i + 1] = xv[i + 1] / 16.0f;
+        xt[i + 2] = xv[i + 2] / 256.0f;
+        xt[i + 3] = xv[i + 3] / 4096.0f;
+      }
+      const uint16_t* ws = (const uint16_t*)(w + e0 / 2);
+      float accum = 0.f;
+      for (int i = 0; i < 4; ++i) {
+        float t = xt[4 * i] * (float)(ws[i] & 0x000f);
+        t = mac(t, xt[4 * i + 1], (float)(ws[i] & 0x00f0), fma);
+        t = mac(t, xt[4 * i + 2], (float)(ws[i] & 0x0f00), fma);
+        t = mac(t, xt[4 * i + 3], (float)(ws[i] & 0xf000), fma);
+        accum = accum + t;
+      }
+      const float sc = orc_bf16_to_f32(scales[e0 / 32]), bi = orc_bf16_to_f32(biases[e0 / 32]);
+      result = result + (fma ? fmaf(sc, accum, sum * bi) : sc * accum + sum * bi);
+    }
+    lanes[lane] = result;
+  }
+  return fold32(lanes, tree);
+}
+
+float orc_affine8_row_dot_ref32(const uint8_t* w, const bf16_t* scales, const bf16_t* biases, int K, const float* x,
+                                int fma, int tree) {
+  float lanes[32];
+  for (int lane = 0; lane < 32; ++lane) {
+    float result = 0.f;
+    for (int k = 0; k + 8 * lane < K; k += 256) {
+      const int e0 = k + 8 * lane;
+      float sum = 0.f, accum = 0.f;
+      for (int i = 0; i < 8; ++i) sum = sum + x[e0 + i];
+      for (int i = 0; i < 8; ++i) accum = mac(accum, x[e0 + i], (float)w[e0 + i], fma);
+      const float sc = orc_bf16_to_f32(scales[e0 / 64]), bi = orc_bf16_to_f32(biases[e0 / 64]);
+      result = result + (fma ? fmaf(sc, accum, sum * bi) : sc * accum + sum * bi);
+    }
+    lanes[lane] = result;
+  }
+  return fold32(lanes, tree);
+}
+
 /* 0: this build's 64-lane order (the default, what the library implements);
- * 1 + tree + 3 * fma: the reference's 32-lane schedule in one of its six readings.
- * Process-global; tests that change it put it back. */
+ * 1 + tree + 3 * fma: the reference's 32-lane schedule in one of its six readings (k-quant and
+ * affine mat-vecs alike). Process-global; tests that change it put it back. */
 int orc_row_order = 0;
 ORC_API void orc_set_row_order(int mode) { orc_row_order = mode; }

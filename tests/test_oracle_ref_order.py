@@ -1,5 +1,6 @@
-"""The k-quant mat-vec in the reference's 32-lane schedule (oracle/orc_ref_order.c), pinned
-like the canonical one (float64 product, one-hot columns), and the measurement it exists for:
+"""The k-quant and mlx-affine mat-vecs in the reference's 32-lane schedule
+(oracle/orc_ref_order.c), pinned like the canonical ones (float64 product, one-hot columns), and
+the measurement they exist for:
 how often router expert ids and greedy tokens change when only the fp32 summation order
 changes. Six readings of the reference's order (three simd_sum trees x contraction on / off)
 are compared with this build's 64-lane order. CPU only.
@@ -108,3 +109,110 @@ def test_how_often_integer_results_depend_on_the_order(capsys):
                   f"leaves the canonical one after {toks[mode][0]} tokens")
     # rare, not impossible: at most 2 % of the router ids
     assert all(v[0] <= 0.02 * T * 8 for v in router.values()), router
+
+
+def _affine_dequant(lin):
+    s = util.bf16_to_f32(lin.scales).astype(np.float64)
+    b = util.bf16_to_f32(lin.biases).astype(np.float64)
+    if lin.mode == "affine8":
+        return lin.w.astype(np.float64) * np.repeat(s, 64, 1) + np.repeat(b, 64, 1)
+    words = lin.w.view(np.uint32)
+    i = np.arange(lin.K)
+    q = (words[:, i // 8] >> (4 * (i % 8)).astype(np.uint32)) & 15      # mlx: eight codes a word, lowest first
+    return q.astype(np.float64) * np.repeat(s, 32, 1) + np.repeat(b, 32, 1)
+
+
+def _affine_qmv(lin, xb):
+    y = np.empty((xb.shape[0], lin.O), np.uint16)
+    if lin.mode == "affine8":
+        oracle().orc_affine8_qmv(p(lin.w), p(lin.scales), p(lin.biases), lin.O, lin.K, p(xb), xb.shape[0], p(y))
+    else:
+        oracle().orc_affine4_gather_qmv(p(lin.w), p(lin.scales), p(lin.biases), 1, lin.O, lin.K, p(xb), None, None,
+                                        xb.shape[0], p(y))
+    return y
+
+
+@pytest.mark.parametrize("fmt,K", [("affine4", 2048), ("affine4", 1568), ("affine8", 2048), ("affine8", 448)])
+def test_affine_reference_schedule_matches_float64_and_dequant_columns(fmt, K):
+    """quantized.h's qmv lane schedule (32 lanes x 16 or 8 values a block, the pre-scaled
+    activations against unshifted masks, four products a word) restated: same product as float64
+    and as the canonical order to bf16 rounding, single weights picked out exactly, and a different
+    order in the last bits. K = 1568 / 448 end inside a block of 512 / 256 (the lanes past the end
+    take nothing)."""
+    rng = np.random.default_rng(K)
+    O = 12
+    lin = util.HostLinear.affine4(rng, O, K) if fmt == "affine4" else util.HostLinear.affine8(rng, O, K)
+    W = _affine_dequant(lin)
+    xb = util.bf16_normal(rng, (3, K))
+    want = util.bf16_to_f32(xb).astype(np.float64) @ W.T
+    canon = _affine_qmv(lin, xb)
+    cols = sorted(c for c in set(list(rng.integers(0, K, 24)) + [0, 1, 3, 4, 7, 8, 15, 16, 31, 32, 255, 256, 511, 512, K - 17, K - 1]) if c < K)
+    seen = set()
+    for mode in MODES:
+        oracle().orc_set_row_order(mode)
+        got = _affine_qmv(lin, xb)
+        seen.add(got.tobytes())
+        g = util.bf16_to_f32(got).astype(np.float64)
+        assert np.all(np.abs(g - want) <= 2.0 ** -8 * np.abs(want) + 1e-5 * np.abs(want).max()), mode
+        for col in cols:
+            e = np.zeros((1, K), np.float32); e[0, col] = 1.0
+            y = util.bf16_to_f32(_affine_qmv(lin, util.f32_to_bf16(e)))[0].astype(np.float64)
+            assert np.all(np.abs(y - W[:, col]) <= 2.0 ** -8 * np.abs(W[:, col]) + 1e-12), (mode, col)
+    oracle().orc_set_row_order(0)
+    # bf16 outputs hide most last-bit differences; over 36 outputs at least the orders are not all
+    # byte-equal to the canonical one AND every one of them is within one bf16 step of it
+    c = util.bf16_to_f32(canon).astype(np.float64)
+    for b in seen:
+        g = util.bf16_to_f32(np.frombuffer(b, np.uint16).reshape(canon.shape)).astype(np.float64)
+        assert np.all(np.abs(g - c) <= 2.0 ** -7 * np.abs(c) + 1e-6)
+
+
+def test_how_often_the_affine_artifact_depends_on_the_order(capsys):
+    """The published artifact's layout (4-bit affine group-32 projections, experts and lm_head,
+    8-bit router and shared gate) under the reference's schedule against this build's: router
+    ids of one MoE block and teacher-forced greedy tokens of the tiny model."""
+    rng = np.random.default_rng(12)
+    H, E, I, k, T = 512, 64, 256, 8, 64
+    moe = util.HostMoe(rng, H=H, E=E, I=I, top_k=k, gate_kind=util.AFFINE4)
+    xb = util.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32))
+    oracle().orc_set_row_order(0)
+    _, inds0, _, _ = util.orc_moe_block(moe, xb, T)
+    router = {}
+    for mode in MODES:
+        oracle().orc_set_row_order(mode)
+        _, inds, _, _ = util.orc_moe_block(moe, xb, T)
+        router[mode] = (int((inds != inds0).sum()), int(sum(set(a) != set(b) for a, b in zip(inds, inds0))))
+    oracle().orc_set_row_order(0)
+    s = synth.SynthModel(synth.TINY, seed=5, with_mtp=False, affine="affine4", trunk="affine4")
+    prompt = np.random.default_rng(6).integers(0, 2048, 12).astype(np.uint32)
+    n = 120
+    r = synth.OracleRun(s, 256)
+    base = r.generate(prompt, n, prefill_step=4)
+    r.close()
+    seq = np.concatenate([prompt, np.array(base[:-1], np.uint32)])
+
+    def forced_tokens():
+        r = synth.OracleRun(s, 256)
+        out = []
+        for i in range(0, len(seq), 4):
+            h = r.forward(seq[i:i + 4])
+            lg = r.logits(h)
+            t = np.empty(len(h), np.uint32)
+            oracle().orc_greedy_rows(p(lg), len(h), lg.shape[1], p(t), None)
+            out += list(t)
+        r.close()
+        return out[len(prompt) - 1:]
+
+    assert forced_tokens() == base
+    toks = {}
+    for mode in MODES:
+        oracle().orc_set_row_order(mode)
+        toks[mode] = sum(a != b for a, b in zip(forced_tokens(), base))
+    oracle().orc_set_row_order(0)
+    with capsys.disabled():
+        print("\n4-bit affine artifact layout, summation-order sensitivity (mode = 1 + tree + 3 * fma):")
+        for mode in MODES:
+            print(f"  mode {mode}: router ids differing {router[mode][0]} of {T * k} (tokens with another expert set: "
+                  f"{router[mode][1]} of {T}); greedy tokens differing at the same prefix {toks[mode]} of {n}")
+    assert all(v[0] <= 0.03 * T * k for v in router.values()), router
+    assert all(v <= 0.1 * n for v in toks.values()), toks
