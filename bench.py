@@ -478,7 +478,106 @@ def ceiling(orn, ctx, np):
     res["word_between_workgroups"] = rows
     for b in (flag, out4, sink):
         b.free()
+
+    # -- what one vector instruction costs (2048 workgroups x 256 threads x 8 chains x 4096)
+    lib.ornith_probe_valu_name.restype = C.c_char_p
+    dx = ctx.to_device(np.array([1e-3, 2e-3, 3e-3, 4e-3], np.float32))
+    dp = ctx.to_device(np.full(4, 0x47000007, np.uint32))   # halves: f16 7.0 and the f16 subnormal 7 * 2^-24
+    wgs, iters = 2048, 4096
+    dout = ctx.alloc(wgs * 256 * 4)
+    rows = []
+    for op in range(lib.ornith_probe_valu_count()):
+        best = 1e30
+        for rep in range(3):
+            ctx.sync()
+            ctx.timer_begin()
+            probe(lib.ornith_probe_valu(ctx.h, op, wgs, iters, dx.ptr, dp.ptr, dout.ptr), "probe_valu")
+            ms = ctx.timer_end()
+            if rep:
+                best = min(best, ms)
+        text = lib.ornith_probe_valu_name(op).decode()
+        name = " + ".join(part.split()[0] for part in text.split("\n\t"))   # mnemonics only; a pair counts as one
+        rows.append({"instruction": name, "ms": round(best, 3),
+                     "T_lane_ops_s": round(wgs * 256 * iters * 8 / (best * 1e-3) / 1e12, 1)})
+    res["vector_instruction_rate"] = rows
+
+    # -- what a kernel argument costs: a struct read by a scalar load, or preloaded flat arguments
+    didx = ctx.to_device(np.array([3], np.uint32))
+    ddata = ctx.alloc(64 << 10)
+    ddata.zero()
+    wg = 512
+    dst = ctx.alloc(wg * 32)
+    scrub = ctx.alloc(64 << 20)
+    rows = []
+    for flat in (0, 1):
+        acc = []
+        for rep in range(6):
+            scrub.zero()   # a launch of something else between two probes, as in a decode step
+            probe(lib.ornith_probe_kernarg(ctx.h, flat, wg, didx.ptr, ddata.ptr, dst.ptr), "probe_kernarg")
+            st = dst.download(np.int64, (wg, 4)).astype(np.float64) / 100.0
+            if rep:
+                acc.append([np.mean(st[:, 1] - st[:, 0]), np.mean(st[:, 2] - st[:, 1]), np.mean(st[:, 3] - st[:, 2])])
+        m = np.mean(np.array(acc), axis=0)
+        rows.append({"arguments": "leading flat arguments (preloaded)" if flat else "one struct (scalar load)",
+                     "us_until_the_argument_is_in_a_register": round(float(m[0]), 3),
+                     "us_dependent_scalar_load": round(float(m[1]), 3), "us_dependent_vector_load": round(float(m[2]), 3)})
+    res["kernel_argument"] = rows
+    for b in (dx, dp, dout, didx, ddata, dst, scrub):
+        b.free()
     print(json.dumps({"ceiling": res}), flush=True)
+
+
+def pair_marks(orn, ctx, model, np, n_layers, T):
+    """Phase time stamps of the expert up + down pair as the model launches it (one launch of a
+    stamped build: `ORN_EXTRA_FLAGS=-DORN_TIMING python ornith-rs_amd/build.py`): every workgroup
+    stores the 100 MHz clock at its phase boundaries; printed as percentiles over the launch's
+    workgroups, in us after the launch's first workgroup started."""
+    lib = orn.lib()
+    if not hasattr(lib, "ornith_debug_marks_up"):
+        sys.exit("bench.py --pair-marks needs the stamped build: ORN_EXTRA_FLAGS=-DORN_TIMING python ornith-rs_amd/build.py")
+    rng = np.random.default_rng(123)
+    H, I, E, k = 2048, 512, 256, 8
+    moes = [model.moe_weights(i) for i in range(n_layers)]
+    x = ctx.to_device(orn.f32_to_bf16(rng.standard_normal((T, H)).astype(np.float32)))
+    gates = [ctx.alloc(T * E * 2) for _ in moes]
+    egate = ctx.alloc(T * 2)
+    inds, scores = ctx.alloc(T * k * 4), ctx.alloc(T * k * 2)
+    act, out = ctx.alloc((T * k + T) * I * 2), ctx.alloc(T * H * 2)
+    for w, g in zip(moes, gates):
+        ctx.linear_matmul(_Lin(w.router), x, T, g)
+        ctx.linear_matmul(_Lin(w.sh_egate), x, T, egate)
+    us = _time_loop(ctx, lambda i: orn.moe_experts_from_gates(ctx, moes[i % n_layers], x, T, gates[i % n_layers], egate,
+                                                              inds, scores, act, out), 200, n_layers)
+    orn.moe_experts_from_gates(ctx, moes[n_layers // 2], x, T, gates[n_layers // 2], egate, inds, scores, act, out)
+    ctx.sync()
+    up = (C.c_longlong * (2048 * 8))()
+    down = (C.c_longlong * (1024 * 8))()
+    lib.ornith_debug_marks_up(up)
+    lib.ornith_debug_marks_down(down)
+    a = np.frombuffer(up, np.int64).reshape(2048, 8).astype(np.float64)
+    a = a[a[:, 4] > 0]
+    d = np.frombuffer(down, np.int64).reshape(1024, 8).astype(np.float64)
+    d = d[d[:, 5] > 0]
+    t0, t1 = a[:, 0].min(), d[:, 0].min()
+
+    def row(name, v, base):
+        v = (v - base) / 100.0
+        return {"phase": name, "min": round(float(v.min()), 2), "p10": round(float(np.percentile(v, 10)), 2),
+                "median": round(float(np.median(v)), 2), "p90": round(float(np.percentile(v, 90)), 2), "max": round(float(v.max()), 2)}
+
+    routed = a[:, 5] > 0
+    res = {"verify_width": T, "us_per_pair_stamped_build": round(us, 2),
+           "up": {"workgroups": len(a), "phases": [
+               row("start", a[:, 0], t0), row("gates in registers (routed workgroups)", a[routed, 6], t0),
+               row("routing made (routed workgroups)", a[routed, 5], t0),
+               row("weight loads issued", a[:, 1], t0), row("activations loaded", a[:, 2], t0),
+               row("first two rows done", a[:, 3], t0), row("end", a[:, 4], t0),
+               row("shared expert's workgroups: weight loads issued", a[~routed, 1], t0),
+               row("shared expert's workgroups: end", a[~routed, 4], t0)]},
+           "down": {"workgroups": len(d), "starts_us_after_the_up_launch": round(float((t1 - t0) / 100.0), 2), "phases": [
+               row("start", d[:, 0], t1), row("weight loads issued", d[:, 1], t1), row("activations loaded", d[:, 2], t1),
+               row("sums done (wavefront 0)", d[:, 3], t1), row("after the barrier", d[:, 4], t1), row("end", d[:, 5], t1)]}}
+    print(json.dumps({"pair_marks": res}), flush=True)
 
 
 def config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name):
@@ -575,7 +674,10 @@ def main():
                     help="only the A/B of the MoE block's launch structure (option fuse_moe_one = 0, 1, 2)")
     ap.add_argument("--ceiling", action="store_true",
                     help="only the machine probes: empty launches, stream-only launches of the expert kernels' shapes, "
-                         "a long read, the workgroup-to-die rule, the latency of a word between workgroups")
+                         "a long read, the workgroup-to-die rule, the latency of a word between workgroups, the rate "
+                         "of single vector instructions, the cost of a kernel argument")
+    ap.add_argument("--pair-marks", action="store_true",
+                    help="only the phase time stamps of the expert pair (needs the library built with -DORN_TIMING)")
     ap.add_argument("--warm-cold", action="store_true",
                     help="only the mat-vec timings on re-used, unread and just-read weights")
     args = ap.parse_args()
@@ -620,6 +722,8 @@ def main():
         return
     if args.moe_ab:
         return moe_ab(orn, ctx, model, np, args.layers)
+    if args.pair_marks:
+        return pair_marks(orn, ctx, model, np, args.layers, args.depth + 1)
     if args.config5:
         print(json.dumps(config5(args, orn, ctx, synth, np, model, ws, cfg, dev_name)), flush=True)
         return

@@ -839,6 +839,21 @@ ORNITH_API int ornith_probe_stream(ornith_ctx* ctx, const void* d_src, size_t by
 ORNITH_API int ornith_probe_read(ornith_ctx* ctx, const void* d_src, size_t bytes, void* d_sink);
 ORNITH_API int ornith_probe_xcc(ornith_ctx* ctx, int workgroups, uint32_t* d_out);
 ORNITH_API int ornith_probe_handoff(ornith_ctx* ctx, void* d_flag, void* d_out4, int producer, int consumer, int mode);
+/* probe_valu: one launch of `workgroups` x 256 threads, every thread running 8 x `iters` of one
+ * vector instruction (op 0 .. ornith_probe_valu_count() - 1, named by ornith_probe_valu_name):
+ * what the instructions of the dequantizing mat-vecs cost each. d_x: 4 floats, d_p: 4 words,
+ * d_out: workgroups x 256 floats. probe_kernarg: the same small kernel with its arguments in a
+ * struct (flat = 0: read through a scalar load when the wavefront starts) or as leading flat
+ * arguments (flat = 1: preloaded into scalar registers with the wavefront); every workgroup
+ * stores four 64-bit stamps of the 100 MHz clock: entry, argument in a register, after a
+ * dependent scalar load, after a dependent vector load. d_idx: one word below 256, d_data:
+ * 64 KB, d_out: workgroups x 4 x int64. */
+ORNITH_API int ornith_probe_valu_count(void);
+ORNITH_API const char* ornith_probe_valu_name(int op);
+ORNITH_API int ornith_probe_valu(ornith_ctx* ctx, int op, int workgroups, int iters, const void* d_x, const void* d_p,
+                                 void* d_out);
+ORNITH_API int ornith_probe_kernarg(ornith_ctx* ctx, int flat, int workgroups, const void* d_idx, const void* d_data,
+                                    void* d_out);
 
 #ifdef __cplusplus
 }

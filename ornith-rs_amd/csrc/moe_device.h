@@ -19,6 +19,10 @@ __device__ __forceinline__ bf16_t swiglu_bf16(float g, float u) {
   return dm_f2bf(s * ub);
 }
 
+#ifndef ORN_TOPK_STAMP
+#define ORN_TOPK_STAMP()
+#endif
+
 template <int S>
 __device__ __forceinline__ uint32_t dm_xor_lane_u32(uint32_t v) {
   return __builtin_bit_cast(uint32_t, dm_xor_lane<S>(__builtin_bit_cast(float, v)));
@@ -76,6 +80,7 @@ __device__ __forceinline__ void router_topk_wave(const bf16_t* gates_row, int k,
 #pragma unroll
   for (int i = 0; i < PER; ++i) m = v[i] > m ? v[i] : m;
   m = dm_wave_max<64>(m);
+  ORN_TOPK_STAMP();  // debug builds: the gates are in registers here
   float s = 0.f;
 #pragma unroll
   for (int i = 0; i < PER; ++i) {

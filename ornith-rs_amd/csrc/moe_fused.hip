@@ -25,6 +25,13 @@
 // nothing but the index list), then the activation loads, and only then computes.
 #include "handoff.h"
 #include "kq_device.h"
+#ifdef ORN_TIMING
+#include "rt.h"
+// debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch
+__device__ long long g_up_marks[2048][8];
+#define UP_MARK(i) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if (threadIdx.x == 0 && bl__ < 2048) g_up_marks[bl__][i] = wall_clock64(); } while (0)
+#define ORN_TOPK_STAMP() UP_MARK(6)  // in the top-k: the gates have arrived
+#endif
 #include "moe_device.h"
 #include "norm_device.h"
 #include "rt.h"
@@ -54,9 +61,6 @@ struct UpArgs {
 
 // grid (ceil(I / (RPW * 4 * ITERS)), T*k + T), 256 threads
 #ifdef ORN_TIMING
-// debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch
-__device__ long long g_up_marks[2048][8];
-#define UP_MARK(i) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if (threadIdx.x == 0 && bl__ < 2048) g_up_marks[bl__][i] = wall_clock64(); } while (0)
 __device__ long long g_down_marks[1024][8];
 #define DOWN_MARK(i) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if ((threadIdx.x & 63) == 0 && (threadIdx.x >> 6) == (i >> 3) && bl__ < 1024) g_down_marks[bl__][i & 7] = wall_clock64(); } while (0)
 #else
@@ -65,6 +69,25 @@ __device__ long long g_down_marks[1024][8];
 #endif
 
 // ROUTE: the routing is made in the head of the launch (a.gates) instead of read (a.inds)
+#ifdef ORN_NOACC
+// measurement build only (-DORN_NOACC): the two expert kernels with the dequantizing arithmetic
+// taken out -- every load, the routing, the activation conversion, the reductions, swiglu and
+// the combine stay; a row's sum is a fold of its loaded registers. What such a build takes is
+// what the launch structure costs without the mat-vec's own vector work (results are garbage).
+__device__ __forceinline__ float noacc_fold(const Q4Row& r, float x) {
+  return __uint_as_float((r.q.x ^ r.q.y ^ r.q.z ^ r.q.w ^ r.s0 ^ r.s1 ^ r.s2 ^ r.dmw) & 0x3fffffffu) + x;
+}
+__device__ __forceinline__ float noacc_fold(const Q6Row& r, float x) {
+  return __uint_as_float((r.qa.x ^ r.qa.y ^ r.qa.z ^ r.qa.w ^ r.qb.x ^ r.qb.y ^ r.qb.z ^ r.qb.w ^ r.qh.x ^ r.qh.y ^
+                          r.qh.z ^ r.qh.w ^ r.sc.x ^ r.sc.y ^ r.d) & 0x3fffffffu) + x;
+}
+__device__ __forceinline__ float noacc_x(const Q4Lane<1>& L) { return L.sl[0] + L.sh[0]; }
+__device__ __forceinline__ float noacc_x(const Q6Lane<1>& L) { return L.x[0][0][0] + L.x[0][1][5] + L.x[0][2][9] + L.x[0][3][15]; }
+#define ORN_KL_ACC(row, L, acc) acc[0] = noacc_fold(row, noacc_x(L))
+#else
+#define ORN_KL_ACC(row, L, acc) KL::accumulate(row, L, acc)
+#endif
+
 // The leading flat arguments repeat what decides a workgroup's expert (the library is built with
 // kernel-argument preloading: they are in scalar registers when the wavefront starts, so the
 // gates / ids are asked for while the argument block is still being fetched).
@@ -143,10 +166,10 @@ __global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* h_gates, cons
 #pragma unroll
     for (int it = 0; it < ITERS; it += 2) {
       float g0[1] = {0.f}, u0[1] = {0.f}, g1[1] = {0.f}, u1[1] = {0.f};
-      KL::accumulate(rg[it], L, g0);
-      KL::accumulate(ru[it], L, u0);
-      KL::accumulate(rg[it + 1], L, g1);
-      KL::accumulate(ru[it + 1], L, u1);
+      ORN_KL_ACC(rg[it], L, g0);
+      ORN_KL_ACC(ru[it], L, u0);
+      ORN_KL_ACC(rg[it + 1], L, g1);
+      ORN_KL_ACC(ru[it + 1], L, u1);
       const float red = dm_wave_sum4(g0[0], u0[0], g1[0], u1[0], lane);
       // lanes [0,16): gate row it, [32,48): up row it, [16,32): gate row it+1, [48,64): up row it+1;
       // after the halves trade places every lane holds a row's gate and up sums, and lanes 0
@@ -162,8 +185,8 @@ __global__ __launch_bounds__(256) void moe_up_kernel(const bf16_t* h_gates, cons
     for (int it = 0; it < ITERS; ++it) {
       const int o = base + it * RPW + slot;
       float ag[1] = {0.f}, au[1] = {0.f};
-      KL::accumulate(rg[it], L, ag);
-      KL::accumulate(ru[it], L, au);
+      ORN_KL_ACC(rg[it], L, ag);
+      ORN_KL_ACC(ru[it], L, au);
       const float g = dm_wave_sum<LPR>(ag[0]);
       const float u = dm_wave_sum<LPR>(au[0]);
       if (c == 0 && o < a.I) a.act[(size_t)r * a.I + o] = swiglu_bf16(g, u);
@@ -236,7 +259,7 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(const uint8_
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     float acc[1] = {0.f};
-    KL::accumulate(rr[it], L, acc);
+    ORN_KL_ACC(rr[it], L, acc);
     const float v = dm_wave_sum<LPR>(acc[0]);
     if (c == 0) yl[j][it * RPW + slot] = dm_rb(v);  // expert outputs are bf16 in the unfused path
   }

@@ -2,7 +2,8 @@
 // launch of the expert kernel's shape costs when it only streams its bytes, what a long read
 // sustains, where workgroups land, and how long a word written by one workgroup takes to be
 // seen by another. They price the decode kernels against the machine instead of against the
-// 8 TB/s figure alone. No reference counterpart; nothing in the decode path calls them.
+// 8 TB/s figure alone; what single vector instructions and kernel arguments cost. No reference
+// counterpart; nothing in the decode path calls them.
 #include "rt.h"
 
 namespace {
@@ -97,9 +98,130 @@ __global__ __launch_bounds__(64) void probe_handoff_kernel(uint32_t* flag, long 
   }
 }
 
+// ---- what one vector instruction costs: eight independent chains of the same instruction per
+// thread, 256 threads a workgroup. The instruction is a template parameter so that the loop
+// holds nothing else; the operands are harmless for every instruction in the list.
+#define ORN_PROBE_OPS(X)                                                                \
+  X(0, "v_fmac_f32 %0, %1, %2")                                                         \
+  X(1, "v_mul_f32 %0, %1, %0")                                                          \
+  X(2, "v_add_f32 %0, %1, %0")                                                          \
+  X(3, "v_and_b32 %0, %2, %0")                                                          \
+  X(4, "v_lshrrev_b32 %0, 1, %0")                                                       \
+  X(5, "v_cvt_f32_ubyte1 %0, %0")                                                       \
+  X(6, "v_cvt_f32_f16 %0, %0")                                                          \
+  X(7, "v_and_or_b32 %0, %0, %2, %2")                                                   \
+  X(8, "v_perm_b32 %0, %0, %2, %2")                                                     \
+  X(9, "v_bfe_u32 %0, %0, 4, 4")                                                        \
+  X(10, "v_pk_add_f16 %0, %0, %2")                                                      \
+  X(11, "v_fma_mix_f32 %0, %1, %2, %0 op_sel:[0,0,0] op_sel_hi:[0,1,0]")                \
+  X(12, "v_cvt_f32_ubyte1 %0, %2\n\tv_fmac_f32 %0, %1, %0")
+
+template <int OP>
+__global__ __launch_bounds__(256) void probe_valu_kernel(const float* xin, const uint32_t* pin, float* out, int iters) {
+  const float x = xin[threadIdx.x & 3];
+  const uint32_t p = pin[threadIdx.x & 3];
+  float a0 = 0.f, a1 = 1.f, a2 = 2.f, a3 = 3.f, a4 = 4.f, a5 = 5.f, a6 = 6.f, a7 = 7.f;
+  for (int i = 0; i < iters; ++i) {
+#define X(N, S)                                          \
+  if constexpr (OP == N) {                               \
+    asm volatile(S : "+v"(a0) : "v"(x), "v"(p));         \
+    asm volatile(S : "+v"(a1) : "v"(x), "v"(p));         \
+    asm volatile(S : "+v"(a2) : "v"(x), "v"(p));         \
+    asm volatile(S : "+v"(a3) : "v"(x), "v"(p));         \
+    asm volatile(S : "+v"(a4) : "v"(x), "v"(p));         \
+    asm volatile(S : "+v"(a5) : "v"(x), "v"(p));         \
+    asm volatile(S : "+v"(a6) : "v"(x), "v"(p));         \
+    asm volatile(S : "+v"(a7) : "v"(x), "v"(p));         \
+  }
+    ORN_PROBE_OPS(X)
+#undef X
+  }
+  out[blockIdx.x * 256 + threadIdx.x] = a0 + a1 + a2 + a3 + a4 + a5 + a6 + a7;
+}
+constexpr int kProbeOps = 13;
+#define X(N, S) S,
+const char* const kProbeOpNames[kProbeOps] = {ORN_PROBE_OPS(X)};
+#undef X
+
+// ---- what a kernel argument costs. The same kernel twice: its arguments as one struct (read
+// through a scalar load when the wavefront starts, as most kernels of this library take theirs)
+// and as leading flat arguments (preloaded into scalar registers with the wavefront). Each
+// workgroup stamps the 100 MHz clock at entry, when the argument is in a register, after a scalar
+// load that depends on it and after a vector load that depends on that.
+struct ProbeArgPack {
+  const uint32_t* p[6];
+  int n[4];
+};
+__device__ __forceinline__ void probe_kernarg_body(const uint32_t* idx, const uint32_t* data, long long* out,
+                                                   long long t0) {
+  uint64_t v = (uint64_t)idx;
+  asm volatile("" : "+s"(v));
+  const long long t1 = wall_clock64();
+  uint32_t i2 = __builtin_amdgcn_readfirstlane(*reinterpret_cast<const uint32_t*>(v));
+  asm volatile("" : "+s"(i2));
+  const long long t2 = wall_clock64();
+  uint32_t w = data[(i2 & 255u) * 64 + threadIdx.x];
+  asm volatile("" : "+v"(w));
+  const long long t3 = wall_clock64();
+  if (threadIdx.x == 0) {
+    long long* o = out + blockIdx.x * 4;
+    o[0] = t0;
+    o[1] = t1;
+    o[2] = t2;
+    o[3] = t3 + (w == 0x12345u);
+  }
+}
+__global__ __launch_bounds__(256) void probe_kernarg_struct_kernel(ProbeArgPack a, long long* out) {
+  const long long t0 = wall_clock64();
+  probe_kernarg_body(a.p[1], a.p[2], out, t0);
+}
+__global__ __launch_bounds__(256) void probe_kernarg_flat_kernel(const uint32_t* idx, const uint32_t* data, long long* out) {
+  const long long t0 = wall_clock64();
+  probe_kernarg_body(idx, data, out, t0);
+}
+
 }  // namespace
 
 extern "C" {
+
+// One launch of `workgroups` x 256 threads, each thread running 8 x `iters` of instruction `op`
+// (ornith_probe_valu_name(op) names it; ops 0 .. ornith_probe_valu_count() - 1). d_x: 4 floats,
+// d_p: 4 words (a word whose halves are small f16 values keeps every instruction finite),
+// d_out: workgroups * 256 floats.
+int ornith_probe_valu_count(void) { return kProbeOps; }
+const char* ornith_probe_valu_name(int op) { return op >= 0 && op < kProbeOps ? kProbeOpNames[op] : ""; }
+int ornith_probe_valu(ornith_ctx* ctx, int op, int workgroups, int iters, const void* d_x, const void* d_p, void* d_out) {
+  ORN_REQUIRE(ctx && d_x && d_p && d_out && op >= 0 && op < kProbeOps && workgroups >= 1 && iters >= 1,
+              "probe_valu: bad argument");
+  switch (op) {
+#define X(N, S)                                                                                                   \
+  case N:                                                                                                         \
+    hipLaunchKernelGGL(probe_valu_kernel<N>, dim3(workgroups), dim3(256), 0, ctx->stream, (const float*)d_x,      \
+                       (const uint32_t*)d_p, (float*)d_out, iters);                                               \
+    break;
+    ORN_PROBE_OPS(X)
+#undef X
+  }
+  ORN_LAUNCH_CHECK("probe_valu_kernel");
+  return ORNITH_OK;
+}
+
+// flat = 0: the arguments in a struct; 1: as leading flat arguments. d_idx: one word (an index
+// below 256), d_data: 64 KB, d_out: workgroups x 4 x int64 (the four stamps).
+int ornith_probe_kernarg(ornith_ctx* ctx, int flat, int workgroups, const void* d_idx, const void* d_data, void* d_out) {
+  ORN_REQUIRE(ctx && d_idx && d_data && d_out && workgroups >= 1, "probe_kernarg: bad argument");
+  if (flat) {
+    hipLaunchKernelGGL(probe_kernarg_flat_kernel, dim3(workgroups), dim3(256), 0, ctx->stream, (const uint32_t*)d_idx,
+                       (const uint32_t*)d_data, (long long*)d_out);
+  } else {
+    ProbeArgPack a{};
+    a.p[1] = (const uint32_t*)d_idx;
+    a.p[2] = (const uint32_t*)d_data;
+    hipLaunchKernelGGL(probe_kernarg_struct_kernel, dim3(workgroups), dim3(256), 0, ctx->stream, a, (long long*)d_out);
+  }
+  ORN_LAUNCH_CHECK("probe_kernarg_kernel");
+  return ORNITH_OK;
+}
 
 int ornith_probe_empty(ornith_ctx* ctx, int workgroups, int threads, int with_args, int launches) {
   ORN_REQUIRE(ctx && workgroups >= 1 && threads >= 1 && threads <= 1024 && launches >= 1, "probe_empty: bad argument");
