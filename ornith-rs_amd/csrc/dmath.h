@@ -65,9 +65,8 @@ __device__ __forceinline__ float dm_h2f(f16_t h) {
 // exp(x): reduce by ln2 in two pieces, degree-5 polynomial, exponent from bits.
 // x < -87 gives +0 and x > 88 gives +inf, so subnormal results never occur.
 __device__ __forceinline__ float dm_exp(float x) {
-  if (x != x) return x;
-  if (x > 88.0f) return DM_INF;
-  if (x < -87.0f) return 0.0f;
+  // no branches: the polynomial is worked out for every input and the special cases are
+  // selected afterwards (outside [-87, 88] its value is never used; a NaN stays that NaN)
   float n = __builtin_rintf(x * 1.44269504088896341f);
   float r = dm_fma(n, -0.693359375f, x);
   r = dm_fma(n, 2.12194440e-4f, r);
@@ -79,8 +78,12 @@ __device__ __forceinline__ float dm_exp(float x) {
   p = dm_fma(p, r, 5.0000001201e-1f);
   float r2 = r * r;
   float e = dm_fma(p, r2, r) + 1.0f;
-  int ni = (int)n;
-  return e * __uint_as_float((uint32_t)(ni + 127) << 23);
+  // n as an integer: n is integral and, where the result is used, within [-126, 127]
+  const int ni = (int)__builtin_fminf(__builtin_fmaxf(n, -200.0f), 200.0f);
+  float v = e * __uint_as_float((uint32_t)(ni + 127) << 23);
+  v = x < -87.0f ? 0.0f : v;
+  v = x > 88.0f ? DM_INF : v;
+  return x != x ? x : v;
 }
 
 // log(x), x finite normal > 0.

@@ -42,6 +42,21 @@ __device__ __forceinline__ uint32_t dm_wave_max_u32(uint32_t v) {
   return v;
 }
 
+// max over the 64 lanes with v_max_f32 (NaN operands lose, as under `v > m ? v : m`; +0 / -0 may
+// come out with the other sign, which exp(v - m) does not see)
+__device__ __forceinline__ float router_wave_max(float v) {
+  float a, b;
+  dm_row_swap<32>(v, a, b);
+  v = __builtin_fmaxf(a, b);
+  dm_row_swap<16>(v, a, b);
+  v = __builtin_fmaxf(a, b);
+  v = __builtin_fmaxf(v, dm_xor_lane<8>(v));
+  v = __builtin_fmaxf(v, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xF, 0xF, false)));
+  v = __builtin_fmaxf(v, dm_xor_lane<2>(v));
+  v = __builtin_fmaxf(v, dm_xor_lane<1>(v));
+  return v;
+}
+
 // Lane l holds gates [l*PER, (l+1)*PER) of the row. All 64 lanes must be active.
 // E = 64 * PER <= 1024 so an index fits 10 bits: a candidate is the single integer
 // (bf16 probability bits << 16 | index) + 1, whose order is exactly (value, index) for
@@ -78,8 +93,8 @@ __device__ __forceinline__ void router_topk_wave(const bf16_t* gates_row, int k,
     for (int i = 0; i < PER; ++i) v[i] = dm_bf2f(g[i]);
   }
 #pragma unroll
-  for (int i = 0; i < PER; ++i) m = v[i] > m ? v[i] : m;
-  m = dm_wave_max<64>(m);
+  for (int i = 0; i < PER; ++i) m = __builtin_fmaxf(m, v[i]);
+  m = router_wave_max(m);
   ORN_TOPK_STAMP();  // debug builds: the gates are in registers here
   float s = 0.f;
 #pragma unroll
@@ -109,10 +124,12 @@ __device__ __forceinline__ void router_topk_wave(const bf16_t* gates_row, int k,
   uint32_t mine = 0;  // lane r keeps round r's winner; one store after the rounds
   for (int r = 0; r < k; ++r) {
     const uint32_t win = dm_wave_max_u32(key[0]);
-    const bool won = key[0] == win;  // keys are distinct (the index is in them) unless 0
+    // keys are distinct (the index is in them) unless 0; the winner's list moves up through a
+    // lane mask (bit selects: no condition register between the steps)
+    const uint32_t stay = key[0] == win ? 0u : 0xffffffffu;
 #pragma unroll
-    for (int i = 0; i + 1 < PER; ++i) key[i] = won ? key[i + 1] : key[i];
-    key[PER - 1] = won ? 0u : key[PER - 1];
+    for (int i = 0; i + 1 < PER; ++i) key[i] = (key[i] & stay) | (key[i + 1] & ~stay);
+    key[PER - 1] &= stay;
     mine = lane == r ? win : mine;
   }
   if (lane < k) {
