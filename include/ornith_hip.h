@@ -95,6 +95,9 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *   "gdn_block_chunks" (ORNITH_GDN_BLOCK_CHUNKS, default 64): chunks one prepare / scan launch
  *               pair of that recurrence covers (longer calls go block by block so that the
  *               block's operands stay in the last-level cache); same results for any value
+ *   "fuse_attn_prep" (ORNITH_FUSE_ATTN_PREP, default 1): ornith_attn_decode lets the attention
+ *               launch do the prep of its own rows (norm, RoPE, KV append) at decode widths
+ *               (0: a prep launch first); bit-identical
  *   "fuse_moe_one" (ORNITH_FUSE_MOE_ONE, default 0): the MoE block's phases as ranges of
  *               workgroups of ONE launch that hand their intermediates over through memory
  *               (1: router + up + down, 2: up + down after a router launch). Bit-identical,
@@ -373,6 +376,17 @@ ORNITH_API int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, co
                                         const void* d_v_cache, const void* d_qg, int T, int Hq,
                                         int Hkv, int hd, int offset, const int* d_offset, int cap,
                                         float scale, void* d_out);
+/* ornith_attn_prep followed by ornith_sdpa_decode_gated on the same rows, as Attention::forward
+ * runs them (src/model/qwen3_5.rs:430-474), host-side offset: the same results and the same
+ * cache contents; at decode widths (T <= 8, a context short enough for the one-workgroup-per-
+ * block form) one launch does both -- every workgroup makes its query row and the call's new
+ * key rows itself, and the caches are written as a side effect. d_q_rot is only written when
+ * the prep runs as its own launch. */
+ORNITH_API int ornith_attn_decode(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const void* d_vx,
+                                  const void* d_q_norm_w, const void* d_k_norm_w, int T, int Hq, int Hkv,
+                                  int hd, int rope_dims, float eps, const float* d_cos, const float* d_sin,
+                                  int table_npos, int offset, int cap, float scale, void* d_q_rot,
+                                  void* d_k_cache, void* d_v_cache, void* d_out);
 /* sdpa_unfused (src/ops/sdpa.rs:386-461) for the rows of a prompt chunk, with the same output
  * gate: causal flash attention on the matrix cores, head_dim 256. Same arguments as
  * sdpa_decode_gated (host-side offset only), which forwards to it from 32 rows up; agrees

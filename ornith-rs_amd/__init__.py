@@ -363,6 +363,15 @@ def sdpa_decode_gated(self, q_rot, k_cache, v_cache, qg, T, Hq, Hkv, hd, offset,
                                           out.ptr), "sdpa_decode_gated")
 
 
+@_ctx_method
+def attn_decode(self, qg, kx, vx, qw, kw, T, Hq, Hkv, hd, rope_dims, eps, cos_t, sin_t, npos, offset, cap, scale,
+                q_rot, k_cache, v_cache, out):
+    """ornith_attn_decode: prep + attention of the same rows, one launch where the shape allows."""
+    _check(lib().ornith_attn_decode(self.h, qg.ptr, kx.ptr, vx.ptr, qw.ptr, kw.ptr, T, Hq, Hkv, hd, rope_dims,
+                                    C.c_float(eps), cos_t.ptr, sin_t.ptr, npos, offset, cap, C.c_float(scale),
+                                    q_rot.ptr, k_cache.ptr, v_cache.ptr, out.ptr), "attn_decode")
+
+
 # ---- greedy selection ----------------------------------------------------------------
 @_ctx_method
 def greedy_rows(self, logits, rows, V, tokens, lse=None):

@@ -44,7 +44,70 @@ struct PrepArgs {
   float eps;
 };
 
-// one wavefront per (head, token); PER = hd / 64 contiguous channels per lane
+// The per-head prep of one row by one wavefront (PER = hd / 64 contiguous channels a lane), in
+// two steps so that a caller can put other loads between the request and the arithmetic:
+// prep_issue asks for the row, the norm weight and the lane's cos / sin entries; prep_finish
+// returns the normed, rotated values (rounded to bf16 by whoever stores them).
+template <int PER>
+struct PrepRegs {
+  bf16_t x[PER], w[PER];
+  float c[PER], s[PER];
+};
+
+template <int PER>
+__device__ __forceinline__ void prep_issue(const bf16_t* src, const bf16_t* w, const float* cos_t, const float* sin_t,
+                                           int pos, int half, int lane, PrepRegs<PER>& g) {
+#pragma unroll
+  for (int i = 0; i < PER; ++i) g.x[i] = src[lane * PER + i];
+  if (w) {
+#pragma unroll
+    for (int i = 0; i < PER; ++i) g.w[i] = w[lane * PER + i];
+    const int hl = half / PER;
+    const bool lowg = lane < hl, rot = lane < 2 * hl;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int e = (lowg ? lane : lane - hl) * PER + i;
+      g.c[i] = rot ? cos_t[(size_t)pos * half + e] : 0.f;
+      g.s[i] = rot ? sin_t[(size_t)pos * half + e] : 0.f;
+    }
+  }
+}
+
+template <int PER>
+__device__ __forceinline__ void prep_finish(const PrepRegs<PER>& g, bool normed, int half, float eps, int lane,
+                                            float (&x)[PER]) {
+  constexpr int HD = 64 * PER;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) x[i] = dm_bf2f(g.x[i]);
+  if (!normed) return;
+  float a = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) a = dm_fma(x[i], x[i], a);
+  const float inv = dm_rsqrt(dm_wave_sum<64>(a) / (float)HD + eps);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) x[i] = dm_rb(dm_bf2f(g.w[i]) * dm_rb(x[i] * inv));
+  // rotate pairs (e, e + half), e < half; the partner channel lives hl lanes away
+  const int hl = half / PER;
+  const bool lowg = lane < hl, rot = lane < 2 * hl;
+  const int partner = lowg ? lane + hl : lane - hl;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const float other = __shfl(x[i], partner & 63, 64);
+    if (rot) {
+      float r;
+      if (lowg) {
+        r = x[i] * g.c[i];
+        r = dm_fma(-other, g.s[i], r);
+      } else {
+        r = other * g.s[i];
+        r = dm_fma(x[i], g.c[i], r);
+      }
+      x[i] = r;  // rounded on store
+    }
+  }
+}
+
+// one wavefront per (head, token)
 template <int PER>
 __global__ __launch_bounds__(64) void attn_prep_kernel(PrepArgs p) {
   constexpr int HD = 64 * PER;
@@ -69,38 +132,10 @@ __global__ __launch_bounds__(64) void attn_prep_kernel(PrepArgs p) {
     src = p.vx + ((size_t)t * p.Hkv + h) * HD;
     dst = p.v_cache + ((size_t)h * p.cap + pos) * HD;
   }
+  PrepRegs<PER> g;
+  prep_issue<PER>(src, w, p.cos_t, p.sin_t, pos, p.half, lane, g);
   float x[PER];
-#pragma unroll
-  for (int i = 0; i < PER; ++i) x[i] = dm_bf2f(src[lane * PER + i]);
-  if (w) {
-    float a = 0.f;
-#pragma unroll
-    for (int i = 0; i < PER; ++i) a = dm_fma(x[i], x[i], a);
-    const float inv = dm_rsqrt(dm_wave_sum<64>(a) / (float)HD + p.eps);
-#pragma unroll
-    for (int i = 0; i < PER; ++i) x[i] = dm_rb(dm_bf2f(w[lane * PER + i]) * dm_rb(x[i] * inv));
-    // rotate pairs (e, e + half), e < half; the partner channel lives hl lanes away
-    const int hl = p.half / PER;
-    const bool lowg = lane < hl, rot = lane < 2 * hl;
-    const int partner = lowg ? lane + hl : lane - hl;
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const float other = __shfl(x[i], partner & 63, 64);
-      if (rot) {
-        const int e = (lowg ? lane : lane - hl) * PER + i;
-        const float c = p.cos_t[(size_t)pos * p.half + e], s = p.sin_t[(size_t)pos * p.half + e];
-        float r;
-        if (lowg) {
-          r = x[i] * c;
-          r = dm_fma(-other, s, r);
-        } else {
-          r = other * s;
-          r = dm_fma(x[i], c, r);
-        }
-        x[i] = r;  // rounded on store
-      }
-    }
-  }
+  prep_finish<PER>(g, w != nullptr, p.half, p.eps, lane, x);
 #pragma unroll
   for (int i = 0; i < PER; ++i) dst[lane * PER + i] = dm_f2bf(x[i]);
 }
@@ -159,11 +194,19 @@ __device__ __forceinline__ float sdpa_pair_tree(const float* p, int stride) {
   return t[0];
 }
 
-template <int HD>
-__global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sdpa_partial_kernel(SdpaArgs p) {
+//
+// PREP: the launch also does attn_prep's work (the per-head norm, RoPE and the KV append), so
+// that no prep launch precedes it: wavefront 0 makes the query row of this (row, head) from the
+// raw projection, wavefronts 1 .. t + 1 the key rows of the call's new positions that lie in this
+// block (they go into the staged block in place of the cache's rows, which are not yet written),
+// the new value rows are read from the raw projection, and the workgroup of a KV group's first
+// head stores its own row's key and value to the cache. Static offset, T <= 8.
+template <int HD, bool PREP>
+__global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void sdpa_partial_kernel(SdpaArgs p,
+                                                                                                           PrepArgs q) {
   const int b = blockIdx.x, hq = blockIdx.y, t = blockIdx.z, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int offset = p.d_offset ? *p.d_offset : p.offset;
+  const int offset = PREP ? p.offset : (p.d_offset ? *p.d_offset : p.offset);
   const int last = min(offset + t, p.cap - 1);
   if (b * ATT_KB > last) return;
   const int hk = hq / (p.Hq / p.Hkv);
@@ -188,6 +231,23 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
   const bf16_t* kbase = p.k_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD;
   const bf16_t* vblk = p.v_cache + ((size_t)hk * p.cap + (size_t)b * ATT_KB) * HD + 8 * piece;
   u32x4 kreg[NLD], vreg[NLD];
+  // PREP: this wavefront's row of the prep (0: none, 1: the query, 2: a new key row at kpos);
+  // its few loads go out ahead of the block's, so that they are back first
+  constexpr int PER = HD / 64;
+  PrepRegs<PER> pg;
+  int task = 0, kpos = 0;
+  const bool first_of_group = hq % (p.Hq / p.Hkv) == 0;
+  if constexpr (PREP) {
+    if (wave == 0) {
+      task = 1;
+      prep_issue<PER>(q.qg + ((size_t)t * p.Hq + hq) * 2 * HD, q.qw, q.cos_t, q.sin_t, offset + t, q.half, lane, pg);
+    } else if (wave <= t + 1 && (offset + wave - 1) / ATT_KB == b) {
+      task = 2;
+      kpos = offset + wave - 1;
+      prep_issue<PER>(q.kx + ((size_t)(wave - 1) * p.Hkv + hk) * HD, q.kw, q.cos_t, q.sin_t, kpos, q.half, lane, pg);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
 #pragma unroll
   for (int c = 0; c < NKC; ++c)
 #pragma unroll
@@ -195,20 +255,58 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
       kreg[c * KPC + i] = *reinterpret_cast<const u32x4*>(
           kbase + (size_t)min(krow0 + KRS * i, nvalid - 1) * HD + c * KC + 8 * kpc);
 #pragma unroll
-  for (int u = 0; u < NLD; ++u)
-    vreg[u] = *reinterpret_cast<const u32x4*>(vblk + (size_t)min(row0 + RPU * u, nvalid - 1) * HD);
+  for (int u = 0; u < NLD; ++u) {
+    const int vr = min(row0 + RPU * u, nvalid - 1);
+    const bf16_t* src = vblk + (size_t)vr * HD;
+    // a position of this call: its value row is still in the projection's output
+    if (PREP && b * ATT_KB + vr >= offset)
+      src = q.vx + ((size_t)(b * ATT_KB + vr - offset) * p.Hkv + hk) * HD + 8 * piece;
+    vreg[u] = *reinterpret_cast<const u32x4*>(src);
+  }
   // the output gate of a finishing block is requested with everything else
   bf16_t gate_pre = 0;
   if (p.finish && tid < HD) gate_pre = p.qg[((size_t)t * p.Hq + hq) * 2 * HD + HD + tid];
-  if (tid < HD) qs[tid] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq) * HD + tid]);
+  if constexpr (!PREP)
+    if (tid < HD) qs[tid] = p.scale * dm_bf2f(p.q_rot[((size_t)t * p.Hq + hq) * HD + tid]);
 
   // scores: thread (key, panel) runs the chain over the panel's 64 channels
 #pragma unroll
   for (int c = 0; c < NKC; ++c)
 #pragma unroll
-    for (int i = 0; i < KPC; ++i)
-      *reinterpret_cast<u32x4*>(stage + c * (ATT_KB * KROW) + (krow0 + KRS * i) * KROW + 16 * kpc) =
-          kreg[c * KPC + i];
+    for (int i = 0; i < KPC; ++i) {
+      const int dest = krow0 + KRS * i;
+      // PREP: the rows of this call's positions come from the wavefronts that make them
+      if (PREP && b * ATT_KB + dest >= offset && dest < nvalid) continue;
+      *reinterpret_cast<u32x4*>(stage + c * (ATT_KB * KROW) + dest * KROW + 16 * kpc) = kreg[c * KPC + i];
+    }
+  if constexpr (PREP) {
+    if (task) {
+      float x[PER];
+      prep_finish<PER>(pg, true, q.half, q.eps, lane, x);
+      if (task == 1) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) qs[lane * PER + i] = p.scale * dm_bf2f(dm_f2bf(x[i]));  // q_rot is bf16
+      } else {
+        const int dest = kpos - b * ATT_KB, ch = lane * PER;
+        bf16_t* row = reinterpret_cast<bf16_t*>(stage + (ch / KC) * (ATT_KB * KROW) + dest * KROW) + ch % KC;
+        bf16_t* crow = q.k_cache + ((size_t)hk * p.cap + kpos) * HD + ch;
+        const bool append = first_of_group && wave - 1 == t;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const bf16_t v = dm_f2bf(x[i]);
+          row[i] = v;
+          if (append) crow[i] = v;
+        }
+      }
+    }
+    // this row's value row to the cache (the thread that holds its piece unclamped)
+    if (first_of_group && b == (offset + t) / ATT_KB) {
+#pragma unroll
+      for (int u = 0; u < NLD; ++u)
+        if (b * ATT_KB + row0 + RPU * u == offset + t)
+          *reinterpret_cast<u32x4*>(q.v_cache + ((size_t)hk * p.cap + offset + t) * HD + 8 * piece) = vreg[u];
+    }
+  }
   __syncthreads();
   const int key = tid & (ATT_KB - 1), grp = tid >> 8;  // four wavefronts a group
   if (grp < NKC) {
@@ -540,11 +638,10 @@ int ornith_rope_table(ornith_ctx* ctx, int npos, int dims, double theta, float* 
   return rc;
 }
 
-int ornith_attn_prep(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const void* d_vx,
-                     const void* d_q_norm_w, const void* d_k_norm_w, int T, int Hq, int Hkv, int hd,
-                     int rope_dims, float eps, const float* d_cos, const float* d_sin, int table_npos,
-                     int offset, const int* d_offset, int cap, void* d_q_rot, void* d_k_cache,
-                     void* d_v_cache) {
+static int prep_args(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const void* d_vx, const void* d_q_norm_w,
+                     const void* d_k_norm_w, int T, int Hq, int Hkv, int hd, int rope_dims, float eps,
+                     const float* d_cos, const float* d_sin, int table_npos, int offset, const int* d_offset, int cap,
+                     void* d_q_rot, void* d_k_cache, void* d_v_cache, PrepArgs* out) {
   ORN_REQUIRE(ctx && d_qg && d_kx && d_vx && d_q_norm_w && d_k_norm_w && d_cos && d_sin && d_q_rot &&
                   d_k_cache && d_v_cache,
               "attn_prep: null argument");
@@ -578,7 +675,12 @@ int ornith_attn_prep(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const 
   p.npos = table_npos;
   p.half = half;
   p.eps = eps;
-  dim3 grid(Hq + 2 * Hkv, T);
+  *out = p;
+  return ORNITH_OK;
+}
+
+static int prep_launch(ornith_ctx* ctx, const PrepArgs& p, int hd) {
+  dim3 grid(p.Hq + 2 * p.Hkv, p.T);
   if (hd == 256)
     hipLaunchKernelGGL(attn_prep_kernel<4>, grid, dim3(64), 0, ctx->stream, p);
   else
@@ -587,15 +689,35 @@ int ornith_attn_prep(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const 
   return ORNITH_OK;
 }
 
-int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d_k_cache,
-                             const void* d_v_cache, const void* d_qg, int T, int Hq, int Hkv, int hd,
-                             int offset, const int* d_offset, int cap, float scale, void* d_out) {
+int ornith_attn_prep(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const void* d_vx,
+                     const void* d_q_norm_w, const void* d_k_norm_w, int T, int Hq, int Hkv, int hd,
+                     int rope_dims, float eps, const float* d_cos, const float* d_sin, int table_npos,
+                     int offset, const int* d_offset, int cap, void* d_q_rot, void* d_k_cache,
+                     void* d_v_cache) {
+  PrepArgs p;
+  int rc = prep_args(ctx, d_qg, d_kx, d_vx, d_q_norm_w, d_k_norm_w, T, Hq, Hkv, hd, rope_dims, eps, d_cos, d_sin,
+                     table_npos, offset, d_offset, cap, d_q_rot, d_k_cache, d_v_cache, &p);
+  if (rc) return rc;
+  return prep_launch(ctx, p, hd);
+}
+
+// prep != null: the prep of the same rows has not been launched yet; it is done inside the
+// attention launch where that launch's form can (the 1024-thread form, T <= 8, static offset), by
+// its own launch first otherwise
+static int sdpa_decode(ornith_ctx* ctx, const void* d_q_rot, const void* d_k_cache, const void* d_v_cache,
+                       const void* d_qg, int T, int Hq, int Hkv, int hd, int offset, const int* d_offset, int cap,
+                       float scale, void* d_out, const PrepArgs* prep) {
   ORN_REQUIRE(ctx && d_q_rot && d_k_cache && d_v_cache && d_qg && d_out, "sdpa_decode: null argument");
   ORN_REQUIRE(hd == 256 || hd == 128, "sdpa_decode: head_dim %d (128 or 256)", hd);
   // prompt chunks: the matrix-core kernel (outside the exact window, like the projections)
-  if (T >= kPrefillRows && hd == 256 && !d_offset)
+  if (T >= kPrefillRows && hd == 256 && !d_offset) {
+    if (prep) {
+      int rc = prep_launch(ctx, *prep, hd);
+      if (rc) return rc;
+    }
     return ornith_sdpa_prefill_gated(ctx, d_q_rot, d_k_cache, d_v_cache, d_qg, T, Hq, Hkv, hd, offset, cap,
                                      scale, d_out);
+  }
   ORN_REQUIRE(T >= 1 && T <= 64 && Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "sdpa_decode: T=%d Hq=%d Hkv=%d",
               T, Hq, Hkv);
   ORN_REQUIRE(offset >= 0 && offset + T <= cap, "sdpa_decode: rows [%d,%d) exceed capacity %d", offset,
@@ -639,6 +761,15 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   const bool many = live > 2L * ctx->compute_units || four;
   // one key block for every row, in the kernel form that knows how to finish: no merge launch
   p.finish = (last_max < ATT_KB && !many) ? 1 : 0;
+  const bool fold = prep && !many && !d_offset && T <= 8 && ornith_option_fuse_attn_prep();
+  PrepArgs pq{};
+  if (prep) {
+    pq = *prep;
+    if (!fold) {
+      const int rcp = prep_launch(ctx, pq, hd);
+      if (rcp) return rcp;
+    }
+  }
   if (many) {
     const dim3 g4(nblk, Hq / 4, T);
     if (hd == 256) {
@@ -651,18 +782,28 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
   } else if (hd == 256) {
     // 150 KB of LDS a block (the whole key block staged at once): asked for once per kernel
     if (!(ctx->lds_attr_set & 1)) {
-      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<256>,
+      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<256, false>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<256>()));
+      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<256, true>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<256>()));
       ctx->lds_attr_set |= 1;
     }
-    hipLaunchKernelGGL((sdpa_partial_kernel<256>), grid, dim3(SDPA_NT), sdpa_stage_bytes<256>(), ctx->stream, p);
+    if (fold)
+      hipLaunchKernelGGL((sdpa_partial_kernel<256, true>), grid, dim3(SDPA_NT), sdpa_stage_bytes<256>(), ctx->stream, p, pq);
+    else
+      hipLaunchKernelGGL((sdpa_partial_kernel<256, false>), grid, dim3(SDPA_NT), sdpa_stage_bytes<256>(), ctx->stream, p, pq);
   } else {
     if (!(ctx->lds_attr_set & 2)) {
-      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<128>,
+      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<128, false>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<128>()));
+      ORN_HIP(hipFuncSetAttribute((const void*)sdpa_partial_kernel<128, true>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, sdpa_stage_bytes<128>()));
       ctx->lds_attr_set |= 2;
     }
-    hipLaunchKernelGGL((sdpa_partial_kernel<128>), grid, dim3(SDPA_NT), sdpa_stage_bytes<128>(), ctx->stream, p);
+    if (fold)
+      hipLaunchKernelGGL((sdpa_partial_kernel<128, true>), grid, dim3(SDPA_NT), sdpa_stage_bytes<128>(), ctx->stream, p, pq);
+    else
+      hipLaunchKernelGGL((sdpa_partial_kernel<128, false>), grid, dim3(SDPA_NT), sdpa_stage_bytes<128>(), ctx->stream, p, pq);
   }
   ORN_LAUNCH_CHECK("sdpa_partial_kernel");
   if (p.finish) return ORNITH_OK;
@@ -672,6 +813,25 @@ int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d
     hipLaunchKernelGGL(sdpa_merge_kernel<128>, dim3(Hq, T), dim3(128), 0, ctx->stream, p);
   ORN_LAUNCH_CHECK("sdpa_merge_kernel");
   return ORNITH_OK;
+}
+
+int ornith_sdpa_decode_gated(ornith_ctx* ctx, const void* d_q_rot, const void* d_k_cache,
+                             const void* d_v_cache, const void* d_qg, int T, int Hq, int Hkv, int hd,
+                             int offset, const int* d_offset, int cap, float scale, void* d_out) {
+  return sdpa_decode(ctx, d_q_rot, d_k_cache, d_v_cache, d_qg, T, Hq, Hkv, hd, offset, d_offset, cap, scale, d_out,
+                     nullptr);
+}
+
+int ornith_attn_decode(ornith_ctx* ctx, const void* d_qg, const void* d_kx, const void* d_vx,
+                       const void* d_q_norm_w, const void* d_k_norm_w, int T, int Hq, int Hkv, int hd,
+                       int rope_dims, float eps, const float* d_cos, const float* d_sin, int table_npos,
+                       int offset, int cap, float scale, void* d_q_rot, void* d_k_cache, void* d_v_cache,
+                       void* d_out) {
+  PrepArgs p;
+  int rc = prep_args(ctx, d_qg, d_kx, d_vx, d_q_norm_w, d_k_norm_w, T, Hq, Hkv, hd, rope_dims, eps, d_cos, d_sin,
+                     table_npos, offset, nullptr, cap, d_q_rot, d_k_cache, d_v_cache, &p);
+  if (rc) return rc;
+  return sdpa_decode(ctx, d_q_rot, d_k_cache, d_v_cache, d_qg, T, Hq, Hkv, hd, offset, nullptr, cap, scale, d_out, &p);
 }
 
 }  // extern "C"

@@ -187,12 +187,10 @@ static int attention_block(ornith_model* m, const AttnLayer& a, void* d_x, int T
     else
       TRY(ornith_linear_matmul_multi(ctx, ws, 3, d_x, T, ys));
   }
-  TRY(ornith_attn_prep(ctx, qg, kx, vx, a.q_norm, a.k_norm, T, c.num_attention_heads,
-                       c.num_key_value_heads, c.head_dim, c.rope_dims, c.rms_norm_eps, m->d_cos,
-                       m->d_sin, m->rope_npos, offset, nullptr, cap, q_rot, k_cache, v_cache));
   const float scale = 1.0f / sqrtf((float)c.head_dim);
-  return ornith_sdpa_decode_gated(ctx, q_rot, k_cache, v_cache, qg, T, c.num_attention_heads,
-                                  c.num_key_value_heads, c.head_dim, offset, nullptr, cap, scale, att);
+  return ornith_attn_decode(ctx, qg, kx, vx, a.q_norm, a.k_norm, T, c.num_attention_heads,
+                            c.num_key_value_heads, c.head_dim, c.rope_dims, c.rms_norm_eps, m->d_cos, m->d_sin,
+                            m->rope_npos, offset, cap, scale, q_rot, k_cache, v_cache, att);
 }
 
 static int forward_rows(ornith_model* m, ornith_caches* cc, const uint32_t* d_tokens, int T,

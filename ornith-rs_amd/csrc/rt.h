@@ -114,6 +114,7 @@ extern "C" int ornith_kq_matmul_multi(ornith_ctx* ctx, const ornith_kmatrix* con
 int ornith_option_gemm_reg();  // 1: expert-gathered prefill GEMM with the weights dequantized into MFMA operand registers; 0: through LDS
 int ornith_option_gdn_block_chunks();  // 64-token chunks a launch pair of the chunked gated-delta recurrence takes
 int ornith_option_gemm_duo();  // 1: prefill GEMM with producer and consumer wavefronts; 0: every wavefront does both in turn
+int ornith_option_fuse_attn_prep();  // 1: the attention launch does its own prep at decode widths
 int ornith_option_kq_iters();      // output rows per wavefront pass of the mat-vec kernels; 0 = by shape
 int ornith_option_moe_up_iters();  // rows per wavefront of the fused gate+up kernel; 0 = by shape
 int ornith_option_moe_down_iters();  // column groups per workgroup of the expert down kernel; 0 = by shape

@@ -50,7 +50,8 @@ Option g_options[] = {{"fuse_moe", "ORNITH_FUSE_MOE", 1, -1},
                       {"moe_down_iters", "ORNITH_MOE_DOWN_ITERS", 0, -1},
                       {"gdn_chunked", "ORNITH_GDN_CHUNKED", 1, -1},
                       {"gemm_reg", "ORNITH_GEMM_REG", 1, -1},
-                      {"gdn_block_chunks", "ORNITH_GDN_BLOCK_CHUNKS", 64, -1}};
+                      {"gdn_block_chunks", "ORNITH_GDN_BLOCK_CHUNKS", 64, -1},
+                      {"fuse_attn_prep", "ORNITH_FUSE_ATTN_PREP", 1, -1}};
 int option_value(int i) {
   Option& o = g_options[i];
   if (o.value < 0) {
@@ -73,6 +74,7 @@ int ornith_option_moe_down_iters() { return option_value(10); }
 int ornith_option_gdn_chunked() { return option_value(11); }
 int ornith_option_gemm_reg() { return option_value(12); }
 int ornith_option_gdn_block_chunks() { return option_value(13); }
+int ornith_option_fuse_attn_prep() { return option_value(14); }
 int ornith_option_ho_spins() { return option_value(9) < 1 ? 1 : option_value(9); }
 
 int ornith_check_handoffs(ornith_ctx* ctx) {

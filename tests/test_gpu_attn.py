@@ -20,6 +20,10 @@ def _mk(rng, T, Hq, Hkv, hd, cap, offset):
 
 @pytest.mark.parametrize("T,Hq,Hkv,hd,cap,offset", [
     (1, 16, 2, 256, 4096, 4000), (2, 16, 2, 256, 4096, 255), (4, 16, 2, 256, 4096, 1021),
+    # decode widths in short contexts (prep folded into the attention launch): first rows of a
+    # cache, new rows across the end of a key block, the widest folded call, head_dim 128
+    (1, 16, 2, 256, 4096, 0), (2, 16, 2, 256, 4096, 51), (4, 16, 2, 256, 4096, 254), (8, 16, 2, 256, 4096, 250),
+    (8, 16, 2, 256, 4096, 100), (3, 8, 2, 128, 1024, 255), (5, 4, 4, 256, 512, 300),
     (3, 4, 1, 256, 512, 0), (2, 4, 2, 128, 768, 300), (1, 2, 2, 256, 256, 7),
     # many live key blocks: the launch switches to its 256-thread form (same sums)
     (4, 16, 2, 256, 4096, 4000), (4, 16, 2, 128, 4096, 3000),
@@ -52,4 +56,13 @@ def test_attention_bit_exact(orn, ctx, T, Hq, Hkv, hd, cap, offset):
         ctx.sdpa_decode_gated(dq, dkc, dvc, d[0], T, Hq, Hkv, hd, 0 if use_dev_offset else offset, cap, hd ** -0.5, dout, d_offset=doff)
         assert np.array_equal(dout.download(np.uint16, want.shape), want), use_dev_offset
         if doff: doff.free()
+    # prep + attention as one call (one launch at decode widths in short contexts, a prep launch
+    # first otherwise; with the fold switched off it is always two): same output, same caches
+    for fold in (1, 0):
+        orn.set_option("fuse_attn_prep", fold)
+        dkc.upload(kc); dvc.upload(vc); dout.zero()
+        ctx.attn_decode(*d, T, Hq, Hkv, hd, rd, 1e-6, dc, ds, cap, offset, cap, hd ** -0.5, dq, dkc, dvc, dout)
+        assert np.array_equal(dout.download(np.uint16, want.shape), want), ("attn_decode", fold)
+        assert np.array_equal(dkc.download(np.uint16, kc.shape), wkc) and np.array_equal(dvc.download(np.uint16, vc.shape), wvc), fold
+    orn.set_option("fuse_attn_prep", 1)
     for b in d + [dkc, dvc, dq, dout, dc, ds]: b.free()
