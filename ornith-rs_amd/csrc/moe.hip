@@ -28,6 +28,10 @@ bool moe_one_launch(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_
 bool moe_affine4_supported(const ornith_moe_weights* w);
 int moe_affine4_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, const uint32_t* d_inds,
                         const void* d_scores, const void* d_egate, void* d_act, void* d_out, const void* d_gates);
+// ... and for dense bf16 experts (the MTP head's block)
+bool moe_dense_supported(const ornith_moe_weights* w);
+int moe_dense_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, const uint32_t* d_inds,
+                      const void* d_scores, const void* d_egate, void* d_act, void* d_out, const void* d_gates);
 int moe_fused_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T,
                       const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act,
                       void* d_out, int phases, const void* d_gates);
@@ -381,16 +385,20 @@ static int moe_block_impl(ornith_ctx* ctx, const ornith_moe_weights* w, const vo
                              ctx->stream));
     return ORNITH_OK;
   }
-  if (ornith_option_fuse_moe() && ex_affine4 && moe_affine4_supported(w)) {
-    // the published artifact's block in three launches: router + shared-expert gate (one launch
-    // when their formats match), then the two expert launches of moe_affine4.hip, the softmax +
-    // top-k in the head of the first where the expert count allows
+  const bool pair_a4 = ex_affine4 && moe_affine4_supported(w), pair_dense = w->ex_dense && moe_dense_supported(w);
+  if (ornith_option_fuse_moe() && (pair_a4 || pair_dense)) {
+    // the published artifact's block, and the MTP head's dense one, in three launches: router +
+    // shared-expert gate (one launch when their formats match), then the two expert launches of
+    // moe_affine4.hip, the softmax + top-k in the head of the first where the expert count allows
     const ornith_linear* in2[2] = {&w->router, &w->sh_egate};
     void* out2[2] = {gates, eg};
     TRY(ornith_linear_matmul_multi(ctx, in2, 2, d_x, T, out2));
     const bool topk_in_up = E % 64 == 0 && E <= 1024 && ((E / 64) & (E / 64 - 1)) == 0 && k <= 16;
     if (!topk_in_up) TRY(launch_router(ctx, gates, T, E, k, inds, scores, nullptr, nullptr, nullptr));
-    TRY(moe_affine4_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, topk_in_up ? gates : nullptr));
+    if (pair_a4)
+      TRY(moe_affine4_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, topk_in_up ? gates : nullptr));
+    else
+      TRY(moe_dense_experts(ctx, w, d_x, T, inds, scores, eg, act, d_out, topk_in_up ? gates : nullptr));
     if (d_inds_out)
       ORN_HIP(hipMemcpyAsync(d_inds_out, inds, 4 * (size_t)T * k, hipMemcpyDeviceToDevice, ctx->stream));
     if (d_scores_out)

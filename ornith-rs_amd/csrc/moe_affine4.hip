@@ -1,6 +1,8 @@
-// The expert half of the MoE block for the published artifact's format: routed and shared
-// experts in mlx 4-bit affine, group 32 (/root/reference/src/ops/quantized.rs:311-333,531-589;
-// the operator path: moe.hip). Two launches that mirror moe_up_kernel / moe_down_kernel
+// The expert half of the MoE block for the two formats whose row dot is one wavefront a row:
+// the published artifact's (routed and shared experts in mlx 4-bit affine, group 32,
+// /root/reference/src/ops/quantized.rs:311-333,531-589) and the MTP head's (dense bf16 experts,
+// /root/reference/src/model/mtp.rs, gather_mm over [E, O, K] tensors). The operator path is
+// moe.hip. Two launches that mirror moe_up_kernel / moe_down_kernel
 // (moe_fused.hip) in place of five (two gathered mat-vecs, swiglu, the shared expert's down
 // projection, the gathered down projection, the combine):
 //
@@ -12,11 +14,13 @@
 //                   block's tail (router weights, bf16 accumulation in slot order, sigmoid-gated
 //                   shared expert).
 //
-// A row dot is affine4_qmv_kernel's (linear.hip), operation for operation: lane l owns the
+// A 4-bit row dot is affine4_qmv_kernel's (linear.hip), operation for operation: lane l owns the
 // 16-code chunks l + 64c in ascending c, one fma chain a chunk in code order beside the plain
 // sum of its activations, scale * chain + bias * sum per chunk added to the lane's running
-// value, then the 64-lane butterfly. So the two launches give the bits of the operator path
-// and of the oracle (oracle/orc_moe.c).
+// value, then the 64-lane butterfly; a dense one is dense_row_dot (linear_device.h), the
+// function the operator path's kernels call. So the two launches give the bits of the operator
+// path and of the oracle (oracle/orc_moe.c).
+#include "linear_device.h"
 #include "moe_device.h"
 #include "rt.h"
 
@@ -64,9 +68,67 @@ __device__ __forceinline__ float a4_chunk(const A4Mat& m, size_t row, int K, int
   return dm_fma(x.sum, b, p);
 }
 
+// The two formats behind one pair of kernels: a matrix handle, the gate and up rows' dots over
+// one activation row, and NC rows' dots of one matrix.
+struct FmtA4 {
+  using Mat = A4Mat;
+  static __device__ __forceinline__ void dot2(const Mat& wg, const Mat& wu, size_t row, int K, const bf16_t* xr,
+                                              int lane, float& g, float& u) {
+    float ag = 0.f, au = 0.f;
+    for (int j = lane; j < K / 16; j += 64) {
+      A4X x;
+      x.load(xr, j);
+      ag = ag + a4_chunk(wg, row, K, j, x);
+      au = au + a4_chunk(wu, row, K, j, x);
+    }
+    g = dm_wave_sum<64>(ag);
+    u = dm_wave_sum<64>(au);
+  }
+  template <int NC>
+  static __device__ __forceinline__ void dotn(const Mat& w, size_t row0, int c0, int O, int K, const bf16_t* xr,
+                                              int lane, float (&v)[NC]) {
+    float acc[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc[c] = 0.f;
+    for (int jj = lane; jj < K / 16; jj += 64) {
+      A4X x;
+      x.load(xr, jj);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int o = c0 + c < O ? c0 + c : O - 1;
+        acc[c] = acc[c] + a4_chunk(w, row0 + o, K, jj, x);
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) v[c] = dm_wave_sum<64>(acc[c]);
+  }
+};
+
+struct DenseMat {
+  const bf16_t* w;  // [rows, K]
+};
+struct FmtDense {
+  using Mat = DenseMat;
+  static __device__ __forceinline__ void dot2(const Mat& wg, const Mat& wu, size_t row, int K, const bf16_t* xr,
+                                              int lane, float& g, float& u) {
+    g = dense_row_dot(wg.w + row * K, xr, K, lane);
+    u = dense_row_dot(wu.w + row * K, xr, K, lane);
+  }
+  template <int NC>
+  static __device__ __forceinline__ void dotn(const Mat& w, size_t row0, int c0, int O, int K, const bf16_t* xr,
+                                              int lane, float (&v)[NC]) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int o = c0 + c < O ? c0 + c : O - 1;
+      v[c] = dense_row_dot(w.w + (row0 + o) * K, xr, K, lane);
+    }
+  }
+};
+
+template <class F>
 struct A4UpArgs {
-  A4Mat gate, up;        // routed [E * I, K]
-  A4Mat sgate, sup;      // shared [I, K]
+  typename F::Mat gate, up;    // routed [E * I, K]
+  typename F::Mat sgate, sup;  // shared [I, K]
   const bf16_t* x;       // [T, K]
   const uint32_t* inds;  // [T*k], read unless gates is given
   bf16_t* act;           // [T*k + T, I]
@@ -77,13 +139,13 @@ struct A4UpArgs {
 };
 
 // grid (ceil(I / 4), T*k + T), 256 threads: a wavefront an output row
-template <bool ROUTE>
-__global__ __launch_bounds__(256) void moe_up_affine4_kernel(A4UpArgs a) {
+template <class F, bool ROUTE>
+__global__ __launch_bounds__(256) void moe_up_affine4_kernel(A4UpArgs<F> a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = blockIdx.y, routed = a.T * a.k;
   int token;
   size_t row0;
-  A4Mat wg, wu;
+  typename F::Mat wg, wu;
   if (r < routed) {
     token = r / a.k;
     uint32_t e;
@@ -121,20 +183,15 @@ __global__ __launch_bounds__(256) void moe_up_affine4_kernel(A4UpArgs a) {
   const int o = blockIdx.x * 4 + wave;
   if (o >= a.I) return;
   const bf16_t* xr = a.x + (size_t)token * a.K;
-  float ag = 0.f, au = 0.f;
-  for (int j = lane; j < a.K / 16; j += 64) {
-    A4X x;
-    x.load(xr, j);
-    ag = ag + a4_chunk(wg, row0 + o, a.K, j, x);
-    au = au + a4_chunk(wu, row0 + o, a.K, j, x);
-  }
-  const float g = dm_wave_sum<64>(ag), u = dm_wave_sum<64>(au);
+  float g, u;
+  F::dot2(wg, wu, row0 + o, a.K, xr, lane, g, u);
   if (lane == 0) a.act[(size_t)r * a.I + o] = swiglu_bf16(g, u);
 }
 
+template <class F>
 struct A4DownArgs {
-  A4Mat down;            // routed [E * H, I]
-  A4Mat sdown;           // shared [H, I]
+  typename F::Mat down;   // routed [E * H, I]
+  typename F::Mat sdown;  // shared [H, I]
   const bf16_t* act;     // [T*k + T, I]
   const uint32_t* inds;  // [T*k]
   const bf16_t* scores;  // [T*k]
@@ -146,7 +203,8 @@ struct A4DownArgs {
 constexpr int kA4Cols = 8;
 
 // grid (ceil(H / 8), T), 64 * (k + 1) threads
-__global__ __launch_bounds__(64 * (kA4MaxK + 1)) void moe_down_affine4_kernel(A4DownArgs a) {
+template <class F>
+__global__ __launch_bounds__(64 * (kA4MaxK + 1)) void moe_down_affine4_kernel(A4DownArgs<F> a) {
   const int lane = threadIdx.x & 63, j = threadIdx.x >> 6;  // j: expert slot, k = shared
   const int t = blockIdx.y, k = a.k, c0 = blockIdx.x * kA4Cols;
   __shared__ float yl[kA4MaxK + 1][kA4Cols];
@@ -154,7 +212,7 @@ __global__ __launch_bounds__(64 * (kA4MaxK + 1)) void moe_down_affine4_kernel(A4
   __shared__ float gsig;
   const bool shared = j == k;
   const int arow = shared ? a.T * k + t : t * k + j;
-  const A4Mat w = shared ? a.sdown : a.down;
+  const typename F::Mat w = shared ? a.sdown : a.down;
   const size_t row0 = shared ? 0 : (size_t)min(a.inds[t * k + j], (uint32_t)(a.E - 1)) * a.H;
   if (j == 0) {
     // the router weights of this token: denom = ((0+s0)+s1)..., w_j = bf16(s_j / denom)
@@ -166,23 +224,11 @@ __global__ __launch_bounds__(64 * (kA4MaxK + 1)) void moe_down_affine4_kernel(A4
     if (lane == 0) gsig = dm_sigmoid_bf16(dm_bf2f(a.egate[t]));
   }
   const bf16_t* xr = a.act + (size_t)arow * a.I;
-  float acc[kA4Cols];
+  float v[kA4Cols];
+  F::template dotn<kA4Cols>(w, row0, c0, a.H, a.I, xr, lane, v);
 #pragma unroll
-  for (int c = 0; c < kA4Cols; ++c) acc[c] = 0.f;
-  for (int jj = lane; jj < a.I / 16; jj += 64) {
-    A4X x;
-    x.load(xr, jj);
-#pragma unroll
-    for (int c = 0; c < kA4Cols; ++c) {
-      const int o = c0 + c < a.H ? c0 + c : a.H - 1;
-      acc[c] = acc[c] + a4_chunk(w, row0 + o, a.I, jj, x);
-    }
-  }
-#pragma unroll
-  for (int c = 0; c < kA4Cols; ++c) {
-    const float v = dm_wave_sum<64>(acc[c]);
-    if (lane == 0) yl[j][c] = dm_rb(v);  // expert outputs are bf16 in the operator path
-  }
+  for (int c = 0; c < kA4Cols; ++c)
+    if (lane == 0) yl[j][c] = dm_rb(v[c]);  // expert outputs are bf16 in the operator path
   __syncthreads();
   const int col = threadIdx.x;
   if (col < kA4Cols && c0 + col < a.H) {
@@ -220,16 +266,18 @@ bool moe_affine4_supported(const ornith_moe_weights* w) {
   return w->ex_gate.K % 32 == 0 && w->ex_gate.O % 32 == 0;
 }
 
-// act: scratch bf16 [(T*k + T), I]. With d_gates the up launch makes the routing and stores it
-// to d_inds / d_scores (which then are outputs).
-int moe_affine4_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, const uint32_t* d_inds,
-                        const void* d_scores, const void* d_egate, void* d_act, void* d_out, const void* d_gates) {
-  const int E = w->router.O, H = w->router.K, I = w->ex_gate.O, k = w->top_k;
-  A4UpArgs u{};
-  u.gate = mat_of(w->ex_gate);
-  u.up = mat_of(w->ex_up);
-  u.sgate = mat_of(w->sh_gate);
-  u.sup = mat_of(w->sh_up);
+namespace {
+
+template <class F>
+int launch_pair(ornith_ctx* ctx, const ornith_moe_weights* w, const typename F::Mat (&m)[6], const void* d_x, int T,
+                const uint32_t* d_inds, const void* d_scores, const void* d_egate, void* d_act, void* d_out,
+                const void* d_gates) {
+  const int E = w->router.O, H = w->router.K, I = w->sh_gate.O, k = w->top_k;
+  A4UpArgs<F> u{};
+  u.gate = m[0];
+  u.up = m[1];
+  u.sgate = m[2];
+  u.sup = m[3];
   u.x = (const bf16_t*)d_x;
   u.inds = d_inds;
   u.act = (bf16_t*)d_act;
@@ -243,13 +291,13 @@ int moe_affine4_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void
   u.scores_out = (bf16_t*)const_cast<void*>(d_scores);
   const dim3 ugrid((I + 3) / 4, T * k + T);
   if (d_gates)
-    hipLaunchKernelGGL(moe_up_affine4_kernel<true>, ugrid, dim3(256), 0, ctx->stream, u);
+    hipLaunchKernelGGL((moe_up_affine4_kernel<F, true>), ugrid, dim3(256), 0, ctx->stream, u);
   else
-    hipLaunchKernelGGL(moe_up_affine4_kernel<false>, ugrid, dim3(256), 0, ctx->stream, u);
+    hipLaunchKernelGGL((moe_up_affine4_kernel<F, false>), ugrid, dim3(256), 0, ctx->stream, u);
   ORN_LAUNCH_CHECK("moe_up_affine4_kernel");
-  A4DownArgs d{};
-  d.down = mat_of(w->ex_down);
-  d.sdown = mat_of(w->sh_down);
+  A4DownArgs<F> d{};
+  d.down = m[4];
+  d.sdown = m[5];
   d.act = (const bf16_t*)d_act;
   d.inds = d_inds;
   d.scores = (const bf16_t*)d_scores;
@@ -261,7 +309,40 @@ int moe_affine4_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void
   d.H = H;
   d.I = I;
   d.normalize = w->norm_topk_prob;
-  hipLaunchKernelGGL(moe_down_affine4_kernel, dim3((H + kA4Cols - 1) / kA4Cols, T), dim3(64 * (k + 1)), 0, ctx->stream, d);
+  hipLaunchKernelGGL(moe_down_affine4_kernel<F>, dim3((H + kA4Cols - 1) / kA4Cols, T), dim3(64 * (k + 1)), 0,
+                     ctx->stream, d);
   ORN_LAUNCH_CHECK("moe_down_affine4_kernel");
   return ORNITH_OK;
+}
+
+}  // namespace
+
+// act: scratch bf16 [(T*k + T), I]. With d_gates the up launch makes the routing and stores it
+// to d_inds / d_scores (which then are outputs).
+int moe_affine4_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, const uint32_t* d_inds,
+                        const void* d_scores, const void* d_egate, void* d_act, void* d_out, const void* d_gates) {
+  const A4Mat m[6] = {mat_of(w->ex_gate), mat_of(w->ex_up), mat_of(w->sh_gate),
+                      mat_of(w->sh_up),   mat_of(w->ex_down), mat_of(w->sh_down)};
+  return launch_pair<FmtA4>(ctx, w, m, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, d_gates);
+}
+
+// The same two launches for dense bf16 experts (the MTP head's block): routed tensors [E, O, K]
+// and dense shared-expert linears.
+bool moe_dense_supported(const ornith_moe_weights* w) {
+  if (!w->ex_dense || !w->d_ex_gate || !w->d_ex_up || !w->d_ex_down) return false;
+  const ornith_linear* sh[3] = {&w->sh_gate, &w->sh_up, &w->sh_down};
+  for (auto* l : sh)
+    if (l->mode != ORNITH_LIN_DENSE || !l->d_w) return false;
+  if (w->sh_up.O != w->sh_gate.O || w->sh_down.K != w->sh_gate.O || w->sh_gate.K != w->router.K ||
+      w->sh_down.O != w->router.K)
+    return false;
+  if (w->top_k < 1 || w->top_k > kA4MaxK) return false;
+  return w->router.K % 8 == 0 && w->sh_gate.O % 8 == 0;
+}
+
+int moe_dense_experts(ornith_ctx* ctx, const ornith_moe_weights* w, const void* d_x, int T, const uint32_t* d_inds,
+                      const void* d_scores, const void* d_egate, void* d_act, void* d_out, const void* d_gates) {
+  const DenseMat m[6] = {{(const bf16_t*)w->d_ex_gate}, {(const bf16_t*)w->d_ex_up},   {(const bf16_t*)w->sh_gate.d_w},
+                         {(const bf16_t*)w->sh_up.d_w}, {(const bf16_t*)w->d_ex_down}, {(const bf16_t*)w->sh_down.d_w}};
+  return launch_pair<FmtDense>(ctx, w, m, d_x, T, d_inds, d_scores, d_egate, d_act, d_out, d_gates);
 }

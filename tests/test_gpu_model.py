@@ -78,18 +78,23 @@ def test_batch_invariance_chunking_does_not_matter(orn, ctx, tiny):
 
 def test_mtp_head_forward_bit_exact(orn, ctx, tiny):
     s, ws, model = tiny
-    rng = np.random.default_rng(2)
-    head = orn.MtpHead(model, ws, 64)
-    orc = synth.OracleRun(s, 64)
-    hid = util.bf16_normal(rng, (3, s.cfg["hidden_size"]))
-    ids = rng.integers(0, s.cfg["vocab_size"], 3).astype(np.uint32)
-    lg, h1 = head.forward(hid[:1], ids[:1])
-    w1 = orc.mtp_hidden(hid[:1], ids[:1])
-    assert np.array_equal(h1, w1) and np.array_equal(lg, orc.logits(w1))
-    _, h2 = head.forward(hid[1:], ids[1:], want_logits=False)   # two rows at once, cache offset 1
-    assert np.array_equal(h2, orc.mtp_hidden(hid[1:], ids[1:]))
-    assert head.offset == 3
-    head.close(); orc.close()
+    # the head's dense-expert MoE block as two fused expert launches (fuse_moe 1) and as one
+    # launch per operator (0): both the oracle's bits
+    for fuse in (1, 0):
+        orn.set_option("fuse_moe", fuse)
+        rng = np.random.default_rng(2)
+        head = orn.MtpHead(model, ws, 64)
+        orc = synth.OracleRun(s, 64)
+        hid = util.bf16_normal(rng, (3, s.cfg["hidden_size"]))
+        ids = rng.integers(0, s.cfg["vocab_size"], 3).astype(np.uint32)
+        lg, h1 = head.forward(hid[:1], ids[:1])
+        w1 = orc.mtp_hidden(hid[:1], ids[:1])
+        assert np.array_equal(h1, w1) and np.array_equal(lg, orc.logits(w1)), fuse
+        _, h2 = head.forward(hid[1:], ids[1:], want_logits=False)   # two rows at once, cache offset 1
+        assert np.array_equal(h2, orc.mtp_hidden(hid[1:], ids[1:])), fuse
+        assert head.offset == 3
+        head.close(); orc.close()
+    orn.set_option("fuse_moe", 1)
 
 
 def test_frspec_prune_map_and_file_format(orn, ctx, tiny, tmp_path):
