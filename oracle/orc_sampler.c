@@ -150,6 +150,7 @@ static void scan_row(const float* in, int n, int bf16, float* out, float* total_
 }
 
 ORC_API void orc_cumsum_bf16(const bf16_t* x, int n, bf16_t* out) {
+  if (n <= 0) return;
   float* f = (float*)malloc(sizeof(float) * (size_t)n * 2);
   for (int i = 0; i < n; ++i) f[i] = orc_bf16_to_f32(x[i]);
   scan_row(f, n, 1, f + n, NULL);
