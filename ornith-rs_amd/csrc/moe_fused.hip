@@ -212,13 +212,22 @@ constexpr int kMaxK = 8;
 // The leading flat arguments repeat what a routed wavefront needs for its first weight request
 // (the library is built with kernel-argument preloading: they are in scalar registers when the
 // wavefront starts, while the argument block is still being fetched).
+//
+// Wavefront j < k takes routed expert j over the workgroup's ITERS column groups. At ITERS = 4
+// the shared expert's column groups go one each to wavefronts k .. k + 3, so that the compute
+// unit's four SIMDs (wavefronts go round them in order) carry 9 / 9 / 9 / 9 row passes instead of
+// 12 / 8 / 8 / 8 with a single shared wavefront (the passes are what is left to do when the rows
+// arrive: 1.1 us of a 29.5 us block at T = 4); at ITERS = 2 the same split (5 / 5 / 4 / 4 against
+// 6 / 4 / 4 / 4) measured no better, so there one wavefront k takes both groups.
+template <int ITERS>
+constexpr int down_shared_waves() { return ITERS >= 4 ? ITERS : 1; }
 template <int KIND, int LPR, int ITERS>
-__global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(const uint8_t* h_qs, const uint8_t* h_scales,
-                                                                    const uint16_t* h_dm, const uint32_t* h_inds,
-                                                                    int h_k, int h_E, int h_H, int h_I, DownArgs a) {
+__global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe_down_kernel(const uint8_t* h_qs, const uint8_t* h_scales,
+                                                                        const uint16_t* h_dm, const uint32_t* h_inds,
+                                                                        int h_k, int h_E, int h_H, int h_I, DownArgs a) {
   using KL = KqLane<KIND, 1>;
   constexpr int RPW = 64 / LPR, COLS = RPW * ITERS;
-  const int lane = threadIdx.x & 63, j = threadIdx.x >> 6;  // j: expert slot, k = shared
+  const int lane = threadIdx.x & 63, j = threadIdx.x >> 6;  // j < k: expert slot; j >= k: the shared expert's group j - k
   const int slot = lane / LPR, c = lane % LPR;
   const int nb = h_I >> 8;
   const int t = blockIdx.y, k = h_k;
@@ -229,7 +238,9 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(const uint8_
   __shared__ float wj[kMaxK];
   __shared__ float gsig;
 
-  const bool shared = j == k;
+  constexpr bool SPLIT = down_shared_waves<ITERS>() > 1;
+  const bool shared = SPLIT ? j >= k : j == k;
+  const int only = j - k;  // SPLIT: the one column group a shared-expert wavefront takes
   const int arow = shared ? a.T * k + t : t * k + j;
   const KqPtr w = shared ? a.sdown : KqPtr{h_qs, h_scales, h_dm};
   const int64_t row0 = shared ? 0 : (int64_t)min(h_inds[t * k + j], (uint32_t)(h_E - 1)) * h_H;
@@ -238,6 +249,7 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(const uint8_
   typename KL::Row rr[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
+    if (SPLIT && shared && it != only) continue;
     const int o = c0 + it * RPW + slot;
     rr[it] = KL::load(w.qs, w.scales, w.dm, row0 + (o < h_H ? o : h_H - 1), nb, L);
   }
@@ -258,10 +270,11 @@ __global__ __launch_bounds__(64 * (kMaxK + 1)) void moe_down_kernel(const uint8_
   }
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
+    if (SPLIT && shared && it != only) continue;
     float acc[1] = {0.f};
     ORN_KL_ACC(rr[it], L, acc);
     const float v = dm_wave_sum<LPR>(acc[0]);
-    if (c == 0) yl[j][it * RPW + slot] = dm_rb(v);  // expert outputs are bf16 in the unfused path
+    if (c == 0) yl[SPLIT && shared ? k : j][it * RPW + slot] = dm_rb(v);  // expert outputs are bf16 in the unfused path
   }
   DOWN_MARK(3);
   __syncthreads();
@@ -739,7 +752,6 @@ void launch_up(ornith_ctx* ctx, const UpArgs& a, int rows_y) {
 template <int KIND, int LPR>
 void launch_down(ornith_ctx* ctx, const DownArgs& a) {
   constexpr int RPW = 64 / LPR;
-  dim3 block(64 * (a.k + 1));
   const long groups1 = (long)(a.H + RPW - 1) / RPW * a.T;
   const int forced = ornith_option_moe_down_iters();
   // About one workgroup (k + 1 wavefronts) per compute unit is the fastest shape at every verify
@@ -747,6 +759,8 @@ void launch_down(ornith_ctx* ctx, const DownArgs& a) {
   // 9.0 / 6.8 / 9.2, T = 3: 12.6 / 11.4 / 10.0, T = 4: 16.2 / 12.1 / 10.9
   const long cu = ctx->compute_units;
   const int iters = forced ? forced : groups1 >= 3 * cu ? 4 : groups1 >= 2 * cu ? 2 : 1;
+  // k routed wavefronts and the shared expert's (one, or one a column group at four groups)
+  const dim3 block(64 * (a.k + (iters >= 4 ? 4 : 1)));
   if (iters >= 4) {
     dim3 grid((a.H + RPW * 4 - 1) / (RPW * 4), a.T);
     hipLaunchKernelGGL((moe_down_kernel<KIND, LPR, 4>), grid, block, 0, ctx->stream, a.down.qs, a.down.scales,
