@@ -442,9 +442,10 @@ int kq_qmv_multi_prenorm(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n
                          const void* d_y, const void* d_wnorm, float eps, int M, void* d_h_out,
                          void* d_normed_out, void* const* d_ys) {
   if (n < 1 || n > kMaxSeg || M < 1 || M > 4 || ws[0]->K != kPreN) return -1;
-  // Q6_K lanes hold 64 activations per row in registers; with the norm's own registers on top
-  // the M >= 2 kernels lose their occupancy and measured slower than a separate norm launch
-  if (ws[0]->kind == ORNITH_Q6K && M > 1) return -1;
+  // (Q6_K lanes hold 64 activations a row in registers, and the M >= 2 kernels once lost their
+  // occupancy to the norm's own registers on top; they no longer do -- the prologue's registers
+  // are dead before the row loop's peak -- and the launch saved is worth 0.4 % at depth 1 and 1.7 %
+  // at depth 3 in same-box A/B runs, so every width takes the norm in its head now.)
   long total = 0;
   for (int s = 0; s < n; ++s) {
     if (check_matrix(ws[s], "kq_qmv_prenorm")) return -1;
