@@ -500,8 +500,11 @@ struct StepArgs {
 // debug build only: per-workgroup phase time stamps (100 MHz wall clock) of the last launch
 __device__ long long g_gdn_marks[64][8];
 #define GDN_MARK(i) do { if (threadIdx.x == 0 && blockIdx.x < 64) g_gdn_marks[blockIdx.x][i] = wall_clock64(); } while (0)
+// by lane 0 of wavefront w
+#define GDN_MARK_W(i, w) do { if ((int)threadIdx.x == 64 * (w) && blockIdx.x < 64) g_gdn_marks[blockIdx.x][i] = wall_clock64(); } while (0)
 #else
 #define GDN_MARK(i)
+#define GDN_MARK_W(i, w)
 #endif
 
 __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
@@ -517,14 +520,42 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
   const int row = lane >> 3, j = lane & 7, dv = wave * 8 + row;
   const size_t ssz = (size_t)p.Hv * 128 * 128;
   const size_t roff = ((size_t)hv * 128 + dv) * 128 + 4 * j;
-  float s[16];
+  // Loads return in issue order, and the state is 64 KB a workgroup straight from memory: asked
+  // for first, it would hold back the few cached operands of the front-end tasks until it had
+  // arrived, and the front end (conv, norms, projections: 1 - 2 us of dependent arithmetic)
+  // would only start then. So a wavefront asks for its first task's operands first, then for
+  // what the later phases need, then for its state, and works its task off under the state's
+  // trip.
+  const int n_conv = 3 * T, n_ab = a.wa ? 2 * T : 0;
+  const bool early_conv = wave < n_conv && p.K == 4;
+  const bool early_ab = wave >= n_conv && wave < n_conv + n_ab && a.H <= 2048;
+  uint4 e_w8 = make_uint4(0, 0, 0, 0);
+  uint32_t e_xv[4] = {0, 0, 0, 0};
+  uint4 e_dw[4], e_dx[4];
+  if (early_conv) {
+    const int which = wave / T, t = wave - which * T;
+    const int slot = which == 0 ? hk : which == 1 ? p.Hk + hk : 2 * p.Hk + hv;
+    const int c0 = slot * 128 + 2 * lane;
+    e_w8 = *reinterpret_cast<const uint4*>(p.cw + (size_t)c0 * 4);
 #pragma unroll
-  for (int m = 0; m < 4; ++m) {
-    const float4 f = *reinterpret_cast<const float4*>(a.state_in + roff + 32 * m);
-    s[4 * m + 0] = f.x;
-    s[4 * m + 1] = f.y;
-    s[4 * m + 2] = f.z;
-    s[4 * m + 3] = f.w;
+    for (int i = 0; i < 4; ++i) {
+      const int jj = t + i;
+      const bf16_t* src = (jj < S) ? (p.conv_state + (size_t)jj * D) : (p.qkv + (size_t)(jj - S) * D);
+      e_xv[i] = *reinterpret_cast<const uint32_t*>(src + c0);
+    }
+  }
+  if (early_ab) {
+    const int u = wave - n_conv, which = u / T, t = u - which * T;
+    const bf16_t* wr = (which == 0 ? a.wa : a.wb) + (size_t)hv * a.H;
+    const bf16_t* xr = a.xn + (size_t)t * a.H;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int jc = lane + 64 * c;
+      if (jc < a.H / 8) {
+        e_dw[c] = *reinterpret_cast<const uint4*>(wr + 8 * jc);
+        e_dx[c] = *reinterpret_cast<const uint4*>(xr + 8 * jc);
+      }
+    }
   }
   // operands of the later phases that depend on nothing computed here: requested now, so that
   // no phase starts with a trip to memory of its own
@@ -540,10 +571,20 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     bin_pre = p.b_in[tid * p.Hv + hv];
   }
   __builtin_amdgcn_sched_barrier(0);
+  float s[16];
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {
+    const float4 f = *reinterpret_cast<const float4*>(a.state_in + roff + 32 * m);
+    s[4 * m + 0] = f.x;
+    s[4 * m + 1] = f.y;
+    s[4 * m + 2] = f.z;
+    s[4 * m + 3] = f.w;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  GDN_MARK(4);  // every request of this wavefront is out
   const float decay_pre = dm_exp(dm_bf2f(alog_pre));  // needs only a parameter: made under the loads
 
   // 2. front-end tasks: [0, 3T) conv of (q | k | v, token); then the a / b projections
-  const int n_conv = 3 * T, n_ab = a.wa ? 2 * T : 0;
   for (int task = wave; task < n_conv + n_ab; task += 16) {
     if (task < n_conv) {
       const int which = task / T, t = task - which * T;  // 0 q, 1 k, 2 v
@@ -553,13 +594,16 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
       if (p.K == 4) {
         // the usual window: the four taps of both channels are one 16-byte load, and the four
         // input rows are requested together
-        const uint4 w8 = *reinterpret_cast<const uint4*>(p.cw + (size_t)c0 * 4);
-        uint32_t xv[4];
+        uint4 w8 = e_w8;
+        uint32_t xv[4] = {e_xv[0], e_xv[1], e_xv[2], e_xv[3]};
+        if (task != wave) {  // a second task of this wavefront (more than 16 tasks): asked for here
+          w8 = *reinterpret_cast<const uint4*>(p.cw + (size_t)c0 * 4);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int jj = t + i;
-          const bf16_t* src = (jj < S) ? (p.conv_state + (size_t)jj * D) : (p.qkv + (size_t)(jj - S) * D);
-          xv[i] = *reinterpret_cast<const uint32_t*>(src + c0);
+          for (int i = 0; i < 4; ++i) {
+            const int jj = t + i;
+            const bf16_t* src = (jj < S) ? (p.conv_state + (size_t)jj * D) : (p.qkv + (size_t)(jj - S) * D);
+            xv[i] = *reinterpret_cast<const uint32_t*>(src + c0);
+          }
         }
         acc0 = dm_fma(dm_bf2f_lo(xv[0]), dm_bf2f_lo(w8.x), acc0);
         acc0 = dm_fma(dm_bf2f_lo(xv[1]), dm_bf2f_hi(w8.x), acc0);
@@ -604,7 +648,28 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
     } else {
       const int u = task - n_conv, which = u / T, t = u - which * T;  // 0 a, 1 b
       const bf16_t* wr = (which == 0 ? a.wa : a.wb) + (size_t)hv * a.H;
-      const float v = dm_rb(dense_row_dot(wr, a.xn + (size_t)t * a.H, a.H, lane));
+      float v;
+      if (task == wave && early_ab) {
+        // dense_row_dot over the operands asked for at the start: the same chain, the same fold
+        float acc = 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+          if (lane + 64 * c < a.H / 8) {
+            const uint4 wv4 = e_dw[c], xv4 = e_dx[c];
+            acc = dm_fma(dm_bf2f_lo(wv4.x), dm_bf2f_lo(xv4.x), acc);
+            acc = dm_fma(dm_bf2f_hi(wv4.x), dm_bf2f_hi(xv4.x), acc);
+            acc = dm_fma(dm_bf2f_lo(wv4.y), dm_bf2f_lo(xv4.y), acc);
+            acc = dm_fma(dm_bf2f_hi(wv4.y), dm_bf2f_hi(xv4.y), acc);
+            acc = dm_fma(dm_bf2f_lo(wv4.z), dm_bf2f_lo(xv4.z), acc);
+            acc = dm_fma(dm_bf2f_hi(wv4.z), dm_bf2f_hi(xv4.z), acc);
+            acc = dm_fma(dm_bf2f_lo(wv4.w), dm_bf2f_lo(xv4.w), acc);
+            acc = dm_fma(dm_bf2f_hi(wv4.w), dm_bf2f_hi(xv4.w), acc);
+          }
+        }
+        v = dm_rb(dm_wave_sum<64>(acc));
+      } else {
+        v = dm_rb(dense_row_dot(wr, a.xn + (size_t)t * a.H, a.H, lane));
+      }
       // the wavefront that made the projection turns it into the token's decay / beta at
       // once: the two chains of exp / log run side by side in different wavefronts instead of
       // one after the other behind a barrier
@@ -618,6 +683,8 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
       }
     }
   }
+  GDN_MARK_W(7, 0);       // the first conv task's wavefront is through
+  GDN_MARK_W(6, n_conv);  // the first a / b projection's wavefront is through
   if (!a.wa && tid < T) {
     // projections given: decay and beta of token `tid`
     const float sp = softplus_bf16(dm_rb(dm_bf2f(ain_pre) + dm_bf2f(dtb_pre)));
