@@ -246,6 +246,13 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
   const int64_t row0 = shared ? 0 : (int64_t)min(h_inds[t * k + j], (uint32_t)(h_E - 1)) * h_H;
   typename KL::Lane L;
   L.set_chunk(c);
+  // the activation row first: it is a kilobyte the up launch has just written, back long before
+  // the weights, and its conversion then runs under the weights' trip (loads return in issue
+  // order: asked for behind the weights it was converted only after the last of them had arrived;
+  // 0.5 us a pair at T = 2)
+  const void* xrow[1] = {a.act + (size_t)arow * a.I};
+  L.template load_x<false>(xrow, c);
+  __builtin_amdgcn_sched_barrier(0);
   typename KL::Row rr[ITERS];
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
@@ -253,10 +260,8 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
     const int o = c0 + it * RPW + slot;
     rr[it] = KL::load(w.qs, w.scales, w.dm, row0 + (o < h_H ? o : h_H - 1), nb, L);
   }
-  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of the activation loads
+  __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of everything that follows
   DOWN_MARK(1);
-  const void* xrow[1] = {a.act + (size_t)arow * a.I};
-  L.template load_x<false>(xrow, c);
   DOWN_MARK(2);
 
   if (j == 0) {
