@@ -153,8 +153,8 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
 
   // Rows kept in flight per wavefront. Cold weights come from HBM with a latency many
   // times the arithmetic of one row, so every wavefront issues the loads of its first PF
-  // rows before anything else (they depend on nothing), then its activations, and
-  // refills a slot as soon as that row's registers are consumed.
+  // rows at once (they depend on nothing), behind only the few cached operands named
+  // below, and refills a slot as soon as that row's registers are consumed.
   constexpr int PF = (KIND == ORNITH_Q4K) ? (M <= 2 ? 4 : 2) : (M <= 2 ? 2 : 1);
   typename KL::Lane L;
   L.set_chunk(c + 64 * ks);
@@ -175,6 +175,12 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
     prenorm_issue<M>(a.pre, pg);
     __builtin_amdgcn_sched_barrier(0);
   }
+  // activations from memory go first: loads return in issue order, so behind the weight rows the
+  // (cached) activation rows and their conversion would wait for the last weight byte
+  if constexpr (!PRE) {
+    L.template load_x<XF32>(xrow, c + 64 * ks);
+    __builtin_amdgcn_sched_barrier(0);
+  }
   typename KL::Row pf[PF];
 #pragma unroll
   for (int i = 0; i < PF; ++i) pf[i] = KL::load(sg.qs, sg.scales, sg.dm, row_of(i), nb, L);
@@ -187,7 +193,7 @@ __global__ __launch_bounds__(256) void kq_qmv_kernel(KqArgs a) {
     for (int t = 0; t < M; ++t) xrow[t] = &pn.xn[t][0];
   }
   ORN_MARK(2);
-  L.template load_x<XF32>(xrow, c + 64 * ks);
+  if constexpr (PRE) L.template load_x<XF32>(xrow, c + 64 * ks);  // from the normed rows in LDS
   ORN_MARK(3);
 
   for (int it0 = 0; it0 < a.iters; it0 += PF) {
