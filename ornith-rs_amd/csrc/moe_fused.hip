@@ -252,6 +252,10 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
   // 0.5 us a pair at T = 2)
   const void* xrow[1] = {a.act + (size_t)arow * a.I};
   L.template load_x<false>(xrow, c);
+  // likewise the token's router scores (lane i < k holds score i) and its shared-expert gate:
+  // wavefront 0 turns them into the combine weights while its weight rows are on their way
+  const uint16_t score_bits = a.scores[(size_t)t * k + (lane < k ? lane : 0)];
+  const uint16_t egate_bits = a.egate[t];
   __builtin_amdgcn_sched_barrier(0);
   typename KL::Row rr[ITERS];
 #pragma unroll
@@ -266,12 +270,14 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
 
   if (j == 0) {
     // the router weights of this token: denom = ((0+s0)+s1)..., w_j = bf16(s_j / denom)
-    const bf16_t* s = a.scores + (size_t)t * k;
     float denom = 0.f;
-    if (a.normalize)
-      for (int i = 0; i < k; ++i) denom = dm_rb(dm_bf2f(s[i]) + denom);
-    if (lane < k) wj[lane] = a.normalize ? dm_rb(dm_bf2f(s[lane]) / denom) : dm_bf2f(s[lane]);
-    if (lane == 0) gsig = dm_sigmoid_bf16(dm_bf2f(a.egate[t]));
+    if (a.normalize) {
+#pragma unroll
+      for (int i = 0; i < kMaxK; ++i)
+        if (i < k) denom = dm_rb(dm_bf2f((bf16_t)__builtin_amdgcn_readlane((int)score_bits, i)) + denom);
+    }
+    if (lane < k) wj[lane] = a.normalize ? dm_rb(dm_bf2f(score_bits) / denom) : dm_bf2f(score_bits);
+    if (lane == 0) gsig = dm_sigmoid_bf16(dm_bf2f(egate_bits));
   }
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
