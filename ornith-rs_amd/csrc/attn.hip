@@ -166,8 +166,8 @@ struct SdpaArgs {
 // and every value row -- is requested by the 16 wavefronts at once, in 16-byte pieces with
 // eight lanes to a 128-byte line, before anything is computed. The rows then pass through
 // LDS (keys as 64-channel panels with rows padded by 16 bytes to spread the banks; the values
-// take the same memory over once the scores are done). Rows past the last valid key are read
-// from the last one (in bounds) and never added.
+// take the same memory over once the scores are done). Rows past the last valid key are not
+// read, and the chains that would hold only such rows are not run.
 constexpr int SDPA_NT = 1024;
 constexpr int SDPA_KROW = 64 * 2 + 16;  // bytes of a staged 64-channel key row
 
@@ -248,15 +248,22 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
     }
     __builtin_amdgcn_sched_barrier(0);
   }
+  // Rows past the last valid key are neither requested nor staged (a short context leaves most
+  // of the block empty, and a request costs its slot in the compute unit's load path whether or
+  // not the line is cached); what LDS holds in their place is never added to anything.
+  // PREP: nor are the key rows of this call's positions, which come from their wavefronts.
+  auto key_row_staged = [&](int r) { return r < nvalid && !(PREP && b * ATT_KB + r >= offset); };
 #pragma unroll
   for (int c = 0; c < NKC; ++c)
 #pragma unroll
-    for (int i = 0; i < KPC; ++i)
-      kreg[c * KPC + i] = *reinterpret_cast<const u32x4*>(
-          kbase + (size_t)min(krow0 + KRS * i, nvalid - 1) * HD + c * KC + 8 * kpc);
+    for (int i = 0; i < KPC; ++i) {
+      const int r = krow0 + KRS * i;
+      if (key_row_staged(r)) kreg[c * KPC + i] = *reinterpret_cast<const u32x4*>(kbase + (size_t)r * HD + c * KC + 8 * kpc);
+    }
 #pragma unroll
   for (int u = 0; u < NLD; ++u) {
-    const int vr = min(row0 + RPU * u, nvalid - 1);
+    const int vr = row0 + RPU * u;
+    if (vr >= nvalid) continue;
     const bf16_t* src = vblk + (size_t)vr * HD;
     // a position of this call: its value row is still in the projection's output
     if (PREP && b * ATT_KB + vr >= offset)
@@ -275,8 +282,7 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
 #pragma unroll
     for (int i = 0; i < KPC; ++i) {
       const int dest = krow0 + KRS * i;
-      // PREP: the rows of this call's positions come from the wavefronts that make them
-      if (PREP && b * ATT_KB + dest >= offset && dest < nvalid) continue;
+      if (!key_row_staged(dest)) continue;
       *reinterpret_cast<u32x4*>(stage + c * (ATT_KB * KROW) + dest * KROW + 16 * kpc) = kreg[c * KPC + i];
     }
   if constexpr (PREP) {
@@ -308,8 +314,11 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
     }
   }
   __syncthreads();
-  const int key = tid & (ATT_KB - 1), grp = tid >> 8;  // four wavefronts a group
-  if (grp < NKC) {
+  // wavefront w takes panel w % 4 of keys [64 (w / 4), +64): a SIMD (wavefronts go round the four
+  // in order) then holds one panel of every key group, and the groups past the last valid key
+  // drop out of all four SIMDs alike
+  const int grp = wave & 3, key = (wave >> 2) * 64 + lane;
+  if (grp < NKC && (wave >> 2) * 64 < nvalid) {
     u32x4 kws[KC / 8];
 #pragma unroll
     for (int i = 0; i < KC / 8; ++i)
@@ -352,10 +361,12 @@ __global__ __launch_bounds__(SDPA_NT) __attribute__((amdgpu_waves_per_eu(4, 4)))
   // values: thread (channel, group of 64 keys) runs the chain over the group's valid keys
   bf16_t (*vst)[HD] = reinterpret_cast<bf16_t (*)[HD]>(stage);
 #pragma unroll
-  for (int u = 0; u < NLD; ++u) *reinterpret_cast<u32x4*>(&vst[row0 + RPU * u][8 * piece]) = vreg[u];
+  for (int u = 0; u < NLD; ++u)
+    if (row0 + RPU * u < nvalid) *reinterpret_cast<u32x4*>(&vst[row0 + RPU * u][8 * piece]) = vreg[u];
   __syncthreads();  // probabilities and value rows in place (the key panels were last read two barriers ago)
   const int ch = tid % HD, vg = tid / HD;
-  if (vg < NVB) {
+  if (vg < NVB && VB * vg >= nvalid) part[vg * HD + ch] = 0.f;  // a chain with no valid key
+  if (vg < NVB && VB * vg < nvalid) {
     const int prv = __float_as_int(pr[VB * vg + lane]);
     bf16_t vv[VB];
 #pragma unroll
