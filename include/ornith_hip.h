@@ -80,7 +80,8 @@ ORNITH_API int ornith_device_info(ornith_ctx* ctx, char* name, size_t name_len, 
  *               k-quant projections and the MoE experts run as matrix-core GEMMs instead of
  *               exact mat-vecs. The one switch that changes results (to bf16 rounding of the
  *               weights): prefill is outside the exact window in the reference as well.
- *   "kq_iters"  (ORNITH_KQ_ITERS, default 0 = chosen by shape; 1..8): output rows each
+ *   "kq_iters"  (ORNITH_KQ_ITERS, default 0 = chosen by the launch from its shape and from how
+ *               many of its workgroups a compute unit holds; 1..8): output rows each
  *               wavefront of the k-quant mat-vec walks, a tuning knob
  *   "gemm_duo"  (ORNITH_GEMM_DUO, default 1): the 256-row tile of the prefill GEMM runs with
  *               producer and consumer wavefronts (0: every wavefront dequantizes, then

@@ -310,11 +310,49 @@ int layout_segments(KqArgs& a) {
   return blocks;
 }
 
+// Workgroups of a kernel that one compute unit holds at once (its registers and LDS decide:
+// from five for one Q4_K activation row down to one for three or four Q6_K rows, whose lanes
+// keep 64 activations a row in registers). Asked of the runtime once per kernel.
+template <typename Kernel>
+int resident_workgroups(Kernel kernel) {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0) != hipSuccess || n < 1) {
+    (void)hipGetLastError();
+    n = 2;
+  }
+  return n;
+}
+
+// Rows each wavefront walks when the caller leaves it open (a.iters == 0): the fewest with
+// which the whole grid is resident at once, counting at most three workgroups a compute unit.
+// The kernels are bound by latency and vector-ALU issue, not by HBM: a grid larger than the
+// chip holds runs as two rounds of the same chain of latencies (a 9216 x 2048 Q6_K projection
+// of two rows: 9.9 us as 1152 workgroups where 512 fit, 8.6 us as 384; one workgroup too many
+// costs the same second round: 8192 + 4096 Q4_K rows of four activation rows take 19.0 us as
+// 342 + 171 workgroups where 512 fit, 15.8 us as 384), while rows beyond that only lengthen the
+// one round; and beyond three workgroups a compute unit the activations' conversion (and a norm
+// made in the head) is repeated for nothing.
+template <int LPR, int KS>
+int auto_iters(const ornith_ctx* ctx, const KqArgs& a, int grid_y, int resident) {
+  constexpr int rows_per_pass = (64 / LPR) * (4 / KS);
+  const long room = (long)ctx->compute_units * (resident < 3 ? resident : 3);
+  for (int iters = 1; iters < 8; ++iters) {
+    long blocks = 0;
+    for (int s = 0; s < a.nseg; ++s) blocks += (a.seg[s].O + rows_per_pass * iters - 1) / (rows_per_pass * iters);
+    if (blocks * grid_y <= room) return iters;
+  }
+  return 8;
+}
+
 template <int KIND, int LPR, int KS, int M, bool XF32, bool GATHER>
 int launch_one(ornith_ctx* ctx, KqArgs& a, int grid_y) {
+  static const int resident = resident_workgroups(kq_qmv_kernel<KIND, LPR, KS, M, XF32, GATHER>);
+  const int asked = a.iters;
+  if (!asked) a.iters = auto_iters<LPR, KS>(ctx, a, grid_y, resident);
   dim3 grid(layout_segments<LPR, KS>(a), grid_y, 1);
   hipLaunchKernelGGL((kq_qmv_kernel<KIND, LPR, KS, M, XF32, GATHER>), grid, dim3(256), 0,
                      ctx->stream, a);
+  a.iters = asked;
   ORN_LAUNCH_CHECK("kq_qmv_kernel");
   return ORNITH_OK;
 }
@@ -339,6 +377,8 @@ int launch_shape(ornith_ctx* ctx, KqArgs& a, int grid_y) {
 
 template <int KIND, int LPR, int M>
 int launch_pre(ornith_ctx* ctx, KqArgs& a) {
+  static const int resident = resident_workgroups(kq_qmv_kernel<KIND, LPR, 1, M, false, false, true>);
+  if (!a.iters) a.iters = auto_iters<LPR, 1>(ctx, a, 1, resident);
   dim3 grid(layout_segments<LPR, 1>(a), 1, 1);
   hipLaunchKernelGGL((kq_qmv_kernel<KIND, LPR, 1, M, false, false, true>), grid, dim3(256), 0, ctx->stream, a);
   ORN_LAUNCH_CHECK("kq_qmv_kernel<pre-norm>");
@@ -364,22 +404,11 @@ int launch_m(ornith_ctx* ctx, KqArgs& a, int M) {
   }
 }
 
-// rows each wavefront walks: the kernels are bound by VALU issue and by latency, not by
-// HBM, so the converted activations are amortised over as many rows as still leaves
-// about three workgroups per compute unit (measured optimum on 256 CUs for 0.4..55 MB).
-int pick_iters(const ornith_ctx* ctx, int kind, int K, long total_rows, int grid_y, int M = 1) {
-  if (const int forced = ornith_option_kq_iters()) return forced > 8 ? 8 : forced;
-  const int nch = (K >> 8) * (kind == ORNITH_Q4K ? 8 : 4);
-  const int lpr = nch >= 64 ? 64 : nch;
-  const int ks = nch > 64 ? 2 : 1;
-  const int rows_per_pass = (64 / lpr) * (4 / ks);  // rows a block covers per iteration
-  const long blocks_at_1 = (total_rows + rows_per_pass - 1) / rows_per_pass * grid_y;
-  // (three or four activation rows: twice the conversion work to spread, half the workgroups)
-  const long want = M >= 3 ? (long)ctx->compute_units * 3 / 2 : (long)ctx->compute_units * 3;
-  int iters = (int)(blocks_at_1 / want);
-  if (iters < 1) iters = 1;
-  if (iters > 8) iters = 8;
-  return iters;
+// rows each wavefront walks: the option's value when it is set, else 0 = left to the launch,
+// which knows its kernel (auto_iters)
+int pick_iters() {
+  const int forced = ornith_option_kq_iters();
+  return forced > 8 ? 8 : forced;
 }
 
 int check_matrix(const ornith_kmatrix* w, const char* who) {
@@ -452,17 +481,15 @@ int kq_qmv_multi_prenorm(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n
   // occupancy to the norm's own registers on top; they no longer do -- the prologue's registers
   // are dead before the row loop's peak -- and the launch saved is worth 0.4 % at depth 1 and 1.7 %
   // at depth 3 in same-box A/B runs, so every width takes the norm in its head now.)
-  long total = 0;
   for (int s = 0; s < n; ++s) {
     if (check_matrix(ws[s], "kq_qmv_prenorm")) return -1;
     if (ws[s]->E != 1 || ws[s]->kind != ws[0]->kind || ws[s]->K != ws[0]->K || !d_ys[s]) return -1;
-    total += ws[s]->O;
   }
   KqArgs a{};
   a.nseg = n;
   a.K = kPreN;
   a.y_bf16 = 1;
-  a.iters = pick_iters(ctx, ws[0]->kind, kPreN, total, 1, M);
+  a.iters = pick_iters();
   for (int s = 0; s < n; ++s) {
     a.seg[s].qs = (const uint8_t*)ws[s]->d_qs;
     a.seg[s].scales = (const uint8_t*)ws[s]->d_scales;
@@ -482,7 +509,6 @@ int ornith_kq_qmv_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n,
   ORN_REQUIRE(n >= 1 && n <= kMaxSeg, "kq_qmv: %d matrices in one launch (1..%d)", n, kMaxSeg);
   ORN_REQUIRE(M >= 1, "kq_qmv: M=%d", M);
   ORN_REQUIRE(((uintptr_t)d_x & 15) == 0, "kq_qmv: x must be 16-byte aligned");
-  long total = 0;
   for (int s = 0; s < n; ++s) {
     int rc = check_matrix(ws[s], "kq_qmv");
     if (rc) return rc;
@@ -490,7 +516,6 @@ int ornith_kq_qmv_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n,
     ORN_REQUIRE(ws[s]->kind == ws[0]->kind && ws[s]->K == ws[0]->K,
                 "kq_qmv: matrices fused into one launch must share format and width");
     ORN_REQUIRE(d_ys[s], "kq_qmv: null output");
-    total += ws[s]->O;
   }
   const int kind = ws[0]->kind, K = ws[0]->K;
   const size_t xs = ornith_dtype_size(x_dtype), ys = ornith_dtype_size(y_dtype);
@@ -498,7 +523,7 @@ int ornith_kq_qmv_multi(ornith_ctx* ctx, const ornith_kmatrix* const* ws, int n,
   a.nseg = n;
   a.K = K;
   a.y_bf16 = y_dtype == ORNITH_BF16;
-  a.iters = pick_iters(ctx, kind, K, total, 1, M < 4 ? M : 4);
+  a.iters = pick_iters();
   for (int m0 = 0; m0 < M; m0 += 4) {
     const int mw = M - m0 < 4 ? M - m0 : 4;
     a.x = (const char*)d_x + (size_t)m0 * K * xs;
@@ -551,7 +576,7 @@ int ornith_kq_gather_qmv(ornith_ctx* ctx, const ornith_kmatrix* w, const void* d
   a.x_rows = x_rows;
   a.K = w->K;
   a.y_bf16 = y_dtype == ORNITH_BF16;
-  a.iters = pick_iters(ctx, w->kind, w->K, w->O, rows);
+  a.iters = pick_iters();
   if (w->kind == ORNITH_Q4K)
     return x_dtype == ORNITH_F32 ? launch_shape<ORNITH_Q4K, 1, true, true>(ctx, a, rows)
                                  : launch_shape<ORNITH_Q4K, 1, false, true>(ctx, a, rows);
