@@ -577,6 +577,15 @@ def pair_marks(orn, ctx, model, np, n_layers, T):
            "down": {"workgroups": len(d), "starts_us_after_the_up_launch": round(float((t1 - t0) / 100.0), 2), "phases": [
                row("start", d[:, 0], t1), row("weight loads issued", d[:, 1], t1), row("activations loaded", d[:, 2], t1),
                row("sums done (wavefront 0)", d[:, 3], t1), row("after the barrier", d[:, 4], t1), row("end", d[:, 5], t1)]}}
+    if hasattr(lib, "ornith_debug_marks_down_waves"):
+        # per wavefront of the down launch's workgroups (j < k: routed slot j, j >= k: the shared expert)
+        wv = (C.c_longlong * (1024 * 32))()
+        lib.ornith_debug_marks_down_waves(wv)
+        w = np.frombuffer(wv, np.int64).reshape(1024, 32).astype(np.float64)[:len(d)]
+        nw = int((w[0, :16] > 0).sum())
+        res["down"]["by_wavefront_median_us"] = [
+            {"wavefront": j, "rows_in_registers": round(float(np.median(w[:, j] - t1) / 100.0), 2),
+             "sums_done": round(float(np.median(w[:, 16 + j] - t1) / 100.0), 2)} for j in range(nw)]
     print(json.dumps({"pair_marks": res}), flush=True)
 
 

@@ -63,9 +63,14 @@ struct UpArgs {
 #ifdef ORN_TIMING
 __device__ long long g_down_marks[1024][8];
 #define DOWN_MARK(i) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if ((threadIdx.x & 63) == 0 && (threadIdx.x >> 6) == (i >> 3) && bl__ < 1024) g_down_marks[bl__][i & 7] = wall_clock64(); } while (0)
+// every wavefront's own stamps: [0, 16) its rows in registers (it waits for them: a wait the
+// plain build does not have), [16, 32) its sums done
+__device__ long long g_down_wave_marks[1024][32];
+#define DOWN_WAVE_MARK(slot) do { const int bl__ = blockIdx.y * gridDim.x + blockIdx.x; if ((threadIdx.x & 63) == 0 && bl__ < 1024) g_down_wave_marks[bl__][(slot) * 16 + ((threadIdx.x >> 6) & 15)] = wall_clock64(); } while (0)
 #else
 #define UP_MARK(i)
 #define DOWN_MARK(i)
+#define DOWN_WAVE_MARK(slot)
 #endif
 
 // ROUTE: the routing is made in the head of the launch (a.gates) instead of read (a.inds)
@@ -279,6 +284,10 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
     if (lane < k) wj[lane] = a.normalize ? dm_rb(dm_bf2f(score_bits) / denom) : dm_bf2f(score_bits);
     if (lane == 0) gsig = dm_sigmoid_bf16(dm_bf2f(egate_bits));
   }
+#ifdef ORN_TIMING
+  __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0) with the other counters: the rows are here
+  DOWN_WAVE_MARK(0);
+#endif
 #pragma unroll
   for (int it = 0; it < ITERS; ++it) {
     if (SPLIT && shared && it != only) continue;
@@ -288,6 +297,7 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
     if (c == 0) yl[SPLIT && shared ? k : j][it * RPW + slot] = dm_rb(v);  // expert outputs are bf16 in the unfused path
   }
   DOWN_MARK(3);
+  DOWN_WAVE_MARK(1);
   __syncthreads();
   DOWN_MARK(4);
   const int col = threadIdx.x;
@@ -795,6 +805,9 @@ extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_up(long
 }
 extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_down(long long* out) {
   return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_down_marks), sizeof(long long) * 1024 * 8);
+}
+extern "C" __attribute__((visibility("default"))) int ornith_debug_marks_down_waves(long long* out) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_down_wave_marks), sizeof(long long) * 1024 * 32);
 }
 #endif
 
