@@ -668,7 +668,7 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
         }
         v = dm_rb(dm_wave_sum<64>(acc));
       } else {
-        v = dm_rb(dense_row_dot(wr, a.xn + (size_t)t * a.H, a.H, lane));
+        v = dm_rb(dense_row_dot<1>(wr, a.xn + (size_t)t * a.H, a.H, lane));
       }
       // the wavefront that made the projection turns it into the token's decay / beta at
       // once: the two chains of exp / log run side by side in different wavefronts instead of

@@ -111,17 +111,22 @@ struct FmtDense {
   using Mat = DenseMat;
   static __device__ __forceinline__ void dot2(const Mat& wg, const Mat& wu, size_t row, int K, const bf16_t* xr,
                                               int lane, float& g, float& u) {
-    g = dense_row_dot(wg.w + row * K, xr, K, lane);
-    u = dense_row_dot(wu.w + row * K, xr, K, lane);
+    const bf16_t* const rows[2] = {wg.w + row * K, wu.w + row * K};
+    float v[2];
+    dense_rows_dot<2, 4>(rows, xr, K, lane, v);
+    g = v[0];
+    u = v[1];
   }
   template <int NC>
   static __device__ __forceinline__ void dotn(const Mat& w, size_t row0, int c0, int O, int K, const bf16_t* xr,
                                               int lane, float (&v)[NC]) {
+    const bf16_t* rows[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       const int o = c0 + c < O ? c0 + c : O - 1;
-      v[c] = dense_row_dot(w.w + (row0 + o) * K, xr, K, lane);
+      rows[c] = w.w + (row0 + o) * K;
     }
+    dense_rows_dot<NC, 1>(rows, xr, K, lane, v);
   }
 };
 
@@ -214,18 +219,25 @@ __global__ __launch_bounds__(64 * (kA4MaxK + 1)) void moe_down_affine4_kernel(A4
   const int arow = shared ? a.T * k + t : t * k + j;
   const typename F::Mat w = shared ? a.sdown : a.down;
   const size_t row0 = shared ? 0 : (size_t)min(a.inds[t * k + j], (uint32_t)(a.E - 1)) * a.H;
-  if (j == 0) {
-    // the router weights of this token: denom = ((0+s0)+s1)..., w_j = bf16(s_j / denom)
-    const bf16_t* s = a.scores + (size_t)t * k;
-    float denom = 0.f;
-    if (a.normalize)
-      for (int i = 0; i < k; ++i) denom = dm_rb(dm_bf2f(s[i]) + denom);
-    if (lane < k) wj[lane] = a.normalize ? dm_rb(dm_bf2f(s[lane]) / denom) : dm_bf2f(s[lane]);
-    if (lane == 0) gsig = dm_sigmoid_bf16(dm_bf2f(a.egate[t]));
-  }
+  // the token's router scores (lane i < k holds score i) and shared-expert gate are asked for
+  // ahead of the rows and turned into the combine weights once the rows' sums are made: a
+  // loop of loads here, one score a trip to memory, held wavefront 0's rows back by all of them
+  const uint16_t score_bits = a.scores[(size_t)t * k + (lane < k ? lane : 0)];
+  const uint16_t egate_bits = a.egate[t];
   const bf16_t* xr = a.act + (size_t)arow * a.I;
   float v[kA4Cols];
   F::template dotn<kA4Cols>(w, row0, c0, a.H, a.I, xr, lane, v);
+  if (j == 0) {
+    // the router weights of this token: denom = ((0+s0)+s1)..., w_j = bf16(s_j / denom)
+    float denom = 0.f;
+    if (a.normalize) {
+#pragma unroll
+      for (int i = 0; i < kA4MaxK; ++i)
+        if (i < k) denom = dm_rb(dm_bf2f((bf16_t)__builtin_amdgcn_readlane((int)score_bits, i)) + denom);
+    }
+    if (lane < k) wj[lane] = a.normalize ? dm_rb(dm_bf2f(score_bits) / denom) : dm_bf2f(score_bits);
+    if (lane == 0) gsig = dm_sigmoid_bf16(dm_bf2f(egate_bits));
+  }
 #pragma unroll
   for (int c = 0; c < kA4Cols; ++c)
     if (lane == 0) yl[j][c] = dm_rb(v[c]);  // expert outputs are bf16 in the operator path
