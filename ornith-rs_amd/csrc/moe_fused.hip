@@ -331,37 +331,82 @@ struct RouterArgs {
                          // by every workgroup; workgroup 0 stores h and x
 };
 
-// one row of the 8-bit affine / dense mat-vec by one wavefront (the order of linear.hip)
+// One row of the 8-bit affine / dense mat-vec by one wavefront (the order of linear.hip): group
+// j of eight weights on lane j mod 64, a lane's groups in ascending order. The row is a few KB
+// that no earlier launch has touched: a lane asks for all of its groups at once (egate_issue),
+// ahead of the norm's arithmetic, and works them off when the normed row is there (egate_finish).
+// Up to kEgGroups groups a lane (K <= 2048); wider rows take the plain loop.
+constexpr int kEgGroups = 4;
+struct EgRegs {
+  uint4 w[kEgGroups];          // dense: eight bf16 weights; affine: .x .y the eight codes
+  bf16_t s[kEgGroups], b[kEgGroups];
+};
+__device__ __forceinline__ void egate_issue(const RouterArgs& a, int lane, EgRegs& g) {
+#pragma unroll
+  for (int u = 0; u < kEgGroups; ++u) {
+    const int j = lane + 64 * u;
+    if (j >= a.K / 8) continue;
+    if (a.eg_affine) {
+      const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint8_t*>(a.eg_w) + 8 * j);
+      g.w[u] = make_uint4(q.x, q.y, 0, 0);
+      g.s[u] = a.eg_s[j >> 3];
+      g.b[u] = a.eg_b[j >> 3];
+    } else {
+      g.w[u] = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(a.eg_w) + 8 * j);
+    }
+  }
+}
+__device__ __forceinline__ float egate_group(const RouterArgs& a, const uint4& wv, bf16_t sc, bf16_t bi, const uint4& xv,
+                                             float acc_lane) {
+  const float xs[8] = {dm_bf2f_lo(xv.x), dm_bf2f_hi(xv.x), dm_bf2f_lo(xv.y), dm_bf2f_hi(xv.y),
+                       dm_bf2f_lo(xv.z), dm_bf2f_hi(xv.z), dm_bf2f_lo(xv.w), dm_bf2f_hi(xv.w)};
+  if (a.eg_affine) {
+    const uint32_t qw[2] = {wv.x, wv.y};
+    float acc = 0.f, sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float qf = (float)((qw[i >> 2] >> (8 * (i & 3))) & 0xffu);
+      acc = dm_fma(xs[i], qf, acc);
+      sum = sum + xs[i];
+    }
+    float p = dm_bf2f(sc) * acc;
+    p = dm_fma(sum, dm_bf2f(bi), p);
+    return acc_lane + p;
+  }
+  acc_lane = dm_fma(dm_bf2f_lo(wv.x), xs[0], acc_lane);
+  acc_lane = dm_fma(dm_bf2f_hi(wv.x), xs[1], acc_lane);
+  acc_lane = dm_fma(dm_bf2f_lo(wv.y), xs[2], acc_lane);
+  acc_lane = dm_fma(dm_bf2f_hi(wv.y), xs[3], acc_lane);
+  acc_lane = dm_fma(dm_bf2f_lo(wv.z), xs[4], acc_lane);
+  acc_lane = dm_fma(dm_bf2f_hi(wv.z), xs[5], acc_lane);
+  acc_lane = dm_fma(dm_bf2f_lo(wv.w), xs[6], acc_lane);
+  acc_lane = dm_fma(dm_bf2f_hi(wv.w), xs[7], acc_lane);
+  return acc_lane;
+}
+__device__ __forceinline__ float egate_finish(const RouterArgs& a, const EgRegs& g, const bf16_t* xr, int lane) {
+  float acc_lane = 0.f;
+#pragma unroll
+  for (int u = 0; u < kEgGroups; ++u) {
+    const int j = lane + 64 * u;
+    if (j >= a.K / 8) continue;
+    acc_lane = egate_group(a, g.w[u], g.s[u], g.b[u], *reinterpret_cast<const uint4*>(xr + 8 * j), acc_lane);
+  }
+  return dm_wave_sum<64>(acc_lane);
+}
 __device__ __forceinline__ float egate_row_dot(const RouterArgs& a, const bf16_t* xr, int lane) {
   float acc_lane = 0.f;
   for (int j = lane; j < a.K / 8; j += 64) {
-    const uint4 xv = *reinterpret_cast<const uint4*>(xr + 8 * j);
-    const float xs[8] = {dm_bf2f_lo(xv.x), dm_bf2f_hi(xv.x), dm_bf2f_lo(xv.y), dm_bf2f_hi(xv.y),
-                         dm_bf2f_lo(xv.z), dm_bf2f_hi(xv.z), dm_bf2f_lo(xv.w), dm_bf2f_hi(xv.w)};
+    uint4 wv;
+    bf16_t sc = 0, bi = 0;
     if (a.eg_affine) {
       const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint8_t*>(a.eg_w) + 8 * j);
-      const uint32_t qw[2] = {q.x, q.y};
-      float acc = 0.f, sum = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float qf = (float)((qw[i >> 2] >> (8 * (i & 3))) & 0xffu);
-        acc = dm_fma(xs[i], qf, acc);
-        sum = sum + xs[i];
-      }
-      float p = dm_bf2f(a.eg_s[j >> 3]) * acc;
-      p = dm_fma(sum, dm_bf2f(a.eg_b[j >> 3]), p);
-      acc_lane = acc_lane + p;
+      wv = make_uint4(q.x, q.y, 0, 0);
+      sc = a.eg_s[j >> 3];
+      bi = a.eg_b[j >> 3];
     } else {
-      const uint4 wv = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(a.eg_w) + 8 * j);
-      acc_lane = dm_fma(dm_bf2f_lo(wv.x), xs[0], acc_lane);
-      acc_lane = dm_fma(dm_bf2f_hi(wv.x), xs[1], acc_lane);
-      acc_lane = dm_fma(dm_bf2f_lo(wv.y), xs[2], acc_lane);
-      acc_lane = dm_fma(dm_bf2f_hi(wv.y), xs[3], acc_lane);
-      acc_lane = dm_fma(dm_bf2f_lo(wv.z), xs[4], acc_lane);
-      acc_lane = dm_fma(dm_bf2f_hi(wv.z), xs[5], acc_lane);
-      acc_lane = dm_fma(dm_bf2f_lo(wv.w), xs[6], acc_lane);
-      acc_lane = dm_fma(dm_bf2f_hi(wv.w), xs[7], acc_lane);
+      wv = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(a.eg_w) + 8 * j);
     }
+    acc_lane = egate_group(a, wv, sc, bi, *reinterpret_cast<const uint4*>(xr + 8 * j), acc_lane);
   }
   return dm_wave_sum<64>(acc_lane);
 }
@@ -380,9 +425,16 @@ __global__ __launch_bounds__(256) void moe_router_kernel(const bf16_t* h_res, co
   __shared__ PreNormLds<M> pn;
   const bool pre = h_res != nullptr;
   if (blockIdx.x == gridDim.x - 1) {
-    if (pre) prenorm_rows<M>(a.pre, false, pn);
+    const bool narrow = a.K / 8 <= 64 * kEgGroups;
+    PreNormRegs<M> pg;
+    EgRegs eg;
+    if (pre) prenorm_issue<M>(a.pre, pg);
+    if (narrow && wave < M) egate_issue(a, lane, eg);
+    __builtin_amdgcn_sched_barrier(0);
+    if (pre) prenorm_finish<M>(a.pre, pg, false, pn);
     if (wave < M) {
-      const float e = egate_row_dot(a, pre ? &pn.xn[wave][0] : a.x + (size_t)wave * a.K, lane);
+      const bf16_t* xr = pre ? &pn.xn[wave][0] : a.x + (size_t)wave * a.K;
+      const float e = narrow ? egate_finish(a, eg, xr, lane) : egate_row_dot(a, xr, lane);
       if (lane == 0) a.egate[wave] = dm_f2bf(e);
     }
     return;
