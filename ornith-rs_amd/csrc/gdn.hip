@@ -529,6 +529,9 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
   const int n_conv = 3 * T, n_ab = a.wa ? 2 * T : 0;
   const bool early_conv = wave < n_conv && p.K == 4;
   const bool early_ab = wave >= n_conv && wave < n_conv + n_ab && a.H <= 2048;
+  // with more than 16 tasks (four rows: 12 + 8) a conv wavefront's second task is a projection:
+  // its operands go out now as well, into the registers a projection wavefront uses
+  const bool early_ab2 = !early_ab && wave + 16 >= n_conv && wave + 16 < n_conv + n_ab && a.H <= 2048;
   uint4 e_w8 = make_uint4(0, 0, 0, 0);
   uint32_t e_xv[4] = {0, 0, 0, 0};
   uint4 e_dw[4], e_dx[4];
@@ -544,8 +547,8 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
       e_xv[i] = *reinterpret_cast<const uint32_t*>(src + c0);
     }
   }
-  if (early_ab) {
-    const int u = wave - n_conv, which = u / T, t = u - which * T;
+  if (early_ab || early_ab2) {
+    const int u = (early_ab ? wave : wave + 16) - n_conv, which = u / T, t = u - which * T;
     const bf16_t* wr = (which == 0 ? a.wa : a.wb) + (size_t)hv * a.H;
     const bf16_t* xr = a.xn + (size_t)t * a.H;
 #pragma unroll
@@ -649,7 +652,7 @@ __global__ __launch_bounds__(1024) void gdn_step_kernel(StepArgs a) {
       const int u = task - n_conv, which = u / T, t = u - which * T;  // 0 a, 1 b
       const bf16_t* wr = (which == 0 ? a.wa : a.wb) + (size_t)hv * a.H;
       float v;
-      if (task == wave && early_ab) {
+      if ((task == wave && early_ab) || (task == wave + 16 && early_ab2)) {
         // dense_row_dot over the operands asked for at the start: the same chain, the same fold
         float acc = 0.f;
 #pragma unroll
