@@ -255,8 +255,24 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
   // the weights, and its conversion then runs under the weights' trip (loads return in issue
   // order: asked for behind the weights it was converted only after the last of them had arrived;
   // 0.5 us a pair at T = 2)
-  const void* xrow[1] = {a.act + (size_t)arow * a.I};
-  L.template load_x<false>(xrow, c);
+  // With fewer than 64 lanes a row the rows of a wavefront pass share their activations: a
+  // lane asks for one 16-byte piece of the row (one load instruction a wavefront where every
+  // lane fetching its own 64 or 128 bytes takes four or eight; 0.2 us a pair at T = 2, 0.4-0.5
+  // at T = 3 and 4) and LDS hands out the chunks once the piece is there.
+  constexpr int XROW = LPR * (KIND == ORNITH_Q4K ? 32 : 64);  // activations a row (== I)
+  constexpr bool X_VIA_LDS = LPR < 64;
+  constexpr int XP = X_VIA_LDS ? (XROW / 8 + 63) / 64 : 1;  // 16-byte pieces a lane
+  __shared__ __align__(16) bf16_t xs[X_VIA_LDS ? kMaxK + down_shared_waves<ITERS>() : 1][X_VIA_LDS ? XROW : 8];
+  const bf16_t* arow_p = a.act + (size_t)arow * a.I;
+  uint4 xpiece[XP];
+  if constexpr (X_VIA_LDS) {
+#pragma unroll
+    for (int p = 0; p < XP; ++p)
+      if (8 * (lane + 64 * p) < XROW) xpiece[p] = *reinterpret_cast<const uint4*>(arow_p + 8 * (lane + 64 * p));
+  } else {
+    const void* xrow[1] = {arow_p};
+    L.template load_x<false>(xrow, c);
+  }
   // likewise the token's router scores (lane i < k holds score i) and its shared-expert gate:
   // wavefront 0 turns them into the combine weights while its weight rows are on their way
   const uint16_t score_bits = a.scores[(size_t)t * k + (lane < k ? lane : 0)];
@@ -271,6 +287,14 @@ __global__ __launch_bounds__(64 * (kMaxK + down_shared_waves<ITERS>())) void moe
   }
   __builtin_amdgcn_sched_barrier(0);  // keep the weight loads ahead of everything that follows
   DOWN_MARK(1);
+  if constexpr (X_VIA_LDS) {
+    // (a wavefront reads back only what it wrote itself: its LDS accesses complete in order)
+#pragma unroll
+    for (int p = 0; p < XP; ++p)
+      if (8 * (lane + 64 * p) < XROW) *reinterpret_cast<uint4*>(&xs[j][8 * (lane + 64 * p)]) = xpiece[p];
+    const void* xrow[1] = {&xs[j][0]};
+    L.template load_x<false>(xrow, c);
+  }
   DOWN_MARK(2);
 
   if (j == 0) {
