@@ -54,7 +54,7 @@ EXPERT_BYTES = 2 * 589_824 + 860_160       # gate + up (Q4_K 512x2048) + down (Q
 # carried from that profile and labelled so.
 _KIB = 1024
 PROFILE_TRAFFIC = {
-    "pair": {"bytes": int(round(((9569.7 + 7095.1) * 2.0 + (36.2 + 8.0) * 1.0) * _KIB)), "algorithmic_bytes": 33_557_094,
+    "pair": {"bytes": int(round(((9565.6 + 7095.0) * 2.0 + (36.1 + 8.0) * 1.0) * _KIB)), "algorithmic_bytes": 33_557_094,
              "kernel": "moe_up_kernel<0, 64, 2, true> + moe_down_kernel<1, 8, 2> (T = 2, the router's picks)"},
     "up_alone": {"bytes": int(round((9865.3 * 2.0 + 36.0 * 1.0) * _KIB)), "algorithmic_bytes": 20_080_704,
                  "kernel": "moe_up_kernel<0, 64, 2, false> (T = 2, 17 experts)"},
