@@ -99,29 +99,33 @@ __global__ __launch_bounds__(RB) void radix_hist_kernel(const bf16_t* x, int neg
   if (tid < 256) table[(size_t)tid * nblk + blockIdx.x] = h[tid];
 }
 
-// in-place exclusive scan of m counters by one workgroup, in tiles of 1024 consecutive
-// counters (coalesced). Up to 64 tiles are fetched into registers before the first is
-// scanned, so the walk over the tiles never waits on memory. One barrier a tile: the
-// wavefront totals of consecutive tiles alternate between two LDS rows, and every thread keeps
-// the running total itself.
+// in-place exclusive scan of m counters (a multiple of 4, 16-byte aligned) by one workgroup, in
+// tiles of 4096 consecutive counters: a thread takes four neighbours as one 16-byte load, so a
+// 62 k table is 16 tiles (a barrier and a wavefront scan each; with a counter a thread it was
+// 61). All tiles are fetched into registers before the first is scanned, so the walk never
+// waits on memory. One barrier a tile: the wavefront totals of consecutive tiles alternate
+// between two LDS rows, and every thread keeps the running total itself. Integer sums: the
+// result does not depend on the grouping.
 __global__ __launch_bounds__(RB) void radix_scan_kernel(uint32_t* table, int m) {
-  constexpr int NW = RB / 64;
+  constexpr int NW = RB / 64, TILE = 4 * RB;
   __shared__ uint32_t wtot[2][NW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  constexpr int G = 64;
+  constexpr int G = 16;
   uint32_t carry = 0;
-  for (int t0 = 0; t0 * RB < m; t0 += G) {
-    uint32_t v[G];
+  for (int t0 = 0; t0 * TILE < m; t0 += G) {
+    uint4 v[G];
 #pragma unroll
     for (int t = 0; t < G; ++t) {
-      const int j = (t0 + t) * RB + tid;
-      v[t] = j < m ? table[j] : 0u;
+      const int j = (t0 + t) * TILE + 4 * tid;
+      v[t] = j < m ? *reinterpret_cast<const uint4*>(table + j) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int t = 0; t < G; ++t) {
-      if ((t0 + t) * RB >= m) break;
-      // inclusive scan inside the wavefront, then across the 16 wavefront totals
-      uint32_t x = v[t];
+      if ((t0 + t) * TILE >= m) break;
+      // the thread's four, inclusive scan of the sums inside the wavefront, then across the 16
+      // wavefront totals
+      const uint32_t p1 = v[t].x, p2 = p1 + v[t].y, p3 = p2 + v[t].z, own = p3 + v[t].w;
+      uint32_t x = own;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
         const uint32_t o = __shfl_up(x, d, 64);
@@ -136,8 +140,9 @@ __global__ __launch_bounds__(RB) void radix_scan_kernel(uint32_t* table, int m) 
         before += w < wave ? c : 0u;
         total += c;
       }
-      const int j = (t0 + t) * RB + tid;
-      if (j < m) table[j] = before + x - v[t];
+      const int j = (t0 + t) * TILE + 4 * tid;
+      const uint32_t b = before + x - own;
+      if (j < m) *reinterpret_cast<uint4*>(table + j) = make_uint4(b, b + p1, b + p2, b + p3);
       carry += total;
     }
     __syncthreads();  // (G is even: the next round starts on row 0 again, which tile G - 2 used)
