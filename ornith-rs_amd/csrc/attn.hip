@@ -588,37 +588,58 @@ __global__ __launch_bounds__(256) void sdpa_partial_many_kernel(SdpaArgs p) {
   }
 }
 
-// grid (Hq, T), HD threads: merge blocks ascending, divide, gate
+// grid (Hq, T), HD threads: merge blocks ascending, divide, gate.
+// Thread b fetches block b's maximum and sum (one load each for the whole row), every thread
+// asks for its channel's partial outputs of up to kMergeAhead blocks at once, and the block
+// weights exp(m_b - M) are made once (thread b) and shared through LDS; the sums over the blocks
+// stay one ascending fma chain per thread. (A loop that fetched the maxima one by one and then
+// eight blocks at a time was a dozen trips to memory for a 27-block row.)
+constexpr int kMergeAhead = 32;
 template <int HD>
 __global__ __launch_bounds__(HD) void sdpa_merge_kernel(SdpaArgs p) {
   const int h = blockIdx.x, t = blockIdx.y, d = threadIdx.x;
+  const int lane = d & 63, wave = d >> 6;
   const int offset = p.d_offset ? *p.d_offset : p.offset;
   const int last = min(offset + t, p.cap - 1);
   const int nb = last / ATT_KB + 1;
   const size_t pi = ((size_t)t * p.Hq + h) * p.nblk;
+  __shared__ float sw[kMergeAhead], sl[kMergeAhead];
+  __shared__ float red[HD / 64];
+  const bf16_t gate_bits = p.qg[((size_t)t * p.Hq + h) * 2 * HD + HD + d];
+  // the row's maximum: every thread over its blocks d, d + HD, ..., then over the workgroup
   float M = -DM_INF;
-  for (int b = 0; b < nb; ++b) M = p.part_m[pi + b] > M ? p.part_m[pi + b] : M;
+  for (int b = d; b < nb; b += HD) {
+    const float m = p.part_m[pi + b];
+    M = m > M ? m : M;
+  }
+  M = dm_wave_max<64>(M);
+  if (lane == 0) red[wave] = M;
+  __syncthreads();
+  M = red[0];
+#pragma unroll
+  for (int w = 1; w < HD / 64; ++w) M = red[w] > M ? red[w] : M;
   float L = 0.f, O = 0.f;
-  // eight blocks' partial sums are asked for together (the sums keep their ascending order)
-  for (int b0 = 0; b0 < nb; b0 += 8) {
-    float pm[8], pl[8], po[8];
+  for (int b0 = 0; b0 < nb; b0 += kMergeAhead) {
+    const int n = min(kMergeAhead, nb - b0);
+    float po[kMergeAhead];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int b = min(b0 + u, nb - 1);
-      pm[u] = p.part_m[pi + b];
-      pl[u] = p.part_l[pi + b];
-      po[u] = p.part_o[(pi + b) * HD + d];
+    for (int u = 0; u < kMergeAhead; ++u) po[u] = p.part_o[(pi + b0 + min(u, n - 1)) * HD + d];
+    __syncthreads();  // the previous round's weights have been read
+    if (d < n) {
+      sw[d] = dm_exp(p.part_m[pi + b0 + d] - M);
+      sl[d] = p.part_l[pi + b0 + d];
     }
+    __syncthreads();
 #pragma unroll
-    for (int u = 0; u < 8; ++u)
-      if (b0 + u < nb) {
-        const float w = dm_exp(pm[u] - M);
-        L = dm_fma(pl[u], w, L);
+    for (int u = 0; u < kMergeAhead; ++u)
+      if (u < n) {
+        const float w = sw[u];
+        L = dm_fma(sl[u], w, L);
         O = dm_fma(po[u], w, O);
       }
   }
   const float att = dm_rb(O / L);
-  const float g = dm_sigmoid_bf16(dm_bf2f(p.qg[((size_t)t * p.Hq + h) * 2 * HD + HD + d]));
+  const float g = dm_sigmoid_bf16(dm_bf2f(gate_bits));
   p.out[((size_t)t * p.Hq + h) * HD + d] = dm_f2bf(g * att);
 }
 
