@@ -354,10 +354,20 @@ __global__ __launch_bounds__(RB) void cat_scale_kernel(const bf16_t* lp, int n, 
   }
 }
 
-// w = isinf(m) ? (x == m) : exp(x - m), in place over x
-__global__ __launch_bounds__(RB) void cat_weights_kernel(float* x, int n, const float* pmax, int nch) {
+// w = isinf(m) ? (x == m) : exp(x - m), in place over x (m: the row maximum from the chunk
+// maxima), and in the same launch the chunk's scan_local_kernel<false> over those weights (the
+// weight is scanned from the register it was made in: same values, same order as a launch of
+// its own). `init`, when given, is the search's (first, last) pair, reset here by one thread.
+__global__ __launch_bounds__(RB) void cat_weights_scan_kernel(float* x, int n, const float* pmax, int nch,
+                                                              float* vloc, float* segoff, float* chunk_tot,
+                                                              uint32_t* init) {
   __shared__ float red[RB / 64];
+  __shared__ float seg[RB / 64], so[RB / 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i = blockIdx.x * RB + tid;
+  if (init && blockIdx.x == 0 && tid == 0) {
+    init[0] = 0xffffffffu;
+    init[1] = 0u;
+  }
   float m = -DM_INF;
   for (int c = tid; c < nch; c += RB) m = pmax[c] > m ? pmax[c] : m;
   m = dm_wave_max<64>(m);
@@ -366,10 +376,31 @@ __global__ __launch_bounds__(RB) void cat_weights_kernel(float* x, int n, const 
   m = red[0];
 #pragma unroll
   for (int w = 1; w < RB / 64; ++w) m = red[w] > m ? red[w] : m;
-  if (i >= n) return;
   const bool inf = m == DM_INF || m == -DM_INF;
-  const float v = x[i];
-  x[i] = inf ? (v == m ? 1.f : 0.f) : dm_exp(v - m);
+  float v = 0.f;
+  if (i < n) {
+    const float xv = x[i];
+    v = inf ? (xv == m ? 1.f : 0.f) : dm_exp(xv - m);
+    x[i] = v;
+  }
+#pragma unroll
+  for (int s = 1; s < 64; s <<= 1) {
+    const float o = __shfl_up(v, s, 64);
+    if (lane >= s) v = add_r<false>(v, o);
+  }
+  if (lane == 63) seg[wave] = v;
+  __syncthreads();
+  if (tid == 0) {
+    float off = 0.f;
+    for (int g = 0; g < RB / 64; ++g) {
+      so[g] = off;
+      off = add_r<false>(off, seg[g]);
+    }
+    chunk_tot[blockIdx.x] = off;
+  }
+  __syncthreads();
+  if (i < n) vloc[i] = v;
+  if (lane == 0) segoff[blockIdx.x * (RB / 64) + wave] = so[wave];
 }
 
 // u = min(float(bits) / 2^32, nextafter(1, 0)) * total; first index with cdf > u, last with w > 0
@@ -491,10 +522,8 @@ int categorical_impl(ornith_ctx* ctx, const bf16_t* lp, int V, double temp, uint
   float scale;
   memcpy(&scale, &u, 4);
   hipLaunchKernelGGL(cat_scale_kernel, dim3(nch), dim3(RB), 0, ctx->stream, lp, V, scale, x, pmax);
-  hipLaunchKernelGGL(cat_weights_kernel, dim3(nch), dim3(RB), 0, ctx->stream, x, V, pmax, nch);
-  hipLaunchKernelGGL(scan_local_kernel<false>, dim3(nch), dim3(RB), 0, ctx->stream, x, V, b.vloc,
-                     b.segoff, b.chunk_tot);
-  hipLaunchKernelGGL(cat_init_kernel, dim3(1), dim3(1), 0, ctx->stream, fl);
+  hipLaunchKernelGGL(cat_weights_scan_kernel, dim3(nch), dim3(RB), 0, ctx->stream, x, V, pmax, nch, b.vloc,
+                     b.segoff, b.chunk_tot, fl);
   hipLaunchKernelGGL(cat_search_kernel, dim3(nch), dim3(RB), 0, ctx->stream, b.vloc, b.segoff,
                      b.chunk_tot, x, V, nch, bits, fl, false);
   hipLaunchKernelGGL(cat_pick_kernel, dim3(1), dim3(1), 0, ctx->stream, fl, token);
@@ -522,9 +551,8 @@ int weights_impl(ornith_ctx* ctx, const bf16_t* lp, int V, double temp, float* w
   float scale;
   memcpy(&scale, &u, 4);
   hipLaunchKernelGGL(cat_scale_kernel, dim3(nch), dim3(RB), 0, ctx->stream, lp, V, scale, w, pmax);
-  hipLaunchKernelGGL(cat_weights_kernel, dim3(nch), dim3(RB), 0, ctx->stream, w, V, pmax, nch);
-  hipLaunchKernelGGL(scan_local_kernel<false>, dim3(nch), dim3(RB), 0, ctx->stream, w, V, b.vloc, b.segoff,
-                     b.chunk_tot);
+  hipLaunchKernelGGL(cat_weights_scan_kernel, dim3(nch), dim3(RB), 0, ctx->stream, w, V, pmax, nch, b.vloc,
+                     b.segoff, b.chunk_tot, (uint32_t*)nullptr);
   hipLaunchKernelGGL(weights_total_kernel, dim3(1), dim3(RB), 0, ctx->stream, b.chunk_tot, nch, w, V);
   ORN_LAUNCH_CHECK("sampler weights kernels");
   return ORNITH_OK;
