@@ -222,13 +222,12 @@ __device__ __forceinline__ float add_r(float a, float b) {
   return BF16 ? dm_rb(r) : r;
 }
 
-// stage 1: segment-local inclusive scans, segment offsets inside the chunk, chunk totals
+// stage 1: segment-local inclusive scans, segment offsets inside the chunk, chunk totals.
+// `v` is the calling thread's element (0 past the end); every thread of the workgroup calls.
 template <bool BF16>
-__global__ __launch_bounds__(RB) void scan_local_kernel(const float* in, int n, float* vloc,
-                                                        float* segoff, float* chunk_tot) {
+__device__ __forceinline__ void scan_local_body(float v, int n, float* vloc, float* segoff, float* chunk_tot) {
   __shared__ float seg[RB / 64], so[RB / 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i = blockIdx.x * RB + tid;
-  float v = i < n ? in[i] : 0.f;
 #pragma unroll
   for (int s = 1; s < 64; s <<= 1) {
     const float o = __shfl_up(v, s, 64);
@@ -247,6 +246,18 @@ __global__ __launch_bounds__(RB) void scan_local_kernel(const float* in, int n, 
   __syncthreads();
   if (i < n) vloc[i] = v;
   if (lane == 0) segoff[blockIdx.x * (RB / 64) + wave] = so[wave];
+}
+template <bool BF16>
+__global__ __launch_bounds__(RB) void scan_local_kernel(const float* in, int n, float* vloc,
+                                                        float* segoff, float* chunk_tot) {
+  const int i = blockIdx.x * RB + threadIdx.x;
+  scan_local_body<BF16>(i < n ? in[i] : 0.f, n, vloc, segoff, chunk_tot);
+}
+// the same over out[j] = bf16(exp(lp[S[j]])) made on the way in (the sorted probabilities of top-p)
+__global__ __launch_bounds__(RB) void gather_exp_scan_kernel(const bf16_t* lp, const uint32_t* S, int n,
+                                                             float* vloc, float* segoff, float* chunk_tot) {
+  const int j = blockIdx.x * RB + threadIdx.x;
+  scan_local_body<true>(j < n ? dm_rb(dm_exp(dm_bf2f(lp[S[j]]))) : 0.f, n, vloc, segoff, chunk_tot);
 }
 
 // base of this chunk (sum of the chunk totals before it, left to right) and the row total
@@ -314,12 +325,6 @@ __global__ __launch_bounds__(RB) void top_p_apply_kernel(const float* vloc, cons
   out[t] = c > thresh ? lp[t] : kNegInf;
 }
 
-// sorted_probs[j] = bf16(exp(lp[S[j]])), kept as float
-__global__ void gather_exp_kernel(const bf16_t* lp, const uint32_t* S, int n, float* out) {
-  const int j = blockIdx.x * blockDim.x + threadIdx.x;
-  if (j < n) out[j] = dm_rb(dm_exp(dm_bf2f(lp[S[j]])));
-}
-
 __global__ void widen_bf16_kernel(const bf16_t* in, int n, float* out) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) out[i] = dm_bf2f(in[i]);
@@ -362,7 +367,6 @@ __global__ __launch_bounds__(RB) void cat_weights_scan_kernel(float* x, int n, c
                                                               float* vloc, float* segoff, float* chunk_tot,
                                                               uint32_t* init) {
   __shared__ float red[RB / 64];
-  __shared__ float seg[RB / 64], so[RB / 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i = blockIdx.x * RB + tid;
   if (init && blockIdx.x == 0 && tid == 0) {
     init[0] = 0xffffffffu;
@@ -383,24 +387,7 @@ __global__ __launch_bounds__(RB) void cat_weights_scan_kernel(float* x, int n, c
     v = inf ? (xv == m ? 1.f : 0.f) : dm_exp(xv - m);
     x[i] = v;
   }
-#pragma unroll
-  for (int s = 1; s < 64; s <<= 1) {
-    const float o = __shfl_up(v, s, 64);
-    if (lane >= s) v = add_r<false>(v, o);
-  }
-  if (lane == 63) seg[wave] = v;
-  __syncthreads();
-  if (tid == 0) {
-    float off = 0.f;
-    for (int g = 0; g < RB / 64; ++g) {
-      so[g] = off;
-      off = add_r<false>(off, seg[g]);
-    }
-    chunk_tot[blockIdx.x] = off;
-  }
-  __syncthreads();
-  if (i < n) vloc[i] = v;
-  if (lane == 0) segoff[blockIdx.x * (RB / 64) + wave] = so[wave];
+  scan_local_body<false>(v, n, vloc, segoff, chunk_tot);
 }
 
 // u = min(float(bits) / 2^32, nextafter(1, 0)) * total; first index with cdf > u, last with w > 0
@@ -477,13 +464,12 @@ size_t scan_workspace(int n) { return (size_t)n * 4 + (size_t)nchunks(n) * (RB /
 int top_p_impl(ornith_ctx* ctx, const bf16_t* lp, int V, double top_p, bf16_t* out, ScratchCursor& sc) {
   const int nch = nchunks(V);
   uint32_t* S = sc.take<uint32_t>(V);
-  float* sp = sc.take<float>(V);
+  (void)sc.take<float>(V);  // (kept: the workspace layout callers size for)
   ScanBufs b = scan_bufs(sc, V);
   int rc = argsort_impl(ctx, lp, V, 0, S, sc);
   if (rc) return rc;
-  hipLaunchKernelGGL(gather_exp_kernel, dim3(nch), dim3(RB), 0, ctx->stream, lp, S, V, sp);
-  hipLaunchKernelGGL(scan_local_kernel<true>, dim3(nch), dim3(RB), 0, ctx->stream, sp, V, b.vloc,
-                     b.segoff, b.chunk_tot);
+  hipLaunchKernelGGL(gather_exp_scan_kernel, dim3(nch), dim3(RB), 0, ctx->stream, lp, S, V, b.vloc, b.segoff,
+                     b.chunk_tot);
   // weak-typed scalar: 1 - top_p rounded to the array's dtype
   const float t32 = (float)(1.0 - top_p);
   uint32_t u;
