@@ -333,9 +333,9 @@ int resident_workgroups(Kernel kernel) {
 // one round; and beyond three workgroups a compute unit the activations' conversion (and a norm
 // made in the head) is repeated for nothing.
 template <int LPR, int KS>
-int auto_iters(const ornith_ctx* ctx, const KqArgs& a, int grid_y, int resident) {
+int auto_iters(const ornith_ctx* ctx, const KqArgs& a, int grid_y, int resident, int most = 3) {
   constexpr int rows_per_pass = (64 / LPR) * (4 / KS);
-  const long room = (long)ctx->compute_units * (resident < 3 ? resident : 3);
+  const long room = (long)ctx->compute_units * (resident < most ? resident : most);
   for (int iters = 1; iters < 8; ++iters) {
     long blocks = 0;
     for (int s = 0; s < a.nseg; ++s) blocks += (a.seg[s].O + rows_per_pass * iters - 1) / (rows_per_pass * iters);
@@ -378,7 +378,9 @@ int launch_shape(ornith_ctx* ctx, KqArgs& a, int grid_y) {
 template <int KIND, int LPR, int M>
 int launch_pre(ornith_ctx* ctx, KqArgs& a) {
   static const int resident = resident_workgroups(kq_qmv_kernel<KIND, LPR, 1, M, false, false, true>);
-  if (!a.iters) a.iters = auto_iters<LPR, 1>(ctx, a, 1, resident);
+  // (with the norm in its head a Q6_K launch, whose lanes take 64 weights a pass, measures best
+  // at no more than two workgroups a compute unit: 9216 rows of one activation row 8.0 -> 7.4 us)
+  if (!a.iters) a.iters = auto_iters<LPR, 1>(ctx, a, 1, resident, KIND == ORNITH_Q6K ? 2 : 3);
   dim3 grid(layout_segments<LPR, 1>(a), 1, 1);
   hipLaunchKernelGGL((kq_qmv_kernel<KIND, LPR, 1, M, false, false, true>), grid, dim3(256), 0, ctx->stream, a);
   ORN_LAUNCH_CHECK("kq_qmv_kernel<pre-norm>");
