@@ -183,3 +183,52 @@ def test_errors_are_reported_not_fatal(orn, ctx):
         ctx.kq_qmv(w, dx, orn.F32, 1, dy, orn.F32)
     for b in (dx, dy): b.free()
     w.free()
+
+
+def test_launch_sizing_never_changes_bits(orn, ctx):
+    """The rows a wavefront walks (chosen by the launch from its kernel's residency, or forced
+    through the kq_iters option) only shape the grid: every output bit stays the same, for the
+    plain mat-vec and for the one that makes the layer's norm in its head, ragged row counts and
+    several matrices a launch included."""
+    import ctypes as C
+    rng = np.random.default_rng(77)
+    lib = orn.lib()
+    try:
+        for kind, K, Os in ((Q4K, 2048, (1000,)), (Q6K, 2048, (520, 36)), (Q4K, 4096, (300,)), (Q6K, 4096, (130,))):
+            ts = [util.make_kq(kind, rng, 1, O, K) for O in Os]
+            lins = [orn.Linear.kquant(ctx, kind, *t, O, K) for t, O in zip(ts, Os)]
+            for M in (1, 2, 3, 4):
+                x = util.bf16_normal(rng, (M, K))
+                dx = ctx.to_device(x)
+                ys = [ctx.alloc(M * O * 2) for O in Os]
+                got = {}
+                for it in (0, 1, 3, 8):
+                    orn.set_option("kq_iters", it)
+                    ctx.linear_matmul_multi(lins, dx, M, ys)
+                    got[it] = [y.download(np.uint16, (M * O,)) for y, O in zip(ys, Os)]
+                for it in (1, 3, 8):
+                    for a, b in zip(got[0], got[it]):
+                        assert np.array_equal(a, b), (kind, K, M, it)
+                if K != 2048:
+                    continue
+                # norm in the head of the launch
+                res, yv = util.bf16_normal(rng, (M, K)), util.bf16_normal(rng, (M, K))
+                wn = ctx.to_device(util.bf16_normal(rng, (K,)))
+                dres, dyv = ctx.to_device(res), ctx.to_device(yv)
+                h, nm = ctx.alloc(M * K * 2), ctx.alloc(M * K * 2)
+                n = len(Os)
+                wp = (C.c_void_p * n)(*[C.cast(C.pointer(l.s), C.c_void_p) for l in lins])
+                yp = (C.c_void_p * n)(*[y.ptr for y in ys])
+                got = {}
+                for it in (0, 1, 2, 5, 8):
+                    orn.set_option("kq_iters", it)
+                    rc = lib.ornith_add_rms_linear_multi(ctx.h, wp, n, dres.ptr, dyv.ptr, wn.ptr, C.c_float(1e-6), M,
+                                                         h.ptr, nm.ptr, yp)
+                    assert rc == 0
+                    got[it] = [y.download(np.uint16, (M * O,)) for y, O in zip(ys, Os)] + \
+                              [h.download(np.uint16, (M * K,)), nm.download(np.uint16, (M * K,))]
+                for it in (1, 2, 5, 8):
+                    for a, b in zip(got[0], got[it]):
+                        assert np.array_equal(a, b), ("prenorm", kind, M, it)
+    finally:
+        orn.set_option("kq_iters", 0)
